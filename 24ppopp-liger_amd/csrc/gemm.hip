@@ -1,0 +1,318 @@
+// gemm.hip -- hand-written GEMMs for gfx950: the cuBLAS calls of the reference's launch vector.
+//
+//   gemm_f16_generic   128x128x32 tiles, 4 waves (2x2), MFMA 16x16x32 f16 -> fp32, any shape / stride /
+//                      alignment, both weight layouts, optional fused epilogue.  Correctness workhorse
+//                      (edge tiles, decomposed sub-ranges, attention GEMMs, small models).
+//   gemm_f32_generic   64x64x16 VALU tiles for the fp32 plumbing configuration.
+// The large aligned prefill shapes are routed to the pipelined kernels in gemm_fast.hip.
+#include "gemm_common.cuh"
+
+namespace lg {
+
+int launch_gemm_fast_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t stream, bool* handled);
+
+// ---------------------------------------------------------------------------------------------------
+// fp16 generic kernel
+// ---------------------------------------------------------------------------------------------------
+constexpr int GB_M = 128, GB_N = 128, GB_K = 32;
+constexpr int GA_STRIDE = GB_K + 8;    // halves per row of the [rows][k] tiles (80 B: conflict-light b128 reads)
+constexpr int GBKN_STRIDE = GB_N + 8;  // halves per row of the [k][n] tile
+
+// loads 8 consecutive halves p[0..7] with per-element bound `valid` (0..8); ALIGNED -> one 16-byte load
+template <bool ALIGNED>
+__device__ __forceinline__ half8_t load8(const half_t* p, int valid) {
+    half8_t r = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (valid <= 0) return r;
+    if (ALIGNED) {
+        if (valid >= 8) return *reinterpret_cast<const half8_t*>(p);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+        if (i < valid) r[i] = p[i];
+    return r;
+}
+
+template <int WL, int EPI, bool ALIGNED>
+__global__ __launch_bounds__(256) void gemm_f16_generic(GemmArgs g) {
+    __shared__ __attribute__((aligned(16))) half_t As[GB_M * GA_STRIDE];
+    __shared__ __attribute__((aligned(16))) half_t Bs[(WL == W_NK) ? GB_N * GA_STRIDE : GB_K * GBKN_STRIDE];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;  // 2x2 waves, 64x64 each
+    const int m0 = blockIdx.y * GB_M, n0 = blockIdx.x * GB_N;
+    const half_t* X = g.X + (int64_t)blockIdx.z * g.strideX;
+    const half_t* W = g.W + (int64_t)blockIdx.z * g.strideW;
+    half_t* Y = g.Y + (int64_t)blockIdx.z * g.strideY;
+
+    float4_t acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    half8_t ra[2], rb[2];
+    auto gload = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int v = tid + 256 * i;
+            {   // X tile: 128 rows x 4 k-vectors
+                const int row = v >> 2, kv = v & 3;
+                const int m = m0 + row, k = k0 + kv * 8;
+                ra[i] = load8<ALIGNED>(X + (int64_t)m * g.ldx + k, (m < g.M) ? (g.K - k) : 0);
+            }
+            if (WL == W_NK) {  // W tile: 128 n-rows x 4 k-vectors
+                const int row = v >> 2, kv = v & 3;
+                const int n = n0 + row, k = k0 + kv * 8;
+                rb[i] = load8<ALIGNED>(W + (int64_t)n * g.ldw + k, (n < g.N) ? (g.K - k) : 0);
+            } else {           // W tile: 32 k-rows x 16 n-vectors
+                const int row = v >> 4, nv = v & 15;
+                const int k = k0 + row, n = n0 + nv * 8;
+                rb[i] = load8<ALIGNED>(W + (int64_t)k * g.ldw + n, (k < g.K) ? (g.N - n) : 0);
+            }
+        }
+    };
+    auto lstore = [&]() {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int v = tid + 256 * i;
+            *reinterpret_cast<half8_t*>(&As[(v >> 2) * GA_STRIDE + (v & 3) * 8]) = ra[i];
+            if (WL == W_NK)
+                *reinterpret_cast<half8_t*>(&Bs[(v >> 2) * GA_STRIDE + (v & 3) * 8]) = rb[i];
+            else
+                *reinterpret_cast<half8_t*>(&Bs[(v >> 4) * GBKN_STRIDE + (v & 15) * 8]) = rb[i];
+        }
+    };
+
+    const int l16 = lane & 15, lk = lane >> 4;  // row inside a 16-row MFMA tile, k-chunk (8 halves) index
+    gload(0);
+    for (int k0 = 0; k0 < g.K; k0 += GB_K) {
+        __syncthreads();  // previous tile fully consumed
+        lstore();
+        __syncthreads();
+        if (k0 + GB_K < g.K) gload(k0 + GB_K);
+
+        half8_t a[4], b[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            a[i] = *reinterpret_cast<const half8_t*>(&As[(wm * 64 + i * 16 + l16) * GA_STRIDE + lk * 8]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (WL == W_NK) {
+                b[j] = *reinterpret_cast<const half8_t*>(&Bs[(wn * 64 + j * 16 + l16) * GA_STRIDE + lk * 8]);
+            } else {
+                const int col = wn * 64 + j * 16 + 4 * (l16 & 3);
+                const int krow = lk * 8 + (l16 >> 2);
+                half4_t lo = lds_read_tr4(&Bs[krow * GBKN_STRIDE + col]);
+                half4_t hi = lds_read_tr4(&Bs[(krow + 4) * GBKN_STRIDE + col]);
+                b[j] = half8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            }
+        }
+        // operands swapped so that each lane owns 4 consecutive output columns (n) of one row (m):
+        //   acc[i][j][r] = Y[m_tile(i) + lane%16][n_tile(j) + 4*(lane/16) + r]
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[i][j] = mfma16(b[j], a[i], acc[i][j]);
+    }
+
+    const bool vec_ok = ALIGNED && (EPI == LG_EPI_BIAS_HEADS ? (g.epi.d % 4 == 0) : (g.ldy % 4 == 0));
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int m = m0 + wm * 64 + i * 16 + l16;
+            const int n = n0 + wn * 64 + j * 16 + 4 * lk;
+            switch (EPI) {
+                case LG_EPI_NONE: epilogue_store4<LG_EPI_NONE>(g, Y, m, n, acc[i][j], vec_ok); break;
+                case LG_EPI_BIAS: epilogue_store4<LG_EPI_BIAS>(g, Y, m, n, acc[i][j], vec_ok); break;
+                case LG_EPI_BIAS_GELU: epilogue_store4<LG_EPI_BIAS_GELU>(g, Y, m, n, acc[i][j], vec_ok); break;
+                default: epilogue_store4<LG_EPI_BIAS_HEADS>(g, Y, m, n, acc[i][j], vec_ok); break;
+            }
+        }
+}
+
+template <int WL, bool ALIGNED>
+static void launch_generic_epi(const GemmArgs& g, dim3 grid, hipStream_t stream) {
+    switch (g.epi.kind) {
+        case LG_EPI_NONE: hipLaunchKernelGGL((gemm_f16_generic<WL, LG_EPI_NONE, ALIGNED>), grid, dim3(256), 0, stream, g); break;
+        case LG_EPI_BIAS: hipLaunchKernelGGL((gemm_f16_generic<WL, LG_EPI_BIAS, ALIGNED>), grid, dim3(256), 0, stream, g); break;
+        case LG_EPI_BIAS_GELU: hipLaunchKernelGGL((gemm_f16_generic<WL, LG_EPI_BIAS_GELU, ALIGNED>), grid, dim3(256), 0, stream, g); break;
+        default: hipLaunchKernelGGL((gemm_f16_generic<WL, LG_EPI_BIAS_HEADS, ALIGNED>), grid, dim3(256), 0, stream, g); break;
+    }
+}
+
+static int gemm_f16_dispatch(GemmArgs g, int wlayout, int batch, hipStream_t stream) {
+    if (g.M == 0 || g.N == 0 || batch == 0) return LG_OK;
+    if (g.K == 0) { set_error("gemm: k == 0 is not supported"); return LG_ERR_INVALID; }
+    bool handled = false;
+    int rc = launch_gemm_fast_f16(g, wlayout, batch, stream, &handled);
+    if (handled) return rc;
+    const bool aligned = aligned16(g.X) && aligned16(g.W) && aligned16(g.Y) && (g.ldx % 8 == 0) && (g.ldw % 8 == 0) &&
+                         (g.strideX % 8 == 0) && (g.strideW % 8 == 0) && (g.strideY % 4 == 0) &&
+                         (g.K % 8 == 0) && (wlayout == W_NK || g.N % 8 == 0) &&
+                         (g.epi.kind == LG_EPI_BIAS_HEADS || (((uintptr_t)g.Y & 7u) == 0));
+    dim3 grid((g.N + GB_N - 1) / GB_N, (g.M + GB_M - 1) / GB_M, batch);
+    if (grid.y > 65535 || grid.z > 65535) { set_error("gemm: problem too large for the generic grid"); return LG_ERR_INVALID; }
+    if (wlayout == W_NK) {
+        if (aligned) launch_generic_epi<W_NK, true>(g, grid, stream); else launch_generic_epi<W_NK, false>(g, grid, stream);
+    } else {
+        if (aligned) launch_generic_epi<W_KN, true>(g, grid, stream); else launch_generic_epi<W_KN, false>(g, grid, stream);
+    }
+    return check_launch("gemm_f16");
+}
+
+// ---------------------------------------------------------------------------------------------------
+// fp32 generic kernel (plumbing configuration): 64x64x16 tiles, 256 threads, 4x4 outputs per thread
+// ---------------------------------------------------------------------------------------------------
+struct GemmArgsF32 {
+    int M, N, K;
+    const float* X; int64_t ldx; int64_t strideX;
+    const float* W; int64_t ldw; int64_t strideW;
+    float* Y;       int64_t ldy; int64_t strideY;
+};
+
+template <int WL>
+__global__ __launch_bounds__(256) void gemm_f32_generic(GemmArgsF32 g) {
+    __shared__ float As[16][64 + 4];  // [k][m]
+    __shared__ float Bs[16][64 + 4];  // [k][n]
+    const int tid = threadIdx.x;
+    const int tx = tid & 15, ty = tid >> 4;  // 16x16 threads, 4x4 outputs each
+    const int m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+    const float* X = g.X + (int64_t)blockIdx.z * g.strideX;
+    const float* W = g.W + (int64_t)blockIdx.z * g.strideW;
+    float* Y = g.Y + (int64_t)blockIdx.z * g.strideY;
+    float acc[4][4] = {};
+    for (int k0 = 0; k0 < g.K; k0 += 16) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int e = tid + 256 * i;  // 1024 elements per tile
+            {
+                const int r = e >> 4, kk = e & 15;  // X: 64 rows x 16 k, k fastest
+                const int m = m0 + r, k = k0 + kk;
+                As[kk][r] = (m < g.M && k < g.K) ? X[(int64_t)m * g.ldx + k] : 0.f;
+            }
+            if (WL == W_NK) {
+                const int r = e >> 4, kk = e & 15;
+                const int n = n0 + r, k = k0 + kk;
+                Bs[kk][r] = (n < g.N && k < g.K) ? W[(int64_t)n * g.ldw + k] : 0.f;
+            } else {
+                const int kk = e >> 6, c = e & 63;  // W: 16 k x 64 n, n fastest
+                const int n = n0 + c, k = k0 + kk;
+                Bs[kk][c] = (n < g.N && k < g.K) ? W[(int64_t)k * g.ldw + n] : 0.f;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < 16; ++kk) {
+            float a[4], b[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[i] = As[kk][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) b[j] = Bs[kk][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int m = m0 + ty * 4 + i, n = n0 + tx * 4 + j;
+            if (m < g.M && n < g.N) Y[(int64_t)m * g.ldy + n] = acc[i][j];
+        }
+}
+
+static int gemm_f32_dispatch(const GemmArgsF32& g, int wlayout, int batch, hipStream_t stream) {
+    if (g.M == 0 || g.N == 0 || batch == 0) return LG_OK;
+    if (g.K == 0) { set_error("gemm: k == 0 is not supported"); return LG_ERR_INVALID; }
+    dim3 grid((g.N + 63) / 64, (g.M + 63) / 64, batch);
+    if (grid.y > 65535 || grid.z > 65535) { set_error("gemm: problem too large for the generic grid"); return LG_ERR_INVALID; }
+    if (wlayout == W_NK) hipLaunchKernelGGL((gemm_f32_generic<W_NK>), grid, dim3(256), 0, stream, g);
+    else hipLaunchKernelGGL((gemm_f32_generic<W_KN>), grid, dim3(256), 0, stream, g);
+    return check_launch("gemm_f32");
+}
+
+// cuBLAS column-major arguments -> row-major problem; returns LG_OK or sets the error text
+static int check_blas_args(const char* what, int transa, int transb, int m, int n, int k, const void* A, int lda,
+                           const void* B, int ldb, const void* C, int ldc, int batch) {
+    if (transb != 0 || (transa != 0 && transa != 1)) { set_error("%s: only (N,N) and (T,N) are supported", what); return LG_ERR_INVALID; }
+    if (m < 0 || n < 0 || k < 0 || batch < 0) { set_error("%s: negative dimension", what); return LG_ERR_INVALID; }
+    if (m == 0 || n == 0 || batch == 0) return LG_OK;
+    if (!A || !B || !C) { set_error("%s: null pointer", what); return LG_ERR_INVALID; }
+    const int min_lda = transa ? k : m;
+    if (lda < (min_lda > 1 ? min_lda : 1) || ldb < (k > 1 ? k : 1) || ldc < (m > 1 ? m : 1)) {
+        set_error("%s: leading dimension too small (lda=%d ldb=%d ldc=%d for m=%d n=%d k=%d)", what, lda, ldb, ldc, m, n, k);
+        return LG_ERR_INVALID;
+    }
+    return LG_OK;
+}
+
+}  // namespace lg
+
+using namespace lg;
+
+extern "C" {
+
+int lg_gemm_strided_batched_f16(int transa, int transb, int m, int n, int k, const void* A, int lda, int64_t strideA,
+                                const void* B, int ldb, int64_t strideB, void* C, int ldc, int64_t strideC, int batch,
+                                void* stream) {
+    int rc = check_blas_args("gemm_f16", transa, transb, m, n, k, A, lda, B, ldb, C, ldc, batch);
+    if (rc) return rc;
+    GemmArgs g;
+    g.M = n; g.N = m; g.K = k;
+    g.X = (const half_t*)B; g.ldx = ldb; g.strideX = strideB;
+    g.W = (const half_t*)A; g.ldw = lda; g.strideW = strideA;
+    g.Y = (half_t*)C; g.ldy = ldc; g.strideY = strideC;
+    g.epi = Epilogue{LG_EPI_NONE, nullptr, 0, 0};
+    return gemm_f16_dispatch(g, transa ? W_NK : W_KN, batch, (hipStream_t)stream);
+}
+
+int lg_gemm_f16(int transa, int transb, int m, int n, int k, const void* A, int lda, const void* B, int ldb, void* C,
+                int ldc, void* stream) {
+    return lg_gemm_strided_batched_f16(transa, transb, m, n, k, A, lda, 0, B, ldb, 0, C, ldc, 0, 1, stream);
+}
+
+int lg_gemm_fused_f16(int transa, int m, int n, int k, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
+                      int epilogue, const void* bias, int epi_arg0, int epi_arg1, void* stream) {
+    int rc = check_blas_args("gemm_fused_f16", transa, 0, m, n, k, A, lda, B, ldb, C, ldc, 1);
+    if (rc) return rc;
+    if (epilogue < LG_EPI_NONE || epilogue > LG_EPI_BIAS_HEADS) { set_error("gemm_fused_f16: unknown epilogue %d", epilogue); return LG_ERR_INVALID; }
+    if (epilogue != LG_EPI_NONE && !bias) { set_error("gemm_fused_f16: epilogue needs a bias"); return LG_ERR_INVALID; }
+    if (epilogue == LG_EPI_BIAS_HEADS) {
+        const int seq = epi_arg0, d = epi_arg1;
+        if (seq <= 0 || d <= 0 || m % d != 0 || n % seq != 0 || d % 4 != 0) {
+            set_error("gemm_fused_f16: heads epilogue needs seq | tokens, size_per_head | features, size_per_head %% 4 == 0");
+            return LG_ERR_INVALID;
+        }
+    }
+    GemmArgs g;
+    g.M = n; g.N = m; g.K = k;
+    g.X = (const half_t*)B; g.ldx = ldb; g.strideX = 0;
+    g.W = (const half_t*)A; g.ldw = lda; g.strideW = 0;
+    g.Y = (half_t*)C; g.ldy = ldc; g.strideY = 0;
+    g.epi = Epilogue{epilogue, (const half_t*)bias, epi_arg0, epi_arg1};
+    return gemm_f16_dispatch(g, transa ? W_NK : W_KN, 1, (hipStream_t)stream);
+}
+
+int lg_gemm_strided_batched_f32(int transa, int transb, int m, int n, int k, const float* A, int lda, int64_t strideA,
+                                const float* B, int ldb, int64_t strideB, float* C, int ldc, int64_t strideC, int batch,
+                                void* stream) {
+    int rc = check_blas_args("gemm_f32", transa, transb, m, n, k, A, lda, B, ldb, C, ldc, batch);
+    if (rc) return rc;
+    GemmArgsF32 g;
+    g.M = n; g.N = m; g.K = k;
+    g.X = B; g.ldx = ldb; g.strideX = strideB;
+    g.W = A; g.ldw = lda; g.strideW = strideA;
+    g.Y = C; g.ldy = ldc; g.strideY = strideC;
+    return gemm_f32_dispatch(g, transa ? W_NK : W_KN, batch, (hipStream_t)stream);
+}
+
+int lg_gemm_f32(int transa, int transb, int m, int n, int k, const float* A, int lda, const float* B, int ldb, float* C,
+                int ldc, void* stream) {
+    return lg_gemm_strided_batched_f32(transa, transb, m, n, k, A, lda, 0, B, ldb, 0, C, ldc, 0, 1, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,77 @@
+// gemm_common.cuh -- operand descriptors, epilogues and MFMA helpers shared by the GEMM kernels.
+//
+// All kernels here use the row-major view of the reference's column-major cuBLAS calls:
+//     Y[M, N] (ldy) = X[M, K] (ldx) * W,      W given either as [K, N] (W_KN) or as [N, K] (W_NK).
+// M = tokens, N = output features, K = reduction.
+#pragma once
+#include "common.cuh"
+
+namespace lg {
+
+enum WLayout { W_KN = 0, W_NK = 1 };
+
+struct Epilogue {
+    int kind;             // LG_EPI_*
+    const half_t* bias;   // [N] or nullptr
+    int seq;              // LG_EPI_BIAS_HEADS: tokens per sequence
+    int d;                // LG_EPI_BIAS_HEADS: size_per_head
+};
+
+struct GemmArgs {
+    int M, N, K;
+    const half_t* X; int64_t ldx; int64_t strideX;
+    const half_t* W; int64_t ldw; int64_t strideW;
+    half_t* Y;       int64_t ldy; int64_t strideY;
+    Epilogue epi;
+};
+
+__device__ __forceinline__ float4_t mfma16(half8_t a, half8_t b, float4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+
+typedef __attribute__((address_space(3))) short4_t lds_short4_t;
+
+// Transposed 4x16 LDS read (gfx950 ds_read_b64_tr_b16).  Within each group of 16 lanes, source lane s
+// supplies the address of 4 consecutive halves; destination lane j = 4a + c receives, for r = 0..3, element c
+// of source lane (a + 4r).  With source lane s pointing at row (s/4), columns 4*(s%4).. of a [k][n] tile,
+// lane j ends up with tile[k0..k0+3][j]: four consecutive k for one n -- the MFMA operand order.
+__device__ __forceinline__ half4_t lds_read_tr4(const half_t* p) {
+    short4_t r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_t*)p);
+    return __builtin_bit_cast(half4_t, r);
+}
+
+// Applies the epilogue to 4 consecutive output columns n..n+3 of token row m and stores them.
+template <int EPI>
+__device__ __forceinline__ void epilogue_store4(const GemmArgs& g, half_t* Yb, int m, int n, float4_t acc, bool vec_ok) {
+    if (m >= g.M || n >= g.N) return;
+    float v[4] = {acc[0], acc[1], acc[2], acc[3]};
+    if (EPI != LG_EPI_NONE) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            if (n + r < g.N) v[r] += (float)g.epi.bias[n + r];
+    }
+    if (EPI == LG_EPI_BIAS_GELU) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[r] = gelu_tanh(v[r]);
+    }
+    int64_t base;
+    if (EPI == LG_EPI_BIAS_HEADS) {
+        // [M = b*seq + s, N = head*d + e]  ->  [b, head, s, e]
+        const int b = m / g.epi.seq, s = m % g.epi.seq;
+        const int head = n / g.epi.d, e = n % g.epi.d;
+        const int heads = g.N / g.epi.d;
+        base = (((int64_t)b * heads + head) * g.epi.seq + s) * (int64_t)g.epi.d + e;  // n..n+3 stay inside one head (d % 4 == 0)
+    } else {
+        base = (int64_t)m * g.ldy + n;
+    }
+    if (vec_ok && n + 3 < g.N) {
+        half4_t o = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+        *reinterpret_cast<half4_t*>(Yb + base) = o;
+    } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            if (n + r < g.N) Yb[base + r] = (half_t)v[r];
+    }
+}
+
+}  // namespace lg

@@ -1,0 +1,204 @@
+// runtime.hip -- error state, thin HIP runtime wrappers and synthetic-data fill kernels.
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "common.cuh"
+
+namespace lg {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+int check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        set_error("%s: %s", what, hipGetErrorString(e));
+        return LG_ERR_LAUNCH;
+    }
+    return LG_OK;
+}
+
+static int rt(hipError_t e, const char* what) {
+    if (e == hipSuccess) return LG_OK;
+    set_error("%s: %s", what, hipGetErrorString(e));
+    return LG_ERR_LAUNCH;
+}
+
+// ---- counter-based Irwin-Hall(8) generator; integer work + two rounded fp32 ops --------------------
+__device__ __forceinline__ uint64_t splitmix64(uint64_t z) {
+    z += 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+static uint64_t splitmix64_host(uint64_t z) {
+    z += 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+__device__ __forceinline__ uint32_t sum16x4(uint64_t r) {
+    return (uint32_t)(r & 0xffffu) + (uint32_t)((r >> 16) & 0xffffu) + (uint32_t)((r >> 32) & 0xffffu) +
+           (uint32_t)(r >> 48);
+}
+
+template <typename T>
+__global__ void fill_normal_kernel(T* out, int64_t n, uint64_t key, float mean, float stddev) {
+    const float inv_sigma = 0x1.3988e2p-16f;  // 1/sqrt(8*(65536^2-1)/12)
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        uint64_t a = splitmix64(key + 2ull * (uint64_t)i);
+        uint64_t b = splitmix64(key + 2ull * (uint64_t)i + 1ull);
+        int32_t s = (int32_t)(sum16x4(a) + sum16x4(b)) - 262140;
+        float z = __fmul_rn((float)s, inv_sigma);
+        float v = __fadd_rn(__fmul_rn(stddev, z), mean);  // never contracted into an FMA
+        out[i] = (T)v;
+    }
+}
+
+template <typename T>
+__global__ void fill_const_kernel(T* out, int64_t n, float value) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        out[i] = (T)value;
+}
+
+template <typename T>
+__global__ void fill_causal_mask_kernel(T* mask, int batch, int seq) {
+    const int64_t n = (int64_t)batch * seq * seq;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        const int col = (int)(i % seq);
+        const int row = (int)((i / seq) % seq);
+        mask[i] = (T)(col <= row ? 1.0f : 0.0f);
+    }
+}
+
+static int grid_for(int64_t n, int block) {
+    int64_t g = (n + block - 1) / block;
+    if (g > 65536) g = 65536;
+    if (g < 1) g = 1;
+    return (int)g;
+}
+
+template <typename T>
+static int fill_normal(T* out, int64_t n, uint64_t seed, uint64_t tensor_id, float mean, float stddev, void* stream) {
+    if (n < 0 || (n > 0 && !out)) { set_error("fill_normal: bad arguments"); return LG_ERR_INVALID; }
+    if (n == 0) return LG_OK;
+    const uint64_t key = splitmix64_host(seed * 0x100000001B3ull + tensor_id);
+    hipLaunchKernelGGL(fill_normal_kernel<T>, dim3(grid_for(n, 256)), dim3(256), 0, (hipStream_t)stream, out, n, key,
+                       mean, stddev);
+    return check_launch("fill_normal");
+}
+template <typename T>
+static int fill_const(T* out, int64_t n, float value, void* stream) {
+    if (n < 0 || (n > 0 && !out)) { set_error("fill_const: bad arguments"); return LG_ERR_INVALID; }
+    if (n == 0) return LG_OK;
+    hipLaunchKernelGGL(fill_const_kernel<T>, dim3(grid_for(n, 256)), dim3(256), 0, (hipStream_t)stream, out, n, value);
+    return check_launch("fill_const");
+}
+template <typename T>
+static int fill_causal(T* mask, int batch, int seq, void* stream) {
+    if (batch <= 0 || seq <= 0 || !mask) { set_error("fill_causal_mask: bad arguments"); return LG_ERR_INVALID; }
+    const int64_t n = (int64_t)batch * seq * seq;
+    hipLaunchKernelGGL(fill_causal_mask_kernel<T>, dim3(grid_for(n, 256)), dim3(256), 0, (hipStream_t)stream, mask,
+                       batch, seq);
+    return check_launch("fill_causal_mask");
+}
+
+}  // namespace lg
+
+using namespace lg;
+
+extern "C" {
+
+const char* lg_last_error(void) { return lg::g_err; }
+const char* lg_version(void) { return "liger-hip 0.1 (gfx950)"; }
+
+int lg_device_info(char* name, int name_len, int* cu_count, int* clock_khz, int* mem_clock_khz, int* bus_width_bits,
+                   size_t* total_mem) {
+    int dev = 0;
+    int rc = rt(hipGetDevice(&dev), "hipGetDevice");
+    if (rc) return rc;
+    hipDeviceProp_t p;
+    rc = rt(hipGetDeviceProperties(&p, dev), "hipGetDeviceProperties");
+    if (rc) return rc;
+    if (name && name_len > 0) {
+        strncpy(name, p.gcnArchName, (size_t)name_len - 1);
+        name[name_len - 1] = 0;
+    }
+    if (cu_count) *cu_count = p.multiProcessorCount;
+    if (clock_khz) *clock_khz = p.clockRate;
+    if (mem_clock_khz) *mem_clock_khz = p.memoryClockRate;
+    if (bus_width_bits) *bus_width_bits = p.memoryBusWidth;
+    if (total_mem) *total_mem = p.totalGlobalMem;
+    return LG_OK;
+}
+
+int lg_malloc(void** ptr, size_t bytes) { return rt(hipMalloc(ptr, bytes), "hipMalloc"); }
+int lg_free(void* ptr) { return rt(hipFree(ptr), "hipFree"); }
+int lg_memcpy_h2d(void* dst, const void* src, size_t bytes) {
+    return rt(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice), "hipMemcpy h2d");
+}
+int lg_memcpy_d2h(void* dst, const void* src, size_t bytes) {
+    return rt(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost), "hipMemcpy d2h");
+}
+int lg_memcpy_d2d_async(void* dst, const void* src, size_t bytes, void* stream) {
+    return rt(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, (hipStream_t)stream), "hipMemcpyAsync d2d");
+}
+int lg_memset_async(void* dst, int value, size_t bytes, void* stream) {
+    return rt(hipMemsetAsync(dst, value, bytes, (hipStream_t)stream), "hipMemsetAsync");
+}
+int lg_device_synchronize(void) { return rt(hipDeviceSynchronize(), "hipDeviceSynchronize"); }
+int lg_stream_create(void** stream) {
+    hipStream_t s = nullptr;
+    int rc = rt(hipStreamCreateWithFlags(&s, hipStreamNonBlocking), "hipStreamCreateWithFlags");
+    *stream = (void*)s;
+    return rc;
+}
+int lg_stream_destroy(void* stream) { return rt(hipStreamDestroy((hipStream_t)stream), "hipStreamDestroy"); }
+int lg_stream_synchronize(void* stream) { return rt(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize"); }
+int lg_stream_wait_event(void* stream, void* event) {
+    return rt(hipStreamWaitEvent((hipStream_t)stream, (hipEvent_t)event, 0), "hipStreamWaitEvent");
+}
+int lg_event_create(void** event) {
+    hipEvent_t e = nullptr;
+    int rc = rt(hipEventCreate(&e), "hipEventCreate");
+    *event = (void*)e;
+    return rc;
+}
+int lg_event_destroy(void* event) { return rt(hipEventDestroy((hipEvent_t)event), "hipEventDestroy"); }
+int lg_event_record(void* event, void* stream) {
+    return rt(hipEventRecord((hipEvent_t)event, (hipStream_t)stream), "hipEventRecord");
+}
+int lg_event_synchronize(void* event) { return rt(hipEventSynchronize((hipEvent_t)event), "hipEventSynchronize"); }
+int lg_event_query(void* event) {
+    hipError_t e = hipEventQuery((hipEvent_t)event);
+    if (e == hipSuccess) return LG_OK;
+    if (e == hipErrorNotReady) return 3;
+    return rt(e, "hipEventQuery");
+}
+int lg_event_elapsed_ms(float* ms, void* start, void* stop) {
+    return rt(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop), "hipEventElapsedTime");
+}
+
+int lg_fill_normal_f32(float* out, int64_t n, uint64_t seed, uint64_t tensor_id, float mean, float stddev, void* stream) {
+    return fill_normal<float>(out, n, seed, tensor_id, mean, stddev, stream);
+}
+int lg_fill_normal_f16(void* out, int64_t n, uint64_t seed, uint64_t tensor_id, float mean, float stddev, void* stream) {
+    return fill_normal<half_t>((half_t*)out, n, seed, tensor_id, mean, stddev, stream);
+}
+int lg_fill_const_f32(float* out, int64_t n, float value, void* stream) { return fill_const<float>(out, n, value, stream); }
+int lg_fill_const_f16(void* out, int64_t n, float value, void* stream) {
+    return fill_const<half_t>((half_t*)out, n, value, stream);
+}
+int lg_fill_causal_mask_f32(float* mask, int batch, int seq, void* stream) { return fill_causal<float>(mask, batch, seq, stream); }
+int lg_fill_causal_mask_f16(void* mask, int batch, int seq, void* stream) {
+    return fill_causal<half_t>((half_t*)mask, batch, seq, stream);
+}
+
+}  // extern "C"

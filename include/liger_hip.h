@@ -1,0 +1,179 @@
+/*
+ * liger_hip.h -- C ABI of the MI355X (gfx950) device library behind Liger's launch vector.
+ *
+ * Every entry point replaces one host launcher (or cuBLAS call) that the reference's adaptors in
+ * src/layer/func_wrapper.h bind into a FuncWrap.  Conventions, identical to the reference's:
+ *   - asynchronous: work is enqueued on `stream` (a hipStream_t passed as void*; NULL = default
+ *     stream) and the call returns without waiting;
+ *   - device pointers are owned by the caller; nothing here allocates or frees (lg_malloc & co.
+ *     below are thin runtime wrappers for host code that does not include HIP headers);
+ *   - several kernels work in place, exactly where the reference's do.
+ * Differences: every function returns an int status instead of asserting --
+ *   LG_OK, LG_ERR_INVALID (bad / unsupported shape or pointer), LG_ERR_LAUNCH (HIP error; text via
+ *   lg_last_error()).  A C++ wrapper that wants the reference's `void` signatures may ignore it.
+ * Suffix _f32 / _f16 = the reference's explicit float / half template instantiations; fp16 data is
+ * IEEE binary16 (`uint16_t` storage, passed as void*).  fp16 kernels compute in fp32 and round once.
+ */
+#ifndef LIGER_HIP_H
+#define LIGER_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LG_OK 0
+#define LG_ERR_INVALID 1
+#define LG_ERR_LAUNCH 2
+
+#define LG_F32 0
+#define LG_F16 1
+
+/* ---- library / device ------------------------------------------------------------------------ */
+const char* lg_last_error(void);
+const char* lg_version(void);
+/* Fills name (gcnArchName), CU count, engine clock (kHz), memory clock (kHz), bus width (bits),
+ * total device memory (bytes).  Used by the bench to print the roofline denominators. */
+int lg_device_info(char* name, int name_len, int* cu_count, int* clock_khz, int* mem_clock_khz,
+                   int* bus_width_bits, size_t* total_mem);
+
+/* ---- thin runtime wrappers (context.h:20-29, schedule.h:62-63,226-241, init.h:58-59,269-275) ---- */
+int lg_malloc(void** ptr, size_t bytes);
+int lg_free(void* ptr);
+int lg_memcpy_h2d(void* dst, const void* src, size_t bytes);
+int lg_memcpy_d2h(void* dst, const void* src, size_t bytes);
+int lg_memcpy_d2d_async(void* dst, const void* src, size_t bytes, void* stream);
+int lg_memset_async(void* dst, int value, size_t bytes, void* stream);
+int lg_device_synchronize(void);
+int lg_stream_create(void** stream);          /* non-blocking stream, default priority */
+int lg_stream_destroy(void* stream);
+int lg_stream_synchronize(void* stream);
+int lg_stream_wait_event(void* stream, void* event);
+int lg_event_create(void** event);            /* timing-enabled */
+int lg_event_destroy(void* event);
+int lg_event_record(void* event, void* stream);
+int lg_event_synchronize(void* event);
+int lg_event_query(void* event);              /* LG_OK when complete, LG_ERR_LAUNCH + 1 (=3) when not ready */
+int lg_event_elapsed_ms(float* ms, void* start, void* stop);
+
+/* Deterministic synthetic data on the device: out[i] = mean + stddev * z_i with z from the
+ * counter-based Irwin-Hall(8) generator keyed by (seed, tensor_id).  Bit-identical to the CPU
+ * oracle's generator.  No reference counterpart (the reference never initialises a buffer). */
+int lg_fill_normal_f32(float* out, int64_t n, uint64_t seed, uint64_t tensor_id, float mean, float stddev,
+                       void* stream);
+int lg_fill_normal_f16(void* out, int64_t n, uint64_t seed, uint64_t tensor_id, float mean, float stddev,
+                       void* stream);
+int lg_fill_const_f32(float* out, int64_t n, float value, void* stream);
+int lg_fill_const_f16(void* out, int64_t n, float value, void* stream);
+/* mask[b,i,j] = (j <= i) as 0/1 in T: the lower-triangular attr_mask for causal prefill */
+int lg_fill_causal_mask_f32(float* mask, int batch, int seq, void* stream);
+int lg_fill_causal_mask_f16(void* mask, int batch, int seq, void* stream);
+
+/* ---- element-wise / normalisation  (src/cuda/cuda_kernels.cuh:23-43) ---------------------------- */
+/* layer_norm<T>                        cuda_kernels.cuh:41-43, cuda_kernels.cu:510-532 */
+int lg_layer_norm_f32(const float* in, const float* gamma, const float* beta, float* out, int m, int n,
+                      void* stream);
+int lg_layer_norm_f16(const void* in, const void* gamma, const void* beta, void* out, int m, int n,
+                      void* stream);
+/* add_bias_act_kernelLauncher<T> (GELU-tanh, in place)   cuda_kernels.cuh:23-24, cuda_kernels.cu:302-319 */
+int lg_add_bias_act_f32(float* out, const float* bias, int m, int n, void* stream);
+int lg_add_bias_act_f16(void* out, const void* bias, int m, int n, void* stream);
+/* add_bias_input_layernorm_kernelLauncher<T> (in place on out)   cuda_kernels.cuh:26-30.
+ * Unlike the reference (n <= 1024 / 2048) any n is accepted. */
+int lg_add_bias_input_layernorm_f32(float* out, const float* input, const float* bias, const float* gamma,
+                                    const float* beta, int m, int n, void* stream);
+int lg_add_bias_input_layernorm_f16(void* out, const void* input, const void* bias, const void* gamma,
+                                    const void* beta, int m, int n, void* stream);
+/* add_bias_input_layernorm_2_kernelLauncher<T>   cuda_kernels.cuh:32-36 */
+int lg_add_bias_input_layernorm_2_f32(const float* input, const float* gamma, const float* beta,
+                                      const float* bias, float* output, float* norm_output, int m, int n,
+                                      void* stream);
+int lg_add_bias_input_layernorm_2_f16(const void* input, const void* gamma, const void* beta, const void* bias,
+                                      void* output, void* norm_output, int m, int n, void* stream);
+/* add_bias_input_kernelLauncher<T>   cuda_kernels.cuh:38-39 */
+int lg_add_bias_input_f32(float* output, const float* bias, const float* input, int m, int n, void* stream);
+int lg_add_bias_input_f16(void* output, const void* bias, const void* input, int m, int n, void* stream);
+
+/* ---- attention helpers  (src/cuda/attention_kernels.cuh:6-54) ------------------------------------ */
+/* add_QKV_bias_transpose_kernelLauncher<T>   attention_kernels.cuh:6-21.  Any head_num*size_per_head. */
+int lg_add_qkv_bias_transpose_f32(float* q_buf, float* k_buf, float* v_buf, const float* Q, const float* bias_Q,
+                                  const float* K, const float* bias_K, const float* V, const float* bias_V,
+                                  int batch, int seq, int head_num, int size_per_head, void* stream);
+int lg_add_qkv_bias_transpose_f16(void* q_buf, void* k_buf, void* v_buf, const void* Q, const void* bias_Q,
+                                  const void* K, const void* bias_K, const void* V, const void* bias_V,
+                                  int batch, int seq, int head_num, int size_per_head, void* stream);
+/* add_fusedQKV_bias_transpose_kernelLauncher<T>   attention_kernels.cuh:23-34 */
+int lg_add_fused_qkv_bias_transpose_f32(float* q_buf, float* k_buf, float* v_buf, const float* QKV,
+                                        const float* qkv_bias, int batch, int seq, int head_num,
+                                        int size_per_head, void* stream);
+int lg_add_fused_qkv_bias_transpose_f16(void* q_buf, void* k_buf, void* v_buf, const void* QKV,
+                                        const void* qkv_bias, int batch, int seq, int head_num,
+                                        int size_per_head, void* stream);
+/* attn_softmax_kernelLauncher<T> (in place)   attention_kernels.cuh:36-44.  Any seq (the reference needs
+ * seq <= 1024 fp32 / 2048 fp16).  `scalar` is passed as float and rounded to T as the reference stores it. */
+int lg_attn_softmax_f32(float* buffer, const float* attr_mask, int batch, int seq, int head_num, float scalar,
+                        void* stream);
+int lg_attn_softmax_f16(void* buffer, const void* attr_mask, int batch, int seq, int head_num, float scalar,
+                        void* stream);
+/* transpose_kernelLauncher<T>   attention_kernels.cuh:46-54.  No batch*head*seq % 4 restriction. */
+int lg_transpose_f32(float* dst, const float* src, int batch, int seq, int head_num, int size_per_head,
+                     void* stream);
+int lg_transpose_f16(void* dst, const void* src, int batch, int seq, int head_num, int size_per_head,
+                     void* stream);
+
+/* ---- GEMM  (cuBLAS as called through func_wrapper.h:20-37) --------------------------------------- */
+/* cublasGemmEx subset the reference uses: column-major, alpha = 1, beta = 0, C = op(A) * B.
+ * transa: 0 = N (linear.h:47-49,99-101), 1 = T (bert_layer.h:145-149); transb must be 0.
+ * In row-major words: C'[n, m] = B'[n, k] * W where W is A seen row-major: [k, m] (transa = 0) or
+ * [m, k] (transa = 1).  fp16: fp32 accumulate (the reference accumulates in fp16). */
+int lg_gemm_f32(int transa, int transb, int m, int n, int k, const float* A, int lda, const float* B, int ldb,
+                float* C, int ldc, void* stream);
+int lg_gemm_f16(int transa, int transb, int m, int n, int k, const void* A, int lda, const void* B, int ldb,
+                void* C, int ldc, void* stream);
+/* cublasGemmStridedBatchedEx, same subset.  func_wrapper.h:30-37 */
+int lg_gemm_strided_batched_f32(int transa, int transb, int m, int n, int k, const float* A, int lda,
+                                int64_t strideA, const float* B, int ldb, int64_t strideB, float* C, int ldc,
+                                int64_t strideC, int batch, void* stream);
+int lg_gemm_strided_batched_f16(int transa, int transb, int m, int n, int k, const void* A, int lda,
+                                int64_t strideA, const void* B, int ldb, int64_t strideB, void* C, int ldc,
+                                int64_t strideC, int batch, void* stream);
+
+/* Epilogues for lg_gemm_fused_f16 */
+#define LG_EPI_NONE 0
+#define LG_EPI_BIAS 1      /* C = acc + bias[m-index]                    */
+#define LG_EPI_BIAS_GELU 2 /* C = gelu_tanh(acc + bias[m-index])   == lg_gemm + lg_add_bias_act        */
+#define LG_EPI_BIAS_HEADS 3 /* C is written as [batch, head, seq, d] == lg_gemm + lg_add_qkv_bias_transpose
+                               for one of Q/K/V; needs seq and size_per_head in `epi_arg0/1`            */
+/* lg_gemm_f16 with a fused epilogue (the bias / GELU / head-transpose kernels that follow the GEMMs in
+ * the launch vector, bert_layer.h:54-56,139-142, folded into the GEMM's store).  No reference
+ * counterpart; results equal the two-kernel sequence up to one fp16 rounding. */
+int lg_gemm_fused_f16(int transa, int m, int n, int k, const void* A, int lda, const void* B, int ldb, void* C,
+                      int ldc, int epilogue, const void* bias, int epi_arg0, int epi_arg1, void* stream);
+
+/* ---- attention kernels with no reference counterpart --------------------------------------------- */
+/* Fused prefill attention over [B,h,S,d] buffers: out = softmax(q k^T * scalar + maskterm) v with the
+ * reference's softmax semantics (-10000 additive mask, +1e-6 in the denominator); replaces launch-vector
+ * entries 4,5,6 (and 7 when out_layout = 1).  causal != 0: implicit lower-triangular mask (attr_mask
+ * ignored, may be NULL); causal == 0: attr_mask [B,S,S] of 0/1 or NULL for all ones.
+ * out_layout 0: [B,h,S,d]; 1: [B,S,h,d] (= transpose-back fused).  size_per_head must be 64 or 128. */
+int lg_attn_prefill_f16(const void* q_buf, const void* k_buf, const void* v_buf, const void* attr_mask,
+                        void* out, int batch, int seq, int head_num, int size_per_head, float scalar,
+                        int causal, int out_layout, void* stream);
+/* Decode attention: q [B,h,d]; k_cache, v_cache [B,h,max_len,d] with `len` valid positions; out [B,h,d].
+ * workspace: float buffer of lg_attn_decode_workspace_bytes(...) bytes (split-KV partials), caller-owned. */
+size_t lg_attn_decode_workspace_bytes(int batch, int head_num, int size_per_head, int max_len);
+int lg_attn_decode_f16(const void* q, const void* k_cache, const void* v_cache, void* out, void* workspace,
+                       int batch, int head_num, int size_per_head, int len, int max_len, float scalar,
+                       void* stream);
+/* Adds the Q/K/V biases to one new token per sequence ([B, h*d] rows straight from the QKV GEMMs), writes
+ * q -> q_out [B,h,d] and appends k, v at position `pos` of the caches [B,h,max_len,d]. */
+int lg_kv_append_f16(void* q_out, void* k_cache, void* v_cache, const void* Q, const void* bias_Q, const void* K,
+                     const void* bias_K, const void* V, const void* bias_V, int batch, int head_num,
+                     int size_per_head, int pos, int max_len, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

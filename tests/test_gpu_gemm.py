@@ -1,0 +1,116 @@
+"""GPU parity for the GEMM entry points (cuBLAS-convention C ABI) against the CPU oracle."""
+import numpy as np
+import pytest
+
+from tests.conftest import max_rel_err
+
+pytestmark = pytest.mark.gpu
+SUF = {0: "f32", 1: "f16"}
+
+
+def rnd(po, n, tid, dt, std=1.0):
+    return po.fill_normal(n, 0, tid, 0.0, std, dt)
+
+
+# (tokens, out_features, k): aligned, ragged, tiny, skinny (decode-like)
+SHAPES = [(64, 256, 256), (128, 128, 32), (130, 136, 72), (1, 8, 8), (33, 70, 19), (32, 1024, 512), (257, 96, 1000),
+          (512, 384, 160)]
+
+
+@pytest.mark.parametrize("dt", [0, 1])
+@pytest.mark.parametrize("transa", [0, 1])
+@pytest.mark.parametrize("M,N,K", SHAPES)
+def test_gemm(dev, po, dt, transa, M, N, K):
+    """Row-major Y[M,N] = X[M,K] W, called as cublasGemmEx(transa, N, m=N, n=M, k=K, A=W, B=X, C=Y)."""
+    X = rnd(po, M * K, 30, dt).reshape(M, K)
+    W = rnd(po, K * N, 31, dt, 0.05).reshape(K, N)
+    ref = po.gemm(X, W, dt)
+    if transa:
+        A = np.ascontiguousarray(W.T)  # [N, K] row-major == column-major k x m with lda = K
+        lda = K
+    else:
+        A = W                          # [K, N] row-major == column-major m x k with lda = N
+        lda = N
+    dA, dX = dev.up(A, dt), dev.up(X, dt)
+    dY = dev.empty((M, N), dt)
+    dev.call("lg_gemm_" + SUF[dt], transa, 0, N, M, K, dA, lda, dX, K, dY, N)
+    assert max_rel_err(dev.down(dY), ref) < (2e-5 if dt == 0 else 2e-3)
+    # the oracle's own cuBLAS-convention entry must agree with its row-major one
+    C2 = np.zeros((M, N), dtype=np.float32)
+    po.gemm_ex(transa, 0, N, M, K, A, lda, X, K, C2, N, dt)
+    assert max_rel_err(C2, ref) < 1e-5
+
+
+@pytest.mark.parametrize("dt", [0, 1])
+def test_gemm_subrange_concatenation_is_exact(dev, po, dt):
+    """Decomposition invariant: computing column slices / row slices of Y separately (pointer offsets, same
+    leading dimensions) reproduces the full product bit for bit (the K order is unchanged)."""
+    M, N, K = 256, 512, 320
+    X = rnd(po, M * K, 32, dt).reshape(M, K)
+    W = rnd(po, K * N, 33, dt, 0.05).reshape(K, N)
+    dW, dX = dev.up(W, dt), dev.up(X, dt)
+    full = dev.empty((M, N), dt)
+    s = SUF[dt]
+    es = 4 if dt == 0 else 2
+    dev.call("lg_gemm_" + s, 0, 0, N, M, K, dW, N, dX, K, full, N)
+    # split output features (the reference's axis, utils.h:218-260) at 3/8
+    cols = dev.empty((M, N), dt)
+    n1 = N * 3 // 8
+    dev.call("lg_gemm_" + s, 0, 0, n1, M, K, dW, N, dX, K, cols, N)
+    dev.call("lg_gemm_" + s, 0, 0, N - n1, M, K, dW.data_ptr() + n1 * es, N, dX, K, cols.data_ptr() + n1 * es, N)
+    assert np.array_equal(dev.down(cols), dev.down(full))
+    # split token rows at 5/8
+    rows = dev.empty((M, N), dt)
+    m1 = M * 5 // 8
+    dev.call("lg_gemm_" + s, 0, 0, N, m1, K, dW, N, dX, K, rows, N)
+    dev.call("lg_gemm_" + s, 0, 0, N, M - m1, K, dW, N, dX.data_ptr() + m1 * K * es, K, rows.data_ptr() + m1 * N * es, N)
+    assert np.array_equal(dev.down(rows), dev.down(full))
+
+
+@pytest.mark.parametrize("dt", [0, 1])
+@pytest.mark.parametrize("B,h,S,d", [(2, 4, 32, 64), (1, 3, 80, 128), (1, 2, 33, 24)])
+def test_attention_batched_gemms(dev, po, dt, B, h, S, d):
+    """qk_gemm and qkv_gemm exactly as bert_layer.h:145-163 issues them."""
+    nb = B * h
+    q = rnd(po, nb * S * d, 34, dt).reshape(nb, S, d)
+    k = rnd(po, nb * S * d, 35, dt).reshape(nb, S, d)
+    v = rnd(po, nb * S * d, 36, dt).reshape(nb, S, d)
+    s = SUF[dt]
+    ref_qk = np.zeros((nb, S, S), dtype=np.float32)
+    po.gemm_strided_batched(1, 0, S, S, d, k, d, S * d, q, d, S * d, ref_qk, S, S * S, nb, dt)
+    assert max_rel_err(ref_qk, np.einsum("bqd,bkd->bqk", q.astype(np.float64), k.astype(np.float64))) < 2e-3
+    dq, dk, dv = dev.up(q, dt), dev.up(k, dt), dev.up(v, dt)
+    dqk = dev.empty((nb, S, S), dt)
+    dev.call("lg_gemm_strided_batched_" + s, 1, 0, S, S, d, dk, d, S * d, dq, d, S * d, dqk, S, S * S, nb)
+    assert max_rel_err(dev.down(dqk), ref_qk) < (2e-5 if dt == 0 else 2e-3)
+    p = np.abs(ref_qk) / np.abs(ref_qk).sum(-1, keepdims=True)
+    p = po.round_f16(p) if dt else p
+    ref_o = np.zeros((nb, S, d), dtype=np.float32)
+    po.gemm_strided_batched(0, 0, d, S, S, v, d, S * d, p, S, S * S, ref_o, d, S * d, nb, dt)
+    do = dev.empty((nb, S, d), dt)
+    dev.call("lg_gemm_strided_batched_" + s, 0, 0, d, S, S, dv, d, S * d, dev.up(p, dt), S, S * S, do, d, S * d, nb)
+    assert max_rel_err(dev.down(do), ref_o) < (2e-5 if dt == 0 else 2e-3)
+
+
+@pytest.mark.parametrize("transa", [0, 1])
+def test_gemm_fused_epilogues(dev, po, transa):
+    B, S, h, d, K = 2, 48, 4, 64, 192
+    M, N = B * S, h * d
+    X = rnd(po, M * K, 37, 1).reshape(M, K)
+    W = rnd(po, K * N, 38, 1, 0.05).reshape(K, N)
+    bias = rnd(po, N, 39, 1, 0.3)
+    A, lda = (np.ascontiguousarray(W.T), K) if transa else (W, N)
+    dA, dX, dB = dev.up(A, 1), dev.up(X, 1), dev.up(bias, 1)
+    # two-kernel references on the GPU itself and from the oracle
+    y = po.gemm(X, W, 1)
+    ref_gelu = po.add_bias_gelu(y.copy(), bias, 1)
+    out = dev.empty((M, N), 1)
+    dev.call("lg_gemm_fused_f16", transa, N, M, K, dA, lda, dX, K, out, N, dev.capi.EPI_BIAS_GELU, dB, 0, 0)
+    assert max_rel_err(dev.down(out), ref_gelu) < 4e-3
+    ref_heads, _, _ = po.add_qkv_bias_transpose(y, bias, y, bias, y, bias, B, S, h, d, 1)
+    out = dev.empty((B, h, S, d), 1)
+    dev.call("lg_gemm_fused_f16", transa, N, M, K, dA, lda, dX, K, out, N, dev.capi.EPI_BIAS_HEADS, dB, S, d)
+    assert max_rel_err(dev.down(out), ref_heads) < 2e-3
+    out = dev.empty((M, N), 1)
+    dev.call("lg_gemm_fused_f16", transa, N, M, K, dA, lda, dX, K, out, N, dev.capi.EPI_BIAS, dB, 0, 0)
+    assert max_rel_err(dev.down(out), po.round_f16(y + bias)) < 2e-3

@@ -1,0 +1,142 @@
+"""GPU parity: every reference-shaped kernel, called through the C ABI, against the CPU oracle.
+
+Tolerances: fp32 kernels 2e-5 relative to the largest reference magnitude; fp16 kernels must meet the
+stated bar (max rel err <= 1e-2) and are additionally held to a few fp16 ulps element-wise where the
+operation is a single rounding away from the oracle.
+"""
+import numpy as np
+import pytest
+
+from tests.conftest import max_rel_err
+
+pytestmark = pytest.mark.gpu
+
+F16_TOL = 1e-2   # the stated tolerance
+SUF = {0: "f32", 1: "f16"}
+
+
+def rnd(po, n, tid, dt, std=1.0, mean=0.0):
+    return po.fill_normal(n, 0, tid, mean, std, dt)
+
+
+def tol(dt):
+    return 2e-5 if dt == 0 else 2e-3
+
+
+@pytest.mark.parametrize("dt", [0, 1])
+@pytest.mark.parametrize("m,n", [(64, 256), (5, 12288), (3, 1000), (7, 37), (2, 16392), (1, 40000), (0, 64)])
+def test_layer_norm(dev, po, dt, m, n):
+    x = rnd(po, m * n, 1, dt).reshape(m, n) * 3 + 0.5
+    x = po.round_f16(x) if dt else x
+    g = rnd(po, n, 2, dt, 0.1, 1.0)
+    b = rnd(po, n, 3, dt, 0.1)
+    ref = po.layer_norm(x, g, b, dt)
+    dx, dg, db = dev.up(x, dt), dev.up(g, dt), dev.up(b, dt)
+    out = dev.empty((m, n), dt)
+    dev.call("lg_layer_norm_" + SUF[dt], dx, dg, db, out, m, n)
+    if m:
+        assert max_rel_err(dev.down(out), ref) < tol(dt)
+
+
+@pytest.mark.parametrize("dt", [0, 1])
+@pytest.mark.parametrize("m,n", [(64, 1024), (4, 16384), (3, 100), (5, 7)])
+def test_add_bias_gelu(dev, po, dt, m, n):
+    x = rnd(po, m * n, 4, dt, 2.0).reshape(m, n)
+    bias = rnd(po, n, 5, dt, 0.5)
+    ref = po.add_bias_gelu(x.copy(), bias, dt)
+    dx, dbias = dev.up(x, dt), dev.up(bias, dt)
+    dev.call("lg_add_bias_act_" + SUF[dt], dx, dbias, m, n)
+    assert max_rel_err(dev.down(dx), ref) < (2e-5 if dt == 0 else 4e-3)
+
+
+@pytest.mark.parametrize("dt", [0, 1])
+@pytest.mark.parametrize("m,n", [(16, 256), (4, 12288), (3, 1001)])
+def test_add_bias_input_layernorm_family(dev, po, dt, m, n):
+    out0 = rnd(po, m * n, 6, dt).reshape(m, n)
+    inp = rnd(po, m * n, 7, dt).reshape(m, n)
+    bias = rnd(po, n, 8, dt, 0.2)
+    g = rnd(po, n, 9, dt, 0.1, 1.0)
+    b = rnd(po, n, 10, dt, 0.1)
+    s = SUF[dt]
+    # add_bias_input_layernorm (in place)
+    ref = po.add_bias_input_layernorm(out0.copy(), inp, bias, g, b, dt)
+    d_out = dev.up(out0, dt)
+    dev.call("lg_add_bias_input_layernorm_" + s, d_out, dev.up(inp, dt), dev.up(bias, dt), dev.up(g, dt), dev.up(b, dt), m, n)
+    assert max_rel_err(dev.down(d_out), ref) < tol(dt)
+    # add_bias_input_layernorm_2 (two outputs)
+    ref_sum, ref_norm = po.add_bias_input_layernorm_2(inp, g, b, bias, out0.copy(), dt)
+    d_out = dev.up(out0, dt)
+    d_norm = dev.empty((m, n), dt)
+    dev.call("lg_add_bias_input_layernorm_2_" + s, dev.up(inp, dt), dev.up(g, dt), dev.up(b, dt), dev.up(bias, dt), d_out, d_norm, m, n)
+    assert max_rel_err(dev.down(d_out), ref_sum) < tol(dt)
+    assert max_rel_err(dev.down(d_norm), ref_norm) < tol(dt)
+    # add_bias_input
+    ref = po.add_bias_input(out0.copy(), bias, inp, dt)
+    d_out = dev.up(out0, dt)
+    dev.call("lg_add_bias_input_" + s, d_out, dev.up(bias, dt), dev.up(inp, dt), m, n)
+    assert max_rel_err(dev.down(d_out), ref) < tol(dt)
+
+
+@pytest.mark.parametrize("dt", [0, 1])
+@pytest.mark.parametrize("B,S,h,d", [(2, 32, 4, 64), (2, 8, 12, 128), (1, 5, 3, 20), (3, 7, 2, 9)])
+def test_qkv_bias_transpose_and_back(dev, po, dt, B, S, h, d):
+    n = h * d
+    M = B * S
+    Q, K, V = (rnd(po, M * n, 11 + i, dt).reshape(M, n) for i in range(3))
+    bq, bk, bv = (rnd(po, n, 14 + i, dt, 0.3) for i in range(3))
+    rq, rk, rv = po.add_qkv_bias_transpose(Q, bq, K, bk, V, bv, B, S, h, d, dt)
+    s = SUF[dt]
+    dq, dk, dv = (dev.empty((B, h, S, d), dt) for _ in range(3))
+    dev.call("lg_add_qkv_bias_transpose_" + s, dq, dk, dv, dev.up(Q, dt), dev.up(bq, dt), dev.up(K, dt), dev.up(bk, dt),
+             dev.up(V, dt), dev.up(bv, dt), B, S, h, d)
+    for got, ref in ((dq, rq), (dk, rk), (dv, rv)):
+        assert max_rel_err(dev.down(got), ref) < tol(dt)
+    # packed variant must give the same three buffers
+    QKV = np.ascontiguousarray(np.stack([Q, K, V], axis=1))  # [M, 3, n]
+    bias = np.concatenate([bq, bk, bv])
+    fq, fk, fv = (dev.empty((B, h, S, d), dt) for _ in range(3))
+    dev.call("lg_add_fused_qkv_bias_transpose_" + s, fq, fk, fv, dev.up(QKV, dt), dev.up(bias, dt), B, S, h, d)
+    for got, ref in ((fq, dq), (fk, dk), (fv, dv)):
+        assert np.array_equal(dev.down(got), dev.down(ref))
+    # transpose back: exact permutation
+    back = dev.empty((B, S, h, d), dt)
+    dev.call("lg_transpose_" + s, back, dq, B, S, h, d)
+    assert np.array_equal(dev.down(back), po.transpose(dev.down(dq)))
+
+
+@pytest.mark.parametrize("dt", [0, 1])
+@pytest.mark.parametrize("B,h,S,causal", [(2, 4, 32, False), (2, 3, 512, True), (1, 2, 77, True), (1, 1, 2048, False),
+                                           (1, 2, 4100, True)])
+def test_attn_softmax(dev, po, dt, B, h, S, causal):
+    qk = rnd(po, B * h * S * S, 20, dt, 4.0).reshape(B, h, S, S)
+    if causal:
+        mask = np.broadcast_to(np.tril(np.ones((S, S), dtype=np.float32)), (B, S, S)).copy()
+    else:
+        mask = (rnd(po, B * S * S, 21, 0).reshape(B, S, S) > -1.0).astype(np.float32)
+        mask[:, :, 0] = 1.0
+    scalar = 1.0 / np.sqrt(64.0)
+    ref = po.attn_softmax(qk.copy(), mask, scalar, dt)
+    d = dev.up(qk, dt)
+    dev.call("lg_attn_softmax_" + SUF[dt], d, dev.up(mask, dt), B, S, h, float(scalar))
+    got = dev.down(d)
+    # probabilities are <= 1; absolute error is the meaningful measure
+    assert np.abs(got - ref).max() < (2e-6 if dt == 0 else 2e-3)
+    assert np.abs(got.sum(-1) - 1.0).max() < (1e-4 if dt == 0 else 2e-2)
+
+
+def test_error_paths(dev):
+    x = dev.empty((4, 8), 0)
+    assert dev.call_rc("lg_layer_norm_f32", x, x, x, x, 4, 0) == dev.capi.ERR_INVALID
+    assert "bad shape" in dev.capi.last_error()
+    assert dev.call_rc("lg_add_bias_act_f32", x, x, -1, 8) == dev.capi.ERR_INVALID
+    assert dev.call_rc("lg_gemm_f32", 0, 1, 4, 4, 4, x, 4, x, 4, x, 4) == dev.capi.ERR_INVALID
+    assert dev.call_rc("lg_gemm_f32", 0, 0, 8, 4, 8, x, 4, x, 8, x, 8) == dev.capi.ERR_INVALID  # lda < m
+
+
+def test_fill_normal_matches_oracle_bitwise(dev, po):
+    for dt in (0, 1):
+        n = 100003
+        t = dev.empty((n,), dt)
+        dev.call("lg_fill_normal_" + SUF[dt], t, n, 7, 42, 0.25, 0.02)
+        ref = po.fill_normal(n, 7, 42, 0.25, 0.02, dt)
+        assert np.array_equal(dev.down(t), ref)
