@@ -266,7 +266,7 @@ int lg_gemm_strided_batched_f16(int transa, int transb, int m, int n, int k, con
     g.X = (const half_t*)B; g.ldx = ldb; g.strideX = strideB;
     g.W = (const half_t*)A; g.ldw = lda; g.strideW = strideA;
     g.Y = (half_t*)C; g.ldy = ldc; g.strideY = strideC;
-    g.epi = Epilogue{LG_EPI_NONE, nullptr, 0, 0};
+    g.epi = Epilogue{LG_EPI_NONE, nullptr, 0, 0, 0};
     return gemm_f16_dispatch(g, transa ? W_NK : W_KN, batch, (hipStream_t)stream);
 }
 
@@ -276,24 +276,28 @@ int lg_gemm_f16(int transa, int transb, int m, int n, int k, const void* A, int 
 }
 
 int lg_gemm_fused_f16(int transa, int m, int n, int k, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
-                      int epilogue, const void* bias, int epi_arg0, int epi_arg1, void* stream) {
-    int rc = check_blas_args("gemm_fused_f16", transa, 0, m, n, k, A, lda, B, ldb, C, ldc, 1);
+                      int epilogue, const void* bias, int epi_arg0, int epi_arg1, int epi_arg2, void* stream) {
+    int rc = check_blas_args("gemm_fused_f16", transa, 0, m, n, k, A, lda, B, ldb, C,
+                             epilogue == LG_EPI_BIAS_HEADS ? (m > 1 ? m : 1) : ldc, 1);
     if (rc) return rc;
     if (epilogue < LG_EPI_NONE || epilogue > LG_EPI_BIAS_HEADS) { set_error("gemm_fused_f16: unknown epilogue %d", epilogue); return LG_ERR_INVALID; }
     if (epilogue != LG_EPI_NONE && !bias) { set_error("gemm_fused_f16: epilogue needs a bias"); return LG_ERR_INVALID; }
     if (epilogue == LG_EPI_BIAS_HEADS) {
         const int seq = epi_arg0, d = epi_arg1;
-        if (seq <= 0 || d <= 0 || m % d != 0 || n % seq != 0 || d % 4 != 0) {
-            set_error("gemm_fused_f16: heads epilogue needs seq | tokens, size_per_head | features, size_per_head %% 4 == 0");
+        if (seq <= 0 || d <= 0 || m % d != 0 || n % seq != 0 || d % 4 != 0 || ldc < seq ||
+            (epi_arg2 != 0 && epi_arg2 < m / d)) {
+            set_error("gemm_fused_f16: heads epilogue needs seq | tokens, size_per_head | features, size_per_head %% 4 == 0, "
+                      "ldc (rows per head slot) >= seq, heads_total >= features / size_per_head");
             return LG_ERR_INVALID;
         }
+        if (epi_arg2 == 0) epi_arg2 = m / d;
     }
     GemmArgs g;
     g.M = n; g.N = m; g.K = k;
     g.X = (const half_t*)B; g.ldx = ldb; g.strideX = 0;
     g.W = (const half_t*)A; g.ldw = lda; g.strideW = 0;
     g.Y = (half_t*)C; g.ldy = ldc; g.strideY = 0;
-    g.epi = Epilogue{epilogue, (const half_t*)bias, epi_arg0, epi_arg1};
+    g.epi = Epilogue{epilogue, (const half_t*)bias, epi_arg0, epi_arg1, epi_arg2};
     return gemm_f16_dispatch(g, transa ? W_NK : W_KN, 1, (hipStream_t)stream);
 }
 

@@ -15,6 +15,7 @@ struct Epilogue {
     const half_t* bias;   // [N] or nullptr
     int seq;              // LG_EPI_BIAS_HEADS: tokens per sequence
     int d;                // LG_EPI_BIAS_HEADS: size_per_head
+    int heads_total;      // LG_EPI_BIAS_HEADS: heads per batch entry in the destination (>= N / d)
 };
 
 struct GemmArgs {
@@ -56,11 +57,10 @@ __device__ __forceinline__ void epilogue_store4(const GemmArgs& g, half_t* Yb, i
     }
     int64_t base;
     if (EPI == LG_EPI_BIAS_HEADS) {
-        // [M = b*seq + s, N = head*d + e]  ->  [b, head, s, e]
+        // [M = b*seq + s, N = head*d + e]  ->  [b, head, s, e] with ldy rows reserved per (b, head)
         const int b = m / g.epi.seq, s = m % g.epi.seq;
         const int head = n / g.epi.d, e = n % g.epi.d;
-        const int heads = g.N / g.epi.d;
-        base = (((int64_t)b * heads + head) * g.epi.seq + s) * (int64_t)g.epi.d + e;  // n..n+3 stay inside one head (d % 4 == 0)
+        base = (((int64_t)b * g.epi.heads_total + head) * g.ldy + s) * (int64_t)g.epi.d + e;  // n..n+3 stay inside one head (d % 4 == 0)
     } else {
         base = (int64_t)m * g.ldy + n;
     }

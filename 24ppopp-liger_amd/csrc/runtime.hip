@@ -51,13 +51,15 @@ __device__ __forceinline__ uint32_t sum16x4(uint64_t r) {
 
 template <typename T>
 __global__ void fill_normal_kernel(T* out, int64_t n, uint64_t key, float mean, float stddev) {
+#pragma clang fp contract(off)  // the multiply and the add must round separately to match the CPU generator
     const float inv_sigma = 0x1.3988e2p-16f;  // 1/sqrt(8*(65536^2-1)/12)
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
         uint64_t a = splitmix64(key + 2ull * (uint64_t)i);
         uint64_t b = splitmix64(key + 2ull * (uint64_t)i + 1ull);
         int32_t s = (int32_t)(sum16x4(a) + sum16x4(b)) - 262140;
-        float z = __fmul_rn((float)s, inv_sigma);
-        float v = __fadd_rn(__fmul_rn(stddev, z), mean);  // never contracted into an FMA
+        const float z = (float)s * inv_sigma;
+        float v = stddev * z;
+        v = v + mean;
         out[i] = (T)v;
     }
 }

@@ -1,0 +1,205 @@
+"""ctypes binding of lib/libliger_host.so: the C++ launch-vector runtime (layer assembly, Sample, Scheduler).
+
+No compute and no fallback here; importing raises if the native libraries are missing.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+from . import capi
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "lib", "libliger_host.so")
+
+POST_NORESID, PRE_LN_RESID = 0, 1
+POLICY_CLASSIC, POLICY_RESOURCE = 0, 1
+SPLIT_OUT_COLS, SPLIT_TOKEN_ROWS = 0, 1
+MODE_SEQUENTIAL, MODE_LIGER = 0, 1
+
+_i, _i64, _u64, _f, _d, _p = C.c_int, C.c_int64, C.c_uint64, C.c_float, C.c_double, C.c_void_p
+
+
+class Report(C.Structure):
+    _fields_ = [("records", _i), ("avg_latency_ms", _d), ("p99_latency_ms", _d), ("avg_gpu_ms", _d),
+                ("avg_queue_ms", _d), ("total_duration_ms", _d), ("throughput", _d), ("rounds", _i),
+                ("secondary_launches", _i), ("splits", _i), ("profile_misses", _i)]
+
+    def as_dict(self):
+        return {n: getattr(self, n) for n, _ in self._fields_}
+
+
+SIGNATURES = {
+    "lgh_first_error": (_i, [C.c_char_p, _i]),
+    "lgh_clear_error": (None, []),
+    "lgh_model_create": (_p, [_i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _u64]),
+    "lgh_model_kernels_per_layer": (_i, [_p, _i]),
+    "lgh_model_workspace_elems": (_i64, [_p, _i, _i]),
+    "lgh_model_stream": (_p, [_p]),
+    "lgh_model_param_count": (_i, [_p]),
+    "lgh_model_param_info": (_i, [_p, _i, C.c_char_p, _i, C.POINTER(_p), C.POINTER(_i64)]),
+    "lgh_model_describe": (_i, [_p, _i, _i, _i, C.c_char_p, _i]),
+    "lgh_model_run": (_i, [_p, _p, _p, _i, _i, _p, _p, _i]),
+    "lgh_model_run_decode": (_i, [_p, _p, _p, _i, _i, _i, _p, _p]),
+    "lgh_model_time_kernels": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, C.POINTER(_f), _i]),
+    "lgh_sched_create": (_p, [_p, _i, _f, _i, _i, _i, _i, _i, _i]),
+    "lgh_sched_profile": (_i, [_p, _i, _i, _i, _i, _i]),
+    "lgh_sched_profile_decode": (_i, [_p, _i, _i, _i]),
+    "lgh_sched_save": (_i, [_p, C.c_char_p, C.c_char_p]),
+    "lgh_sched_load": (_i, [_p, C.c_char_p, C.c_char_p]),
+    "lgh_sched_lookup": (_f, [_p, _i, _i, _i]),
+    "lgh_sched_sub_lookup": (_i, [_p, _i, _i, _i, C.POINTER(_f), _i]),
+    "lgh_sched_run_trace": (_i, [_p, _i, C.POINTER(_d), C.POINTER(_i), C.POINTER(_i), C.POINTER(_i), _i, C.POINTER(Report)]),
+    "lgh_summarize": (_i, [C.POINTER(_d), C.POINTER(_d), _i, _d, C.POINTER(Report)]),
+    "lgh_make_poisson_trace": (_i, [_d, _i, _i, _i, _i, _i, _i, _u64, C.POINTER(_d), C.POINTER(_i)]),
+}
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError("libliger_host.so is not built (expected at %s); run __graft_entry__.build()" % LIB_PATH)
+    lib = C.CDLL(LIB_PATH, mode=C.RTLD_GLOBAL)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+lib = _load()
+
+
+def first_error():
+    buf = C.create_string_buffer(1024)
+    code = lib.lgh_first_error(buf, 1024)
+    return code, buf.value.decode()
+
+
+def check(rc, what):
+    if rc != 0:
+        code, text = first_error()
+        lib.lgh_clear_error()
+        raise capi.LigerError("%s failed (%d): %s" % (what, code or rc, text))
+
+
+def summarize(cpu_ms, gpu_ms, total_duration_ms):
+    cpu = (C.c_double * len(cpu_ms))(*cpu_ms)
+    gpu = (C.c_double * len(gpu_ms))(*gpu_ms)
+    r = Report()
+    check(lib.lgh_summarize(cpu, gpu, len(cpu_ms), total_duration_ms, C.byref(r)), "lgh_summarize")
+    return r.as_dict()
+
+
+def make_poisson_trace(lam, n, batch, seq_lo, seq_hi, seq_round, n_decode, seed):
+    arr = (C.c_double * n)()
+    seq = (C.c_int * n)()
+    check(lib.lgh_make_poisson_trace(lam, n, batch, seq_lo, seq_hi, seq_round, n_decode, seed, arr, seq), "lgh_make_poisson_trace")
+    return [{"arrival_s": arr[i], "batch": batch, "seq": seq[i], "n_decode": n_decode} for i in range(n)]
+
+
+class Model:
+    """One tensor-parallel shard of a stack of encoder layers, assembled as launch vectors by the C++ runtime."""
+
+    def __init__(self, dtype, max_batch, max_seq, head_num, size_per_head, layer_num=1, world_size=1, ffn_inner=0,
+                 norm_mode=POST_NORESID, causal=False, fused=False, max_cache_len=0, factor=8, seed=0):
+        lib.lgh_clear_error()
+        self.h = lib.lgh_model_create(dtype, max_batch, max_seq, head_num, size_per_head, layer_num, world_size, ffn_inner,
+                                      norm_mode, int(causal), int(fused), max_cache_len, factor, seed)
+        if not self.h:
+            check(1, "lgh_model_create")
+        self.dtype = dtype
+        self.hidden = head_num * size_per_head
+        self.layer_num = layer_num
+        self.es = 2 if dtype == capi.F16 else 4
+
+    def kernels_per_layer(self, decode=False):
+        return lib.lgh_model_kernels_per_layer(self.h, int(decode))
+
+    def workspace_elems(self, batch, seq):
+        return lib.lgh_model_workspace_elems(self.h, batch, seq)
+
+    @property
+    def stream(self):
+        return lib.lgh_model_stream(self.h)
+
+    def params(self):
+        """name -> (device pointer, element count)"""
+        out = {}
+        for i in range(lib.lgh_model_param_count(self.h)):
+            name = C.create_string_buffer(128)
+            ptr, n = _p(), _i64()
+            check(lib.lgh_model_param_info(self.h, i, name, 128, C.byref(ptr), C.byref(n)), "lgh_model_param_info")
+            out[name.value.decode()] = (ptr.value, n.value)
+        return out
+
+    def download_params(self):
+        """name -> float32 numpy array (exact values of the device parameters)"""
+        res = {}
+        for name, (ptr, n) in self.params().items():
+            raw = np.empty(n, dtype=np.float16 if self.dtype == capi.F16 else np.float32)
+            capi.check(capi.lib.lg_memcpy_d2h(raw.ctypes.data_as(_p), _p(ptr), n * self.es), "lg_memcpy_d2h")
+            res[name] = raw.astype(np.float32)
+        return res
+
+    def describe(self, batch, seq, decode_past=-1):
+        buf = C.create_string_buffer(1 << 16)
+        n = lib.lgh_model_describe(self.h, batch, seq, decode_past, buf, 1 << 16)
+        if n < 0:
+            check(1, "lgh_model_describe")
+        rows = [ln.split("|") for ln in buf.value.decode().strip().split("\n") if ln]
+        return [{"idx": int(r[0]), "label": r[1], "type": r[2], "class": r[3]} for r in rows]
+
+    def run(self, input_ptr, output_ptr, batch, seq, workspace_ptr=None, stream=None, cache_slot=-1):
+        check(lib.lgh_model_run(self.h, input_ptr, output_ptr, batch, seq, workspace_ptr, stream, cache_slot), "lgh_model_run")
+
+    def run_decode(self, input_ptr, output_ptr, batch, past, cache_slot=0, workspace_ptr=None, stream=None):
+        check(lib.lgh_model_run_decode(self.h, input_ptr, output_ptr, batch, past, cache_slot, workspace_ptr, stream),
+              "lgh_model_run_decode")
+
+    def time_kernels(self, input_ptr, output_ptr, batch, seq, decode_past=-1, cache_slot=-1, iters=20, trials=3):
+        out = (C.c_float * 4096)()
+        n = lib.lgh_model_time_kernels(self.h, input_ptr, output_ptr, batch, seq, decode_past, cache_slot, iters, trials, out, 4096)
+        if n < 0:
+            check(1, "lgh_model_time_kernels")
+        return [out[i] for i in range(n)]
+
+
+class Scheduler:
+    def __init__(self, model, schedule_deep=6, contention_factor=0.8, policy=POLICY_RESOURCE, axis=SPLIT_OUT_COLS,
+                 seq_bucket=1, ignore_num=0, pool_count=0, ctx_batch=1):
+        lib.lgh_clear_error()
+        self.model = model
+        self.h = lib.lgh_sched_create(model.h, schedule_deep, contention_factor, policy, axis, seq_bucket, ignore_num,
+                                      pool_count, ctx_batch)
+        if not self.h:
+            check(1, "lgh_sched_create")
+
+    def profile(self, bs, seq_lo, seq_hi, seq_step=1, itr=20):
+        check(lib.lgh_sched_profile(self.h, bs, seq_lo, seq_hi, seq_step, itr), "lgh_sched_profile")
+
+    def profile_decode(self, bs, past, itr=20):
+        check(lib.lgh_sched_profile_decode(self.h, bs, past, itr), "lgh_sched_profile_decode")
+
+    def save(self, main_file, sub_file):
+        check(lib.lgh_sched_save(self.h, main_file.encode(), sub_file.encode()), "lgh_sched_save")
+
+    def load(self, main_file, sub_file):
+        check(lib.lgh_sched_load(self.h, main_file.encode(), sub_file.encode()), "lgh_sched_load")
+
+    def lookup(self, name, bs, seq):
+        return lib.lgh_sched_lookup(self.h, name, bs, seq)
+
+    def sub_lookup(self, name, bs, seq):
+        out = (C.c_float * 64)()
+        n = lib.lgh_sched_sub_lookup(self.h, name, bs, seq, out, 64)
+        return None if n < 0 else [out[i] for i in range(n)]
+
+    def run_trace(self, trace, mode):
+        n = len(trace)
+        arr = (C.c_double * n)(*[t["arrival_s"] for t in trace])
+        bs = (C.c_int * n)(*[t["batch"] for t in trace])
+        sq = (C.c_int * n)(*[t["seq"] for t in trace])
+        nd = (C.c_int * n)(*[t.get("n_decode", 0) for t in trace])
+        r = Report()
+        check(lib.lgh_sched_run_trace(self.h, mode, arr, bs, sq, nd, n, C.byref(r)), "lgh_sched_run_trace")
+        return r.as_dict()

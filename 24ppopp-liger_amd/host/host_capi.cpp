@@ -1,0 +1,320 @@
+// host_capi.cpp -- C API over the C++ launch-vector runtime, for drivers that are not C++ (tests, bench).
+//
+// A model handle owns a Bert_Model<T> (T = float or liger::half), its default workspace and two stream contexts.
+// Nothing here computes: vectors are built by the layer classes and launched entry by entry through FuncWrap.
+#include <cstring>
+#include <memory>
+#include <string>
+
+#include "layers.h"
+#include "scheduler.h"
+
+using namespace liger;
+
+namespace {
+
+struct SchedBase {
+    virtual ~SchedBase() {}
+    virtual void configure(int deep, float contention, int policy, int axis, int seq_bucket, int ignore_num) = 0;
+    virtual void make_pool(int count, int ctx_batch) = 0;
+    virtual void profile(int bs, int seq_lo, int seq_hi, int seq_step, int itr) = 0;
+    virtual void profile_decode(int bs, int past, int itr) = 0;
+    virtual bool save(const char* main_file, const char* sub_file) = 0;
+    virtual bool load(const char* main_file, const char* sub_file) = 0;
+    virtual Report run(int mode, const std::vector<TraceRequest>& trace, int* counters) = 0;
+    virtual float lookup(int name, int bs, int seq) = 0;
+    virtual int sub_lookup(int name, int bs, int seq, float* out, int cap) = 0;
+};
+
+struct ModelBase {
+    virtual SchedBase* make_scheduler() = 0;
+    virtual ~ModelBase() {}
+    virtual std::vector<FuncWrap> build(void* in, void* out, int batch, int seq, void* ws, int slot) = 0;
+    virtual std::vector<FuncWrap> build_decode(void* in, void* out, int batch, int past, int slot, void* ws) = 0;
+    virtual int64_t workspace_elems(int batch, int seq) = 0;
+    virtual int kernels_per_layer(bool decode) = 0;
+    virtual std::vector<ParamRef> params() = 0;
+    virtual size_t elem_size() = 0;
+    BertInitParam P;
+    StaticInitParam S;
+    void* default_ws = nullptr;
+    int64_t default_ws_elems = 0;
+    DynamicInitParam* stream0 = nullptr;
+    void *io_in = nullptr, *io_out = nullptr;  // default request buffers [max_batch * max_seq, hidden]
+};
+
+template <typename T>
+struct SchedT : SchedBase {
+    std::unique_ptr<Scheduler<T, Bert_Model<T>>> s;
+    void configure(int deep, float contention, int policy, int axis, int seq_bucket, int ignore_num) override {
+        s->schedule_deep = deep; s->contention_factor = contention; s->policy = (class_policy)policy;
+        s->axis = (split_axis)axis; s->seq_bucket = seq_bucket; s->ignore_num = ignore_num;
+    }
+    void make_pool(int count, int ctx_batch) override { s->make_pool(count, ctx_batch); }
+    void profile(int bs, int seq_lo, int seq_hi, int seq_step, int itr) override {
+        s->profile(bs, bs + 1, seq_lo, seq_hi + 1, "", "", seq_step, itr);
+    }
+    void profile_decode(int bs, int past, int itr) override { s->profile_decode(bs, past, itr); }
+    bool save(const char* a, const char* b) override {
+        return MainDictToFile(s->profiling_res_dict, a) && SubDictToFile(s->profiling_decompse_res_dict, b);
+    }
+    bool load(const char* a, const char* b) override {
+        return MainFileToDict(a, s->profiling_res_dict) && SubFileToDict(b, s->profiling_decompse_res_dict);
+    }
+    Report run(int mode, const std::vector<TraceRequest>& trace, int* counters) override {
+        s->reset_run();
+        s->serving(trace);
+        if (mode == 0) s->run_sequential(); else s->run_stream_sync();
+        Report r = s->output_recording(false);
+        if (counters) { counters[0] = s->rounds; counters[1] = s->secondary_launches; counters[2] = s->splits; counters[3] = s->profile_misses; }
+        return r;
+    }
+    float lookup(int name, int bs, int seq) override { return s->lookup(name, bs, seq); }
+    int sub_lookup(int name, int bs, int seq, float* out, int cap) override {
+        auto it = s->profiling_decompse_res_dict.find({name, bs, seq});
+        if (it == s->profiling_decompse_res_dict.end()) return -1;
+        int n = (int)it->second.size();
+        for (int i = 0; i < n && i < cap; ++i) out[i] = it->second[i];
+        return n;
+    }
+};
+
+template <typename T>
+struct ModelT : ModelBase {
+    std::unique_ptr<Bert_Model<T>> m;
+    SchedBase* make_scheduler() override {
+        auto* st = new SchedT<T>();
+        BertInitParam P2 = P;
+        st->s.reset(new Scheduler<T, Bert_Model<T>>(m.get(), P2, S, (T*)io_in, (T*)io_out));
+        return st;
+    }
+    std::vector<FuncWrap> build(void* in, void* out, int batch, int seq, void* ws, int slot) override {
+        return m->forward((T*)in, (T*)out, batch, seq, (T*)(ws ? ws : default_ws), slot);
+    }
+    std::vector<FuncWrap> build_decode(void* in, void* out, int batch, int past, int slot, void* ws) override {
+        return m->forward_decode((T*)in, (T*)out, batch, past, slot, (T*)(ws ? ws : default_ws));
+    }
+    int64_t workspace_elems(int batch, int seq) override { return m->workspace_elems(batch, seq); }
+    int kernels_per_layer(bool decode) override { return m->kernels_per_layer(decode); }
+    std::vector<ParamRef> params() override { return m->params(); }
+    size_t elem_size() override { return sizeof(T); }
+};
+
+int fail(const char* msg) {
+    if (error_state().code == 0) {
+        error_state().code = LG_ERR_INVALID;
+        error_state().text = msg;
+    }
+    return LG_ERR_INVALID;
+}
+
+bool shape_ok(ModelBase* mb, int batch, int seq) {
+    return mb && batch > 0 && seq > 0 && batch <= mb->P.max_batch_size && seq <= mb->P.max_seq_len;
+}
+
+}  // namespace
+
+extern "C" {
+
+int lgh_first_error(char* buf, int len) {
+    if (buf && len > 0) {
+        strncpy(buf, error_state().text.c_str(), (size_t)len - 1);
+        buf[len - 1] = 0;
+    }
+    return first_error();
+}
+void lgh_clear_error(void) { clear_error(); }
+
+// dtype 0 = fp32, 1 = fp16.  head_num and ffn_inner are GLOBAL sizes; the model holds the 1/world_size shard.
+void* lgh_model_create(int dtype, int max_batch, int max_seq, int head_num, int size_per_head, int layer_num, int world_size,
+                       int ffn_inner, int norm_mode, int causal, int fused, int max_cache_len, int factor, uint64_t seed) {
+    if (max_batch <= 0 || max_seq <= 0 || head_num <= 0 || size_per_head <= 0 || layer_num <= 0 || world_size <= 0 ||
+        head_num % world_size != 0 || (ffn_inner > 0 && ffn_inner % world_size != 0) || (dtype != 0 && dtype != 1)) {
+        fail("lgh_model_create: bad configuration");
+        return nullptr;
+    }
+    if (fused && dtype != 1) { fail("lgh_model_create: the fused assembly is fp16 only"); return nullptr; }
+    if (max_cache_len > 0 && !fused) { fail("lgh_model_create: the KV cache needs the fused assembly"); return nullptr; }
+    BertInitParam P(max_batch, max_seq, head_num, size_per_head, layer_num, 0, factor, 0);
+    P.ffn_inner = ffn_inner; P.norm_mode = norm_mode; P.causal = causal; P.fused = fused; P.max_cache_len = max_cache_len;
+    StaticInitParam S(0, world_size, dtype);
+    const int hidden = head_num * size_per_head;
+    ModelBase* mb = nullptr;
+    if (dtype == 1) {
+        auto* m = new ModelT<half>();
+        m->P = P; m->S = S;
+        m->default_ws_elems = Bert_Encoder<half>::workspace_elems(P, S, max_batch, max_seq);
+        m->default_ws = dev_alloc<half>(m->default_ws_elems);
+        m->m.reset(new Bert_Model<half>(P, S, hidden, hidden, (half*)m->default_ws));
+        m->m->init_weights(seed);
+        mb = m;
+    } else {
+        auto* m = new ModelT<float>();
+        m->P = P; m->S = S;
+        m->default_ws_elems = Bert_Encoder<float>::workspace_elems(P, S, max_batch, max_seq);
+        m->default_ws = dev_alloc<float>(m->default_ws_elems);
+        m->m.reset(new Bert_Model<float>(P, S, hidden, hidden, (float*)m->default_ws));
+        m->m->init_weights(seed);
+        mb = m;
+    }
+    mb->P.kernel_num = mb->kernels_per_layer(false);
+    mb->stream0 = new DynamicInitParam();
+    {
+        const size_t io_bytes = (size_t)max_batch * max_seq * hidden * mb->elem_size();
+        mb->io_in = dev_alloc<char>(io_bytes);
+        mb->io_out = dev_alloc<char>(io_bytes);
+        if (dtype == 1) dev_fill_normal((half*)mb->io_in, (int64_t)(io_bytes / 2), seed, 7, 0.f, 1.f);
+        else dev_fill_normal((float*)mb->io_in, (int64_t)(io_bytes / 4), seed, 7, 0.f, 1.f);
+        note_status(lg_device_synchronize(), "lg_device_synchronize");
+    }
+    if (first_error()) return nullptr;
+    return mb;
+}
+
+int lgh_model_kernels_per_layer(void* model, int decode) { return model ? ((ModelBase*)model)->kernels_per_layer(decode != 0) : -1; }
+int64_t lgh_model_workspace_elems(void* model, int batch, int seq) { return model ? ((ModelBase*)model)->workspace_elems(batch, seq) : -1; }
+void* lgh_model_stream(void* model) { return model ? ((ModelBase*)model)->stream0->stream : nullptr; }
+
+int lgh_model_param_count(void* model) { return model ? (int)((ModelBase*)model)->params().size() : -1; }
+int lgh_model_param_info(void* model, int idx, char* name, int name_len, void** ptr, int64_t* elems) {
+    if (!model) return fail("lgh_model_param_info: null model");
+    auto ps = ((ModelBase*)model)->params();
+    if (idx < 0 || idx >= (int)ps.size()) return fail("lgh_model_param_info: index out of range");
+    if (name && name_len > 0) { strncpy(name, ps[idx].name.c_str(), (size_t)name_len - 1); name[name_len - 1] = 0; }
+    if (ptr) *ptr = ps[idx].ptr;
+    if (elems) *elems = ps[idx].elems;
+    return LG_OK;
+}
+
+// Writes "idx|label|type|class\n" per entry of the vector forward() (or forward_decode()) would return.
+int lgh_model_describe(void* model, int batch, int seq, int decode_past, char* buf, int len) {
+    ModelBase* mb = (ModelBase*)model;
+    if (!shape_ok(mb, batch, decode_past >= 0 ? 1 : seq)) return fail("lgh_model_describe: bad shape");
+    std::vector<FuncWrap> v = decode_past >= 0 ? mb->build_decode(mb->default_ws, mb->default_ws, batch, decode_past, 0, nullptr)
+                                               : mb->build(mb->default_ws, mb->default_ws, batch, seq, nullptr, -1);
+    std::string s;
+    const char* tn[3] = {"COMMUNICATION", "COMPUTATION", "GEMM"};
+    const char* cn[3] = {"MFMA_BOUND", "HBM_BOUND", "LINK_BOUND"};
+    for (size_t i = 0; i < v.size(); ++i)
+        s += std::to_string(i) + "|" + v[i].label + "|" + tn[v[i].type] + "|" + cn[v[i].rclass] + "\n";
+    if (buf && len > 0) { strncpy(buf, s.c_str(), (size_t)len - 1); buf[len - 1] = 0; }
+    return (int)v.size();
+}
+
+// Builds the launch vector and launches every entry in order on `stream` (NULL -> the model's own stream).
+// Does not synchronise.  cache_slot >= 0 routes K/V into the KV cache (fused assembly).
+int lgh_model_run(void* model, void* input, void* output, int batch, int seq, void* workspace, void* stream, int cache_slot) {
+    ModelBase* mb = (ModelBase*)model;
+    if (!shape_ok(mb, batch, seq) || !input || !output) return fail("lgh_model_run: bad arguments");
+    DynamicInitParam D(stream ? stream : mb->stream0->stream, 0);
+    for (auto& f : mb->build(input, output, batch, seq, workspace, cache_slot)) f.callback(D);
+    return first_error();
+}
+
+int lgh_model_run_decode(void* model, void* input, void* output, int batch, int past, int cache_slot, void* workspace, void* stream) {
+    ModelBase* mb = (ModelBase*)model;
+    if (!mb || batch <= 0 || batch > mb->P.max_batch_size || past < 0 || past >= mb->P.max_cache_len || cache_slot < 0 ||
+        cache_slot + batch > mb->P.max_batch_size || !input || !output)
+        return fail("lgh_model_run_decode: bad arguments");
+    DynamicInitParam D(stream ? stream : mb->stream0->stream, 0);
+    for (auto& f : mb->build_decode(input, output, batch, past, cache_slot, workspace)) f.callback(D);
+    return first_error();
+}
+
+// Times every entry of the launch vector the way the reference's profiler does (schedule.h:93-112): 2 warm-up
+// launches, then `iters` launches between two events on the launch stream, minimum over `trials`.  ms_out gets one
+// value per entry; returns the number of entries.
+int lgh_model_time_kernels(void* model, void* input, void* output, int batch, int seq, int decode_past, int cache_slot,
+                           int iters, int trials, float* ms_out, int ms_cap) {
+    ModelBase* mb = (ModelBase*)model;
+    if (!mb || !input || !output || iters <= 0 || trials <= 0) return fail("lgh_model_time_kernels: bad arguments");
+    std::vector<FuncWrap> v = decode_past >= 0 ? mb->build_decode(input, output, batch, decode_past, cache_slot, nullptr)
+                                               : mb->build(input, output, batch, seq, nullptr, cache_slot);
+    if ((int)v.size() > ms_cap) return fail("lgh_model_time_kernels: output array too small");
+    DynamicInitParam& D = *mb->stream0;
+    void *e0 = nullptr, *e1 = nullptr;
+    note_status(lg_event_create(&e0), "lg_event_create");
+    note_status(lg_event_create(&e1), "lg_event_create");
+    // run the whole vector once so that every entry sees valid inputs
+    for (auto& f : v) f.callback(D);
+    note_status(lg_stream_synchronize(D.stream), "lg_stream_synchronize");
+    for (size_t i = 0; i < v.size(); ++i) ms_out[i] = profile_callback(v[i], D, e0, e1, iters, trials);
+    lg_event_destroy(e0);
+    lg_event_destroy(e1);
+    return first_error() ? -1 : (int)v.size();
+}
+
+
+// ---- scheduler ---------------------------------------------------------------------------------------------------
+struct LghReport {
+    int records;
+    double avg_latency_ms, p99_latency_ms, avg_gpu_ms, avg_queue_ms, total_duration_ms, throughput;
+    int rounds, secondary_launches, splits, profile_misses;
+};
+
+// policy: 0 = classic (communication vs rest), 1 = resource classes (MFMA-bound vs HBM-bound)
+// axis: 0 = split output features (the reference's axis), 1 = split token rows
+void* lgh_sched_create(void* model, int schedule_deep, float contention_factor, int policy, int axis, int seq_bucket,
+                       int ignore_num, int pool_count, int ctx_batch) {
+    ModelBase* mb = (ModelBase*)model;
+    if (!mb || schedule_deep < 1 || contention_factor < 0 || pool_count < 0 || ctx_batch < 0 ||
+        (int64_t)pool_count * ctx_batch > mb->P.max_batch_size) {
+        fail("lgh_sched_create: bad arguments (pool_count * ctx_batch must not exceed the model's max_batch)");
+        return nullptr;
+    }
+    SchedBase* s = mb->make_scheduler();
+    s->configure(schedule_deep, contention_factor, policy, axis, seq_bucket < 1 ? 1 : seq_bucket, ignore_num);
+    if (pool_count > 0) s->make_pool(pool_count, ctx_batch);
+    return first_error() ? nullptr : s;
+}
+int lgh_sched_profile(void* sched, int bs, int seq_lo, int seq_hi, int seq_step, int itr) {
+    if (!sched || bs <= 0 || seq_lo <= 0 || seq_hi < seq_lo || seq_step <= 0 || itr <= 0) return fail("lgh_sched_profile: bad arguments");
+    ((SchedBase*)sched)->profile(bs, seq_lo, seq_hi, seq_step, itr);
+    return first_error();
+}
+int lgh_sched_profile_decode(void* sched, int bs, int past, int itr) {
+    if (!sched || bs <= 0 || past < 0 || itr <= 0) return fail("lgh_sched_profile_decode: bad arguments");
+    ((SchedBase*)sched)->profile_decode(bs, past, itr);
+    return first_error();
+}
+int lgh_sched_save(void* sched, const char* main_file, const char* sub_file) {
+    return (sched && ((SchedBase*)sched)->save(main_file, sub_file)) ? LG_OK : fail("lgh_sched_save: cannot write");
+}
+int lgh_sched_load(void* sched, const char* main_file, const char* sub_file) {
+    return (sched && ((SchedBase*)sched)->load(main_file, sub_file)) ? LG_OK : fail("lgh_sched_load: cannot read or parse");
+}
+float lgh_sched_lookup(void* sched, int name, int bs, int seq) { return sched ? ((SchedBase*)sched)->lookup(name, bs, seq) : -1.f; }
+int lgh_sched_sub_lookup(void* sched, int name, int bs, int seq, float* out, int cap) {
+    return sched ? ((SchedBase*)sched)->sub_lookup(name, bs, seq, out, cap) : -1;
+}
+// mode 0 = sequential baseline (run_sequential), 1 = interleaved (run_stream_sync).  Replays the trace in real time.
+int lgh_sched_run_trace(void* sched, int mode, const double* arrival_s, const int* batch, const int* seq, const int* n_decode,
+                        int n, LghReport* out) {
+    if (!sched || n < 0 || !out) return fail("lgh_sched_run_trace: bad arguments");
+    std::vector<TraceRequest> tr;
+    for (int i = 0; i < n; ++i) tr.push_back({arrival_s[i], batch[i], seq[i], n_decode ? n_decode[i] : 0});
+    int c[4] = {0, 0, 0, 0};
+    Report r = ((SchedBase*)sched)->run(mode, tr, c);
+    out->records = r.records; out->avg_latency_ms = r.avg_latency_ms; out->p99_latency_ms = r.p99_latency_ms;
+    out->avg_gpu_ms = r.avg_gpu_ms; out->avg_queue_ms = r.avg_queue_ms; out->total_duration_ms = r.total_duration_ms;
+    out->throughput = r.throughput; out->rounds = c[0]; out->secondary_launches = c[1]; out->splits = c[2]; out->profile_misses = c[3];
+    return first_error();
+}
+// the report arithmetic alone (known-answer tests against the reference's published logs)
+int lgh_summarize(const double* cpu_ms, const double* gpu_ms, int n, double total_duration_ms, LghReport* out) {
+    if (n < 0 || !out) return fail("lgh_summarize: bad arguments");
+    Report r = summarize_records(std::vector<double>(cpu_ms, cpu_ms + n), std::vector<double>(gpu_ms, gpu_ms + n), total_duration_ms);
+    out->records = r.records; out->avg_latency_ms = r.avg_latency_ms; out->p99_latency_ms = r.p99_latency_ms;
+    out->avg_gpu_ms = r.avg_gpu_ms; out->avg_queue_ms = r.avg_queue_ms; out->total_duration_ms = r.total_duration_ms;
+    out->throughput = r.throughput; out->rounds = out->secondary_launches = out->splits = out->profile_misses = 0;
+    return LG_OK;
+}
+int lgh_make_poisson_trace(double lambda, int n, int batch, int seq_lo, int seq_hi, int seq_round, int n_decode, uint64_t seed,
+                           double* arrival_s, int* seq_out) {
+    if (lambda <= 0 || n < 0 || seq_lo <= 0 || seq_hi < seq_lo) return fail("lgh_make_poisson_trace: bad arguments");
+    auto tr = make_poisson_trace(lambda, n, batch, seq_lo, seq_hi, seq_round, n_decode, seed);
+    for (int i = 0; i < n; ++i) { arrival_s[i] = tr[i].arrival_s; seq_out[i] = tr[i].seq; }
+    return LG_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,576 @@
+// layers.h -- layer assembly: classes that own device weights and emit the launch vector.
+//
+// Counterpart of the reference's src/layer/linear.h (Linear_Row :16-64, Linear_Col :68-109), operator.h
+// (LayerNorm :16-41), bert_layer.h (Bert_MLP :19-63, Bert_MHA :65-176) and bert.h (Bert_Encoder :18-80,
+// Bert_Model :83-118).  Same class names, constructor arguments and `forward(...) -> vector<FuncWrap>` contract;
+// no GPU work happens in forward().  Deliberate differences:
+//   * weights, biases, gamma/beta and masks are initialised (seeded generator) -- the reference leaves every
+//     buffer uninitialised because it only measures time;
+//   * workspace slices are computed per request from (batch, seq) and are sized correctly (the reference sizes
+//     the score buffer as B*S*n and multiplies element offsets by sizeof(T));
+//   * tensor parallelism appears only as `/ world_size` on the shard dimensions, exactly as in the reference,
+//     but the all-reduce entry after a row-parallel GEMM is not emitted (single-GPU build: one shard at its real
+//     shape, exchange out of scope);
+//   * optional assemblies: pre-LN with residuals built from the reference's fused residual kernels, a fused
+//     assembly (epilogue-fused GEMMs + one attention kernel) and a decode step over a KV cache.
+#pragma once
+#include <cmath>
+#include <map>
+#include <memory>
+
+#include "func_wrapper.h"
+
+namespace liger {
+
+template <typename T>
+inline T* dev_alloc(size_t elems) {
+    void* p = nullptr;
+    note_status(lg_malloc(&p, (elems ? elems : 1) * sizeof(T)), "lg_malloc");
+    return (T*)p;
+}
+template <typename T>
+inline void dev_fill_normal(T* p, int64_t n, uint64_t seed, uint64_t tensor_id, float mean, float stddev) {
+    if (dtype_of<T>::value == LG_F16) note_status(lg_fill_normal_f16(p, n, seed, tensor_id, mean, stddev, nullptr), "lg_fill_normal_f16");
+    else note_status(lg_fill_normal_f32((float*)p, n, seed, tensor_id, mean, stddev, nullptr), "lg_fill_normal_f32");
+}
+template <typename T>
+inline void dev_fill_const(T* p, int64_t n, float v) {
+    if (dtype_of<T>::value == LG_F16) note_status(lg_fill_const_f16(p, n, v, nullptr), "lg_fill_const_f16");
+    else note_status(lg_fill_const_f32((float*)p, n, v, nullptr), "lg_fill_const_f32");
+}
+
+inline int64_t align_up(int64_t x, int64_t a = 128) { return (x + a - 1) / a * a; }
+
+// Named parameters of a layer, for tests that download / upload them.
+struct ParamRef {
+    std::string name;
+    void* ptr;
+    int64_t elems;
+};
+
+// ---------------------------------------------------------------------------------------------------
+// Linear layers.  Y[M, N'] = X[M, K'] * W with W stored row-major [K', N'] (the layout cuBLAS's (N,N) call in
+// the reference implies: column-major N' x K' with lda = N').
+// ---------------------------------------------------------------------------------------------------
+template <typename T>
+class Linear_Col {  // linear.h:68-109: output features split across ranks
+  public:
+    int k, n;  // GLOBAL in/out features
+    T* weights;
+    StaticInitParam SParams;
+    std::vector<FuncWrap> FuncWrapVec;
+
+    Linear_Col(const StaticInitParam& SParams_, const int& k_, const int& n_) : k(k_), n(n_), SParams(SParams_) {
+        weights = dev_alloc<T>((size_t)k * n / SParams.world_size);
+    }
+    int n_local() const { return n / SParams.world_size; }
+    void init_weights(uint64_t seed, uint64_t tensor_id, float stddev = 0.02f) {
+        dev_fill_normal(weights, (int64_t)k * n_local(), seed, tensor_id, 0.f, stddev);
+    }
+    GemmDesc desc(T* input, T* output, int m) const {
+        GemmDesc g;
+        g.valid = true; g.dtype = dtype_of<T>::value; g.transa = 0;
+        g.m = n_local(); g.n = m; g.k = k;
+        g.A = weights; g.lda = n_local(); g.B = input; g.ldb = k; g.C = output; g.ldc = n_local();
+        return g;
+    }
+    std::vector<FuncWrap> forward(T* input, T* output, int m) {
+        FuncWrapVec.clear();
+        GemmDesc g = desc(input, output, m);
+        FuncWrapVec.push_back(FuncWrap(1.0f, GEMM, [g](const DynamicInitParam& D) { GemmEx(D, g); }, g, "linear_col"));
+        return FuncWrapVec;
+    }
+};
+
+template <typename T>
+class Linear_Row {  // linear.h:16-64: input features split across ranks; partial sums
+  public:
+    int k, n;
+    T* weights;
+    StaticInitParam SParams;
+    std::vector<FuncWrap> FuncWrapVec;
+
+    Linear_Row(const StaticInitParam& SParams_, const int& k_, const int& n_) : k(k_), n(n_), SParams(SParams_) {
+        weights = dev_alloc<T>((size_t)k * n / SParams.world_size);
+    }
+    int k_local() const { return k / SParams.world_size; }
+    void init_weights(uint64_t seed, uint64_t tensor_id, float stddev = 0.02f) {
+        dev_fill_normal(weights, (int64_t)k_local() * n, seed, tensor_id, 0.f, stddev);
+    }
+    GemmDesc desc(T* input, T* output, int m) const {
+        GemmDesc g;
+        g.valid = true; g.dtype = dtype_of<T>::value; g.transa = 0;
+        g.m = n; g.n = m; g.k = k_local();
+        g.A = weights; g.lda = n; g.B = input; g.ldb = k_local(); g.C = output; g.ldc = n;
+        return g;
+    }
+    std::vector<FuncWrap> forward(T* input, T* output, int m) {
+        FuncWrapVec.clear();
+        GemmDesc g = desc(input, output, m);
+        FuncWrapVec.push_back(FuncWrap(2.0f, GEMM, [g](const DynamicInitParam& D) { GemmEx(D, g); }, g, "linear_row"));
+        // linear.h:55-60 appends the all-reduce of m*n elements here when world_size != 1.  The exchange between
+        // GPUs is outside this single-GPU build, so the vector holds this rank's partial product only.
+        return FuncWrapVec;
+    }
+};
+
+template <typename T>
+class LayerNorm {  // operator.h:16-41
+  public:
+    int k;
+    T* gamma;
+    T* beta;
+    StaticInitParam SParams;
+    std::vector<FuncWrap> FuncWrapVec;
+
+    LayerNorm(const StaticInitParam& SParams_, const int& k_) : k(k_), SParams(SParams_) {
+        gamma = dev_alloc<T>(k);
+        beta = dev_alloc<T>(k);
+        dev_fill_const(gamma, k, 1.0f);
+        dev_fill_const(beta, k, 0.0f);
+    }
+    void init_weights(uint64_t seed, uint64_t tensor_id) {
+        dev_fill_normal(gamma, k, seed, tensor_id, 1.0f, 0.1f);
+        dev_fill_normal(beta, k, seed, tensor_id + 1, 0.0f, 0.1f);
+    }
+    std::vector<FuncWrap> forward(T* input, T* output, int m) {
+        FuncWrapVec.clear();
+        T *g = gamma, *b = beta;
+        int kk = k;
+        FuncWrapVec.push_back(FuncWrap(0.1f, COMPUTATION,
+                                       [=](const DynamicInitParam& D) { Layer_Norm<T>(input, g, b, output, m, kk, D); },
+                                       "layer_norm"));
+        return FuncWrapVec;
+    }
+};
+
+// ---------------------------------------------------------------------------------------------------
+// MLP  (bert_layer.h:19-63)
+// ---------------------------------------------------------------------------------------------------
+template <typename T>
+class Bert_MLP {
+  public:
+    int k, n, intermediate_size;  // GLOBAL sizes
+    int mlp_ratio = 4;
+    StaticInitParam SParam;
+    BertInitParam BertParams;
+    T* linear_row_output;  // default inner buffer
+    T* bias;               // [F local]   (bert_layer.h:45)
+    T* bias2;              // [k] FFN-2 bias: only used by the pre-LN assembly
+    Linear_Col<T>* linear_col;
+    Linear_Row<T>* linear_row;
+    std::vector<FuncWrap> FuncWrapVec;
+
+    Bert_MLP(const BertInitParam& BertParams_, const StaticInitParam& SParam_, const int& k_, const int& n_, T* workspace)
+        : k(k_), n(n_), SParam(SParam_), BertParams(BertParams_), linear_row_output(workspace) {
+        intermediate_size = BertParams.ffn_inner > 0 ? BertParams.ffn_inner : n * mlp_ratio;
+        linear_col = new Linear_Col<T>(SParam, k, intermediate_size);
+        linear_row = new Linear_Row<T>(SParam, intermediate_size, k);
+        bias = dev_alloc<T>(f_local());
+        bias2 = dev_alloc<T>(k);
+        dev_fill_const(bias, f_local(), 0.f);
+        dev_fill_const(bias2, k, 0.f);
+    }
+    int f_local() const { return intermediate_size / SParam.world_size; }
+    void init_weights(uint64_t seed, uint64_t base) {
+        linear_col->init_weights(seed, base + 0);
+        linear_row->init_weights(seed, base + 1);
+        dev_fill_normal(bias, f_local(), seed, base + 2, 0.f, 0.02f);
+        dev_fill_normal(bias2, k, seed, base + 3, 0.f, 0.02f);
+    }
+    void params(const std::string& prefix, std::vector<ParamRef>& out) {
+        out.push_back({prefix + "w1", linear_col->weights, (int64_t)k * f_local()});
+        out.push_back({prefix + "b1", bias, f_local()});
+        out.push_back({prefix + "w2", linear_row->weights, (int64_t)f_local() * k});
+        out.push_back({prefix + "b2", bias2, k});
+    }
+    // inner: [m, F local] scratch.  idx 11, 12, 13 of the launch vector (fused: 2 entries).
+    std::vector<FuncWrap> forward(T* input, T* output, int m, T* inner = nullptr) {
+        FuncWrapVec.clear();
+        if (!inner) inner = linear_row_output;
+        const int F = f_local();
+        if (BertParams.fused && dtype_of<T>::value == LG_F16) {
+            GemmDesc g = linear_col->desc(input, inner, m);
+            g.epilogue = LG_EPI_BIAS_GELU;
+            g.bias = bias;
+            FuncWrapVec.push_back(FuncWrap(1.0f, GEMM, [g](const DynamicInitParam& D) { GemmEx(D, g); }, g, "ffn1+bias+gelu"));
+        } else {
+            std::vector<FuncWrap> v = linear_col->forward(input, inner, m);
+            v[0].label = "ffn1";
+            FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
+            T* b = bias;
+            FuncWrapVec.push_back(FuncWrap(0.2f, COMPUTATION,
+                                           [=](const DynamicInitParam& D) { Add_bias_act_kernelLauncher<T>(inner, b, m, F, D); },
+                                           "bias+gelu"));
+        }
+        std::vector<FuncWrap> v = linear_row->forward(inner, output, m);
+        v[0].label = "ffn2";
+        FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
+        return FuncWrapVec;
+    }
+};
+
+// ---------------------------------------------------------------------------------------------------
+// Multi-head attention  (bert_layer.h:65-176)
+// ---------------------------------------------------------------------------------------------------
+template <typename T>
+struct MhaBuffers {  // per-request slices, all in elements of T
+    T *q, *k, *v, *q_buf, *k_buf, *v_buf, *qk_buf, *attn_trans_out, *attn_out;
+    void* decode_ws;  // split-KV partials of the decode attention
+};
+
+template <typename T>
+class Bert_MHA {
+  public:
+    int k, n;
+    float scalar;
+    Linear_Col<T>* linear_q_col;
+    Linear_Col<T>* linear_k_col;
+    Linear_Col<T>* linear_v_col;
+    Linear_Row<T>* linear_w_row;
+    StaticInitParam SParam;
+    BertInitParam BertParams;
+    T *q_bias, *k_bias, *v_bias, *w_bias;
+    T* workspace;
+    std::map<int, T*> masks;  // seq -> attr_mask [max_batch, seq, seq] (all ones, or lower-triangular if causal)
+    T *k_cache = nullptr, *v_cache = nullptr;  // [max_batch, heads, max_cache_len, d] when max_cache_len > 0
+    std::vector<FuncWrap> FuncWrapVec;
+
+    Bert_MHA(const BertInitParam& BertParams_, const StaticInitParam& SParam_, const int& k_, const int& n_, T* workspace_)
+        : k(k_), n(n_), SParam(SParam_), BertParams(BertParams_), workspace(workspace_) {
+        scalar = 1.0f / sqrtf((float)BertParams.size_per_head);  // bert_layer.h:94
+        linear_q_col = new Linear_Col<T>(SParam, k, n);
+        linear_k_col = new Linear_Col<T>(SParam, k, n);
+        linear_v_col = new Linear_Col<T>(SParam, k, n);
+        linear_w_row = new Linear_Row<T>(SParam, k, n);
+        q_bias = dev_alloc<T>(hl()); k_bias = dev_alloc<T>(hl()); v_bias = dev_alloc<T>(hl());
+        w_bias = dev_alloc<T>(n);
+        dev_fill_const(q_bias, hl(), 0.f); dev_fill_const(k_bias, hl(), 0.f); dev_fill_const(v_bias, hl(), 0.f);
+        dev_fill_const(w_bias, n, 0.f);
+        if (BertParams.max_cache_len > 0) {
+            const size_t ce = (size_t)BertParams.max_batch_size * heads() * BertParams.max_cache_len * BertParams.size_per_head;
+            k_cache = dev_alloc<T>(ce);
+            v_cache = dev_alloc<T>(ce);
+            note_status(lg_memset_async(k_cache, 0, ce * sizeof(T), nullptr), "lg_memset_async");
+            note_status(lg_memset_async(v_cache, 0, ce * sizeof(T), nullptr), "lg_memset_async");
+        }
+    }
+    int heads() const { return BertParams.head_num / SParam.world_size; }
+    int hl() const { return heads() * BertParams.size_per_head; }
+    void init_weights(uint64_t seed, uint64_t base) {
+        linear_q_col->init_weights(seed, base + 0);
+        linear_k_col->init_weights(seed, base + 1);
+        linear_v_col->init_weights(seed, base + 2);
+        linear_w_row->init_weights(seed, base + 3);
+        dev_fill_normal(q_bias, hl(), seed, base + 4, 0.f, 0.02f);
+        dev_fill_normal(k_bias, hl(), seed, base + 5, 0.f, 0.02f);
+        dev_fill_normal(v_bias, hl(), seed, base + 6, 0.f, 0.02f);
+        dev_fill_normal(w_bias, n, seed, base + 7, 0.f, 0.02f);
+    }
+    void params(const std::string& prefix, std::vector<ParamRef>& out) {
+        out.push_back({prefix + "wq", linear_q_col->weights, (int64_t)k * hl()});
+        out.push_back({prefix + "wk", linear_k_col->weights, (int64_t)k * hl()});
+        out.push_back({prefix + "wv", linear_v_col->weights, (int64_t)k * hl()});
+        out.push_back({prefix + "bq", q_bias, hl()});
+        out.push_back({prefix + "bk", k_bias, hl()});
+        out.push_back({prefix + "bv", v_bias, hl()});
+        out.push_back({prefix + "wo", linear_w_row->weights, (int64_t)hl() * n});
+        out.push_back({prefix + "bo", w_bias, n});
+    }
+    static int64_t score_elems(const BertInitParam& P, const StaticInitParam& S, int batch, int seq) {
+        const bool fused = P.fused && dtype_of<T>::value == LG_F16;
+        return fused ? 0 : align_up((int64_t)batch * (P.head_num / S.world_size) * seq * seq);
+    }
+    static int64_t decode_ws_elems(const BertInitParam& P, const StaticInitParam& S, int batch) {
+        if (P.max_cache_len <= 0) return 0;
+        const size_t bytes = lg_attn_decode_workspace_bytes(batch, P.head_num / S.world_size, P.size_per_head, P.max_cache_len);
+        return align_up((int64_t)((bytes + sizeof(T) - 1) / sizeof(T)));
+    }
+    static int64_t workspace_elems(const BertInitParam& P, const StaticInitParam& S, int batch, int seq) {
+        const int64_t M = (int64_t)batch * seq, hl_ = (int64_t)(P.head_num / S.world_size) * P.size_per_head;
+        return 8 * align_up(M * hl_) + score_elems(P, S, batch, seq) + decode_ws_elems(P, S, batch);
+    }
+    MhaBuffers<T> slice(T* ws, int batch, int seq) const {
+        const int64_t M = (int64_t)batch * seq, a = align_up(M * hl());
+        MhaBuffers<T> b;
+        b.q = ws; b.k = b.q + a; b.v = b.k + a;
+        b.q_buf = b.v + a; b.k_buf = b.q_buf + a; b.v_buf = b.k_buf + a;
+        b.attn_trans_out = b.v_buf + a; b.attn_out = b.attn_trans_out + a;
+        b.qk_buf = b.attn_out + a;
+        b.decode_ws = b.qk_buf + score_elems(BertParams, SParam, batch, seq);
+        return b;
+    }
+    T* mask_for(int seq) {
+        auto it = masks.find(seq);
+        if (it != masks.end()) return it->second;
+        const int64_t e = (int64_t)BertParams.max_batch_size * seq * seq;
+        T* m = dev_alloc<T>(e);
+        if (BertParams.causal) {
+            if (dtype_of<T>::value == LG_F16) note_status(lg_fill_causal_mask_f16(m, BertParams.max_batch_size, seq, nullptr), "lg_fill_causal_mask_f16");
+            else note_status(lg_fill_causal_mask_f32((float*)m, BertParams.max_batch_size, seq, nullptr), "lg_fill_causal_mask_f32");
+        } else {
+            dev_fill_const(m, e, 1.0f);
+        }
+        note_status(lg_device_synchronize(), "lg_device_synchronize");
+        masks[seq] = m;
+        return m;
+    }
+
+    // idx 0..8 of the launch vector (9 entries); fused assembly: 5 entries.
+    // cache_slot >= 0 (fused only): K/V are written straight into the KV cache rows [cache_slot, cache_slot+batch).
+    std::vector<FuncWrap> forward(T* input, T* output, int batch_size, int seq_len, T* ws = nullptr, int cache_slot = -1) {
+        FuncWrapVec.clear();
+        if (!ws) ws = workspace;
+        const MhaBuffers<T> b = slice(ws, batch_size, seq_len);
+        const int M = batch_size * seq_len, h = heads(), d = BertParams.size_per_head;
+        const int dt = dtype_of<T>::value;
+        const float sc = scalar;
+        if (BertParams.fused && dt == LG_F16) {
+            T* kdst = b.k_buf;
+            T* vdst = b.v_buf;
+            int kv_rows = seq_len;
+            if (cache_slot >= 0 && k_cache) {
+                kv_rows = BertParams.max_cache_len;
+                kdst = k_cache + (int64_t)cache_slot * h * kv_rows * d;
+                vdst = v_cache + (int64_t)cache_slot * h * kv_rows * d;
+            }
+            Linear_Col<T>* lin[3] = {linear_q_col, linear_k_col, linear_v_col};
+            T* dst[3] = {b.q_buf, kdst, vdst};
+            const T* bias[3] = {q_bias, k_bias, v_bias};
+            const char* lab[3] = {"q_gemm+bias+heads", "k_gemm+bias+heads", "v_gemm+bias+heads"};
+            for (int t = 0; t < 3; ++t) {
+                GemmDesc g = lin[t]->desc(input, dst[t], M);
+                g.epilogue = LG_EPI_BIAS_HEADS;
+                g.bias = bias[t];
+                g.epi_seq = seq_len; g.epi_d = d; g.epi_heads_total = h;
+                g.ldc = (t == 0) ? seq_len : kv_rows;  // rows per (batch, head) slot of the destination
+                FuncWrapVec.push_back(FuncWrap(1.0f, GEMM, [g](const DynamicInitParam& D) { GemmEx(D, g); }, g, lab[t]));
+            }
+            T* qb = b.q_buf; T* ao = b.attn_out;
+            const int causal = BertParams.causal;
+            FuncWrapVec.push_back(FuncWrap(0.8f, COMPUTATION, [=](const DynamicInitParam& D) {
+                note_status(lg_attn_prefill_f16(qb, kdst, vdst, nullptr, ao, batch_size, seq_len, h, d, kv_rows, sc, causal, 1,
+                                                D.stream), "lg_attn_prefill_f16");
+            }, "attn_prefill_fused", MFMA_BOUND));
+            std::vector<FuncWrap> v = linear_w_row->forward(b.attn_out, output, M);
+            v[0].label = "out_proj";
+            FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
+            return FuncWrapVec;
+        }
+
+        // qkv linear  (bert_layer.h:128-135)
+        std::vector<FuncWrap> v = linear_q_col->forward(input, b.q, M); v[0].label = "q_gemm";
+        FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
+        v = linear_k_col->forward(input, b.k, M); v[0].label = "k_gemm";
+        FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
+        v = linear_v_col->forward(input, b.v, M); v[0].label = "v_gemm";
+        FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
+        // bias + transpose  (:139-142)
+        T *qbias = q_bias, *kbias = k_bias, *vbias = v_bias;
+        FuncWrapVec.push_back(FuncWrap(0.2f, COMPUTATION, [=](const DynamicInitParam& D) {
+            Add_QKV_bias_transpose<T>(b.q_buf, b.k_buf, b.v_buf, b.q, qbias, b.k, kbias, b.v, vbias, batch_size, seq_len, h, d, D);
+        }, "qkv_bias_transpose"));
+        // qk  (:145-150)
+        FuncWrapVec.push_back(FuncWrap(0.3f, COMPUTATION, [=](const DynamicInitParam& D) {
+            GemmStridedBatchedEx(D, dt, 1, 0, seq_len, seq_len, d, b.k_buf, d, (long long)seq_len * d, b.q_buf, d,
+                                 (long long)seq_len * d, b.qk_buf, seq_len, (long long)seq_len * seq_len, batch_size * h);
+        }, "qk_gemm", MFMA_BOUND));
+        // softmax  (:153-155)
+        T* mask = mask_for(seq_len);
+        FuncWrapVec.push_back(FuncWrap(0.2f, COMPUTATION, [=](const DynamicInitParam& D) {
+            Attn_softmax_kernel<T>(b.qk_buf, mask, batch_size, seq_len, h, sc, D);
+        }, "softmax"));
+        // qkv  (:158-163)
+        FuncWrapVec.push_back(FuncWrap(0.3f, COMPUTATION, [=](const DynamicInitParam& D) {
+            GemmStridedBatchedEx(D, dt, 0, 0, d, seq_len, seq_len, b.v_buf, d, (long long)seq_len * d, b.qk_buf, seq_len,
+                                 (long long)seq_len * seq_len, b.attn_trans_out, d, (long long)seq_len * d, batch_size * h);
+        }, "pv_gemm", MFMA_BOUND));
+        // transpose back  (:166-168)
+        FuncWrapVec.push_back(FuncWrap(0.1f, COMPUTATION, [=](const DynamicInitParam& D) {
+            Transpose_kernel<T>(b.attn_out, b.attn_trans_out, batch_size, seq_len, h, d, D);
+        }, "transpose_back"));
+        // linear row  (:171)
+        v = linear_w_row->forward(b.attn_out, output, M); v[0].label = "out_proj";
+        FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
+        return FuncWrapVec;
+    }
+
+    // One decode step for `batch` sequences whose cache rows start at cache_slot: Q/K/V GEMMs on one token each,
+    // bias + append to the cache at position `past`, attention over past+1 positions, output projection.
+    // No reference counterpart (the reference has no KV cache).  fp16 only.
+    std::vector<FuncWrap> forward_decode(T* input, T* output, int batch, int past, int cache_slot, T* ws = nullptr) {
+        FuncWrapVec.clear();
+        if (!ws) ws = workspace;
+        const MhaBuffers<T> b = slice(ws, batch, 1);
+        const int h = heads(), d = BertParams.size_per_head, Lmax = BertParams.max_cache_len;
+        const float sc = scalar;
+        std::vector<FuncWrap> v = linear_q_col->forward(input, b.q, batch); v[0].label = "q_gemm(decode)"; v[0].rclass = HBM_BOUND;
+        FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
+        v = linear_k_col->forward(input, b.k, batch); v[0].label = "k_gemm(decode)"; v[0].rclass = HBM_BOUND;
+        FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
+        v = linear_v_col->forward(input, b.v, batch); v[0].label = "v_gemm(decode)"; v[0].rclass = HBM_BOUND;
+        FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
+        T* kc = k_cache + (int64_t)cache_slot * h * Lmax * d;
+        T* vc = v_cache + (int64_t)cache_slot * h * Lmax * d;
+        T *qbias = q_bias, *kbias = k_bias, *vbias = v_bias;
+        void* dws = b.decode_ws;
+        FuncWrapVec.push_back(FuncWrap(0.05f, COMPUTATION, [=](const DynamicInitParam& D) {
+            note_status(lg_kv_append_f16(b.q_buf, kc, vc, b.q, qbias, b.k, kbias, b.v, vbias, batch, h, d, past, Lmax, D.stream), "lg_kv_append_f16");
+        }, "kv_append"));
+        FuncWrapVec.push_back(FuncWrap(0.15f, COMPUTATION, [=](const DynamicInitParam& D) {
+            note_status(lg_attn_decode_f16(b.q_buf, kc, vc, b.attn_out, dws, batch, h, d, past + 1, Lmax, sc, D.stream), "lg_attn_decode_f16");
+        }, "attn_decode"));
+        v = linear_w_row->forward(b.attn_out, output, batch); v[0].label = "out_proj(decode)"; v[0].rclass = HBM_BOUND;
+        FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
+        return FuncWrapVec;
+    }
+};
+
+// ---------------------------------------------------------------------------------------------------
+// Encoder layer and model  (bert.h:18-118)
+// ---------------------------------------------------------------------------------------------------
+template <typename T>
+class Bert_Encoder {
+    int k, n;
+    StaticInitParam SParam;
+    BertInitParam BertParam;
+    T* workspace;
+    std::vector<FuncWrap> FuncWrapVec;
+
+  public:
+    Bert_MHA<T>* MHA;
+    Bert_MLP<T>* MLP;
+    LayerNorm<T>* ln_mha;
+    LayerNorm<T>* ln_mlp;
+
+    Bert_Encoder(const BertInitParam& BertParams, const StaticInitParam& SParam_, const int& k_, const int& n_, T* workspace_)
+        : k(k_), n(n_), SParam(SParam_), BertParam(BertParams), workspace(workspace_) {
+        MHA = new Bert_MHA<T>(BertParams, SParam, k, n, workspace);
+        MLP = new Bert_MLP<T>(BertParams, SParam, k, n, workspace);
+        ln_mha = new LayerNorm<T>(SParam, k);
+        ln_mlp = new LayerNorm<T>(SParam, k);
+    }
+    void init_weights(uint64_t seed, uint64_t base) {
+        MHA->init_weights(seed, base + 0);
+        MLP->init_weights(seed, base + 8);
+        ln_mha->init_weights(seed, base + 12);
+        ln_mlp->init_weights(seed, base + 14);
+    }
+    void params(const std::string& prefix, std::vector<ParamRef>& out) {
+        MHA->params(prefix, out);
+        out.push_back({prefix + "ln1_g", ln_mha->gamma, k});
+        out.push_back({prefix + "ln1_b", ln_mha->beta, k});
+        MLP->params(prefix, out);
+        out.push_back({prefix + "ln2_g", ln_mlp->gamma, k});
+        out.push_back({prefix + "ln2_b", ln_mlp->beta, k});
+    }
+    static int64_t workspace_elems(const BertInitParam& P, const StaticInitParam& S, int batch, int seq) {
+        const int hidden = P.head_num * P.size_per_head;
+        const int F = (P.ffn_inner > 0 ? P.ffn_inner : 4 * hidden) / S.world_size;
+        const int64_t M = (int64_t)batch * seq;
+        return Bert_MHA<T>::workspace_elems(P, S, batch, seq) + align_up(M * F) + 4 * align_up(M * hidden);
+    }
+
+    // bert.h:59-79: MHA -> LN -> MLP -> LN (POST_NORESID).  PRE_LN_RESID chains layer_norm -> MHA ->
+    // add_bias_input_layernorm_2 -> MLP -> add_bias_input.
+    std::vector<FuncWrap> forward(T* input, T* output, int batch_size, int seq_len, T* ws = nullptr, int cache_slot = -1,
+                                  int decode_past = -1) {
+        FuncWrapVec.clear();
+        if (!ws) ws = workspace;
+        const bool decode = decode_past >= 0;
+        const int seq = decode ? 1 : seq_len;
+        const int M = batch_size * seq;
+        T* attn_ws = ws;
+        T* mlp_inner = attn_ws + Bert_MHA<T>::workspace_elems(BertParam, SParam, batch_size, seq);
+        T* mha_out = mlp_inner + align_up((int64_t)M * MLP->f_local());
+        T* ln_mha_out = mha_out + align_up((int64_t)M * n);
+        T* mlp_out = ln_mha_out + align_up((int64_t)M * n);
+        T* pre_ln_out = mlp_out + align_up((int64_t)M * n);
+        auto append = [&](std::vector<FuncWrap> v) { FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end()); };
+        auto mha = [&](T* in, T* out) {
+            return decode ? MHA->forward_decode(in, out, batch_size, decode_past, cache_slot, attn_ws)
+                          : MHA->forward(in, out, batch_size, seq_len, attn_ws, cache_slot);
+        };
+        auto mlp = [&](T* in, T* out) {
+            std::vector<FuncWrap> v = MLP->forward(in, out, M, mlp_inner);
+            if (decode) for (auto& f : v) f.rclass = HBM_BOUND;
+            return v;
+        };
+        if (BertParam.norm_mode == POST_NORESID) {
+            append(mha(input, mha_out));
+            append(ln_mha->forward(mha_out, ln_mha_out, M));
+            append(mlp(ln_mha_out, mlp_out));
+            append(ln_mlp->forward(mlp_out, output, M));
+        } else {
+            append(ln_mha->forward(input, pre_ln_out, M));
+            append(mha(pre_ln_out, mha_out));
+            T *g = ln_mlp->gamma, *bt = ln_mlp->beta, *wb = MHA->w_bias;
+            const int nn = n;
+            FuncWrapVec.push_back(FuncWrap(0.1f, COMPUTATION, [=](const DynamicInitParam& D) {
+                Add_bias_input_layernorm_2_kernelLauncher<T>(input, g, bt, wb, mha_out, ln_mha_out, M, nn, D);
+            }, "residual+bias+layer_norm"));
+            append(mlp(ln_mha_out, output));
+            T* b2 = MLP->bias2;
+            FuncWrapVec.push_back(FuncWrap(0.1f, COMPUTATION, [=](const DynamicInitParam& D) {
+                Add_bias_input_kernelLauncher<T>(output, b2, mha_out, M, nn, D);
+            }, "residual+bias"));
+        }
+        return FuncWrapVec;
+    }
+};
+
+template <typename T>
+class Bert_Model {
+  public:
+    int k, n;
+    StaticInitParam SParam;
+    BertInitParam BertParams;
+    std::vector<Bert_Encoder<T>*> encoders;
+    std::vector<FuncWrap> FuncWrapVec;
+    T* workspace;
+
+    Bert_Model(const BertInitParam& BertParams_, const StaticInitParam& SParam_, const int& k_, const int& n_, T* workspace_)
+        : k(k_), n(n_), SParam(SParam_), BertParams(BertParams_), workspace(workspace_) {
+        for (int i = 0; i < BertParams.layer_num; i++) encoders.push_back(new Bert_Encoder<T>(BertParams, SParam, k, n, workspace));
+    }
+    void init_weights(uint64_t seed) {
+        for (size_t i = 0; i < encoders.size(); ++i) encoders[i]->init_weights(seed, 1000 * (i + 1));
+        note_status(lg_device_synchronize(), "lg_device_synchronize");
+    }
+    std::vector<ParamRef> params() {
+        std::vector<ParamRef> out;
+        for (size_t i = 0; i < encoders.size(); ++i) encoders[i]->params("layer" + std::to_string(i) + ".", out);
+        return out;
+    }
+    int64_t workspace_elems(int batch, int seq) const { return Bert_Encoder<T>::workspace_elems(BertParams, SParam, batch, seq); }
+    // entries per layer of the vector forward() returns for this configuration
+    int kernels_per_layer(bool decode = false) const {
+        const bool fused = BertParams.fused && dtype_of<T>::value == LG_F16;
+        int mha = decode ? 6 : (fused ? 5 : 9);
+        int mlp = fused ? 2 : 3;
+        return mha + mlp + 2 + (BertParams.norm_mode == PRE_LN_RESID ? 1 : 0);
+    }
+
+    // bert.h:104-115: layer 0 input -> output, later layers output -> output (in place through the workspace)
+    std::vector<FuncWrap> forward(T* input, T* output, int batch_size, int seq_len, T* ws = nullptr, int cache_slot = -1) {
+        FuncWrapVec.clear();
+        if (!ws) ws = workspace;
+        for (int i = 0; i < BertParams.layer_num; i++) {
+            std::vector<FuncWrap> v = encoders[i]->forward(i == 0 ? input : output, output, batch_size, seq_len, ws, cache_slot);
+            FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
+        }
+        return FuncWrapVec;
+    }
+    // one decode step through all layers (KV caches must have been filled by a fused prefill with the same slot)
+    std::vector<FuncWrap> forward_decode(T* input, T* output, int batch_size, int past, int cache_slot, T* ws = nullptr) {
+        FuncWrapVec.clear();
+        if (!ws) ws = workspace;
+        for (int i = 0; i < BertParams.layer_num; i++) {
+            std::vector<FuncWrap> v = encoders[i]->forward(i == 0 ? input : output, output, batch_size, 1, ws, cache_slot, past);
+            FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
+        }
+        return FuncWrapVec;
+    }
+};
+
+}  // namespace liger

@@ -1,0 +1,475 @@
+// scheduler.h -- profile-driven two-stream scheduler with hybrid (host + device event) synchronisation.
+//
+// Counterpart of the reference's src/schedule.h (Scheduler<T, MODEL>: profile :79-157, serve :159-172, update_vec
+// :175-202, run_sequential :204-219, run_stream_sync :221-278, run_stop :280-282, request simulator :285-321,
+// output_recording :325-350).  Same structure: a request thread builds launch vectors and queues Samples; the
+// scheduler thread runs rounds -- the primary request launches one run of same-class kernels on stream 0, then up to
+// contention_factor x (profiled time of that run) worth of other-class kernels of the waiting requests is launched
+// on stream 1, splitting a GEMM when only a fraction fits.  The host blocks on an event recorded before the LAST
+// kernel of the previous round (so it prepares the next round while that kernel runs) and stream 1 is gated on the
+// END of the previous round by a device-side event wait.
+// Differences: a mutex-protected queue and an atomic stop flag (the reference shares a std::queue and a bool between
+// threads unguarded); per-request input/output/workspace/KV-cache contexts (the reference shares one set between all
+// in-flight requests); the class notion is a policy (see sample.h); requests may carry decode steps; the report
+// adds p99; the loop ends when stop has been requested AND all work has drained.
+#pragma once
+#include <algorithm>
+#include <atomic>
+#include <condition_variable>
+#include <deque>
+#include <mutex>
+#include <thread>
+
+#include "layers.h"
+#include "sample.h"
+
+namespace liger {
+
+// Times one launch-vector entry the way the reference's profiler does (schedule.h:93-112): two warm-up launches,
+// device sync, `iters` launches between two events on the launch stream; minimum over `trials`.  Returns ms/launch.
+inline float profile_callback(FuncWrap& f, const DynamicInitParam& D, void* e0, void* e1, int iters = 20, int trials = 3) {
+    float best = 1e30f;
+    for (int t = 0; t < trials; ++t) {
+        f.callback(D);
+        f.callback(D);
+        note_status(lg_device_synchronize(), "lg_device_synchronize");
+        note_status(lg_event_record(e0, D.stream), "lg_event_record");
+        for (int i = 0; i < iters; ++i) f.callback(D);
+        note_status(lg_event_record(e1, D.stream), "lg_event_record");
+        note_status(lg_event_synchronize(e1), "lg_event_synchronize");
+        float ms = 0.f;
+        note_status(lg_event_elapsed_ms(&ms, e0, e1), "lg_event_elapsed_ms");
+        if (ms < best) best = ms;
+    }
+    return best / (float)iters;
+}
+
+struct TraceRequest {
+    double arrival_s;  // offset from the start of the trace
+    int batch, seq, n_decode;
+};
+
+struct Report {
+    int records = 0;
+    double avg_latency_ms = 0, p99_latency_ms = 0, avg_gpu_ms = 0, avg_queue_ms = 0, total_duration_ms = 0, throughput = 0;
+};
+
+// Pure arithmetic of the reference's report (schedule.h:325-348): latency_i = cpu_ms[i] + gpu_ms[i];
+// Average Latency = mean; Throughput = 1000 * count / total_duration_ms.  p99 = nearest-rank percentile.
+inline Report summarize_records(const std::vector<double>& cpu_ms, const std::vector<double>& gpu_ms, double total_duration_ms) {
+    Report r;
+    r.records = (int)std::min(cpu_ms.size(), gpu_ms.size());
+    if (r.records == 0) return r;
+    std::vector<double> lat(r.records);
+    double sl = 0, sg = 0, sq = 0;
+    for (int i = 0; i < r.records; ++i) {
+        lat[i] = cpu_ms[i] + gpu_ms[i];
+        sl += lat[i]; sg += gpu_ms[i]; sq += cpu_ms[i];
+    }
+    r.avg_latency_ms = sl / r.records;
+    r.avg_gpu_ms = sg / r.records;
+    r.avg_queue_ms = sq / r.records;
+    std::sort(lat.begin(), lat.end());
+    int rank = (int)std::ceil(0.99 * r.records);
+    r.p99_latency_ms = lat[std::max(1, rank) - 1];
+    r.total_duration_ms = total_duration_ms;
+    r.throughput = total_duration_ms > 0 ? 1000.0 * r.records / total_duration_ms : 0;
+    return r;
+}
+
+// Deterministic Poisson trace: exponential inter-arrival times with rate lambda (req/s), prompt lengths uniform in
+// [seq_lo, seq_hi] rounded down to a multiple of seq_round (the reference rejects batch*seq % 4 != 0, schedule.h:299).
+inline std::vector<TraceRequest> make_poisson_trace(double lambda, int n, int batch, int seq_lo, int seq_hi, int seq_round,
+                                                    int n_decode, uint64_t seed) {
+    auto next = [&seed]() {
+        seed += 0x9E3779B97F4A7C15ull;
+        uint64_t z = seed;
+        z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+        z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+        return z ^ (z >> 31);
+    };
+    std::vector<TraceRequest> tr;
+    double t = 0;
+    for (int i = 0; i < n; ++i) {
+        const double u = ((double)(next() >> 11) + 0.5) / 9007199254740992.0;  // (0,1)
+        t += -std::log(u) / lambda;
+        int s = seq_lo + (int)(next() % (uint64_t)(seq_hi - seq_lo + 1));
+        if (seq_round > 1) s = std::max(seq_round, s / seq_round * seq_round);
+        tr.push_back({t, batch, s, n_decode});
+    }
+    return tr;
+}
+
+template <class T, class MODELTYPE>
+class Scheduler {
+  public:
+    struct ReqCtx {
+        T *input, *output, *ws, *dec_a, *dec_b;
+        int slot;
+    };
+
+  private:
+    MODELTYPE* _model;
+    std::thread _thread;
+    std::mutex _q_mutex;
+    std::deque<Sample*> _main_q;
+    std::mutex _pool_mutex;
+    std::condition_variable _pool_cv;
+    std::vector<ReqCtx*> _pool;
+    std::atomic<bool> _stop{false};
+    int _next_id = 0;
+
+  public:
+    std::vector<Sample*> exe_vec;
+    int schedule_deep = 6;            // schedule.h:30
+    float contention_factor = 0.8f;   // schedule.h:249
+    class_policy policy = RESOURCE;
+    split_axis axis = SPLIT_OUT_COLS;
+    int seq_bucket = 1;               // durations are looked up at seq rounded up to a multiple of this
+    int ignore_num = 20;              // warm-up records dropped from the report (schedule.h:327)
+    int profile_misses = 0;
+    int rounds = 0, secondary_launches = 0, splits = 0;
+    StaticInitParam SParams;
+    DynamicInitParam DParams0;
+    DynamicInitParam DParams1;
+    MainDict profiling_res_dict;
+    SubDict profiling_decompse_res_dict;
+    BertInitParam BertParams;
+    std::vector<recorder> recs;
+    T *input, *output;  // default buffers (profile / single request), like the reference's members
+    void *Main_EVENT = nullptr, *Wait_EVENT = nullptr;
+
+    Scheduler(MODELTYPE* model, const BertInitParam& BertParams_, const StaticInitParam& SParams_, T* input_, T* output_,
+              const std::string& main_filename = "", const std::string& sub_filename = "")
+        : _model(model), SParams(SParams_), DParams0(-4), DParams1(0), BertParams(BertParams_), input(input_), output(output_) {
+        DParams0.stream_id = 0;
+        DParams1.stream_id = 1;
+        if (!main_filename.empty()) MainFileToDict(main_filename, profiling_res_dict);
+        if (!sub_filename.empty()) SubFileToDict(sub_filename, profiling_decompse_res_dict);
+        note_status(lg_event_create(&Main_EVENT), "lg_event_create");
+        note_status(lg_event_create(&Wait_EVENT), "lg_event_create");
+    }
+    ~Scheduler() {
+        if (_thread.joinable()) _thread.join();
+    }
+
+    // ---- per-request contexts ------------------------------------------------------------------------------
+    // Allocates `count` contexts sized for (max_batch_size, max_seq_len); serve() blocks when all are in flight.
+    void make_pool(int count, int ctx_batch) {
+        const int H = BertParams.head_num * BertParams.size_per_head;
+        const int64_t io = (int64_t)ctx_batch * BertParams.max_seq_len * H;
+        const int64_t we = _model->workspace_elems(ctx_batch, BertParams.max_seq_len);
+        for (int i = 0; i < count; ++i) {
+            ReqCtx* c = new ReqCtx();
+            c->input = dev_alloc<T>(io);
+            c->output = dev_alloc<T>(io);
+            c->ws = dev_alloc<T>(we);
+            c->dec_a = dev_alloc<T>((int64_t)ctx_batch * H);
+            c->dec_b = dev_alloc<T>((int64_t)ctx_batch * H);
+            c->slot = _pool_total * ctx_batch;
+            dev_fill_normal(c->input, io, 1234, 50000 + _pool_total, 0.f, 1.f);
+            _pool.push_back(c);
+            _pool_total++;
+        }
+        note_status(lg_device_synchronize(), "lg_device_synchronize");
+    }
+    ReqCtx* acquire_ctx() {
+        std::unique_lock<std::mutex> lk(_pool_mutex);
+        _pool_cv.wait(lk, [this] { return !_pool.empty(); });
+        ReqCtx* c = _pool.back();
+        _pool.pop_back();
+        return c;
+    }
+    void release_ctx(ReqCtx* c) {
+        { std::lock_guard<std::mutex> lk(_pool_mutex); _pool.push_back(c); }
+        _pool_cv.notify_one();
+    }
+
+    // ---- profile  (schedule.h:79-157) -----------------------------------------------------------------------
+    float lookup(int name, int bs, int seq) {
+        auto it = profiling_res_dict.find({name, bs, seq});
+        if (it != profiling_res_dict.end()) return it->second;
+        if (seq_bucket > 1) {
+            it = profiling_res_dict.find({name, bs, (seq + seq_bucket - 1) / seq_bucket * seq_bucket});
+            if (it != profiling_res_dict.end()) return it->second;
+        }
+        profile_misses++;
+        return 0.f;  // the reference's operator[] yields 0 for a missing key as well
+    }
+
+    void profile_vector(std::vector<FuncWrap>& vec, int count, int name_base, int bs, int key_seq, int itr) {
+        void *e0 = nullptr, *e1 = nullptr;
+        note_status(lg_event_create(&e0), "lg_event_create");
+        note_status(lg_event_create(&e1), "lg_event_create");
+        for (int k = 0; k < count; k++) {
+            kernel_info info = {name_base + k, bs, key_seq};
+            profiling_res_dict[info] = profile_callback(vec[k], DParams0, e0, e1, itr, 3);
+            if (vec[k].type == GEMM && vec[k].args_gemm.valid && BertParams.factor > 1) {
+                std::vector<float> tmp;
+                for (int n = 1; n < BertParams.factor; n++) {
+                    FuncWrap fc = decompose_callback(vec[k], BertParams.factor, n, 0.f, 0, axis);
+                    tmp.push_back(profile_callback(fc, DParams0, e0, e1, itr, 3));
+                }
+                profiling_decompse_res_dict[info] = tmp;
+            }
+        }
+        lg_event_destroy(e0);
+        lg_event_destroy(e1);
+    }
+
+    // Profiles every (bs, seq) in the given ranges with bs*seq % 4 == 0, like the reference; seq advances by seq_step.
+    void profile(int low_bs, int high_bs, int low_sq, int high_sq, const std::string& main_filename,
+                 const std::string& sub_filename, int seq_step = 1, int itr = 20) {
+        for (int i = low_bs; i < high_bs; i++) {
+            for (int j = low_sq; j < high_sq; j += seq_step) {
+                if ((i * j) % 4 != 0) continue;
+                std::vector<FuncWrap> vec = _model->forward(input, output, i, j);
+                // run the layer once so that every kernel is timed on initialised data
+                for (int k = 0; k < BertParams.kernel_num; k++) vec[k].callback(DParams0);
+                profile_vector(vec, BertParams.kernel_num, 0, i, j, itr);
+            }
+        }
+        if (SParams.world_rank == 0) {
+            if (!main_filename.empty()) MainDictToFile(profiling_res_dict, main_filename);
+            if (!sub_filename.empty()) SubDictToFile(profiling_decompse_res_dict, sub_filename);
+        }
+    }
+    // Profiles one decode step at `past` cached positions; keys are {1000 + k, bs, past}.
+    void profile_decode(int bs, int past, int itr = 20) {
+        std::vector<FuncWrap> vec = _model->forward_decode(input, output, bs, past, 0);
+        const int count = _model->kernels_per_layer(true);
+        for (int k = 0; k < count; k++) vec[k].callback(DParams0);
+        profile_vector(vec, count, 1000, bs, past, itr);
+    }
+
+    // ---- serve  (schedule.h:159-172) ------------------------------------------------------------------------
+    // Builds the launch vector of one request (prefill of batch_size x seq_len, then n_decode decode steps), stamps
+    // kernel indices and profiled durations, and queues it.
+    void serve(int batch_size, int seq_len, int n_decode = 0) {
+        ReqCtx* ctx = _pool_total ? acquire_ctx() : nullptr;  // without a pool all requests share the default buffers
+        T* in = ctx ? ctx->input : input;
+        T* out = ctx ? ctx->output : output;
+        T* ws = ctx ? ctx->ws : nullptr;
+        const int slot = (ctx && BertParams.max_cache_len > 0) ? ctx->slot : -1;
+        std::vector<FuncWrap> vec = _model->forward(in, out, batch_size, seq_len, ws, slot);
+        for (int i = 0; i < BertParams.layer_num; i++)
+            for (int j = 0; j < BertParams.kernel_num; j++) {
+                FuncWrap& f = vec[i * BertParams.kernel_num + j];
+                f.name = j;
+                f.duration = lookup(j, batch_size, seq_len);
+            }
+        if (n_decode > 0 && ctx && slot >= 0) {
+            const int H = BertParams.head_num * BertParams.size_per_head;
+            const int kd = _model->kernels_per_layer(true);
+            T* din = ctx->dec_a;
+            T* dout = ctx->dec_b;
+            // the last token's hidden state of every sequence becomes the first decode input
+            {
+                const size_t row_bytes = (size_t)H * sizeof(T);
+                FuncWrap g(0.01f, COMPUTATION, [=](const DynamicInitParam& D) {
+                    for (int b = 0; b < batch_size; ++b)
+                        note_status(lg_memcpy_d2d_async((char*)din + b * row_bytes,
+                                                        (const char*)out + ((size_t)(b + 1) * seq_len - 1) * row_bytes, row_bytes,
+                                                        D.stream), "lg_memcpy_d2d_async");
+                }, "gather_last_token");
+                g.name = 900;
+                g.duration = 0.005f;
+                vec.push_back(g);
+            }
+            for (int t = 0; t < n_decode; ++t) {
+                const int past = seq_len + t;
+                std::vector<FuncWrap> dv = _model->forward_decode(din, dout, batch_size, past, slot, ws);
+                const int key_past = seq_bucket > 1 ? (past + seq_bucket - 1) / seq_bucket * seq_bucket : past;
+                for (size_t j = 0; j < dv.size(); ++j) {
+                    dv[j].name = 1000 + (int)(j % kd);
+                    dv[j].duration = lookup(dv[j].name, batch_size, key_past);
+                }
+                vec.insert(vec.end(), dv.begin(), dv.end());
+                std::swap(din, dout);
+            }
+        }
+        Sample* sample = new Sample(vec, profiling_decompse_res_dict, batch_size, seq_len, BertParams.factor, policy, axis);
+        sample->user = ctx;
+        {
+            std::lock_guard<std::mutex> lk(_q_mutex);
+            sample->id = _next_id++;
+            _main_q.push_back(sample);
+        }
+    }
+
+    size_t queued() {
+        std::lock_guard<std::mutex> lk(_q_mutex);
+        return _main_q.size();
+    }
+
+    // ---- admission / retirement  (schedule.h:175-202) ------------------------------------------------------------
+    void update_vec() {
+        if (!exe_vec.empty() && exe_vec[0]->empty()) {
+            Sample* tmp = exe_vec[0];
+            recs.push_back(tmp->get_recording());
+            exe_vec.erase(exe_vec.begin());
+            _retired.push_back(tmp);
+        }
+        _reclaim();
+        for (size_t i = exe_vec.size(); i < (size_t)schedule_deep; i++) {
+            std::lock_guard<std::mutex> lk(_q_mutex);
+            if (_main_q.empty()) break;
+            exe_vec.push_back(_main_q.front());
+            _main_q.pop_front();
+        }
+        if (exe_vec.empty()) std::this_thread::sleep_for(std::chrono::microseconds(100));
+    }
+
+    bool drained() { return exe_vec.empty() && queued() == 0; }
+
+    // ---- baseline: one request at a time on stream 0  (schedule.h:204-219) -----------------------------------------
+    void run_sequential() {
+        float time_planned = 0;
+        note_status(lg_event_record(Wait_EVENT, DParams0.stream), "lg_event_record");
+        while (!(_stop.load() && drained())) {
+            update_vec();
+            if (!exe_vec.empty()) {
+                note_status(lg_event_synchronize(Wait_EVENT), "lg_event_synchronize");
+                while (!exe_vec.at(0)->empty()) exe_vec.at(0)->dequeue(DParams0, 1, time_planned);
+                note_status(lg_event_record(Wait_EVENT, DParams0.stream), "lg_event_record");
+                rounds++;
+            }
+        }
+        _finish();
+    }
+
+    // ---- Liger: interleave the waiting requests into the primary's windows  (schedule.h:221-278) ----------------------
+    void run_stream_sync() {
+        float time_planned = 0.0f;
+        int main_class = 0;
+        note_status(lg_event_record(Wait_EVENT, DParams0.stream), "lg_event_record");
+        note_status(lg_event_record(Main_EVENT, DParams0.stream), "lg_event_record");
+        while (!(_stop.load() && drained())) {
+            update_vec();
+            if (exe_vec.empty()) continue;
+            // hybrid synchronisation: the host waits for everything before the last kernel of the previous round,
+            // stream 1 waits (on the device) for the end of the previous round
+            note_status(lg_event_synchronize(Wait_EVENT), "lg_event_synchronize");
+            note_status(lg_stream_wait_event(DParams1.stream, Main_EVENT), "lg_stream_wait_event");
+            Sample* head = exe_vec.at(0);
+            while (!head->empty()) {
+                main_class = head->next_class();
+                if (head->is_switch()) {
+                    note_status(lg_event_record(Wait_EVENT, DParams0.stream), "lg_event_record");
+                    time_planned += head->dequeue(DParams0, 1, time_planned);
+                    note_status(lg_event_record(Main_EVENT, DParams0.stream), "lg_event_record");
+                    break;
+                }
+                time_planned += head->dequeue(DParams0, 1, time_planned);
+            }
+            rounds++;
+            time_planned *= contention_factor;
+            for (size_t s = 1; s < exe_vec.size(); s++) {
+                Sample* sub = exe_vec.at(s);
+                while (time_planned > 0 && !sub->empty()) {
+                    if (sub->is_same_class(main_class)) break;
+                    if (sub->duration(0, time_planned) > time_planned) {
+                        if (sub->type() == GEMM && sub->possible_duration(time_planned)) {
+                            splits++;
+                            continue;  // the first piece now fits
+                        }
+                        time_planned = 0.0f;
+                    } else {
+                        time_planned -= sub->dequeue(DParams1, 0, time_planned);
+                        secondary_launches++;
+                    }
+                }
+            }
+            time_planned = 0.0f;
+        }
+        _finish();
+    }
+
+    void run_stop() { _stop.store(true); }
+    void reset_run() {
+        _stop.store(false);
+        for (auto& r : recs) { lg_event_destroy(r.start); lg_event_destroy(r.stop); }
+        recs.clear();
+        rounds = secondary_launches = splits = 0;
+    }
+
+    // ---- request simulator  (schedule.h:285-321) ---------------------------------------------------------------------
+    // Replays `trace` in real time on a second host thread, then requests stop.
+    void serving(const std::vector<TraceRequest>& trace) {
+        if (_thread.joinable()) _thread.join();
+        _thread = std::thread([this, trace]() {
+            const auto t0 = std::chrono::steady_clock::now();
+            for (const auto& r : trace) {
+                std::this_thread::sleep_until(t0 + std::chrono::duration_cast<std::chrono::steady_clock::duration>(
+                                                       std::chrono::duration<double>(r.arrival_s)));
+                serve(r.batch, r.seq, r.n_decode);
+            }
+            run_stop();
+        });
+    }
+    // the reference's generator: `count` requests of max batch, seq = rand() % (max_seq_len - 28) + 16 accepted when
+    // batch*seq % 4 == 0, spaced by rq_interval microseconds
+    std::vector<TraceRequest> reference_trace(int count, unsigned seed = 1) {
+        std::vector<TraceRequest> tr;
+        srand(seed);
+        double t = 0;
+        while ((int)tr.size() < count) {
+            const int bs = BertParams.max_batch_size;
+            const int sq = (rand() % (BertParams.max_seq_len - 28)) + 16;
+            if ((bs * sq) % 4 == 0) {
+                tr.push_back({t, bs, sq, 0});
+                t += BertParams.rq_interval * 1e-6;
+            }
+        }
+        return tr;
+    }
+
+    // ---- report  (schedule.h:325-350) ----------------------------------------------------------------------------------
+    Report output_recording(bool print = true) {
+        std::vector<double> cpu, gpu;
+        const size_t skip = std::min((size_t)std::max(0, ignore_num), recs.size());
+        for (size_t i = skip; i < recs.size(); ++i) {
+            float ms = 0.f;
+            note_status(lg_event_elapsed_ms(&ms, recs[i].start, recs[i].stop), "lg_event_elapsed_ms");
+            cpu.push_back(recs[i].cpu_time * 1000.0);
+            gpu.push_back(ms);
+            if (print) printf("request: %zu, CPU_Time: %f ms, CUDA_Time: %f ms. \n", i - skip, cpu.back(), gpu.back());
+        }
+        float total = 0.f;
+        if (recs.size() > skip) note_status(lg_event_elapsed_ms(&total, recs[skip].start, recs.back().stop), "lg_event_elapsed_ms");
+        Report r = summarize_records(cpu, gpu, total);
+        if (print) {
+            printf("Total_Duration: %f ms. \n", r.total_duration_ms);
+            printf("Throughput: %f samples/s. \n", r.throughput);
+            printf("Average Latency: %f ms. \n", r.avg_latency_ms);
+            printf("P99 Latency: %f ms. \n", r.p99_latency_ms);
+            printf("Total %d records. \n", r.records);
+        }
+        return r;
+    }
+
+  private:
+    std::vector<Sample*> _retired;
+    int _pool_total = 0;
+    // a retired sample's buffers may be reused once its last kernel has finished
+    void _reclaim() {
+        for (size_t i = 0; i < _retired.size();) {
+            Sample* s = _retired[i];
+            if (lg_event_query(s->stop) == LG_OK) {
+                if (s->user) release_ctx((ReqCtx*)s->user);
+                delete s;
+                _retired.erase(_retired.begin() + i);
+            } else {
+                ++i;
+            }
+        }
+    }
+    void _finish() {
+        note_status(lg_stream_synchronize(DParams0.stream), "lg_stream_synchronize");
+        note_status(lg_stream_synchronize(DParams1.stream), "lg_stream_synchronize");
+        _reclaim();
+        if (_thread.joinable()) _thread.join();
+    }
+};
+
+}  // namespace liger

@@ -1,0 +1,170 @@
+#!/usr/bin/env python3
+"""Benchmark of the Liger hot path on one MI355X.
+
+A step is one pass of the launch vector of one GLM-130B-shaped TP=2 layer shard over one prefill batch
+(BASELINE config 2: hidden 12288, 48 of 96 heads x 128, FFN 16384 of 32768, batch 8 x seq 512, causal, fp16).
+Prints one JSON line; `value` is milliseconds per layer-shard with inputs and weights resident in HBM.
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+
+CFG2 = dict(hidden=12288, heads_global=96, d=128, ffn_global=32768, world_size=2, batch=8, seq=512)
+CFG3 = dict(batch=32, cache_len=1024)
+
+
+def gemm_flops_cfg2():
+    M, H, Hl, F = 4096, 12288, 6144, 16384
+    return {"q": 2 * M * H * Hl, "k": 2 * M * H * Hl, "v": 2 * M * H * Hl, "out": 2 * M * Hl * H, "ffn1": 2 * M * H * F, "ffn2": 2 * M * F * H}
+
+
+def cpu_baseline(po, sample_batch=1, sample_seq=256):
+    """Times the CPU oracle (OpenMP C) on a bounded sample of the cfg2 layer: same shard shapes, M = sample rows,
+    and scales linearly to M = 4096 (GEMM time is linear in M; attention at this size is < 1 % of the work)."""
+    import numpy as np
+    H, h, d, F = 12288, 48, 128, 16384
+    Hl = h * d
+    w = {}
+    tid = 1
+    for name, shape, std, mean in (("wq", (H, Hl), 0.02, 0), ("wk", (H, Hl), 0.02, 0), ("wv", (H, Hl), 0.02, 0), ("bq", (Hl,), 0.02, 0),
+                                   ("bk", (Hl,), 0.02, 0), ("bv", (Hl,), 0.02, 0), ("wo", (Hl, H), 0.02, 0), ("ln1_g", (H,), 0.1, 1),
+                                   ("ln1_b", (H,), 0.1, 0), ("w1", (H, F), 0.02, 0), ("b1", (F,), 0.02, 0), ("w2", (F, H), 0.02, 0),
+                                   ("ln2_g", (H,), 0.1, 1), ("ln2_b", (H,), 0.1, 0)):
+        n = int(np.prod(shape))
+        w[name] = po.fill_normal(n, 0, tid, mean, std, po.F16).reshape(shape)
+        tid += 1
+    M = sample_batch * sample_seq
+    x = po.fill_normal(M * H, 0, 99, 0.0, 1.0, po.F16).reshape(M, H)
+    shape = dict(batch=sample_batch, seq=sample_seq, hidden=H, head_num=h, size_per_head=d, ffn_inner=F, causal=1, norm_mode=0, dtype=po.F16)
+    t0 = time.perf_counter()
+    po.encoder_forward(shape, w, x)
+    dt = time.perf_counter() - t0
+    scale = 4096.0 / M
+    return {"value": dt * 1e3 * scale, "unit": "ms/layer-shard", "cores": po.lib().lo_num_threads(), "kind": "port",
+            "sample": "cfg2 layer shard with batch %d x seq %d (M=%d of 4096 rows): %.2f s measured, scaled x%.0f" % (
+                sample_batch, sample_seq, M, dt, scale)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--unfused", action="store_true", help="time the reference-shaped 14-entry assembly instead")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs one GPU's tensor-parallel shard on one GPU; --gpus %d is not supported "
+              "(the all-reduce between GPUs is out of scope)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    liger = importlib.import_module("24ppopp-liger_amd")
+    host = importlib.import_module("24ppopp-liger_amd.host")
+    capi = liger.capi
+    torch.cuda.set_device(0)
+    info = capi.device_info()
+    c = CFG2
+    B, S, H = c["batch"], c["seq"], c["hidden"]
+    M = B * S
+    fused = not args.unfused
+    model = host.Model(capi.F16, 32, S, c["heads_global"], c["d"], layer_num=1, world_size=c["world_size"], ffn_inner=c["ffn_global"],
+                       norm_mode=host.POST_NORESID, causal=True, fused=fused, max_cache_len=CFG3["cache_len"] + 32 if fused else 0,
+                       seed=0)
+    x = torch.empty(M, H, device="cuda", dtype=torch.float16)
+    capi.call("lg_fill_normal_f16", x.data_ptr(), x.numel(), 0, 99, 0.0, 1.0, None)
+    y = torch.empty_like(x)
+    stream = model.stream
+
+    def step():
+        model.run(x.data_ptr(), y.data_ptr(), B, S, None, stream)
+
+    for _ in range(args.warmup):
+        step()
+    capi.call("lg_stream_synchronize", stream)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    capi.call("lg_stream_synchronize", stream)
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # per-kernel durations: HIP events on the launch stream, 2 warm-ups + 20 launches, min of 3 (the reference's profiler protocol)
+    desc = model.describe(B, S)
+    times = model.time_kernels(x.data_ptr(), y.data_ptr(), B, S)
+    kernels = [{"idx": e["idx"], "kernel": e["label"], "class": e["class"], "ms": round(t, 4)} for e, t in zip(desc, times)]
+    fl = gemm_flops_cfg2()
+    label_flops = {"q_gemm": fl["q"], "k_gemm": fl["k"], "v_gemm": fl["v"], "out_proj": fl["out"], "ffn1": fl["ffn1"], "ffn2": fl["ffn2"],
+                   "q_gemm+bias+heads": fl["q"], "k_gemm+bias+heads": fl["k"], "v_gemm+bias+heads": fl["v"], "ffn1+bias+gelu": fl["ffn1"]}
+    gemm_ms = 0.0
+    gemm_fl = 0.0
+    for k in kernels:
+        if k["kernel"] in label_flops:
+            k["tflops"] = round(label_flops[k["kernel"]] / (k["ms"] * 1e-3) / 1e12, 1)
+            gemm_ms += k["ms"]
+            gemm_fl += label_flops[k["kernel"]]
+    # dominant kernel = the FFN GEMM with the largest share of the step
+    dom = max((k for k in kernels if k["kernel"] in label_flops), key=lambda k: k["ms"])
+    dom_fl = label_flops[dom["kernel"]]
+    achieved = dom_fl / (dom["ms"] * 1e-3) / 1e12
+    roofline = {"bound": "mfma", "kernel": dom["kernel"], "achieved": round(achieved, 1), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(achieved / PEAK_FP16_TFLOPS, 4), "traffic": None,
+                "all_gemms_tflops": round(gemm_fl / (gemm_ms * 1e-3) / 1e12, 1)}
+    ln = [k for k in kernels if k["kernel"] == "layer_norm"]
+    ln_gbs = (2 * M * H * 2) / (min(k["ms"] for k in ln) * 1e-3) / 1e9 if ln else None
+
+    # decode step of the same shard (BASELINE config 3): batch 32, one token, 1024 cached positions
+    decode = None
+    if fused:
+        Bd, L = CFG3["batch"], CFG3["cache_len"]
+        xd = torch.empty(Bd, H, device="cuda", dtype=torch.float16)
+        capi.call("lg_fill_normal_f16", xd.data_ptr(), xd.numel(), 0, 98, 0.0, 1.0, None)
+        yd = torch.empty_like(xd)
+        ddesc = model.describe(Bd, 1, decode_past=L - 1)
+        dtimes = model.time_kernels(xd.data_ptr(), yd.data_ptr(), Bd, 1, decode_past=L - 1, cache_slot=0)
+        dk = [{"idx": e["idx"], "kernel": e["label"], "ms": round(t, 4)} for e, t in zip(ddesc, dtimes)]
+        attn = [k for k in dk if k["kernel"] == "attn_decode"][0]
+        kv_bytes = 2 * Bd * 48 * L * 128 * 2
+        w_bytes = (3 * H * 6144 + 6144 * H + 2 * H * 16384) * 2
+        gemm_dec_ms = sum(k["ms"] for k in dk if "gemm" in k["kernel"] or "proj" in k["kernel"] or "ffn" in k["kernel"])
+        decode = {"workload": "cfg3: batch 32, 1 new token, 1024 cached positions", "ms_per_layer_shard": round(sum(dtimes), 4),
+                  "tokens_per_s": round(Bd / (sum(dtimes) * 1e-3), 1), "kernels": dk,
+                  "roofline_attn_decode": {"bound": "hbm", "achieved": round(kv_bytes / (attn["ms"] * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
+                                           "unit": "GB/s", "frac": round(kv_bytes / (attn["ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)},
+                  "skinny_gemms": {"ms": round(gemm_dec_ms, 4), "weight_GBps": round(w_bytes / (gemm_dec_ms * 1e-3) / 1e9, 1)}}
+
+    out = {
+        "metric": "ms/layer-shard prefill (GLM-130B TP=2 shard, B8 S512, causal, fp16)",
+        "value": round(ms_per_step, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "cfg2 prefill: hidden 12288, 48/96 heads x 128, FFN 16384/32768, batch 8 x seq 512, causal; "
+                               + ("fused assembly (9 launches/layer)" if fused else "reference-shaped assembly (14 launches/layer)")},
+        "tokens_per_s": round(M / (ms_per_step * 1e-3), 1),
+        "roofline": roofline,
+        "layer_norm_GBps": round(ln_gbs, 1) if ln_gbs else None,
+        "kernels": kernels,
+        "sum_kernel_ms": round(sum(times), 4),
+        "decode": decode,
+        "device": info,
+        "peaks": {"fp16_mfma_TFLOPs": PEAK_FP16_TFLOPS, "hbm_GBps": PEAK_HBM_GBS},
+    }
+    if not args.no_cpu_baseline:
+        from oracle import pyoracle as po
+        out["cpu_baseline"] = cpu_baseline(po)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -144,23 +144,28 @@ int lg_gemm_strided_batched_f16(int transa, int transb, int m, int n, int k, con
 #define LG_EPI_NONE 0
 #define LG_EPI_BIAS 1      /* C = acc + bias[m-index]                    */
 #define LG_EPI_BIAS_GELU 2 /* C = gelu_tanh(acc + bias[m-index])   == lg_gemm + lg_add_bias_act        */
-#define LG_EPI_BIAS_HEADS 3 /* C is written as [batch, head, seq, d] == lg_gemm + lg_add_qkv_bias_transpose
-                               for one of Q/K/V; needs seq and size_per_head in `epi_arg0/1`            */
+#define LG_EPI_BIAS_HEADS 3 /* C is written as [batch, head, row, d] == lg_gemm + lg_add_qkv_bias_transpose
+                               for one of Q/K/V.  epi_arg0 = seq (tokens per sequence), epi_arg1 =
+                               size_per_head, epi_arg2 = heads per batch entry in C (0 -> m / size_per_head;
+                               larger when C is a slice of a wider buffer), and ldc = rows reserved per
+                               (batch, head) in C (>= seq; > seq when C is a KV cache)                     */
 /* lg_gemm_f16 with a fused epilogue (the bias / GELU / head-transpose kernels that follow the GEMMs in
  * the launch vector, bert_layer.h:54-56,139-142, folded into the GEMM's store).  No reference
  * counterpart; results equal the two-kernel sequence up to one fp16 rounding. */
 int lg_gemm_fused_f16(int transa, int m, int n, int k, const void* A, int lda, const void* B, int ldb, void* C,
-                      int ldc, int epilogue, const void* bias, int epi_arg0, int epi_arg1, void* stream);
+                      int ldc, int epilogue, const void* bias, int epi_arg0, int epi_arg1, int epi_arg2,
+                      void* stream);
 
 /* ---- attention kernels with no reference counterpart --------------------------------------------- */
-/* Fused prefill attention over [B,h,S,d] buffers: out = softmax(q k^T * scalar + maskterm) v with the
- * reference's softmax semantics (-10000 additive mask, +1e-6 in the denominator); replaces launch-vector
- * entries 4,5,6 (and 7 when out_layout = 1).  causal != 0: implicit lower-triangular mask (attr_mask
- * ignored, may be NULL); causal == 0: attr_mask [B,S,S] of 0/1 or NULL for all ones.
- * out_layout 0: [B,h,S,d]; 1: [B,S,h,d] (= transpose-back fused).  size_per_head must be 64 or 128. */
+/* Fused prefill attention: out = softmax(q k^T * scalar + maskterm) v with the reference's softmax
+ * semantics (-10000 additive mask, +1e-6 in the denominator); replaces launch-vector entries 4,5,6 (and 7
+ * when out_layout = 1).  q_buf [B,h,S,d]; k_buf, v_buf [B,h,kv_rows,d] with the S valid rows first
+ * (kv_rows = S for plain buffers, = max_len when they are a KV cache).  causal != 0: implicit
+ * lower-triangular mask (attr_mask ignored, may be NULL); causal == 0: attr_mask [B,S,S] of 0/1 or NULL
+ * for all ones.  out_layout 0: [B,h,S,d]; 1: [B,S,h,d] (= transpose-back fused).  size_per_head: 64 or 128. */
 int lg_attn_prefill_f16(const void* q_buf, const void* k_buf, const void* v_buf, const void* attr_mask,
-                        void* out, int batch, int seq, int head_num, int size_per_head, float scalar,
-                        int causal, int out_layout, void* stream);
+                        void* out, int batch, int seq, int head_num, int size_per_head, int kv_rows,
+                        float scalar, int causal, int out_layout, void* stream);
 /* Decode attention: q [B,h,d]; k_cache, v_cache [B,h,max_len,d] with `len` valid positions; out [B,h,d].
  * workspace: float buffer of lg_attn_decode_workspace_bytes(...) bytes (split-KV partials), caller-owned. */
 size_t lg_attn_decode_workspace_bytes(int batch, int head_num, int size_per_head, int max_len);

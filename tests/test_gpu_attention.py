@@ -46,3 +46,51 @@ def test_kv_append(dev, po, B, h, d, pos, Lmax):
     assert np.array_equal(dev.down(dkc), kc)
     assert np.array_equal(dev.down(dvc), vc)
     assert np.array_equal(dev.down(dq), po.round_f16(Q + bq).reshape(B, h, d))
+
+
+@pytest.mark.parametrize("B,h,S,d,mode,kv_rows,layout", [
+    (2, 3, 128, 128, "causal", 128, 0), (1, 2, 200, 64, "causal", 256, 1), (2, 2, 77, 128, "mask", 77, 1),
+    (1, 1, 512, 128, "none", 512, 0), (1, 2, 1000, 128, "causal", 1024, 1), (1, 1, 5, 64, "causal", 8, 0)])
+def test_attn_prefill_fused(dev, po, B, h, S, d, mode, kv_rows, layout):
+    """Fused attention == qk_gemm -> softmax -> qkv_gemm (-> transpose) of the oracle, fp16 semantics."""
+    q = rnd(po, B * h * S * d, 70).reshape(B, h, S, d)
+    k = rnd(po, B * h * S * d, 71).reshape(B, h, S, d)
+    v = rnd(po, B * h * S * d, 72).reshape(B, h, S, d)
+    scalar = 1.0 / np.sqrt(d)
+    if mode == "mask":
+        mask = (po.fill_normal(B * S * S, 0, 73).reshape(B, S, S) > -0.8).astype(np.float32)
+        mask[:, 3, :] = 0.0  # a fully masked row must still follow the additive -10000 semantics
+        nb = B * h
+        scores = np.zeros((nb, S, S), dtype=np.float32)
+        po.gemm_strided_batched(1, 0, S, S, d, k.reshape(nb, S, d), d, S * d, q.reshape(nb, S, d), d, S * d, scores, S, S * S, nb, 1)
+        po.attn_softmax(scores.reshape(B, h, S, S), mask, scalar, 1)
+        ref = np.zeros((nb, S, d), dtype=np.float32)
+        po.gemm_strided_batched(0, 0, d, S, S, v.reshape(nb, S, d), d, S * d, scores, S, S * S, ref, d, S * d, nb, 1)
+        ref = ref.reshape(B, h, S, d)
+        dmask = dev.up(mask, 1)
+    else:
+        ref = po.attn_prefill(q, k, v, scalar, mode == "causal", 1)
+        dmask = None
+    kpad = np.zeros((B, h, kv_rows, d), dtype=np.float32); vpad = np.full((B, h, kv_rows, d), 7.0, dtype=np.float32)
+    kpad[:, :, :S] = k; vpad[:, :, :S] = v
+    out = dev.empty((B, S, h, d) if layout else (B, h, S, d), 1)
+    dev.call("lg_attn_prefill_f16", dev.up(q, 1), dev.up(kpad, 1), dev.up(vpad, 1), dmask if dmask is not None else 0, out,
+             B, S, h, d, kv_rows, float(scalar), int(mode == "causal"), layout)
+    got = dev.down(out)
+    if layout:
+        got = got.transpose(0, 2, 1, 3)
+    if mode == "mask":
+        # On the fully masked row the reference's half kernel adds -10000 in fp16 (spacing 8 at that magnitude), which
+        # quantises the scores; the fused kernel adds it in fp32.  There the fp32-semantics oracle is the yardstick:
+        # a constant shift cancels and the row is the plain softmax.
+        scores32 = np.zeros((B * h, S, S), dtype=np.float32)
+        nb = B * h
+        po.gemm_strided_batched(1, 0, S, S, d, k.reshape(nb, S, d), d, S * d, q.reshape(nb, S, d), d, S * d, scores32, S, S * S, nb, 0)
+        po.attn_softmax(scores32.reshape(B, h, S, S), mask, scalar, 0)
+        ref32 = np.zeros((nb, S, d), dtype=np.float32)
+        po.gemm_strided_batched(0, 0, d, S, S, v.reshape(nb, S, d), d, S * d, scores32, S, S * S, ref32, d, S * d, nb, 0)
+        ref32 = ref32.reshape(B, h, S, d)
+        assert max_rel_err(got[:, :, 3], ref32[:, :, 3]) < 1e-2
+        got = np.delete(got, 3, axis=2)
+        ref = np.delete(ref, 3, axis=2)
+    assert max_rel_err(got, ref) < 1e-2

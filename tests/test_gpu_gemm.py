@@ -105,12 +105,12 @@ def test_gemm_fused_epilogues(dev, po, transa):
     y = po.gemm(X, W, 1)
     ref_gelu = po.add_bias_gelu(y.copy(), bias, 1)
     out = dev.empty((M, N), 1)
-    dev.call("lg_gemm_fused_f16", transa, N, M, K, dA, lda, dX, K, out, N, dev.capi.EPI_BIAS_GELU, dB, 0, 0)
+    dev.call("lg_gemm_fused_f16", transa, N, M, K, dA, lda, dX, K, out, N, dev.capi.EPI_BIAS_GELU, dB, 0, 0, 0)
     assert max_rel_err(dev.down(out), ref_gelu) < 4e-3
     ref_heads, _, _ = po.add_qkv_bias_transpose(y, bias, y, bias, y, bias, B, S, h, d, 1)
     out = dev.empty((B, h, S, d), 1)
-    dev.call("lg_gemm_fused_f16", transa, N, M, K, dA, lda, dX, K, out, N, dev.capi.EPI_BIAS_HEADS, dB, S, d)
+    dev.call("lg_gemm_fused_f16", transa, N, M, K, dA, lda, dX, K, out, S, dev.capi.EPI_BIAS_HEADS, dB, S, d, 0)
     assert max_rel_err(dev.down(out), ref_heads) < 2e-3
     out = dev.empty((M, N), 1)
-    dev.call("lg_gemm_fused_f16", transa, N, M, K, dA, lda, dX, K, out, N, dev.capi.EPI_BIAS, dB, 0, 0)
+    dev.call("lg_gemm_fused_f16", transa, N, M, K, dA, lda, dX, K, out, N, dev.capi.EPI_BIAS, dB, 0, 0, 0)
     assert max_rel_err(dev.down(out), po.round_f16(y + bias)) < 2e-3

@@ -1,0 +1,100 @@
+"""GPU parity of whole layers assembled by the C++ launch-vector runtime against the CPU oracle.
+
+The model initialises its own parameters on the device (seeded generator); the test downloads them, so the oracle
+sees bit-identical weights.  Tolerance for fp16: max |gpu - oracle| / max |oracle| <= 1e-2 (the stated bar).
+"""
+import importlib
+
+import numpy as np
+import pytest
+
+from tests.conftest import max_rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def host(liger):
+    return importlib.import_module("24ppopp-liger_amd.host")
+
+
+def oracle_weights(params, layer=0):
+    pre = "layer%d." % layer
+    return {k[len(pre):]: v for k, v in params.items() if k.startswith(pre)}
+
+
+def run_layer_case(dev, po, host, dtype, B, S, heads, d, F, norm_mode, causal, fused, ws=1, layers=1, seed=0):
+    H = heads * d
+    m = host.Model(dtype, B, S, heads, d, layer_num=layers, world_size=ws, ffn_inner=F, norm_mode=norm_mode, causal=causal,
+                   fused=fused, seed=seed)
+    params = m.download_params()
+    x = po.fill_normal(B * S * H, seed, 99, 0.0, 1.0, dtype).reshape(B * S, H)
+    dx = dev.up(x, dtype)
+    dy = dev.empty((B * S, H), dtype)
+    m.run(dx.data_ptr(), dy.data_ptr(), B, S, None, dev.stream)
+    got = dev.down(dy)
+    shape = dict(batch=B, seq=S, hidden=H, head_num=heads // ws, size_per_head=d, ffn_inner=(F or 4 * H) // ws,
+                 causal=int(causal), norm_mode=norm_mode, dtype=dtype)
+    ref = x
+    for l in range(layers):
+        ref = po.encoder_forward(shape, oracle_weights(params, l), ref)
+    return got, ref, m
+
+
+def test_cfg1_plumbing_fp32_prelayernorm(dev, po, host):
+    """BASELINE config 1: hidden 256, 4 heads x 64, FFN 1024 (GELU), pre-LayerNorm, batch 2, seq 32, fp32, seed 0."""
+    got, ref, m = run_layer_case(dev, po, host, 0, 2, 32, 4, 64, 1024, host.PRE_LN_RESID, False, False)
+    assert m.kernels_per_layer() == 15
+    assert max_rel_err(got, ref) < 2e-5
+
+
+def test_cfg1_reference_assembly_fp32(dev, po, host):
+    """The order src/layer/bert.h assembles (MHA -> LN -> MLP -> LN), 14 entries per layer on one GPU."""
+    got, ref, m = run_layer_case(dev, po, host, 0, 2, 32, 4, 64, 1024, host.POST_NORESID, False, False)
+    assert m.kernels_per_layer() == 14
+    labels = [e["label"] for e in m.describe(2, 32)]
+    assert labels == ["q_gemm", "k_gemm", "v_gemm", "qkv_bias_transpose", "qk_gemm", "softmax", "pv_gemm", "transpose_back",
+                      "out_proj", "layer_norm", "ffn1", "bias+gelu", "ffn2", "layer_norm"]
+    assert max_rel_err(got, ref) < 2e-5
+
+
+@pytest.mark.parametrize("norm_mode", [0, 1])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("fused", [False, True])
+def test_fp16_layer_small(dev, po, host, norm_mode, causal, fused):
+    got, ref, _ = run_layer_case(dev, po, host, 1, 2, 96, 4, 64, 512, norm_mode, causal, fused)
+    assert max_rel_err(got, ref) < 1e-2
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_fp16_tp2_shard_two_layers(dev, po, host, fused):
+    """One TP=2 shard (half the heads, half the FFN) of a 2-layer stack, GLM-like head size 128, ragged seq."""
+    got, ref, _ = run_layer_case(dev, po, host, 1, 2, 200, 8, 128, 2048, 0, True, fused, ws=2, layers=2)
+    assert max_rel_err(got, ref) < 1e-2
+
+
+def test_decode_step_matches_oracle(dev, po, host):
+    """Fused prefill fills the KV cache, then two decode steps; each is checked against the oracle's decoder step."""
+    B, S, heads, d, F, Lmax = 2, 40, 4, 64, 512, 64
+    H = heads * d
+    m = host.Model(1, B, S, heads, d, layer_num=1, ffn_inner=F, causal=True, fused=True, max_cache_len=Lmax, seed=3)
+    w = oracle_weights(m.download_params())
+    x = po.fill_normal(B * S * H, 3, 99, 0.0, 1.0, 1).reshape(B * S, H)
+    dx, dy = dev.up(x, 1), dev.empty((B * S, H), 1)
+    m.run(dx.data_ptr(), dy.data_ptr(), B, S, None, dev.stream, cache_slot=0)
+    shape = dict(batch=B, seq=S, hidden=H, head_num=heads, size_per_head=d, ffn_inner=F, causal=1, norm_mode=0, dtype=1)
+    ref_prefill = po.encoder_forward(shape, w, x)
+    assert max_rel_err(dev.down(dy), ref_prefill) < 1e-2
+    # oracle-side cache from the same prefill
+    q = po.gemm(x, w["wq"].reshape(H, H), 1); k = po.gemm(x, w["wk"].reshape(H, H), 1); v = po.gemm(x, w["wv"].reshape(H, H), 1)
+    _, kb, vb = po.add_qkv_bias_transpose(q, w["bq"], k, w["bk"], v, w["bv"], B, S, heads, d, 1)
+    kc = np.zeros((B, heads, Lmax, d), dtype=np.float32); vc = np.zeros_like(kc)
+    kc[:, :, :S] = kb; vc[:, :, :S] = vb
+    tok = po.fill_normal(B * H, 3, 100, 0.0, 1.0, 1).reshape(B, H)
+    for step in range(2):
+        dt_in, dt_out = dev.up(tok, 1), dev.empty((B, H), 1)
+        m.run_decode(dt_in.data_ptr(), dt_out.data_ptr(), B, S + step, 0, None, dev.stream)
+        ref = po.decoder_step(shape, w, tok, kc, vc, S + step)
+        got = dev.down(dt_out)
+        assert max_rel_err(got, ref) < 1e-2
+        tok = po.round_f16(ref)
