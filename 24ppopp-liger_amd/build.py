@@ -86,9 +86,26 @@ def build_host(force=True, verbose=False):
     return lib
 
 
+def build_fake_host(force=True):
+    """The same host runtime linked against tests/fake_backend (virtual-time stand-in for the device library):
+    lets the scheduler logic be unit-tested without a GPU.  Test infrastructure; never loaded by the product."""
+    fake_dir = os.path.join(ROOT, "tests", "fake_backend")
+    src = os.path.join(fake_dir, "fake_hip.cpp")
+    if not os.path.exists(src):
+        return None
+    lib = os.path.join(fake_dir, "libliger_host_fake.so")
+    srcs = [os.path.join(HOST, f) for f in sorted(os.listdir(HOST)) if f.endswith(".cpp") and f != "liger_main.cpp"] + [src]
+    hdrs = [os.path.join(HOST, f) for f in os.listdir(HOST) if f.endswith(".h")] + [os.path.join(ROOT, "include", "liger_hip.h")]
+    if force or _stale(lib, srcs + hdrs):
+        _run(["g++", "-O1", "-g", "-std=c++17", "-fPIC", "-Wall", "-Wextra", "-Wno-unused-parameter", "-pthread", "-I",
+              os.path.join(ROOT, "include"), "-I", HOST, "-shared", "-Wl,-Bsymbolic", "-o", lib] + srcs)
+    return lib
+
+
 def build_all(force=True, verbose=False):
     dev = build_device(force=force, verbose=verbose)
     host = build_host(force=force, verbose=verbose)
+    build_fake_host(force=force)
     return dev, host
 
 

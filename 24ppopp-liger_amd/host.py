@@ -50,15 +50,18 @@ SIGNATURES = {
     "lgh_sched_lookup": (_f, [_p, _i, _i, _i]),
     "lgh_sched_sub_lookup": (_i, [_p, _i, _i, _i, C.POINTER(_f), _i]),
     "lgh_sched_run_trace": (_i, [_p, _i, C.POINTER(_d), C.POINTER(_i), C.POINTER(_i), C.POINTER(_i), _i, C.POINTER(Report)]),
+    "lgh_sched_set_profile": (_i, [_p, _i, _i, _i, _f, C.POINTER(_f), _i]),
+    "lgh_sched_serve": (_i, [_p, _i, _i, _i]),
+    "lgh_sched_run_queued": (_i, [_p, _i, C.POINTER(Report)]),
     "lgh_summarize": (_i, [C.POINTER(_d), C.POINTER(_d), _i, _d, C.POINTER(Report)]),
     "lgh_make_poisson_trace": (_i, [_d, _i, _i, _i, _i, _i, _i, _u64, C.POINTER(_d), C.POINTER(_i)]),
 }
 
 
-def _load():
-    if not os.path.exists(LIB_PATH):
-        raise ImportError("libliger_host.so is not built (expected at %s); run __graft_entry__.build()" % LIB_PATH)
-    lib = C.CDLL(LIB_PATH, mode=C.RTLD_GLOBAL)
+def _load(path=LIB_PATH, mode=C.RTLD_GLOBAL):
+    if not os.path.exists(path):
+        raise ImportError("%s is not built; run __graft_entry__.build()" % path)
+    lib = C.CDLL(path, mode=mode)
     for name, (res, args) in SIGNATURES.items():
         fn = getattr(lib, name)
         fn.restype = res
@@ -67,6 +70,15 @@ def _load():
 
 
 lib = _load()
+
+
+def use_library(path):
+    """Rebinds this module to another build of the host runtime.  Exists for the CPU unit tests, which link the same
+    runtime sources against a virtual-time stand-in for the device library; returns the previous binding."""
+    global lib
+    prev = lib
+    lib = _load(path, C.RTLD_LOCAL)
+    return prev
 
 
 def first_error():
@@ -193,6 +205,18 @@ class Scheduler:
         out = (C.c_float * 64)()
         n = lib.lgh_sched_sub_lookup(self.h, name, bs, seq, out, 64)
         return None if n < 0 else [out[i] for i in range(n)]
+
+    def set_profile(self, name, bs, seq, ms, sub=None):
+        arr = (C.c_float * len(sub))(*sub) if sub else None
+        check(lib.lgh_sched_set_profile(self.h, name, bs, seq, ms, arr, len(sub) if sub else 0), "lgh_sched_set_profile")
+
+    def serve(self, bs, seq, n_decode=0):
+        check(lib.lgh_sched_serve(self.h, bs, seq, n_decode), "lgh_sched_serve")
+
+    def run_queued(self, mode):
+        r = Report()
+        check(lib.lgh_sched_run_queued(self.h, mode, C.byref(r)), "lgh_sched_run_queued")
+        return r.as_dict()
 
     def run_trace(self, trace, mode):
         n = len(trace)

@@ -24,6 +24,9 @@ struct SchedBase {
     virtual Report run(int mode, const std::vector<TraceRequest>& trace, int* counters) = 0;
     virtual float lookup(int name, int bs, int seq) = 0;
     virtual int sub_lookup(int name, int bs, int seq, float* out, int cap) = 0;
+    virtual void set_profile(int name, int bs, int seq, float ms, const float* sub, int nsub) = 0;
+    virtual void serve(int bs, int seq, int n_decode) = 0;
+    virtual Report run_queued(int mode, int* counters) = 0;
 };
 
 struct ModelBase {
@@ -70,6 +73,19 @@ struct SchedT : SchedBase {
         return r;
     }
     float lookup(int name, int bs, int seq) override { return s->lookup(name, bs, seq); }
+    void set_profile(int name, int bs, int seq, float ms, const float* sub, int nsub) override {
+        s->profiling_res_dict[{name, bs, seq}] = ms;
+        if (sub && nsub > 0) s->profiling_decompse_res_dict[{name, bs, seq}] = std::vector<float>(sub, sub + nsub);
+    }
+    void serve(int bs, int seq, int n_decode) override { s->serve(bs, seq, n_decode); }
+    Report run_queued(int mode, int* counters) override {
+        s->reset_run();
+        s->run_stop();  // everything is already queued: the loop ends once it has drained
+        if (mode == 0) s->run_sequential(); else s->run_stream_sync();
+        Report r = s->output_recording(false);
+        if (counters) { counters[0] = s->rounds; counters[1] = s->secondary_launches; counters[2] = s->splits; counters[3] = s->profile_misses; }
+        return r;
+    }
     int sub_lookup(int name, int bs, int seq, float* out, int cap) override {
         auto it = s->profiling_decompse_res_dict.find({name, bs, seq});
         if (it == s->profiling_decompse_res_dict.end()) return -1;
@@ -295,6 +311,27 @@ int lgh_sched_run_trace(void* sched, int mode, const double* arrival_s, const in
     for (int i = 0; i < n; ++i) tr.push_back({arrival_s[i], batch[i], seq[i], n_decode ? n_decode[i] : 0});
     int c[4] = {0, 0, 0, 0};
     Report r = ((SchedBase*)sched)->run(mode, tr, c);
+    out->records = r.records; out->avg_latency_ms = r.avg_latency_ms; out->p99_latency_ms = r.p99_latency_ms;
+    out->avg_gpu_ms = r.avg_gpu_ms; out->avg_queue_ms = r.avg_queue_ms; out->total_duration_ms = r.total_duration_ms;
+    out->throughput = r.throughput; out->rounds = c[0]; out->secondary_launches = c[1]; out->splits = c[2]; out->profile_misses = c[3];
+    return first_error();
+}
+// Deterministic variant for tests: requests are queued up front with lgh_sched_serve (no request thread, no real-time
+// arrivals), then lgh_sched_run_queued drains them.
+int lgh_sched_set_profile(void* sched, int name, int bs, int seq, float ms, const float* sub, int nsub) {
+    if (!sched) return fail("lgh_sched_set_profile: null");
+    ((SchedBase*)sched)->set_profile(name, bs, seq, ms, sub, nsub);
+    return LG_OK;
+}
+int lgh_sched_serve(void* sched, int bs, int seq, int n_decode) {
+    if (!sched || bs <= 0 || seq <= 0 || n_decode < 0) return fail("lgh_sched_serve: bad arguments");
+    ((SchedBase*)sched)->serve(bs, seq, n_decode);
+    return first_error();
+}
+int lgh_sched_run_queued(void* sched, int mode, LghReport* out) {
+    if (!sched || !out) return fail("lgh_sched_run_queued: bad arguments");
+    int c[4] = {0, 0, 0, 0};
+    Report r = ((SchedBase*)sched)->run_queued(mode, c);
     out->records = r.records; out->avg_latency_ms = r.avg_latency_ms; out->p99_latency_ms = r.p99_latency_ms;
     out->avg_gpu_ms = r.avg_gpu_ms; out->avg_queue_ms = r.avg_queue_ms; out->total_duration_ms = r.total_duration_ms;
     out->throughput = r.throughput; out->rounds = c[0]; out->secondary_launches = c[1]; out->splits = c[2]; out->profile_misses = c[3];

@@ -1,0 +1,189 @@
+// fake_hip.cpp -- a host-only stand-in for the device library, for unit tests of the launch-vector runtime.
+//
+// TEST INFRASTRUCTURE.  It exports every symbol of include/liger_hip.h but computes nothing: each "kernel launch"
+// appends a record (stream, kernel name, problem size, pointers, virtual start/end time) to a trace and advances a
+// virtual clock by a deterministic cost; streams are timelines, events are timestamps.  With it the Sample / Scheduler
+// policy (src/schedule.h:221-278, src/init.h:121-259 of the reference) can be asserted launch by launch on a machine
+// without a GPU.  Memory "on the device" is ordinary host memory that is never dereferenced by the fake kernels.
+#include <algorithm>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "liger_hip.h"
+
+namespace {
+
+struct Stream { double ready = 0; int id = 0; };
+struct Event { double time = 0; bool recorded = false; };
+struct Launch {
+    int stream; char name[48]; long long a, b, c;  // problem size (m, n, k) or (rows, cols, 0)
+    const void* p0; const void* p1; void* p2; double start, end;
+};
+
+std::mutex g_mu;
+double g_host_now = 0;          // virtual milliseconds
+double g_launch_cost = 0.002;   // host time per launch call
+double g_mfma_rate = 1.0e9;     // flop per virtual ms
+double g_hbm_rate = 1.0e6;      // bytes per virtual ms
+std::vector<Stream*> g_streams;
+std::vector<Launch> g_trace;
+Stream g_default;
+
+Stream* S(void* s) { return s ? (Stream*)s : &g_default; }
+
+int launch(void* stream, const char* name, long long a, long long b, long long c, const void* p0, const void* p1, void* p2, double cost) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    Stream* s = S(stream);
+    g_host_now += g_launch_cost;
+    Launch l;
+    l.stream = s->id;
+    strncpy(l.name, name, sizeof(l.name) - 1);
+    l.name[sizeof(l.name) - 1] = 0;
+    l.a = a; l.b = b; l.c = c; l.p0 = p0; l.p1 = p1; l.p2 = p2;
+    l.start = std::max(s->ready, g_host_now);
+    l.end = l.start + cost;
+    s->ready = l.end;
+    g_trace.push_back(l);
+    return LG_OK;
+}
+double gemm_cost(long long m, long long n, long long k) { return 0.003 + 2.0 * m * n * k / g_mfma_rate; }
+double mem_cost(double bytes) { return 0.003 + bytes / g_hbm_rate; }
+
+}  // namespace
+
+extern "C" {
+
+// ---- test controls -------------------------------------------------------------------------------------------------
+void fake_reset(void) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    g_trace.clear();
+    g_host_now = 0;
+    g_default.ready = 0;
+    for (auto* s : g_streams) s->ready = 0;
+}
+void fake_set_rates(double mfma_flop_per_ms, double hbm_bytes_per_ms, double launch_cost_ms) {
+    g_mfma_rate = mfma_flop_per_ms; g_hbm_rate = hbm_bytes_per_ms; g_launch_cost = launch_cost_ms;
+}
+int fake_trace_count(void) { std::lock_guard<std::mutex> lk(g_mu); return (int)g_trace.size(); }
+int fake_trace_get(int i, int* stream, char* name, int name_len, long long* abc, unsigned long long* ptrs, double* start_end) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (i < 0 || i >= (int)g_trace.size()) return 1;
+    const Launch& l = g_trace[i];
+    *stream = l.stream;
+    strncpy(name, l.name, (size_t)name_len - 1); name[name_len - 1] = 0;
+    abc[0] = l.a; abc[1] = l.b; abc[2] = l.c;
+    ptrs[0] = (unsigned long long)(uintptr_t)l.p0; ptrs[1] = (unsigned long long)(uintptr_t)l.p1; ptrs[2] = (unsigned long long)(uintptr_t)l.p2;
+    start_end[0] = l.start; start_end[1] = l.end;
+    return 0;
+}
+double fake_host_now(void) { return g_host_now; }
+
+// ---- library / runtime ------------------------------------------------------------------------------------------------
+const char* lg_last_error(void) { return "fake backend: no error text"; }
+const char* lg_version(void) { return "liger-fake 0.1 (virtual time)"; }
+int lg_device_info(char* name, int name_len, int* cu, int* clk, int* mclk, int* bus, size_t* mem) {
+    if (name && name_len > 0) { strncpy(name, "fake", (size_t)name_len - 1); name[name_len - 1] = 0; }
+    if (cu) *cu = 256; if (clk) *clk = 2400000; if (mclk) *mclk = 2000000; if (bus) *bus = 8192; if (mem) *mem = (size_t)1 << 38;
+    return LG_OK;
+}
+int lg_malloc(void** ptr, size_t bytes) {
+    // address space only: the fake kernels never touch the memory, so reserve small real blocks and hand out
+    // distinct, correctly spaced addresses from a bump counter
+    static uintptr_t next = 0x100000000ull;
+    std::lock_guard<std::mutex> lk(g_mu);
+    *ptr = (void*)next;
+    next += (bytes + 255) / 256 * 256 + 256;
+    return LG_OK;
+}
+int lg_free(void*) { return LG_OK; }
+int lg_memcpy_h2d(void*, const void*, size_t) { return LG_OK; }
+int lg_memcpy_d2h(void*, const void*, size_t) { return LG_OK; }
+int lg_memcpy_d2d_async(void* dst, const void* src, size_t bytes, void* stream) { return launch(stream, "memcpy_d2d", (long long)bytes, 0, 0, src, nullptr, dst, mem_cost(2.0 * bytes)); }
+int lg_memset_async(void*, int, size_t, void*) { return LG_OK; }
+int lg_device_synchronize(void) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    g_host_now = std::max(g_host_now, g_default.ready);
+    for (auto* s : g_streams) g_host_now = std::max(g_host_now, s->ready);
+    return LG_OK;
+}
+int lg_stream_create(void** stream) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    Stream* s = new Stream();
+    s->id = (int)g_streams.size() + 1;
+    s->ready = g_host_now;
+    g_streams.push_back(s);
+    *stream = s;
+    return LG_OK;
+}
+int lg_stream_destroy(void*) { return LG_OK; }
+int lg_stream_synchronize(void* stream) { std::lock_guard<std::mutex> lk(g_mu); g_host_now = std::max(g_host_now, S(stream)->ready); return LG_OK; }
+int lg_stream_wait_event(void* stream, void* event) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    Event* e = (Event*)event;
+    if (e->recorded) S(stream)->ready = std::max(S(stream)->ready, e->time);
+    return LG_OK;
+}
+int lg_event_create(void** event) { *event = new Event(); return LG_OK; }
+int lg_event_destroy(void* event) { delete (Event*)event; return LG_OK; }
+int lg_event_record(void* event, void* stream) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    Event* e = (Event*)event;
+    e->time = std::max(S(stream)->ready, g_host_now);
+    e->recorded = true;
+    return LG_OK;
+}
+int lg_event_synchronize(void* event) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    Event* e = (Event*)event;
+    if (e->recorded) g_host_now = std::max(g_host_now, e->time);
+    return LG_OK;
+}
+int lg_event_query(void* event) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    Event* e = (Event*)event;
+    return (!e->recorded || e->time <= g_host_now) ? LG_OK : 3;
+}
+int lg_event_elapsed_ms(float* ms, void* start, void* stop) { *ms = (float)(((Event*)stop)->time - ((Event*)start)->time); return LG_OK; }
+
+int lg_fill_normal_f32(float*, int64_t, uint64_t, uint64_t, float, float, void*) { return LG_OK; }
+int lg_fill_normal_f16(void*, int64_t, uint64_t, uint64_t, float, float, void*) { return LG_OK; }
+int lg_fill_const_f32(float*, int64_t, float, void*) { return LG_OK; }
+int lg_fill_const_f16(void*, int64_t, float, void*) { return LG_OK; }
+int lg_fill_causal_mask_f32(float*, int, int, void*) { return LG_OK; }
+int lg_fill_causal_mask_f16(void*, int, int, void*) { return LG_OK; }
+
+// ---- kernels -------------------------------------------------------------------------------------------------------------
+#define EW(name, m, n, es, passes, p0, p1, p2) launch(stream, name, m, n, 0, p0, p1, p2, mem_cost((double)(passes) * (m) * (n) * (es)))
+int lg_layer_norm_f32(const float* in, const float* g, const float*, float* out, int m, int n, void* stream) { return EW("layer_norm", m, n, 4, 2, in, g, out); }
+int lg_layer_norm_f16(const void* in, const void* g, const void*, void* out, int m, int n, void* stream) { return EW("layer_norm", m, n, 2, 2, in, g, out); }
+int lg_add_bias_act_f32(float* out, const float* b, int m, int n, void* stream) { return EW("add_bias_act", m, n, 4, 2, out, b, out); }
+int lg_add_bias_act_f16(void* out, const void* b, int m, int n, void* stream) { return EW("add_bias_act", m, n, 2, 2, out, b, out); }
+int lg_add_bias_input_layernorm_f32(float* out, const float* in, const float*, const float*, const float*, int m, int n, void* stream) { return EW("add_bias_input_layernorm", m, n, 4, 3, in, nullptr, out); }
+int lg_add_bias_input_layernorm_f16(void* out, const void* in, const void*, const void*, const void*, int m, int n, void* stream) { return EW("add_bias_input_layernorm", m, n, 2, 3, in, nullptr, out); }
+int lg_add_bias_input_layernorm_2_f32(const float* in, const float*, const float*, const float*, float* o, float* no, int m, int n, void* stream) { return EW("add_bias_input_layernorm_2", m, n, 4, 4, in, o, no); }
+int lg_add_bias_input_layernorm_2_f16(const void* in, const void*, const void*, const void*, void* o, void* no, int m, int n, void* stream) { return EW("add_bias_input_layernorm_2", m, n, 2, 4, in, o, no); }
+int lg_add_bias_input_f32(float* o, const float*, const float* in, int m, int n, void* stream) { return EW("add_bias_input", m, n, 4, 3, in, nullptr, o); }
+int lg_add_bias_input_f16(void* o, const void*, const void* in, int m, int n, void* stream) { return EW("add_bias_input", m, n, 2, 3, in, nullptr, o); }
+int lg_add_qkv_bias_transpose_f32(float* q, float*, float*, const float* Q, const float*, const float*, const float*, const float*, const float*, int b, int s, int h, int d, void* stream) { return EW("add_qkv_bias_transpose", (long long)b * s, (long long)h * d, 4, 6, Q, nullptr, q); }
+int lg_add_qkv_bias_transpose_f16(void* q, void*, void*, const void* Q, const void*, const void*, const void*, const void*, const void*, int b, int s, int h, int d, void* stream) { return EW("add_qkv_bias_transpose", (long long)b * s, (long long)h * d, 2, 6, Q, nullptr, q); }
+int lg_add_fused_qkv_bias_transpose_f32(float* q, float*, float*, const float* X, const float*, int b, int s, int h, int d, void* stream) { return EW("add_fused_qkv_bias_transpose", (long long)b * s, (long long)h * d, 4, 6, X, nullptr, q); }
+int lg_add_fused_qkv_bias_transpose_f16(void* q, void*, void*, const void* X, const void*, int b, int s, int h, int d, void* stream) { return EW("add_fused_qkv_bias_transpose", (long long)b * s, (long long)h * d, 2, 6, X, nullptr, q); }
+int lg_attn_softmax_f32(float* buf, const float* m, int b, int s, int h, float, void* stream) { return EW("attn_softmax", (long long)b * h * s, s, 4, 2, buf, m, buf); }
+int lg_attn_softmax_f16(void* buf, const void* m, int b, int s, int h, float, void* stream) { return EW("attn_softmax", (long long)b * h * s, s, 2, 2, buf, m, buf); }
+int lg_transpose_f32(float* dst, const float* src, int b, int s, int h, int d, void* stream) { return EW("transpose", (long long)b * s, (long long)h * d, 4, 2, src, nullptr, dst); }
+int lg_transpose_f16(void* dst, const void* src, int b, int s, int h, int d, void* stream) { return EW("transpose", (long long)b * s, (long long)h * d, 2, 2, src, nullptr, dst); }
+
+int lg_gemm_f32(int, int, int m, int n, int k, const float* A, int, const float* B, int, float* C, int, void* stream) { return launch(stream, "gemm", m, n, k, A, B, C, gemm_cost(m, n, k)); }
+int lg_gemm_f16(int, int, int m, int n, int k, const void* A, int, const void* B, int, void* C, int, void* stream) { return launch(stream, "gemm", m, n, k, A, B, C, gemm_cost(m, n, k)); }
+int lg_gemm_strided_batched_f32(int, int, int m, int n, int k, const float* A, int, int64_t, const float* B, int, int64_t, float* C, int, int64_t, int batch, void* stream) { return launch(stream, "gemm_batched", m, n, k, A, B, C, gemm_cost((long long)m * batch, n, k)); }
+int lg_gemm_strided_batched_f16(int, int, int m, int n, int k, const void* A, int, int64_t, const void* B, int, int64_t, void* C, int, int64_t, int batch, void* stream) { return launch(stream, "gemm_batched", m, n, k, A, B, C, gemm_cost((long long)m * batch, n, k)); }
+int lg_gemm_fused_f16(int, int m, int n, int k, const void* A, int, const void* B, int, void* C, int, int, const void*, int, int, int, void* stream) { return launch(stream, "gemm_fused", m, n, k, A, B, C, gemm_cost(m, n, k)); }
+int lg_attn_prefill_f16(const void* q, const void* k, const void*, const void*, void* out, int b, int s, int h, int d, int, float, int, int, void* stream) { return launch(stream, "attn_prefill", (long long)b * h, s, d, q, k, out, gemm_cost((long long)b * h * s, s, 2 * d)); }
+size_t lg_attn_decode_workspace_bytes(int, int, int, int) { return 1024; }
+int lg_attn_decode_f16(const void* q, const void* kc, const void*, void* out, void*, int b, int h, int d, int len, int, float, void* stream) { return launch(stream, "attn_decode", (long long)b * h, len, d, q, kc, out, mem_cost(4.0 * b * h * len * d)); }
+int lg_kv_append_f16(void* q, void* kc, void*, const void* Q, const void*, const void*, const void*, const void*, const void*, int b, int h, int d, int pos, int, void* stream) { return launch(stream, "kv_append", (long long)b * h, pos, d, Q, kc, q, mem_cost(12.0 * b * h * d)); }
+
+}  // extern "C"

@@ -1,0 +1,240 @@
+"""Pins the CPU oracle without the reference (which is CUDA and ships no golden vectors): closed forms, brute force,
+identities, an independent library (numpy / CPU torch) and committed fixtures.  Each check is chosen so that a
+plausible slip (dropped term, wrong sign or index, transposed operand, wrong epsilon) fails it."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as Fn
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def test_half_rounding_matches_ieee(po):
+    rng = np.random.default_rng(0)
+    x = np.concatenate([rng.standard_normal(200000).astype(np.float32) * s for s in (1e-8, 1e-6, 1e-4, 1e-2, 1, 100, 30000, 70000)])
+    x = np.concatenate([x, np.array([0, -0.0, 65504, 65519.9, 65520, 1e9, -1e9, 6e-8, 5.96e-8, 2.98e-8, 2.99e-8, 3e-8, 6.1e-5, 6.10352e-5,
+                                     1.0009765625, 1.00048828125, 1.00146484375], dtype=np.float32)])
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).astype(np.float32)
+    assert np.array_equal(po.round_f16(x), want)
+
+
+def test_fill_normal_golden_words_and_moments(po):
+    words = json.load(open(os.path.join(GOLD, "fill_normal_words.json")))
+    assert [float(v) for v in po.fill_normal(8, 0, 1)] == words["seed0_tid1_n8"]
+    assert [float(v) for v in po.fill_normal(8, 7, 42, 0.25, 0.02)] == words["seed7_tid42_mean0.25_std0.02_n8"]
+    big = po.fill_normal(1000001, 0, 1)
+    assert float(big[-1]) == words["seed0_tid1_at_1000000"]
+    assert abs(big.mean()) < 5e-3 and abs(big.std() - 1.0) < 5e-3
+    assert abs(((big - big.mean()) ** 3).mean()) < 2e-2           # symmetric
+    assert not np.array_equal(po.fill_normal(64, 0, 1), po.fill_normal(64, 0, 2))  # tensor id matters
+    assert not np.array_equal(po.fill_normal(64, 0, 1), po.fill_normal(64, 1, 1))  # seed matters
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (1, 8, 5), (32, 40, 17), (7, 300, 260), (64, 256, 256), (5, 3, 600)])
+def test_gemm_against_brute_force_and_numpy(po, M, N, K):
+    X = po.fill_normal(M * K, 0, 10).reshape(M, K)
+    W = po.fill_normal(K * N, 0, 11).reshape(K, N)
+    Y = po.gemm(X, W)
+    # fp32 accumulation over K terms of magnitude ~1: absolute error well below 1e-4, relative to |Y| ~ sqrt(K)
+    assert np.abs(Y - po.gemm_naive_f64(X, W)).max() < 1e-4
+    assert np.abs(Y - X.astype(np.float64) @ W.astype(np.float64)).max() < 1e-4
+    # a transposed-operand slip would survive symmetric inputs, so check structure explicitly
+    if M >= 2 and N >= 2 and K >= 2:
+        E = np.zeros((K, N), dtype=np.float32)
+        E[1, 0] = 1.0  # picks column 1 of X into output column 0
+        assert np.array_equal(po.gemm(X, E)[:, 0], X[:, 1])
+    if N == K:
+        assert np.array_equal(po.gemm(X, np.eye(K, dtype=np.float32)), X)
+
+
+def test_gemm_ex_is_cublas_column_major(po):
+    """cublasGemmEx semantics: C(m x n, col-major) = op(A) op(B).  Checked against numpy with Fortran-order views."""
+    m, n, k = 7, 5, 9
+    for transa in (0, 1):
+        lda = (k if transa else m) + 2
+        ldb, ldc = k + 1, m + 3
+        A = po.fill_normal(lda * (m if transa else k), 0, 12)
+        B = po.fill_normal(ldb * n, 0, 13)
+        Cm = np.zeros(ldc * n, dtype=np.float32)
+        po.gemm_ex(transa, 0, m, n, k, A, lda, B, ldb, Cm, ldc)
+        Af = A.reshape((m if transa else k), lda).T  # column-major storage: element (i, j) at i + j*lda
+        Aop = Af[:k, :m].T if transa else Af[:m, :k]
+        Bf = B.reshape(n, ldb).T[:k, :n]
+        want = Aop.astype(np.float64) @ Bf.astype(np.float64)
+        got = Cm.reshape(n, ldc).T[:m, :n]
+        assert np.allclose(got, want, rtol=1e-5, atol=1e-5)
+
+
+def test_gemm_strided_batched_matches_attention_einsums(po):
+    nb, S, d = 3, 10, 6
+    q = po.fill_normal(nb * S * d, 0, 14).reshape(nb, S, d)
+    k = po.fill_normal(nb * S * d, 0, 15).reshape(nb, S, d)
+    v = po.fill_normal(nb * S * d, 0, 16).reshape(nb, S, d)
+    qk = np.zeros((nb, S, S), dtype=np.float32)
+    po.gemm_strided_batched(1, 0, S, S, d, k, d, S * d, q, d, S * d, qk, S, S * S, nb)   # bert_layer.h:145-149
+    assert np.allclose(qk, np.einsum("bqd,bkd->bqk", q, k), atol=1e-5)
+    p = np.abs(qk)
+    o = np.zeros((nb, S, d), dtype=np.float32)
+    po.gemm_strided_batched(0, 0, d, S, S, v, d, S * d, p, S, S * S, o, d, S * d, nb)     # bert_layer.h:158-162
+    assert np.allclose(o, np.einsum("bqk,bkd->bqd", p, v), atol=1e-4)
+
+
+def test_layer_norm_closed_forms_and_torch(po):
+    n = 64
+    g = po.fill_normal(n, 0, 20, 1.0, 0.1)
+    b = po.fill_normal(n, 0, 21, 0.0, 0.1)
+    # constant row -> beta exactly (x - mean == 0)
+    assert np.array_equal(po.layer_norm(np.full((1, n), 3.25, dtype=np.float32), g, b), b.reshape(1, n))
+    # +-1 row: mean 0, biased variance 1 -> y = x * rsqrt(1 + 1e-6) * gamma + beta  (eps is 1e-6, not 1e-5)
+    x = np.tile(np.array([-1.0, 1.0], dtype=np.float32), n // 2).reshape(1, n)
+    want = x * (1.0 / np.sqrt(1.0 + 1e-6)) * g + b
+    assert np.allclose(po.layer_norm(x, g, b), want, atol=1e-6)
+    assert not np.allclose(po.layer_norm(x * 1e-2, g, b), x * (1.0 / np.sqrt(1.0 + 1e-5 * 1e4)) * g + b, atol=1e-4)
+    # shift invariance and agreement with torch
+    x = po.fill_normal(5 * n, 0, 22).reshape(5, n) * 2 + 0.3
+    y = po.layer_norm(x, g, b)
+    assert np.allclose(po.layer_norm(x + 7.0, g, b), y, atol=2e-5)
+    t = Fn.layer_norm(torch.from_numpy(x), (n,), torch.from_numpy(g), torch.from_numpy(b), eps=1e-6).numpy()
+    assert np.allclose(y, t, atol=2e-6)
+    # unbiased-variance slip: with n = 2 biased var of [-1, 1] is 1, unbiased is 2
+    y2 = po.layer_norm(np.array([[-1.0, 1.0]], dtype=np.float32), np.ones(2, dtype=np.float32), np.zeros(2, dtype=np.float32))
+    assert np.allclose(y2, [[-1.0, 1.0]], atol=1e-5)
+
+
+def test_bias_gelu_tabulated_and_torch(po):
+    pts = np.array([[0.0, 1.0, -1.0, 3.0, -3.0, 10.0, -10.0, 0.5]], dtype=np.float32)
+    want = [0.0, 0.8411919906, -0.1588080094, 2.9963627, -0.0036373, 10.0, 0.0, 0.3457140]
+    got = po.add_bias_gelu(pts.copy(), np.zeros(8, dtype=np.float32))
+    assert np.allclose(got[0], want, atol=2e-6)
+    x = po.fill_normal(6 * 32, 0, 23, 0.0, 2.0).reshape(6, 32)
+    bias = po.fill_normal(32, 0, 24)
+    t = Fn.gelu(torch.from_numpy(x + bias), approximate="tanh").numpy()
+    assert np.allclose(po.add_bias_gelu(x.copy(), bias), t, atol=2e-6)
+    # fp16 instantiation stays within a couple of half ulps of the exact value
+    xh, bh = po.round_f16(x), po.round_f16(bias)
+    th = Fn.gelu(torch.from_numpy(xh + bh), approximate="tanh").numpy()
+    assert np.abs(po.add_bias_gelu(xh.copy(), bh, 1) - th).max() < 8e-3
+
+
+def test_softmax_identities_and_torch(po):
+    B, h, S = 2, 3, 16
+    scalar = 0.125
+    qk = po.fill_normal(B * h * S * S, 0, 25, 0.0, 3.0).reshape(B, h, S, S)
+    ones = np.ones((B, S, S), dtype=np.float32)
+    p = po.attn_softmax(qk.copy(), ones, scalar)
+    t = torch.softmax(torch.from_numpy(qk) * scalar, -1).numpy()
+    assert np.allclose(p, t, atol=2e-6)
+    # rows sum to sum/(sum + 1e-6), i.e. slightly below one
+    e = np.exp(qk * scalar - (qk * scalar).max(-1, keepdims=True))
+    assert np.allclose(p.sum(-1), e.sum(-1) / (e.sum(-1) + 1e-6), atol=1e-6)
+    # constant scores, all-ones mask -> 1/S * S/(S + 1e-6)
+    c = po.attn_softmax(np.full((1, 1, S, S), 2.5, dtype=np.float32), np.ones((1, S, S), dtype=np.float32), scalar)
+    assert np.allclose(c, 1.0 / (S + 1e-6), atol=1e-7)
+    # masked columns vanish (exp(-10000) == 0 in fp32) and the rest renormalises; mask is shared over heads, indexed [b, q, k]
+    mask = np.ones((B, S, S), dtype=np.float32)
+    mask[1, 2, 5:] = 0.0
+    pm = po.attn_softmax(qk.copy(), mask, scalar)
+    assert np.all(pm[1, :, 2, 5:] == 0.0) and np.allclose(pm[1, :, 2, :5].sum(-1), 1.0, atol=1e-5)
+    assert np.allclose(pm[0], p[0], atol=1e-7) and np.allclose(pm[1, :, 3], p[1, :, 3], atol=1e-7)
+    # shift invariance of the scores
+    assert np.allclose(po.attn_softmax(qk.copy() + 4.0, ones, scalar), p, atol=2e-6)
+    # a fully masked row is the plain softmax (the -10000 cancels): the reference's additive semantics
+    mask0 = np.ones((B, S, S), dtype=np.float32)
+    mask0[0, 4, :] = 0.0
+    p0 = po.attn_softmax(qk.copy(), mask0, scalar)
+    assert np.allclose(p0[0, :, 4], p[0, :, 4], atol=1e-4)
+
+
+def test_transposes_are_the_stated_permutations(po):
+    B, S, h, d = 2, 3, 4, 5
+    n = h * d
+    Q = np.arange(B * S * n, dtype=np.float32).reshape(B * S, n)
+    zero = np.zeros(n, dtype=np.float32)
+    qb, kb, vb = po.add_qkv_bias_transpose(Q, zero, Q + 1000, zero, Q + 2000, zero, B, S, h, d)
+    want = Q.reshape(B, S, h, d).transpose(0, 2, 1, 3)
+    assert np.array_equal(qb, want) and np.array_equal(kb, want + 1000) and np.array_equal(vb, want + 2000)
+    # bias is indexed [head, e] and added per column
+    bias = np.arange(n, dtype=np.float32) * 0.5
+    qb2, _, _ = po.add_qkv_bias_transpose(Q, bias, Q, zero, Q, zero, B, S, h, d)
+    assert np.array_equal(qb2, (Q + bias).reshape(B, S, h, d).transpose(0, 2, 1, 3))
+    # transpose back is the inverse permutation
+    assert np.array_equal(po.transpose(qb).reshape(B * S, n), Q)
+    # packed [M, 3, n] variant gives the same three buffers
+    QKV = np.ascontiguousarray(np.stack([Q, Q + 1000, Q + 2000], axis=1))
+    fq, fk, fv = po.add_fused_qkv_bias_transpose(QKV, np.concatenate([bias, zero, zero]), B, S, h, d)
+    assert np.array_equal(fq, qb2) and np.array_equal(fk, kb) and np.array_equal(fv, vb)
+
+
+def test_fused_residual_kernels_compose_from_layer_norm(po):
+    m, n = 4, 48
+    out = po.fill_normal(m * n, 0, 30).reshape(m, n)
+    inp = po.fill_normal(m * n, 0, 31).reshape(m, n)
+    bias = po.fill_normal(n, 0, 32)
+    g = po.fill_normal(n, 0, 33, 1.0, 0.1)
+    b = po.fill_normal(n, 0, 34, 0.0, 0.1)
+    s = out + inp + bias
+    assert np.allclose(po.add_bias_input_layernorm(out.copy(), inp, bias, g, b), po.layer_norm(s, g, b), atol=2e-6)
+    o2, n2 = po.add_bias_input_layernorm_2(inp, g, b, bias, out.copy())
+    assert np.allclose(o2, s, atol=1e-6) and np.allclose(n2, po.layer_norm(s, g, b), atol=2e-6)
+    assert np.allclose(po.add_bias_input(out.copy(), bias, inp), s, atol=1e-6)
+
+
+def test_decode_equals_last_row_of_causal_prefill(po):
+    """Pins lo_attn_decode (no reference counterpart): decode over L cached positions == the last query row of causal
+    prefill attention over the same L tokens; and causal prefill == the explicit 3-step path with a tril mask."""
+    B, h, d, L = 2, 3, 64, 40
+    q = po.fill_normal(B * h * L * d, 0, 60).reshape(B, h, L, d)
+    k = po.fill_normal(B * h * L * d, 0, 61).reshape(B, h, L, d)
+    v = po.fill_normal(B * h * L * d, 0, 62).reshape(B, h, L, d)
+    scalar = 1.0 / np.sqrt(d)
+    full = po.attn_prefill(q, k, v, scalar, True)
+    dec = po.attn_decode(np.ascontiguousarray(q[:, :, -1, :]), k, v, L, scalar)
+    assert np.abs(dec - full[:, :, -1, :]).max() < 1e-5
+    # shorter length on a longer cache ignores the tail
+    dec20 = po.attn_decode(np.ascontiguousarray(q[:, :, 19, :]), k, v, 20, scalar)
+    assert np.abs(dec20 - full[:, :, 19, :]).max() < 1e-5
+    # against torch
+    sc = torch.from_numpy(q) @ torch.from_numpy(k).transpose(-1, -2) * scalar
+    sc = sc.masked_fill(~torch.tril(torch.ones(L, L, dtype=torch.bool)), float("-inf"))
+    ref = (torch.softmax(sc, -1) @ torch.from_numpy(v)).numpy()
+    assert np.abs(full - ref).max() < 1e-5
+
+
+@pytest.mark.parametrize("mode,key", [(0, "post_noresid"), (1, "pre_ln_resid")])
+def test_encoder_matches_torch_fixture_cfg1(po, mode, key):
+    """BASELINE config 1 layer against the committed torch fixture (tests/golden/make_golden.py)."""
+    from tests.golden.make_golden import cfg1_weights
+    w, x = cfg1_weights()
+    # the oracle's own generator must reproduce the numpy restatement the fixture was made from
+    assert np.array_equal(w["wq"].ravel(), po.fill_normal(256 * 256, 0, 1, 0.0, 0.02))
+    shape = dict(batch=2, seq=32, hidden=256, head_num=4, size_per_head=64, ffn_inner=1024, causal=0, norm_mode=mode, dtype=0)
+    got = po.encoder_forward(shape, w, x)
+    want = np.load(os.path.join(GOLD, "cfg1_layer_torch.npz"))[key]
+    assert np.abs(got - want).max() / np.abs(want).max() < 2e-5
+
+
+def test_decoder_step_equals_prefill_of_extended_sequence(po):
+    """One decode step after a causal prefill of S tokens == row S of a causal prefill of S+1 tokens (same layer)."""
+    B, S, heads, d, F = 2, 12, 2, 16, 64
+    H = heads * d
+    from tests.golden.make_golden import fill_normal
+    names = [("wq", (H, H)), ("wk", (H, H)), ("wv", (H, H)), ("bq", (H,)), ("bk", (H,)), ("bv", (H,)), ("wo", (H, H)),
+             ("ln1_g", (H,)), ("ln1_b", (H,)), ("w1", (H, F)), ("b1", (F,)), ("w2", (F, H)), ("ln2_g", (H,)), ("ln2_b", (H,))]
+    w = {n: fill_normal(int(np.prod(s)), 5, i + 1, 1.0 if n.endswith("_g") else 0.0, 0.1).reshape(s) for i, (n, s) in enumerate(names)}
+    x = fill_normal(B * (S + 1) * H, 5, 99).reshape(B, S + 1, H)
+    shape1 = dict(batch=B, seq=S + 1, hidden=H, head_num=heads, size_per_head=d, ffn_inner=F, causal=1, norm_mode=0, dtype=0)
+    full = po.encoder_forward(shape1, w, np.ascontiguousarray(x.reshape(B * (S + 1), H))).reshape(B, S + 1, H)
+    # build the cache from the first S tokens, then decode token S
+    xs = np.ascontiguousarray(x[:, :S].reshape(B * S, H))
+    kk = po.gemm(xs, w["wk"]); vv = po.gemm(xs, w["wv"])
+    _, kb, vb = po.add_qkv_bias_transpose(kk, w["bq"], kk, w["bk"], vv, w["bv"], B, S, heads, d)
+    Lmax = S + 4
+    kc = np.zeros((B, heads, Lmax, d), dtype=np.float32); vc = np.zeros_like(kc)
+    kc[:, :, :S] = kb; vc[:, :, :S] = vb
+    shape = dict(shape1, seq=S)
+    out = po.decoder_step(shape, w, np.ascontiguousarray(x[:, S]), kc, vc, S)
+    assert np.abs(out - full[:, S]).max() < 1e-4

@@ -1,0 +1,265 @@
+"""Unit tests of the launch-vector runtime (layer assembly, Sample, Scheduler, profile JSON, report) on the CPU.
+
+The runtime is the shipped C++ code; only the device library underneath is replaced by tests/fake_backend, which
+records every launch with virtual timestamps.  Expected launch sequences are derived by hand from the policy the
+reference implements (src/schedule.h:221-278, src/init.h:121-259); the fake's cost model is
+    gemm: 0.003 + 2*m*n*k / 1e9 ms      memory kernels: 0.003 + bytes / 1e6 ms      host launch cost 0.002 ms.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from tests.fake_util import Fake
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+@pytest.fixture()
+def fake():
+    f = Fake()
+    f.set_rates(1.0e9, 1.0e6, 0.002)
+    f.reset()
+    yield f
+    f.close()
+
+
+def small_model(host, fused=True, factor=4, layers=1, max_batch=4, cache=128):
+    return host.Model(1, max_batch, 64, 4, 64, layer_num=layers, ffn_inner=512, causal=True, fused=fused,
+                      max_cache_len=cache if fused else 0, factor=factor, seed=0)
+
+
+def test_launch_vector_shapes_and_order(fake):
+    host = fake.host
+    m = small_model(host, fused=False, cache=0)
+    d = m.describe(2, 32)
+    assert [e["label"] for e in d] == ["q_gemm", "k_gemm", "v_gemm", "qkv_bias_transpose", "qk_gemm", "softmax", "pv_gemm",
+                                       "transpose_back", "out_proj", "layer_norm", "ffn1", "bias+gelu", "ffn2", "layer_norm"]
+    # only the six weight GEMMs are type GEMM (decomposable), as in the reference (bert_layer.h:145-163 tags the batched ones COMPUTATION)
+    assert [e["type"] for e in d].count("GEMM") == 6
+    assert m.kernels_per_layer() == 14
+    mf = small_model(host, fused=True)
+    assert mf.kernels_per_layer() == 9 and mf.kernels_per_layer(decode=True) == 10
+    assert all(e["class"] == "HBM_BOUND" for e in mf.describe(2, 1, decode_past=10))
+    m2 = host.Model(0, 2, 32, 4, 64, layer_num=3, norm_mode=host.PRE_LN_RESID)
+    assert len(m2.describe(2, 32)) == 3 * 15
+    with pytest.raises(host.capi.LigerError):
+        host.Model(1, 2, 32, 5, 64, world_size=2)      # heads not divisible by the TP degree
+    with pytest.raises(host.capi.LigerError):
+        host.Model(0, 2, 32, 4, 64, fused=True)        # fused assembly is fp16 only
+
+
+def test_sequential_run_launches_every_entry_once_in_order(fake):
+    host = fake.host
+    m = small_model(host)
+    s = host.Scheduler(m, pool_count=3, ctx_batch=1)
+    fake.reset()
+    s.serve(1, 64)
+    s.serve(1, 48)
+    r = s.run_queued(host.MODE_SEQUENTIAL)
+    t = fake.trace()
+    assert r["records"] == 2 and r["secondary_launches"] == 0 and r["rounds"] == 2
+    assert len({e["stream"] for e in t}) == 1
+    names = ["gemm_fused"] * 3 + ["attn_prefill", "gemm", "layer_norm", "gemm_fused", "gemm", "layer_norm"]
+    assert [e["name"] for e in t] == names * 2
+    assert [e["n"] for e in t if e["name"] == "gemm"] == [64, 64, 48, 48]
+    assert all(b["start"] >= a["end"] - 1e-12 for a, b in zip(t, t[1:]))
+
+
+def test_classic_policy_degenerates_to_sequential_without_communication(fake):
+    """With COMMUNICATION vs rest as the only classes and no all-reduce entry in a one-GPU vector, nothing may be
+    launched on the secondary stream."""
+    host = fake.host
+    m = small_model(host)
+    s = host.Scheduler(m, policy=host.POLICY_CLASSIC, pool_count=3, ctx_batch=1)
+    s.profile(1, 64, 64, 1, 2)
+    fake.reset()
+    s.serve(1, 64)
+    s.serve(1, 64)
+    r = s.run_queued(host.MODE_LIGER)
+    assert r["secondary_launches"] == 0 and r["splits"] == 0
+    assert len({e["stream"] for e in fake.trace()}) == 1
+
+
+def test_resource_policy_worked_example(fake):
+    """Two identical prefill requests A (primary) and B.  Fused vector: [q k v attn out](MFMA) [ln](HBM) [ffn1 ffn2](MFMA) [ln](HBM).
+    Round 1: A launches q,k,v,attn,out; B's next is MFMA -> same class -> nothing on stream 1.
+    Round 2: A launches ln (0.0695 ms window, x0.8 = 0.0556).  B: q,k,v (0.0124 each), attn (0.0082) fit -> 0.0102 left;
+             out_proj (0.0124) does not fit -> split with profiled fractions [0.0061, 0.0082, 0.0103] -> 2/4 fits ->
+             first piece (128 of 256 output columns) goes to stream 1, remainder (128 columns) stays queued.
+    Round 3: A launches ffn1, ffn2 (MFMA); B's next (remainder of out_proj) is MFMA -> nothing.
+    Round 4: A launches its last ln; B's remainder fits the window and runs on stream 1; B's ln is HBM -> stop.
+    Then B becomes primary and finishes alone on stream 0."""
+    host = fake.host
+    m = small_model(host, factor=4)
+    s = host.Scheduler(m, contention_factor=0.8, policy=host.POLICY_RESOURCE, pool_count=3, ctx_batch=1)
+    s.profile(1, 64, 64, 1, 2)
+    # profiled with 2 launches per timing: the first launch starts one host launch cost (0.002) after the start event,
+    # so the per-launch figure is the kernel cost + 0.001
+    assert abs(s.lookup(0, 1, 64) - (0.003 + 2 * 256 * 64 * 256 / 1e9 + 0.001)) < 1e-6
+    assert abs(s.lookup(5, 1, 64) - (0.003 + 2 * 64 * 256 * 2 / 1e6 + 0.001)) < 1e-6
+    sub = s.sub_lookup(4, 1, 64)
+    assert len(sub) == 3 and all(abs(v - (0.003 + 2 * (64 * (i + 1)) * 64 * 256 / 1e9 + 0.001)) < 1e-6 for i, v in enumerate(sub))
+    assert s.sub_lookup(5, 1, 64) is None  # only GEMM entries are decomposable
+    fake.reset()
+    s.serve(1, 64)
+    s.serve(1, 64)
+    r = s.run_queued(host.MODE_LIGER)
+    t = fake.trace()
+    s0 = min(e["stream"] for e in t)
+    seq = [(e["stream"] - s0, e["name"], e["m"]) for e in t]
+    A1 = [(0, "gemm_fused", 256)] * 3 + [(0, "attn_prefill", 4), (0, "gemm", 256), (0, "layer_norm", 64)]
+    B1 = [(1, "gemm_fused", 256)] * 3 + [(1, "attn_prefill", 4), (1, "gemm", 128)]
+    A2 = [(0, "gemm_fused", 512), (0, "gemm", 256), (0, "layer_norm", 64)]
+    B2 = [(1, "gemm", 128)]
+    B3 = [(0, "layer_norm", 64), (0, "gemm_fused", 512), (0, "gemm", 256), (0, "layer_norm", 64)]
+    assert seq == A1 + B1 + A2 + B2 + B3
+    assert r["secondary_launches"] == 6 and r["splits"] == 1 and r["records"] == 2
+    # the two pieces of B's out_proj tile the output: same weights base + 128 columns (fp16), same activations, C + 128 columns
+    p1, p2 = [e for e in t if e["name"] == "gemm" and e["m"] == 128]
+    assert p2["A"] - p1["A"] == 128 * 2 and p2["C"] - p1["C"] == 128 * 2 and p1["B"] == p2["B"]
+    # stream 1 is gated on the end of the previous primary round (device-side event wait)
+    end_round1 = [e for e in t if e["stream"] == s0][4]["end"]
+    first_b = [e for e in t if e["stream"] != s0][0]
+    assert first_b["start"] >= end_round1 - 1e-12
+    # budget: secondary work launched in a round never exceeds contention_factor x the primary window
+    assert sum(e["end"] - e["start"] for e in t[6:11]) <= 0.8 * (t[5]["end"] - t[5]["start"]) + 1e-9
+    # B moves from stream 1 to stream 0: its first kernel there starts after its last kernel on stream 1 has ended
+    assert t[15]["start"] >= t[14]["end"] - 1e-12
+
+
+@pytest.mark.parametrize("contention,expect_splits", [(0.8, False), (0.12, True), (0.05, True)])
+def test_decode_request_fills_prefill_gemm_windows_and_splits_cover_exactly(fake, contention, expect_splits):
+    """Primary = a prefill request (long MFMA rounds), secondary = a request with decode steps (HBM-bound kernels).
+    Every kernel of every request is launched exactly once and per request in order; decomposed GEMM pieces of the
+    decode request's skinny GEMMs are not produced (they fit), while a swapped case (decode primary, prefill secondary)
+    produces splits whose pieces partition the columns."""
+    host = fake.host
+    m = small_model(host, factor=8)
+    s = host.Scheduler(m, contention_factor=contention, policy=host.POLICY_RESOURCE, seq_bucket=16, pool_count=3, ctx_batch=1)
+    s.profile(1, 48, 64, 16, 2)
+    for past in (48, 64, 80):
+        s.profile_decode(1, past, 2)
+    fake.reset()
+    s.serve(1, 48, 3)   # A: prefill 48 + 3 decode steps
+    s.serve(1, 64, 0)   # B: prefill only
+    r = s.run_queued(host.MODE_LIGER)
+    t = fake.trace()
+    assert r["records"] == 2 and r["profile_misses"] == 0
+    # B's GEMMs (token dimension 64) : total output columns per weight matrix must be covered exactly once
+    weights = {n: (p, p + 2 * cnt) for n, (p, cnt) in m.params().items() if n.split(".")[1] in ("wq", "wk", "wv", "wo", "w1", "w2")}
+    cover = {}
+    for e in t:
+        if e["name"] in ("gemm", "gemm_fused") and e["n"] == 64:
+            owner = [n for n, (lo, hi) in weights.items() if lo <= e["A"] < hi]
+            assert len(owner) == 1
+            cover.setdefault(owner[0], []).append((e["C"], e["m"]))
+    widths = {n.split(".")[1]: sum(m_ for _, m_ in v) for n, v in cover.items()}
+    assert widths == {"wq": 256, "wk": 256, "wv": 256, "wo": 256, "w1": 512, "w2": 256}
+    for n, v in cover.items():
+        v.sort()
+        if n.endswith(("wq", "wk", "wv")):
+            continue  # head-transposed outputs: pieces are whole heads, checked by the width sum above
+        for (c0, m0), (c1, _) in zip(v, v[1:]):
+            assert c1 - c0 == m0 * 2              # contiguous fp16 column ranges: no gap, no overlap
+    assert (r["splits"] > 0) == expect_splits
+    # A's decode kernels: 3 steps x 10 entries, in order, attention lengths 49, 50, 51
+    assert [e["n"] for e in t if e["name"] == "attn_decode"] == [49, 50, 51]
+    assert r["secondary_launches"] > 0
+    # per-request order in virtual time (n == tokens identifies the request for row-shaped kernels)
+    for tokens in (48, 64):
+        mine = [e for e in t if (e["name"] in ("gemm", "gemm_fused") and e["n"] == tokens) or (e["name"] == "layer_norm" and e["m"] == tokens)]
+        assert all(b["start"] >= a["end"] - 1e-12 for a, b in zip(mine, mine[1:]))
+
+
+def test_missing_or_short_profile_never_splits_or_crashes(fake):
+    host = fake.host
+    m = small_model(host, factor=8)
+    s = host.Scheduler(m, policy=host.POLICY_RESOURCE, pool_count=3, ctx_batch=1)
+    # main durations only for the primary's ln (window) and a GEMM that is too long; sub profile shorter than factor-1
+    for k in range(9):
+        s.set_profile(k, 1, 64, 1.0 if k in (5, 8) else 5.0, sub=[0.1, 0.2] if k == 0 else None)
+    fake.reset()
+    s.serve(1, 64)
+    s.serve(1, 64)
+    r = s.run_queued(host.MODE_LIGER)
+    assert r["records"] == 2 and r["splits"] == 0 and r["secondary_launches"] == 0
+    # with no profile at all every lookup misses, durations are 0, windows are 0: still drains, sequentially
+    s2 = host.Scheduler(m, policy=host.POLICY_RESOURCE, pool_count=3, ctx_batch=1)
+    fake.reset()
+    s2.serve(1, 64)
+    s2.serve(1, 32)
+    r2 = s2.run_queued(host.MODE_LIGER)
+    assert r2["records"] == 2 and r2["profile_misses"] == 18 and r2["secondary_launches"] == 0
+
+
+def test_profile_json_roundtrip_and_failure_paths(fake, tmp_path):
+    host = fake.host
+    m = small_model(host)
+    s = host.Scheduler(m, pool_count=0)
+    s.profile(1, 32, 64, 32, 2)
+    a, b = str(tmp_path / "Main_1_64_4_1_64.json"), str(tmp_path / "Sub_1_64_4_1_64.json")
+    s.save(a, b)
+    main = json.load(open(a))
+    sub = json.load(open(b))
+    assert {tuple(sorted(e)) for e in main} == {("batch_size", "duration", "kernel_name", "seq_len")}   # utils.h:106-127 schema
+    assert len(main) == 18 and len(sub) == 12 and all(len(e["duration"]) == 3 for e in sub)            # factor 4 -> 3 fractions
+    s2 = host.Scheduler(m, pool_count=0)
+    s2.load(a, b)
+    for e in main:
+        assert abs(s2.lookup(e["kernel_name"], e["batch_size"], e["seq_len"]) - e["duration"]) < 1e-6
+    # a file in the reference's own writer format (trailing-comma-free, "duration": [ ... ] with a space)
+    open(a, "w").write('[{"kernel_name":0,"batch_size":2,"seq_len":64,"duration":1.5},{"kernel_name":1,"batch_size":2,"seq_len":64,"duration":0.25}]')
+    open(b, "w").write('[{"kernel_name":0,"batch_size":2,"seq_len":64,"duration": [0.2,0.4,0.6]}]')
+    s2.load(a, b)
+    assert s2.lookup(0, 2, 64) == 1.5 and s2.lookup(1, 2, 64) == 0.25 and s2.sub_lookup(0, 2, 64) == pytest.approx([0.2, 0.4, 0.6])
+    for bad in ("", "[{\"kernel_name\":0}]", "{", "[{\"kernel_name\":0,\"batch_size\":1,\"seq_len\":2,\"duration\":[1,2]}]"):
+        open(a, "w").write(bad)
+        with pytest.raises(host.capi.LigerError):
+            s2.load(a, b)
+    with pytest.raises(host.capi.LigerError):
+        s2.load(str(tmp_path / "missing.json"), b)
+
+
+def test_report_arithmetic_reproduces_the_published_logs(fake):
+    """Known-answer test: mean(CPU_Time + CUDA_Time) over the 131 request lines of the reference's published runs gives
+    the printed Average Latency, and 1000 * records / Total_Duration the printed Throughput (schedule.h:325-348)."""
+    host = fake.host
+    logs = json.load(open(os.path.join(GOLD, "reference_logs.json")))
+    for run, avg in (("baseline", 260.409698), ("liger", 199.714066)):
+        d = logs[run]
+        r = host.summarize(d["cpu_ms"], d["gpu_ms"], d["printed"]["Total_Duration"])
+        assert r["records"] == d["printed"]["records"] == 131
+        assert abs(r["avg_latency_ms"] - avg) < 2e-3 and abs(avg - d["printed"]["Average Latency"]) < 1e-9
+        assert abs(r["throughput"] - d["printed"]["Throughput"]) < 1e-3
+        lat = np.sort(np.array(d["cpu_ms"]) + np.array(d["gpu_ms"]))
+        assert r["p99_latency_ms"] == pytest.approx(lat[int(np.ceil(0.99 * 131)) - 1])
+    assert host.summarize([], [], 0.0)["records"] == 0
+
+
+def test_poisson_trace_is_seeded_and_has_the_right_rate(fake):
+    host = fake.host
+    tr = host.make_poisson_trace(8.0, 4000, 1, 128, 1024, 64, 32, 7)
+    assert tr == host.make_poisson_trace(8.0, 4000, 1, 128, 1024, 64, 32, 7)
+    assert tr != host.make_poisson_trace(8.0, 4000, 1, 128, 1024, 64, 32, 8)
+    arr = np.array([t["arrival_s"] for t in tr])
+    gaps = np.diff(np.concatenate([[0.0], arr]))
+    assert np.all(gaps > 0) and abs(gaps.mean() - 1 / 8.0) < 0.01 and abs(gaps.std() - 1 / 8.0) < 0.02   # exponential: mean == std
+    seqs = np.array([t["seq"] for t in tr])
+    assert seqs.min() >= 128 and seqs.max() <= 1024 and np.all(seqs % 64 == 0) and len(set(seqs)) == 15
+    assert all(t["n_decode"] == 32 and t["batch"] == 1 for t in tr)
+
+
+def test_realtime_trace_replay_drains(fake):
+    """The threaded path (request thread + scheduler loop): arrivals in real time, all requests reported."""
+    host = fake.host
+    m = small_model(host)
+    s = host.Scheduler(m, policy=host.POLICY_RESOURCE, pool_count=2, ctx_batch=1, ignore_num=0)
+    s.profile(1, 64, 64, 1, 2)
+    trace = [{"arrival_s": 0.002 * i, "batch": 1, "seq": 64, "n_decode": 0} for i in range(12)]
+    for mode in (host.MODE_SEQUENTIAL, host.MODE_LIGER):
+        fake.reset()
+        r = s.run_trace(trace, mode)
+        assert r["records"] == 12
+        assert len([e for e in fake.trace() if e["name"] == "attn_prefill"]) == 12
