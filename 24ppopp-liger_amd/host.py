@@ -32,12 +32,12 @@ class Report(C.Structure):
 SIGNATURES = {
     "lgh_first_error": (_i, [C.c_char_p, _i]),
     "lgh_clear_error": (None, []),
-    "lgh_model_create": (_p, [_i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _u64]),
+    "lgh_model_create": (_p, [_i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _u64]),
     "lgh_model_kernels_per_layer": (_i, [_p, _i]),
     "lgh_model_workspace_elems": (_i64, [_p, _i, _i]),
     "lgh_model_stream": (_p, [_p]),
     "lgh_model_param_count": (_i, [_p]),
-    "lgh_model_param_info": (_i, [_p, _i, C.c_char_p, _i, C.POINTER(_p), C.POINTER(_i64)]),
+    "lgh_model_param_info": (_i, [_p, _i, C.c_char_p, _i, C.POINTER(_p), C.POINTER(_i64), C.POINTER(_i), C.POINTER(_i), C.POINTER(_i)]),
     "lgh_model_describe": (_i, [_p, _i, _i, _i, C.c_char_p, _i]),
     "lgh_model_run": (_i, [_p, _p, _p, _i, _i, _p, _p, _i]),
     "lgh_model_run_decode": (_i, [_p, _p, _p, _i, _i, _i, _p, _p]),
@@ -113,10 +113,10 @@ class Model:
     """One tensor-parallel shard of a stack of encoder layers, assembled as launch vectors by the C++ runtime."""
 
     def __init__(self, dtype, max_batch, max_seq, head_num, size_per_head, layer_num=1, world_size=1, ffn_inner=0,
-                 norm_mode=POST_NORESID, causal=False, fused=False, max_cache_len=0, factor=8, seed=0):
+                 norm_mode=POST_NORESID, causal=False, fused=False, max_cache_len=0, factor=8, weight_layout=0, seed=0):
         lib.lgh_clear_error()
         self.h = lib.lgh_model_create(dtype, max_batch, max_seq, head_num, size_per_head, layer_num, world_size, ffn_inner,
-                                      norm_mode, int(causal), int(fused), max_cache_len, factor, seed)
+                                      norm_mode, int(causal), int(fused), max_cache_len, factor, weight_layout, seed)
         if not self.h:
             check(1, "lgh_model_create")
         self.dtype = dtype
@@ -134,23 +134,35 @@ class Model:
     def stream(self):
         return lib.lgh_model_stream(self.h)
 
-    def params(self):
-        """name -> (device pointer, element count)"""
+    def param_info(self):
+        """name -> dict(ptr, elems, rows, cols, transposed); rows x cols is the logical [in, out] shape"""
         out = {}
         for i in range(lib.lgh_model_param_count(self.h)):
             name = C.create_string_buffer(128)
             ptr, n = _p(), _i64()
-            check(lib.lgh_model_param_info(self.h, i, name, 128, C.byref(ptr), C.byref(n)), "lgh_model_param_info")
-            out[name.value.decode()] = (ptr.value, n.value)
+            r, c, t = _i(), _i(), _i()
+            check(lib.lgh_model_param_info(self.h, i, name, 128, C.byref(ptr), C.byref(n), C.byref(r), C.byref(c), C.byref(t)),
+                  "lgh_model_param_info")
+            out[name.value.decode()] = dict(ptr=ptr.value, elems=n.value, rows=r.value, cols=c.value, transposed=t.value)
         return out
 
+    def params(self):
+        """name -> (device pointer, element count)"""
+        return {k: (v["ptr"], v["elems"]) for k, v in self.param_info().items()}
+
     def download_params(self):
-        """name -> float32 numpy array (exact values of the device parameters)"""
+        """name -> float32 numpy array with the exact device values; weight matrices come back in the logical [in, out]
+        orientation whatever their storage layout, vectors flat"""
         res = {}
-        for name, (ptr, n) in self.params().items():
+        for name, info in self.param_info().items():
+            n = info["elems"]
             raw = np.empty(n, dtype=np.float16 if self.dtype == capi.F16 else np.float32)
-            capi.check(capi.lib.lg_memcpy_d2h(raw.ctypes.data_as(_p), _p(ptr), n * self.es), "lg_memcpy_d2h")
-            res[name] = raw.astype(np.float32)
+            capi.check(capi.lib.lg_memcpy_d2h(raw.ctypes.data_as(_p), _p(info["ptr"]), n * self.es), "lg_memcpy_d2h")
+            a = raw.astype(np.float32)
+            if info["rows"] > 1:
+                a = a.reshape(info["cols"], info["rows"]).T if info["transposed"] else a.reshape(info["rows"], info["cols"])
+                a = np.ascontiguousarray(a)
+            res[name] = a
         return res
 
     def describe(self, batch, seq, decode_past=-1):

@@ -143,7 +143,8 @@ void lgh_clear_error(void) { clear_error(); }
 
 // dtype 0 = fp32, 1 = fp16.  head_num and ffn_inner are GLOBAL sizes; the model holds the 1/world_size shard.
 void* lgh_model_create(int dtype, int max_batch, int max_seq, int head_num, int size_per_head, int layer_num, int world_size,
-                       int ffn_inner, int norm_mode, int causal, int fused, int max_cache_len, int factor, uint64_t seed) {
+                       int ffn_inner, int norm_mode, int causal, int fused, int max_cache_len, int factor, int weight_layout,
+                       uint64_t seed) {
     if (max_batch <= 0 || max_seq <= 0 || head_num <= 0 || size_per_head <= 0 || layer_num <= 0 || world_size <= 0 ||
         head_num % world_size != 0 || (ffn_inner > 0 && ffn_inner % world_size != 0) || (dtype != 0 && dtype != 1)) {
         fail("lgh_model_create: bad configuration");
@@ -153,6 +154,7 @@ void* lgh_model_create(int dtype, int max_batch, int max_seq, int head_num, int 
     if (max_cache_len > 0 && !fused) { fail("lgh_model_create: the KV cache needs the fused assembly"); return nullptr; }
     BertInitParam P(max_batch, max_seq, head_num, size_per_head, layer_num, 0, factor, 0);
     P.ffn_inner = ffn_inner; P.norm_mode = norm_mode; P.causal = causal; P.fused = fused; P.max_cache_len = max_cache_len;
+    P.weight_layout = weight_layout ? 1 : 0;
     StaticInitParam S(0, world_size, dtype);
     const int hidden = head_num * size_per_head;
     ModelBase* mb = nullptr;
@@ -192,13 +194,17 @@ int64_t lgh_model_workspace_elems(void* model, int batch, int seq) { return mode
 void* lgh_model_stream(void* model) { return model ? ((ModelBase*)model)->stream0->stream : nullptr; }
 
 int lgh_model_param_count(void* model) { return model ? (int)((ModelBase*)model)->params().size() : -1; }
-int lgh_model_param_info(void* model, int idx, char* name, int name_len, void** ptr, int64_t* elems) {
+int lgh_model_param_info(void* model, int idx, char* name, int name_len, void** ptr, int64_t* elems, int* rows, int* cols,
+                         int* transposed) {
     if (!model) return fail("lgh_model_param_info: null model");
     auto ps = ((ModelBase*)model)->params();
     if (idx < 0 || idx >= (int)ps.size()) return fail("lgh_model_param_info: index out of range");
     if (name && name_len > 0) { strncpy(name, ps[idx].name.c_str(), (size_t)name_len - 1); name[name_len - 1] = 0; }
     if (ptr) *ptr = ps[idx].ptr;
     if (elems) *elems = ps[idx].elems;
+    if (rows) *rows = ps[idx].rows;
+    if (cols) *cols = ps[idx].cols;
+    if (transposed) *transposed = ps[idx].transposed;
     return LG_OK;
 }
 

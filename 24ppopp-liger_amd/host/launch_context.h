@@ -94,6 +94,8 @@ class BertInitParam {
     int causal = 0;         // 1 -> lower-triangular attr_mask
     int fused = 0;          // 1 -> bias/GELU/transposes folded into GEMM epilogues, one fused attention kernel
     int max_cache_len = 0;  // > 0 -> layers own a KV cache [max_batch, heads, max_cache_len, d] for decode steps
+    int weight_layout = 0;  // 0: weights stored [in, out] (what the reference's (N,N) cuBLAS call implies);
+                            // 1: stored [out, in] and multiplied with transa = T (both operands K-contiguous)
     BertInitParam() {}
     BertInitParam(int max_batch_size_, int max_seq_len_, int head_num_, int size_per_head_, int layer_num_,
                   int kernel_num_, int factor_, int rq_interval_)

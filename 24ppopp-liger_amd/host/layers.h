@@ -46,6 +46,8 @@ struct ParamRef {
     std::string name;
     void* ptr;
     int64_t elems;
+    int rows = 1, cols = 0;   // logical shape [in, out] of a weight matrix (vectors: rows = 1)
+    int transposed = 0;       // 1: stored as [out, in]
 };
 
 // ---------------------------------------------------------------------------------------------------
@@ -60,18 +62,22 @@ class Linear_Col {  // linear.h:68-109: output features split across ranks
     StaticInitParam SParams;
     std::vector<FuncWrap> FuncWrapVec;
 
-    Linear_Col(const StaticInitParam& SParams_, const int& k_, const int& n_) : k(k_), n(n_), SParams(SParams_) {
+    int weight_layout = 0;  // 0: [k, n_local] row-major; 1: [n_local, k] row-major (multiplied with transa = T)
+
+    Linear_Col(const StaticInitParam& SParams_, const int& k_, const int& n_, int weight_layout_ = 0)
+        : k(k_), n(n_), SParams(SParams_), weight_layout(weight_layout_) {
         weights = dev_alloc<T>((size_t)k * n / SParams.world_size);
     }
+    ParamRef param(const std::string& name) { return ParamRef{name, weights, (int64_t)k * n_local(), k, n_local(), weight_layout}; }
     int n_local() const { return n / SParams.world_size; }
     void init_weights(uint64_t seed, uint64_t tensor_id, float stddev = 0.02f) {
         dev_fill_normal(weights, (int64_t)k * n_local(), seed, tensor_id, 0.f, stddev);
     }
     GemmDesc desc(T* input, T* output, int m) const {
         GemmDesc g;
-        g.valid = true; g.dtype = dtype_of<T>::value; g.transa = 0;
+        g.valid = true; g.dtype = dtype_of<T>::value; g.transa = weight_layout;
         g.m = n_local(); g.n = m; g.k = k;
-        g.A = weights; g.lda = n_local(); g.B = input; g.ldb = k; g.C = output; g.ldc = n_local();
+        g.A = weights; g.lda = weight_layout ? k : n_local(); g.B = input; g.ldb = k; g.C = output; g.ldc = n_local();
         return g;
     }
     std::vector<FuncWrap> forward(T* input, T* output, int m) {
@@ -90,18 +96,22 @@ class Linear_Row {  // linear.h:16-64: input features split across ranks; partia
     StaticInitParam SParams;
     std::vector<FuncWrap> FuncWrapVec;
 
-    Linear_Row(const StaticInitParam& SParams_, const int& k_, const int& n_) : k(k_), n(n_), SParams(SParams_) {
+    int weight_layout = 0;  // 0: [k_local, n] row-major; 1: [n, k_local] row-major (multiplied with transa = T)
+
+    Linear_Row(const StaticInitParam& SParams_, const int& k_, const int& n_, int weight_layout_ = 0)
+        : k(k_), n(n_), SParams(SParams_), weight_layout(weight_layout_) {
         weights = dev_alloc<T>((size_t)k * n / SParams.world_size);
     }
+    ParamRef param(const std::string& name) { return ParamRef{name, weights, (int64_t)k_local() * n, k_local(), n, weight_layout}; }
     int k_local() const { return k / SParams.world_size; }
     void init_weights(uint64_t seed, uint64_t tensor_id, float stddev = 0.02f) {
         dev_fill_normal(weights, (int64_t)k_local() * n, seed, tensor_id, 0.f, stddev);
     }
     GemmDesc desc(T* input, T* output, int m) const {
         GemmDesc g;
-        g.valid = true; g.dtype = dtype_of<T>::value; g.transa = 0;
+        g.valid = true; g.dtype = dtype_of<T>::value; g.transa = weight_layout;
         g.m = n; g.n = m; g.k = k_local();
-        g.A = weights; g.lda = n; g.B = input; g.ldb = k_local(); g.C = output; g.ldc = n;
+        g.A = weights; g.lda = weight_layout ? k_local() : n; g.B = input; g.ldb = k_local(); g.C = output; g.ldc = n;
         return g;
     }
     std::vector<FuncWrap> forward(T* input, T* output, int m) {
@@ -164,8 +174,8 @@ class Bert_MLP {
     Bert_MLP(const BertInitParam& BertParams_, const StaticInitParam& SParam_, const int& k_, const int& n_, T* workspace)
         : k(k_), n(n_), SParam(SParam_), BertParams(BertParams_), linear_row_output(workspace) {
         intermediate_size = BertParams.ffn_inner > 0 ? BertParams.ffn_inner : n * mlp_ratio;
-        linear_col = new Linear_Col<T>(SParam, k, intermediate_size);
-        linear_row = new Linear_Row<T>(SParam, intermediate_size, k);
+        linear_col = new Linear_Col<T>(SParam, k, intermediate_size, BertParams.weight_layout);
+        linear_row = new Linear_Row<T>(SParam, intermediate_size, k, BertParams.weight_layout);
         bias = dev_alloc<T>(f_local());
         bias2 = dev_alloc<T>(k);
         dev_fill_const(bias, f_local(), 0.f);
@@ -179,10 +189,10 @@ class Bert_MLP {
         dev_fill_normal(bias2, k, seed, base + 3, 0.f, 0.02f);
     }
     void params(const std::string& prefix, std::vector<ParamRef>& out) {
-        out.push_back({prefix + "w1", linear_col->weights, (int64_t)k * f_local()});
-        out.push_back({prefix + "b1", bias, f_local()});
-        out.push_back({prefix + "w2", linear_row->weights, (int64_t)f_local() * k});
-        out.push_back({prefix + "b2", bias2, k});
+        out.push_back(linear_col->param(prefix + "w1"));
+        out.push_back({prefix + "b1", bias, f_local(), 1, f_local(), 0});
+        out.push_back(linear_row->param(prefix + "w2"));
+        out.push_back({prefix + "b2", bias2, k, 1, k, 0});
     }
     // inner: [m, F local] scratch.  idx 11, 12, 13 of the launch vector (fused: 2 entries).
     std::vector<FuncWrap> forward(T* input, T* output, int m, T* inner = nullptr) {
@@ -239,10 +249,10 @@ class Bert_MHA {
     Bert_MHA(const BertInitParam& BertParams_, const StaticInitParam& SParam_, const int& k_, const int& n_, T* workspace_)
         : k(k_), n(n_), SParam(SParam_), BertParams(BertParams_), workspace(workspace_) {
         scalar = 1.0f / sqrtf((float)BertParams.size_per_head);  // bert_layer.h:94
-        linear_q_col = new Linear_Col<T>(SParam, k, n);
-        linear_k_col = new Linear_Col<T>(SParam, k, n);
-        linear_v_col = new Linear_Col<T>(SParam, k, n);
-        linear_w_row = new Linear_Row<T>(SParam, k, n);
+        linear_q_col = new Linear_Col<T>(SParam, k, n, BertParams.weight_layout);
+        linear_k_col = new Linear_Col<T>(SParam, k, n, BertParams.weight_layout);
+        linear_v_col = new Linear_Col<T>(SParam, k, n, BertParams.weight_layout);
+        linear_w_row = new Linear_Row<T>(SParam, k, n, BertParams.weight_layout);
         q_bias = dev_alloc<T>(hl()); k_bias = dev_alloc<T>(hl()); v_bias = dev_alloc<T>(hl());
         w_bias = dev_alloc<T>(n);
         dev_fill_const(q_bias, hl(), 0.f); dev_fill_const(k_bias, hl(), 0.f); dev_fill_const(v_bias, hl(), 0.f);
@@ -268,14 +278,14 @@ class Bert_MHA {
         dev_fill_normal(w_bias, n, seed, base + 7, 0.f, 0.02f);
     }
     void params(const std::string& prefix, std::vector<ParamRef>& out) {
-        out.push_back({prefix + "wq", linear_q_col->weights, (int64_t)k * hl()});
-        out.push_back({prefix + "wk", linear_k_col->weights, (int64_t)k * hl()});
-        out.push_back({prefix + "wv", linear_v_col->weights, (int64_t)k * hl()});
-        out.push_back({prefix + "bq", q_bias, hl()});
-        out.push_back({prefix + "bk", k_bias, hl()});
-        out.push_back({prefix + "bv", v_bias, hl()});
-        out.push_back({prefix + "wo", linear_w_row->weights, (int64_t)hl() * n});
-        out.push_back({prefix + "bo", w_bias, n});
+        out.push_back(linear_q_col->param(prefix + "wq"));
+        out.push_back(linear_k_col->param(prefix + "wk"));
+        out.push_back(linear_v_col->param(prefix + "wv"));
+        out.push_back({prefix + "bq", q_bias, hl(), 1, hl(), 0});
+        out.push_back({prefix + "bk", k_bias, hl(), 1, hl(), 0});
+        out.push_back({prefix + "bv", v_bias, hl(), 1, hl(), 0});
+        out.push_back(linear_w_row->param(prefix + "wo"));
+        out.push_back({prefix + "bo", w_bias, n, 1, n, 0});
     }
     static int64_t score_elems(const BertInitParam& P, const StaticInitParam& S, int batch, int seq) {
         const bool fused = P.fused && dtype_of<T>::value == LG_F16;
@@ -458,11 +468,11 @@ class Bert_Encoder {
     }
     void params(const std::string& prefix, std::vector<ParamRef>& out) {
         MHA->params(prefix, out);
-        out.push_back({prefix + "ln1_g", ln_mha->gamma, k});
-        out.push_back({prefix + "ln1_b", ln_mha->beta, k});
+        out.push_back({prefix + "ln1_g", ln_mha->gamma, k, 1, k, 0});
+        out.push_back({prefix + "ln1_b", ln_mha->beta, k, 1, k, 0});
         MLP->params(prefix, out);
-        out.push_back({prefix + "ln2_g", ln_mlp->gamma, k});
-        out.push_back({prefix + "ln2_b", ln_mlp->beta, k});
+        out.push_back({prefix + "ln2_g", ln_mlp->gamma, k, 1, k, 0});
+        out.push_back({prefix + "ln2_b", ln_mlp->beta, k, 1, k, 0});
     }
     static int64_t workspace_elems(const BertInitParam& P, const StaticInitParam& S, int batch, int seq) {
         const int hidden = P.head_num * P.size_per_head;

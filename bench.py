@@ -28,7 +28,7 @@ def gemm_flops_cfg2():
     return {"q": 2 * M * H * Hl, "k": 2 * M * H * Hl, "v": 2 * M * H * Hl, "out": 2 * M * Hl * H, "ffn1": 2 * M * H * F, "ffn2": 2 * M * F * H}
 
 
-def cpu_baseline(po, sample_batch=1, sample_seq=256):
+def cpu_baseline(po, sample_batch=2, sample_seq=512):
     """Times the CPU oracle (OpenMP C) on a bounded sample of the cfg2 layer: same shard shapes, M = sample rows,
     and scales linearly to M = 4096 (GEMM time is linear in M; attention at this size is < 1 % of the work)."""
     import numpy as np
@@ -62,6 +62,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--unfused", action="store_true", help="time the reference-shaped 14-entry assembly instead")
+    ap.add_argument("--weight-layout", type=int, default=1, choices=[0, 1],
+                    help="0: weights stored [in, out] (the reference's cuBLAS (N,N) layout); 1: stored [out, in] (default)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs one GPU's tensor-parallel shard on one GPU; --gpus %d is not supported "
@@ -80,7 +82,7 @@ def main():
     fused = not args.unfused
     model = host.Model(capi.F16, 32, S, c["heads_global"], c["d"], layer_num=1, world_size=c["world_size"], ffn_inner=c["ffn_global"],
                        norm_mode=host.POST_NORESID, causal=True, fused=fused, max_cache_len=CFG3["cache_len"] + 32 if fused else 0,
-                       seed=0)
+                       weight_layout=args.weight_layout, seed=0)
     x = torch.empty(M, H, device="cuda", dtype=torch.float16)
     capi.call("lg_fill_normal_f16", x.data_ptr(), x.numel(), 0, 99, 0.0, 1.0, None)
     y = torch.empty_like(x)
@@ -150,7 +152,8 @@ def main():
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": "cfg2 prefill: hidden 12288, 48/96 heads x 128, FFN 16384/32768, batch 8 x seq 512, causal; "
-                               + ("fused assembly (9 launches/layer)" if fused else "reference-shaped assembly (14 launches/layer)")},
+                               + ("fused assembly (9 launches/layer)" if fused else "reference-shaped assembly (14 launches/layer)")
+                               + ("; weights stored [out, in]" if args.weight_layout else "; weights stored [in, out]")},
         "tokens_per_s": round(M / (ms_per_step * 1e-3), 1),
         "roofline": roofline,
         "layer_norm_GBps": round(ln_gbs, 1) if ln_gbs else None,

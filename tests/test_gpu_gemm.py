@@ -14,7 +14,9 @@ def rnd(po, n, tid, dt, std=1.0):
 
 # (tokens, out_features, k): aligned, ragged, tiny, skinny (decode-like)
 SHAPES = [(64, 256, 256), (128, 128, 32), (130, 136, 72), (1, 8, 8), (33, 70, 19), (32, 1024, 512), (257, 96, 1000),
-          (512, 384, 160)]
+          (512, 384, 160),
+          # multiples of the 256 x 256 x 64 tile: the pipelined kernel
+          (256, 256, 64), (512, 768, 256), (256, 512, 1024), (1024, 2048, 192), (2048, 256, 128)]
 
 
 @pytest.mark.parametrize("dt", [0, 1])
@@ -114,3 +116,33 @@ def test_gemm_fused_epilogues(dev, po, transa):
     out = dev.empty((M, N), 1)
     dev.call("lg_gemm_fused_f16", transa, N, M, K, dA, lda, dX, K, out, N, dev.capi.EPI_BIAS, dB, 0, 0, 0)
     assert max_rel_err(dev.down(out), po.round_f16(y + bias)) < 2e-3
+
+
+@pytest.mark.parametrize("transa", [0, 1])
+def test_gemm_fused_epilogues_on_the_pipelined_kernel(dev, po, transa):
+    """Same epilogues on a tile-aligned problem (256-multiples), which takes the pipelined kernel, incl. a column slice
+    written into a wider head-transposed destination (the decomposition case)."""
+    B, S, h, d, K = 2, 256, 4, 128, 320
+    M, N = B * S, h * d
+    X = rnd(po, M * K, 40, 1).reshape(M, K)
+    W = rnd(po, K * N, 41, 1, 0.05).reshape(K, N)
+    bias = rnd(po, N, 42, 1, 0.3)
+    A, lda = (np.ascontiguousarray(W.T), K) if transa else (W, N)
+    dA, dX, dB = dev.up(A, 1), dev.up(X, 1), dev.up(bias, 1)
+    y = po.gemm(X, W, 1)
+    out = dev.empty((M, N), 1)
+    dev.call("lg_gemm_fused_f16", transa, N, M, K, dA, lda, dX, K, out, N, dev.capi.EPI_BIAS_GELU, dB, 0, 0, 0)
+    assert max_rel_err(dev.down(out), po.add_bias_gelu(y.copy(), bias, 1)) < 4e-3
+    ref_heads, _, _ = po.add_qkv_bias_transpose(y, bias, y, bias, y, bias, B, S, h, d, 1)
+    rows = S + 32  # destination reserves more rows per (batch, head) than the sequence has (a KV cache)
+    out = dev.empty((B, h, rows, d), 1)
+    out.zero_()
+    half = N // 2
+    es = 2
+    a_off = (half * K if transa else half) * es
+    dev.call("lg_gemm_fused_f16", transa, half, M, K, dA, lda, dX, K, out, rows, dev.capi.EPI_BIAS_HEADS, dB, S, d, h)
+    dev.call("lg_gemm_fused_f16", transa, N - half, M, K, dA.data_ptr() + a_off, lda, dX, K,
+             out.data_ptr() + (half // d) * rows * d * es, rows, dev.capi.EPI_BIAS_HEADS, dB.data_ptr() + half * es, S, d, h)
+    got = dev.down(out)
+    assert max_rel_err(got[:, :, :S], ref_heads) < 2e-3
+    assert np.all(got[:, :, S:] == 0)

@@ -23,10 +23,10 @@ def oracle_weights(params, layer=0):
     return {k[len(pre):]: v for k, v in params.items() if k.startswith(pre)}
 
 
-def run_layer_case(dev, po, host, dtype, B, S, heads, d, F, norm_mode, causal, fused, ws=1, layers=1, seed=0):
+def run_layer_case(dev, po, host, dtype, B, S, heads, d, F, norm_mode, causal, fused, ws=1, layers=1, seed=0, weight_layout=0):
     H = heads * d
     m = host.Model(dtype, B, S, heads, d, layer_num=layers, world_size=ws, ffn_inner=F, norm_mode=norm_mode, causal=causal,
-                   fused=fused, seed=seed)
+                   fused=fused, weight_layout=weight_layout, seed=seed)
     params = m.download_params()
     x = po.fill_normal(B * S * H, seed, 99, 0.0, 1.0, dtype).reshape(B * S, H)
     dx = dev.up(x, dtype)
@@ -67,9 +67,19 @@ def test_fp16_layer_small(dev, po, host, norm_mode, causal, fused):
 
 
 @pytest.mark.parametrize("fused", [False, True])
-def test_fp16_tp2_shard_two_layers(dev, po, host, fused):
-    """One TP=2 shard (half the heads, half the FFN) of a 2-layer stack, GLM-like head size 128, ragged seq."""
-    got, ref, _ = run_layer_case(dev, po, host, 1, 2, 200, 8, 128, 2048, 0, True, fused, ws=2, layers=2)
+@pytest.mark.parametrize("weight_layout", [0, 1])
+def test_fp16_tp2_shard_two_layers(dev, po, host, fused, weight_layout):
+    """One TP=2 shard (half the heads, half the FFN) of a 2-layer stack, GLM-like head size 128, ragged seq; weights
+    stored [in, out] (the reference's layout) or [out, in]."""
+    got, ref, _ = run_layer_case(dev, po, host, 1, 2, 200, 8, 128, 2048, 0, True, fused, ws=2, layers=2, weight_layout=weight_layout)
+    assert max_rel_err(got, ref) < 1e-2
+
+
+@pytest.mark.parametrize("weight_layout", [0, 1])
+def test_fp16_layer_on_the_pipelined_gemm(dev, po, host, weight_layout):
+    """Shapes that are multiples of the 256 x 256 x 64 tile, so every weight GEMM takes the pipelined kernel
+    (hidden 1024, 8 heads x 128, FFN 2048, 512 tokens)."""
+    got, ref, _ = run_layer_case(dev, po, host, 1, 2, 256, 8, 128, 2048, 0, True, True, weight_layout=weight_layout)
     assert max_rel_err(got, ref) < 1e-2
 
 
@@ -86,7 +96,7 @@ def test_decode_step_matches_oracle(dev, po, host):
     ref_prefill = po.encoder_forward(shape, w, x)
     assert max_rel_err(dev.down(dy), ref_prefill) < 1e-2
     # oracle-side cache from the same prefill
-    q = po.gemm(x, w["wq"].reshape(H, H), 1); k = po.gemm(x, w["wk"].reshape(H, H), 1); v = po.gemm(x, w["wv"].reshape(H, H), 1)
+    q = po.gemm(x, w["wq"], 1); k = po.gemm(x, w["wk"], 1); v = po.gemm(x, w["wv"], 1)
     _, kb, vb = po.add_qkv_bias_transpose(q, w["bq"], k, w["bk"], v, w["bv"], B, S, heads, d, 1)
     kc = np.zeros((B, heads, Lmax, d), dtype=np.float32); vc = np.zeros_like(kc)
     kc[:, :, :S] = kb; vc[:, :, :S] = vb
