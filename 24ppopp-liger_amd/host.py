@@ -42,6 +42,7 @@ SIGNATURES = {
     "lgh_model_run": (_i, [_p, _p, _p, _i, _i, _p, _p, _i]),
     "lgh_model_run_decode": (_i, [_p, _p, _p, _i, _i, _i, _p, _p]),
     "lgh_model_time_kernels": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, C.POINTER(_f), _i]),
+    "lgh_model_time_one": (_f, [_p, _p, _p, _i, _i, _i, _i, _i, _i]),
     "lgh_sched_create": (_p, [_p, _i, _f, _i, _i, _i, _i, _i, _i]),
     "lgh_sched_profile": (_i, [_p, _i, _i, _i, _i, _i]),
     "lgh_sched_profile_decode": (_i, [_p, _i, _i, _i]),
@@ -52,6 +53,9 @@ SIGNATURES = {
     "lgh_sched_run_trace": (_i, [_p, _i, C.POINTER(_d), C.POINTER(_i), C.POINTER(_i), C.POINTER(_i), _i, C.POINTER(Report)]),
     "lgh_sched_set_profile": (_i, [_p, _i, _i, _i, _f, C.POINTER(_f), _i]),
     "lgh_sched_serve": (_i, [_p, _i, _i, _i]),
+    "lgh_sched_serve_decode": (_i, [_p, _i, _i, _i]),
+    "lgh_sched_set_factor": (_i, [_p, _i]),
+    "lgh_sched_ctx_ptrs": (_i, [_p, _i, C.POINTER(_p), C.POINTER(_p)]),
     "lgh_sched_run_queued": (_i, [_p, _i, C.POINTER(Report)]),
     "lgh_summarize": (_i, [C.POINTER(_d), C.POINTER(_d), _i, _d, C.POINTER(Report)]),
     "lgh_make_poisson_trace": (_i, [_d, _i, _i, _i, _i, _i, _i, _u64, C.POINTER(_d), C.POINTER(_i)]),
@@ -224,6 +228,17 @@ class Scheduler:
 
     def serve(self, bs, seq, n_decode=0):
         check(lib.lgh_sched_serve(self.h, bs, seq, n_decode), "lgh_sched_serve")
+
+    def serve_decode(self, bs, past, n_steps):
+        check(lib.lgh_sched_serve_decode(self.h, bs, past, n_steps), "lgh_sched_serve_decode")
+
+    def set_factor(self, factor):
+        check(lib.lgh_sched_set_factor(self.h, factor), "lgh_sched_set_factor")
+
+    def ctx_ptrs(self, i):
+        a, b = _p(), _p()
+        check(lib.lgh_sched_ctx_ptrs(self.h, i, C.byref(a), C.byref(b)), "lgh_sched_ctx_ptrs")
+        return a.value, b.value
 
     def run_queued(self, mode):
         r = Report()

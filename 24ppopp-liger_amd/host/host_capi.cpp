@@ -26,6 +26,9 @@ struct SchedBase {
     virtual int sub_lookup(int name, int bs, int seq, float* out, int cap) = 0;
     virtual void set_profile(int name, int bs, int seq, float ms, const float* sub, int nsub) = 0;
     virtual void serve(int bs, int seq, int n_decode) = 0;
+    virtual void serve_decode(int bs, int past, int n_steps) = 0;
+    virtual void set_factor(int factor) = 0;
+    virtual bool ctx_ptrs(int i, void** in, void** out) = 0;
     virtual Report run_queued(int mode, int* counters) = 0;
 };
 
@@ -78,6 +81,14 @@ struct SchedT : SchedBase {
         if (sub && nsub > 0) s->profiling_decompse_res_dict[{name, bs, seq}] = std::vector<float>(sub, sub + nsub);
     }
     void serve(int bs, int seq, int n_decode) override { s->serve(bs, seq, n_decode); }
+    void serve_decode(int bs, int past, int n_steps) override { s->serve_decode(bs, past, n_steps); }
+    void set_factor(int factor) override { s->BertParams.factor = factor; }
+    bool ctx_ptrs(int i, void** in, void** out) override {
+        auto* c = s->context(i);
+        if (!c) return false;
+        *in = c->input; *out = c->output;
+        return true;
+    }
     Report run_queued(int mode, int* counters) override {
         s->reset_run();
         s->run_stop();  // everything is already queued: the loop ends once it has drained
@@ -334,6 +345,22 @@ int lgh_sched_serve(void* sched, int bs, int seq, int n_decode) {
     ((SchedBase*)sched)->serve(bs, seq, n_decode);
     return first_error();
 }
+int lgh_sched_serve_decode(void* sched, int bs, int past, int n_steps) {
+    if (!sched || bs <= 0 || past < 0 || n_steps <= 0) return fail("lgh_sched_serve_decode: bad arguments");
+    ((SchedBase*)sched)->serve_decode(bs, past, n_steps);
+    return first_error();
+}
+// decomposition factor used by profile() and by the samples queued afterwards
+int lgh_sched_set_factor(void* sched, int factor) {
+    if (!sched || factor < 1) return fail("lgh_sched_set_factor: bad arguments");
+    ((SchedBase*)sched)->set_factor(factor);
+    return LG_OK;
+}
+// input / output buffers of the i-th per-request context (creation order; requests take contexts in that order)
+int lgh_sched_ctx_ptrs(void* sched, int i, void** input, void** output) {
+    if (!sched || !input || !output || !((SchedBase*)sched)->ctx_ptrs(i, input, output)) return fail("lgh_sched_ctx_ptrs: no such context");
+    return LG_OK;
+}
 int lgh_sched_run_queued(void* sched, int mode, LghReport* out) {
     if (!sched || !out) return fail("lgh_sched_run_queued: bad arguments");
     int c[4] = {0, 0, 0, 0};
@@ -358,6 +385,33 @@ int lgh_make_poisson_trace(double lambda, int n, int batch, int seq_lo, int seq_
     auto tr = make_poisson_trace(lambda, n, batch, seq_lo, seq_hi, seq_round, n_decode, seed);
     for (int i = 0; i < n; ++i) { arrival_s[i] = tr[i].arrival_s; seq_out[i] = tr[i].seq; }
     return LG_OK;
+}
+
+
+// Launches entry `index` of the vector `iters` times back to back between two events on the model's stream (after one
+// full pass of the vector so that its inputs are valid); returns the average milliseconds per launch, or -1.
+float lgh_model_time_one(void* model, void* input, void* output, int batch, int seq, int decode_past, int cache_slot, int index,
+                         int iters) {
+    ModelBase* mb = (ModelBase*)model;
+    if (!mb || !input || !output || iters <= 0) { fail("lgh_model_time_one: bad arguments"); return -1.f; }
+    std::vector<FuncWrap> v = decode_past >= 0 ? mb->build_decode(input, output, batch, decode_past, cache_slot, nullptr)
+                                               : mb->build(input, output, batch, seq, nullptr, cache_slot);
+    if (index < 0 || index >= (int)v.size()) { fail("lgh_model_time_one: index out of range"); return -1.f; }
+    DynamicInitParam& D = *mb->stream0;
+    for (auto& f : v) f.callback(D);
+    note_status(lg_stream_synchronize(D.stream), "lg_stream_synchronize");
+    void *e0 = nullptr, *e1 = nullptr;
+    note_status(lg_event_create(&e0), "lg_event_create");
+    note_status(lg_event_create(&e1), "lg_event_create");
+    note_status(lg_event_record(e0, D.stream), "lg_event_record");
+    for (int i = 0; i < iters; ++i) v[index].callback(D);
+    note_status(lg_event_record(e1, D.stream), "lg_event_record");
+    note_status(lg_event_synchronize(e1), "lg_event_synchronize");
+    float ms = 0.f;
+    note_status(lg_event_elapsed_ms(&ms, e0, e1), "lg_event_elapsed_ms");
+    lg_event_destroy(e0);
+    lg_event_destroy(e1);
+    return first_error() ? -1.f : ms / (float)iters;
 }
 
 }  // extern "C"

@@ -169,15 +169,18 @@ class Scheduler {
             c->slot = _pool_total * ctx_batch;
             dev_fill_normal(c->input, io, 1234, 50000 + _pool_total, 0.f, 1.f);
             _pool.push_back(c);
+            _all_ctx.push_back(c);
             _pool_total++;
         }
         note_status(lg_device_synchronize(), "lg_device_synchronize");
     }
+    // contexts in creation order (tests compare a request's output buffer with a plain sequential run)
+    const ReqCtx* context(int i) const { return (i >= 0 && i < (int)_all_ctx.size()) ? _all_ctx[i] : nullptr; }
     ReqCtx* acquire_ctx() {
         std::unique_lock<std::mutex> lk(_pool_mutex);
         _pool_cv.wait(lk, [this] { return !_pool.empty(); });
-        ReqCtx* c = _pool.back();
-        _pool.pop_back();
+        ReqCtx* c = _pool.front();
+        _pool.erase(_pool.begin());
         return c;
     }
     void release_ctx(ReqCtx* c) {
@@ -289,6 +292,36 @@ class Scheduler {
             }
         }
         Sample* sample = new Sample(vec, profiling_decompse_res_dict, batch_size, seq_len, BertParams.factor, policy, axis);
+        sample->user = ctx;
+        {
+            std::lock_guard<std::mutex> lk(_q_mutex);
+            sample->id = _next_id++;
+            _main_q.push_back(sample);
+        }
+    }
+
+    // Queues a request that consists of decode steps only: `n_steps` single-token steps for `batch_size` sequences that
+    // already have `past` cached positions (cache contents are whatever the slot holds).  No reference counterpart.
+    void serve_decode(int batch_size, int past, int n_steps) {
+        ReqCtx* ctx = _pool_total ? acquire_ctx() : nullptr;
+        T* din = ctx ? ctx->dec_a : input;
+        T* dout = ctx ? ctx->dec_b : output;
+        T* ws = ctx ? ctx->ws : nullptr;
+        const int slot = ctx ? ctx->slot : 0;
+        const int kd = _model->kernels_per_layer(true);
+        std::vector<FuncWrap> vec;
+        for (int t = 0; t < n_steps; ++t) {
+            const int p = past + t;
+            std::vector<FuncWrap> dv = _model->forward_decode(din, dout, batch_size, p, slot, ws);
+            const int key_past = seq_bucket > 1 ? (p + seq_bucket - 1) / seq_bucket * seq_bucket : p;
+            for (size_t j = 0; j < dv.size(); ++j) {
+                dv[j].name = 1000 + (int)(j % kd);
+                dv[j].duration = lookup(dv[j].name, batch_size, key_past);
+            }
+            vec.insert(vec.end(), dv.begin(), dv.end());
+            std::swap(din, dout);
+        }
+        Sample* sample = new Sample(vec, profiling_decompse_res_dict, batch_size, past, BertParams.factor, policy, axis);
         sample->user = ctx;
         {
             std::lock_guard<std::mutex> lk(_q_mutex);
@@ -451,6 +484,7 @@ class Scheduler {
   private:
     std::vector<Sample*> _retired;
     int _pool_total = 0;
+    std::vector<ReqCtx*> _all_ctx;
     // a retired sample's buffers may be reused once its last kernel has finished
     void _reclaim() {
         for (size_t i = 0; i < _retired.size();) {

@@ -23,6 +23,17 @@ CFG2 = dict(hidden=12288, heads_global=96, d=128, ffn_global=32768, world_size=2
 CFG3 = dict(batch=32, cache_len=1024)
 
 
+def measured_traffic(label):
+    """HBM bytes per launch of `label` from the committed rocprofv3 counter runs (FETCH_SIZE + WRITE_SIZE, calibrated
+    against a copy kernel of known size; see profiles/).  None when no measurement is on file."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            k = json.load(f)["kernels"].get(label)
+        return int(k["fetch_bytes"] + k["write_bytes"]) if k else None
+    except (OSError, KeyError, ValueError):
+        return None
+
+
 def gemm_flops_cfg2():
     M, H, Hl, F = 4096, 12288, 6144, 16384
     return {"q": 2 * M * H * Hl, "k": 2 * M * H * Hl, "v": 2 * M * H * Hl, "out": 2 * M * Hl * H, "ffn1": 2 * M * H * F, "ffn2": 2 * M * F * H}
@@ -55,6 +66,101 @@ def cpu_baseline(po, sample_batch=2, sample_seq=512):
                 sample_batch, sample_seq, M, dt, scale)}
 
 
+def kernel_only(args, capi, host, model, x, y, B, S, H, stream):
+    """Launches one kernel repeatedly so that a profiler sees only it (same shapes and buffers as the bench)."""
+    import ctypes as C
+    import torch
+    name = args.kernel_only
+    if name == "copy":
+        # calibration kernel of known traffic: the transpose-back kernel moving 128 MiB in and 128 MiB out
+        src = torch.empty(1, 64, 8192, 128, device="cuda", dtype=torch.float16)
+        capi.call("lg_fill_normal_f16", src.data_ptr(), src.numel(), 0, 5, 0.0, 1.0, None)
+        dst = torch.empty_like(src)
+        for _ in range(args.iters):
+            capi.call("lg_transpose_f16", dst.data_ptr(), src.data_ptr(), 1, 8192, 64, 128, C.c_void_p(stream))
+        capi.call("lg_stream_synchronize", stream)
+        print(json.dumps({"kernel": "copy", "bytes_read": src.numel() * 2, "bytes_written": src.numel() * 2, "iters": args.iters}))
+        return
+    decode = name in ("attn_decode", "kv_append") or name.endswith("(decode)")
+    if decode:
+        Bd, L = CFG3["batch"], CFG3["cache_len"]
+        xd = torch.empty(Bd, H, device="cuda", dtype=torch.float16)
+        capi.call("lg_fill_normal_f16", xd.data_ptr(), xd.numel(), 0, 98, 0.0, 1.0, None)
+        yd = torch.empty_like(xd)
+        desc = model.describe(Bd, 1, decode_past=L - 1)
+        idx = [e["idx"] for e in desc if e["label"] == name]
+        if not idx:
+            sys.exit("no launch-vector entry named %r; have %s" % (name, [e["label"] for e in desc]))
+        ms = host.lib.lgh_model_time_one(model.h, xd.data_ptr(), yd.data_ptr(), Bd, 1, L - 1, 0, idx[0], args.iters)
+    else:
+        desc = model.describe(B, S)
+        idx = [e["idx"] for e in desc if e["label"] == name]
+        if not idx:
+            sys.exit("no launch-vector entry named %r; have %s" % (name, [e["label"] for e in desc]))
+        ms = host.lib.lgh_model_time_one(model.h, x.data_ptr(), y.data_ptr(), B, S, -1, -1, idx[0], args.iters)
+    print(json.dumps({"kernel": name, "iters": args.iters, "avg_ms_hip_events": round(ms, 5)}))
+
+
+def bench_cfg4(capi, host, weight_layout):
+    """BASELINE config 4: a prefill request (batch 4 x seq 512) is decomposed by factor 1, 2, 4, 8 (token rows) and
+    interleaved on two streams with a decode batch (32 sequences, 1024 cached positions, 8 steps); makespan against
+    sequential launch of the same two requests.  The decode batch is the primary request (its HBM-bound kernels open the
+    windows), the prefill's MFMA-bound GEMMs are the ones split to fit them."""
+    c = CFG2
+    out = []
+    model = host.Model(capi.F16, 36, 512, c["heads_global"], c["d"], layer_num=1, world_size=c["world_size"], ffn_inner=c["ffn_global"],
+                       causal=True, fused=True, max_cache_len=1024 + 64, weight_layout=weight_layout, seed=0)
+    for factor in (1, 2, 4, 8):
+        sched = host.Scheduler(model, schedule_deep=6, contention_factor=0.8, policy=host.POLICY_RESOURCE,
+                               axis=host.SPLIT_TOKEN_ROWS, seq_bucket=64, ignore_num=0, pool_count=0)
+        sched.set_factor(factor)
+        sched.profile(4, 512, 512, 1, 10)
+        sched.profile_decode(32, 1024, 10)
+        res = {"factor": factor}
+        for mode, name in ((host.MODE_SEQUENTIAL, "sequential"), (host.MODE_LIGER, "interleaved")):
+            best = None
+            for _ in range(3):
+                sched.serve_decode(32, 1000, 8)
+                sched.serve(4, 512, 0)
+                r = sched.run_queued(mode)
+                if best is None or r["total_duration_ms"] < best["total_duration_ms"]:
+                    best = r
+            res[name] = {"makespan_ms": round(best["total_duration_ms"], 4), "secondary_launches": best["secondary_launches"],
+                         "splits": best["splits"], "rounds": best["rounds"]}
+        res["speedup"] = round(res["sequential"]["makespan_ms"] / res["interleaved"]["makespan_ms"], 4)
+        out.append(res)
+    return {"workload": "cfg4: prefill B4 S512 (split by token rows) || decode B32 L1024 x 8 steps, one layer shard", "results": out}
+
+
+def bench_cfg5(capi, host, weight_layout, n_requests):
+    """BASELINE config 5: Poisson arrivals at 4, 8, 16 req/s through 4 stacked layer shards; prompts U[128, 1024]
+    (rounded to 64), 32 decode tokens each; mean and p99 request latency with interleaving on and off."""
+    c = CFG2
+    pool = 16
+    model = host.Model(capi.F16, pool, 1024, c["heads_global"], c["d"], layer_num=4, world_size=c["world_size"], ffn_inner=c["ffn_global"],
+                       causal=True, fused=True, max_cache_len=1024 + 64, weight_layout=weight_layout, factor=8, seed=0)
+    sched = host.Scheduler(model, schedule_deep=6, contention_factor=0.8, policy=host.POLICY_RESOURCE, axis=host.SPLIT_TOKEN_ROWS,
+                           seq_bucket=64, ignore_num=5, pool_count=pool, ctx_batch=1)
+    t0 = time.perf_counter()
+    sched.profile(1, 128, 1024, 64, 5)
+    for past in range(128, 1024 + 64 + 1, 64):
+        sched.profile_decode(1, min(past, 1024 + 63), 5)
+    prof_s = time.perf_counter() - t0
+    out = []
+    for lam in (4.0, 8.0, 16.0):
+        trace = host.make_poisson_trace(lam, n_requests, 1, 128, 1024, 64, 32, 0)
+        row = {"lambda_req_s": lam, "requests": n_requests}
+        for mode, name in ((host.MODE_SEQUENTIAL, "scheduling_off"), (host.MODE_LIGER, "scheduling_on")):
+            r = sched.run_trace(trace, mode)
+            row[name] = {"mean_latency_ms": round(r["avg_latency_ms"], 3), "p99_latency_ms": round(r["p99_latency_ms"], 3),
+                         "mean_gpu_ms": round(r["avg_gpu_ms"], 3), "mean_queue_ms": round(r["avg_queue_ms"], 3),
+                         "throughput_req_s": round(r["throughput"], 3), "records": r["records"],
+                         "secondary_launches": r["secondary_launches"], "splits": r["splits"], "profile_misses": r["profile_misses"]}
+        out.append(row)
+    return {"workload": "cfg5: 4 layer shards, Poisson arrivals, prompts U[128,1024] rounded to 64, 32 decode tokens", "profile_seconds": round(prof_s, 1),
+            "results": out}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -62,6 +168,13 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--unfused", action="store_true", help="time the reference-shaped 14-entry assembly instead")
+    ap.add_argument("--cfg4", action="store_true", help="also run the decomposition sweep (BASELINE config 4)")
+    ap.add_argument("--cfg5", action="store_true", help="also run the mixed request trace (BASELINE config 5); takes minutes")
+    ap.add_argument("--cfg5-requests", type=int, default=60)
+    ap.add_argument("--kernel-only", default=None,
+                    help="launch only the named launch-vector entry (e.g. 'ffn1+bias+gelu', 'attn_decode', 'layer_norm') or "
+                         "'copy' (a plain 128 MiB read + 128 MiB write kernel) --iters times; for rocprofv3 runs")
+    ap.add_argument("--iters", type=int, default=50)
     ap.add_argument("--weight-layout", type=int, default=1, choices=[0, 1],
                     help="0: weights stored [in, out] (the reference's cuBLAS (N,N) layout); 1: stored [out, in] (default)")
     args = ap.parse_args()
@@ -87,6 +200,10 @@ def main():
     capi.call("lg_fill_normal_f16", x.data_ptr(), x.numel(), 0, 99, 0.0, 1.0, None)
     y = torch.empty_like(x)
     stream = model.stream
+
+    if args.kernel_only:
+        kernel_only(args, capi, host, model, x, y, B, S, H, stream)
+        return
 
     def step():
         model.run(x.data_ptr(), y.data_ptr(), B, S, None, stream)
@@ -121,7 +238,7 @@ def main():
     dom_fl = label_flops[dom["kernel"]]
     achieved = dom_fl / (dom["ms"] * 1e-3) / 1e12
     roofline = {"bound": "mfma", "kernel": dom["kernel"], "achieved": round(achieved, 1), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(achieved / PEAK_FP16_TFLOPS, 4), "traffic": None,
+                "frac": round(achieved / PEAK_FP16_TFLOPS, 4), "traffic": measured_traffic(dom["kernel"]),
                 "all_gemms_tflops": round(gemm_fl / (gemm_ms * 1e-3) / 1e12, 1)}
     ln = [k for k in kernels if k["kernel"] == "layer_norm"]
     ln_gbs = (2 * M * H * 2) / (min(k["ms"] for k in ln) * 1e-3) / 1e9 if ln else None
@@ -143,7 +260,8 @@ def main():
         decode = {"workload": "cfg3: batch 32, 1 new token, 1024 cached positions", "ms_per_layer_shard": round(sum(dtimes), 4),
                   "tokens_per_s": round(Bd / (sum(dtimes) * 1e-3), 1), "kernels": dk,
                   "roofline_attn_decode": {"bound": "hbm", "achieved": round(kv_bytes / (attn["ms"] * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
-                                           "unit": "GB/s", "frac": round(kv_bytes / (attn["ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)},
+                                           "unit": "GB/s", "frac": round(kv_bytes / (attn["ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                                           "traffic": measured_traffic("attn_decode")},
                   "skinny_gemms": {"ms": round(gemm_dec_ms, 4), "weight_GBps": round(w_bytes / (gemm_dec_ms * 1e-3) / 1e9, 1)}}
 
     out = {
@@ -166,6 +284,11 @@ def main():
     if not args.no_cpu_baseline:
         from oracle import pyoracle as po
         out["cpu_baseline"] = cpu_baseline(po)
+    del model
+    if args.cfg4:
+        out["cfg4"] = bench_cfg4(capi, host, args.weight_layout)
+    if args.cfg5:
+        out["cfg5"] = bench_cfg5(capi, host, args.weight_layout, args.cfg5_requests)
     print(json.dumps(out))
 
 
