@@ -57,11 +57,11 @@ def test_interleaved_decomposed_requests_match_sequential_bitwise(dev, host, axi
 def test_prefill_plus_decode_trace_on_gpu(dev, host):
     """Requests with decode steps, profiled on the device, replayed in real time in both modes."""
     heads, d, F = 8, 128, 2048
-    m = host.Model(1, 4, 128, heads, d, layer_num=2, ffn_inner=F, causal=True, fused=True, max_cache_len=160, factor=4, weight_layout=1, seed=5)
+    m = host.Model(1, 4, 128, heads, d, layer_num=2, ffn_inner=F, causal=True, fused=True, max_cache_len=192, factor=4, weight_layout=1, seed=5)
     s = host.Scheduler(m, policy=host.POLICY_RESOURCE, axis=host.SPLIT_TOKEN_ROWS, seq_bucket=32, ignore_num=0, pool_count=4, ctx_batch=1)
     s.profile(1, 64, 128, 32, 3)
     for past in (64, 96, 128, 160):
-        s.profile_decode(1, min(past, 159), 3)
+        s.profile_decode(1, past, 3)
     assert s.lookup(0, 1, 128) > 0 and s.lookup(1004, 1, 128) > 0
     trace = [{"arrival_s": 0.001 * i, "batch": 1, "seq": 64 + 32 * (i % 3), "n_decode": 4} for i in range(10)]
     for mode in (host.MODE_SEQUENTIAL, host.MODE_LIGER):
