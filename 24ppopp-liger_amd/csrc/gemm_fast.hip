@@ -21,6 +21,7 @@
 //   * workgroup ids are remapped so that the 32 workgroups resident on one XCD (ids congruent mod 8) form a compact
 //     4 x 8 block of tiles and share their X / W panels in that XCD's L2.
 #include "gemm_common.cuh"
+#include <type_traits>
 
 namespace lg {
 
@@ -28,7 +29,9 @@ constexpr int FB_M = 256, FB_K = 64;
 constexpr int F_THREADS = 512;
 // The tile is 256 x (64 * NJ) outputs: NJ = 4 -> 256 x 256, NJ = 3 -> 256 x 192 (used when it needs fewer rounds of 256
 // workgroups, e.g. N = 6144: 512 tiles = 2 full rounds instead of 384 tiles = 1.5 rounds)
-constexpr int stage_halves(int NJ) { return FB_M * FB_K + FB_K * 64 * NJ; }  // X tile + W tile per stage
+// LDS: a ring of 3 X tiles and a ring of 2 W tiles (256-wide: 96 + 64 KiB = the whole 160 KiB of a CU)
+constexpr int X_STAGES = 3, W_STAGES = 2;
+constexpr int lds_halves(int NJ) { return X_STAGES * FB_M * FB_K + W_STAGES * FB_K * 64 * NJ; }
 
 typedef __attribute__((address_space(3))) void lds_void_t;
 typedef __attribute__((address_space(1))) const void gbl_void_t;
@@ -47,12 +50,15 @@ __device__ __forceinline__ int swz_b(int k, int blk) { return blk ^ ((k & 3) | (
 template <int WL, int EPI, int NJ>
 __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles_m, int tiles_n) {
     constexpr int FB_N = 64 * NJ;
-    constexpr int F_STAGE_HALVES = stage_halves(NJ);
+    constexpr int X_TILE = FB_M * FB_K, W_TILE = FB_K * FB_N;  // halves per ring slot
     constexpr int WCH = (FB_K * FB_N) / 512 / 8;  // 1 KiB chunks of the W tile per wave (= NJ)
     static_assert(WL == W_NK || NJ == 4, "the [in, out] weight tile layout is written for 256-wide tiles");
-    extern __shared__ __attribute__((aligned(16))) half_t smem[];  // 2 stages x (X tile, W tile)
+    extern __shared__ __attribute__((aligned(16))) half_t smem[];  // X ring (3 tiles), then W ring (2 tiles)
+    half_t* const xring = smem;
+    half_t* const wring = smem + X_STAGES * X_TILE;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: LDS bases stay in scalar registers
     const int wm = wave >> 2, wn = wave & 3;  // 2 x 4 waves; each 128 (M) x 16*NJ (N)
     const int l16 = lane & 15, lk = lane >> 4;
 
@@ -79,36 +85,34 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles
 
     // ---- per-lane global offsets of the 8 direct-to-LDS loads of one k-tile ---------------------------------------------
     // X tile (and W tile when [N, K]): 32 chunks of 1 KiB = 8 rows x 128 B; wave w fills chunks w, w+8, w+16, w+24.
-    int xoff[4], woff[WCH];  // element offsets inside the tile; the launcher guarantees they fit 31 bits
+    unsigned xoff[4], woff[WCH];  // byte offsets inside the tile; the launcher guarantees they fit 32 bits
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int q = i * 8 + wave;
         const int row = q * 8 + (lane >> 3), pos = lane & 7;
         const int c = swz_a(row, pos);  // XOR is an involution: the chunk stored at `pos` is logical chunk pos ^ f(row)
-        xoff[i] = row * (int)g.ldx + c * 8;
+        xoff[i] = (unsigned)(row * (int)g.ldx + c * 8) * 2u;
         if (i >= WCH) continue;
         if (WL == W_NK) {
-            woff[i] = row * (int)g.ldw + c * 8;
+            woff[i] = (unsigned)(row * (int)g.ldw + c * 8) * 2u;
         } else {
             // W tile [64 k][256 n]: chunk q = k-rows 2q, 2q+1 (512 B each)
             const int k = q * 2 + (lane >> 5), p = lane & 31;
             const int blk = swz_b(k, p >> 1);
-            woff[i] = k * (int)g.ldw + (blk * 2 + (p & 1)) * 8;
+            woff[i] = (unsigned)(k * (int)g.ldw + (blk * 2 + (p & 1)) * 8) * 2u;
         }
     }
     const int64_t wstep = (WL == W_KN) ? (int64_t)FB_K * g.ldw : FB_K;
 
-    auto issue = [&](int kt, int stage) {
-        half_t* xs = smem + stage * F_STAGE_HALVES;
-        half_t* ws = xs + FB_M * FB_K;
-        const half_t* xg = X + (int64_t)kt * FB_K;
-        const half_t* wg = W + (int64_t)kt * wstep;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int q = i * 8 + wave;
-            load_lds16(xg + xoff[i], xs + q * 512);
-            if (i < WCH) load_lds16(wg + woff[i], ws + q * 512);
-        }
+    // tile index clamped to the last one: the loop body is branch-free, the extra loads of the last iterations
+    // refill slots nobody reads any more
+    const int ktiles = g.K / FB_K;
+    auto x_tile = [&](int kt) { return reinterpret_cast<const char*>(X + (int64_t)(kt < ktiles ? kt : ktiles - 1) * FB_K); };
+    auto w_tile = [&](int kt) { return reinterpret_cast<const char*>(W + (int64_t)(kt < ktiles ? kt : ktiles - 1) * wstep); };
+    // load l of a k-tile: l < WCH -> chunk l of the W tile, else chunk l - WCH of the X tile (W first: it is needed first)
+    auto issue_one = [&](int l, const char* xg, const char* wg, half_t* xs, half_t* ws) {
+        if (l < WCH) load_lds16(reinterpret_cast<const half_t*>(wg + woff[l]), ws + (l * 8 + wave) * 512);
+        else load_lds16(reinterpret_cast<const half_t*>(xg + xoff[l - WCH]), xs + ((l - WCH) * 8 + wave) * 512);
     };
 
     float4_t acc[8][NJ];
@@ -117,82 +121,80 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles
 #pragma unroll
         for (int j = 0; j < NJ; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    // fragments of k-step ks of the tile in `stage`: 8 row tiles of X, NJ column tiles of W
-    auto read_frags = [&](int stage, int ks, half8_t (&a)[8], half8_t (&b)[NJ]) {
-        const half_t* xs = smem + stage * F_STAGE_HALVES;
-        const half_t* ws = xs + FB_M * FB_K;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
+    // LDS read unit u of k-step ks: u < NJ -> W fragment u, else X fragment u - NJ (W first: every MFMA row needs all of b)
+    auto read_unit = [&](const half_t* xs, const half_t* ws, int ks, int u, half8_t (&a)[8], half8_t (&b)[NJ]) {
+        if (u >= NJ) {
+            const int i = u - NJ;
             const int row = wm * 128 + i * 16 + l16;
             a[i] = *reinterpret_cast<const half8_t*>(&xs[row * FB_K + swz_a(row, ks * 4 + lk) * 8]);
+        } else if (WL == W_NK) {
+            const int row = wn * (16 * NJ) + u * 16 + l16;
+            b[u] = *reinterpret_cast<const half8_t*>(&ws[row * FB_K + swz_a(row, ks * 4 + lk) * 8]);
+        } else {
+            const int blk = wn * 4 + u;                      // 32-byte block = 16 output columns
+            const int k = ks * 32 + lk * 8 + (l16 >> 2);     // this lane's source row of the first 4x16 read
+            const half4_t lo = lds_read_tr4(&ws[k * FB_N + swz_b(k, blk) * 16 + (l16 & 3) * 4]);
+            const half4_t hi = lds_read_tr4(&ws[(k + 4) * FB_N + swz_b(k + 4, blk) * 16 + (l16 & 3) * 4]);
+            b[u] = half8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         }
+    };
+    constexpr int NDS = 8 + NJ;       // LDS read units per k-step
+    constexpr int NMFMA = 8 * NJ;     // MFMAs per k-step
+    constexpr int NLOAD = 4 + WCH;    // global -> LDS loads per k-tile and thread
+    constexpr int DS_SPAN = NMFMA * 3 / 4;  // the reads of a phase are issued under its first 3/4 MFMAs
+    // One phase = the NMFMA MFMAs of one k-step (fragments ma, mb) with the LDS reads of the next k-step (into ra, rb)
+    // and, if LOADS, the global -> LDS loads of a later k-tile placed between them in exactly this order: the
+    // scheduling fence after every MFMA keeps the compiler from regrouping them.  Operands are swapped in the MFMA so
+    // that each lane owns 4 consecutive output columns of one row.
+    auto phase = [&](auto with_loads, half8_t (&ma)[8], half8_t (&mb)[NJ], half8_t (&ra)[8], half8_t (&rb)[NJ],
+                     const half_t* rxs, const half_t* rws, int rks, const char* xg, const char* wg, half_t* lxs,
+                     half_t* lws) {
+        constexpr bool LOADS = decltype(with_loads)::value;
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) {
-            if (WL == W_NK) {
-                const int row = wn * (16 * NJ) + j * 16 + l16;
-                b[j] = *reinterpret_cast<const half8_t*>(&ws[row * FB_K + swz_a(row, ks * 4 + lk) * 8]);
-            } else {
-                const int blk = wn * 4 + j;                      // 32-byte block = 16 output columns
-                const int k = ks * 32 + lk * 8 + (l16 >> 2);     // this lane's source row of the first 4x16 read
-                const half4_t lo = lds_read_tr4(&ws[k * FB_N + swz_b(k, blk) * 16 + (l16 & 3) * 4]);
-                const half4_t hi = lds_read_tr4(&ws[(k + 4) * FB_N + swz_b(k + 4, blk) * 16 + (l16 & 3) * 4]);
-                b[j] = half8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        for (int m = 0; m < NMFMA; ++m) {
+            const int i = m / NJ, j = m % NJ;
+            acc[i][j] = mfma16(mb[j], ma[i], acc[i][j]);
+            if (LOADS) {
+#pragma unroll
+                for (int l = m * NLOAD / NMFMA; l < (m + 1) * NLOAD / NMFMA; ++l) issue_one(l, xg, wg, lxs, lws);
             }
+#pragma unroll
+            for (int u = m * NDS / DS_SPAN; u < (m + 1) * NDS / DS_SPAN && u < NDS; ++u) read_unit(rxs, rws, rks, u, ra, rb);
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
-    // operands swapped so that each lane owns 4 consecutive output columns of one row
-    auto do_mfma = [&](half8_t (&a)[8], half8_t (&b)[NJ]) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-#pragma unroll
-            for (int j = 0; j < NJ; ++j) acc[i][j] = mfma16(b[j], a[i], acc[i][j]);
-    };
-    constexpr int NDS = (WL == W_NK) ? 8 + NJ : 8 + 2 * NJ;  // LDS read instructions per k-step
-    constexpr int NMFMA = 8 * NJ;                             // MFMAs per k-step
-    constexpr int NLOAD = 4 + WCH;                            // global -> LDS loads per k-tile and thread
 
-    const int ktiles = g.K / FB_K;
-    issue(0, 0);
-    if (ktiles > 1) issue(1, 1);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // prologue: X0 W0 X1 W1 X2; everything but X2 must have landed before the first fragments are read
+    for (int t = 0; t < 3; ++t) {
+#pragma unroll
+        for (int l = (t < 2 ? 0 : WCH); l < NLOAD; ++l)
+            issue_one(l, x_tile(t), w_tile(t), xring + t * X_TILE, wring + (t & 1) * W_TILE);
+    }
+    asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
     __syncthreads();
     half8_t a0[8], b0[NJ], a1[8], b1[NJ];
-    read_frags(0, 0, a0, b0);
+#pragma unroll
+    for (int u = 0; u < NDS; ++u) read_unit(xring, wring, 0, u, a0, b0);
 
+    int xslot = 0, xnext = 1;  // kt % 3, (kt + 1) % 3
     for (int kt = 0; kt < ktiles; ++kt) {
-        const int stage = kt & 1;
+        const int wslot = kt & 1;
+        half_t* const xs = xring + xslot * X_TILE;
+        half_t* const ws = wring + wslot * W_TILE;
         // first k-step multiplies while the second k-step's fragments stream in
-        read_frags(stage, 1, a1, b1);
-        do_mfma(a0, b0);
-#pragma unroll
-        for (int i = 0; i < NDS; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // 2 MFMA
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 LDS read
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, NMFMA - 2 * NDS, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        // this wave's loads of tile kt+1 have landed and all of tile kt is in its registers
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        phase(std::false_type{}, a0, b0, a1, b1, xs, ws, 1, nullptr, nullptr, nullptr, nullptr);
+        // all of tile kt is in this wave's registers; its loads of X(kt+1) and W(kt+1) have landed, the four loads of
+        // X(kt+2) issued last may stay in flight across the barrier
+        asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
         __syncthreads();
-        // every wave is past tile kt: its stage takes tile kt+2; tile kt+1's first fragments stream in under the MFMAs
-        if (kt + 2 < ktiles) issue(kt + 2, stage);
-        if (kt + 1 < ktiles) read_frags(stage ^ 1, 0, a0, b0);
-        do_mfma(a1, b1);
-#pragma unroll
-        for (int i = 0; i < NLOAD; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // global -> LDS load
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // LDS read
-        }
-#pragma unroll
-        for (int i = 0; i < NDS - NLOAD; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, NMFMA - 2 * NDS, 0);
-        __builtin_amdgcn_sched_barrier(0);
+        // every wave is past tile kt: its W slot takes W(kt+2), its X slot X(kt+3); tile kt+1's first fragments stream
+        // in under the MFMAs of the second k-step
+        phase(std::true_type{}, a1, b1, a0, b0, xring + xnext * X_TILE, wring + (wslot ^ 1) * W_TILE, 0, x_tile(kt + 3),
+              w_tile(kt + 2), xs, ws);
+        xslot = xnext;
+        xnext = (xnext == X_STAGES - 1) ? 0 : xnext + 1;
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the clamped refills of the last iterations
 
     // ---- epilogue: acc[i][j][r] = Y[m0 + wm*128 + i*16 + l16][n0 + wn*16*NJ + j*16 + 4*lk + r] -----------------------------
 #pragma unroll
@@ -205,7 +207,7 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles
 template <int WL, int NJ>
 static void launch_fast_epi(const GemmArgs& g, int tiles_m, int tiles_n, hipStream_t stream) {
     const dim3 grid(tiles_m * tiles_n), block(F_THREADS);
-    const size_t smem = 2 * stage_halves(NJ) * sizeof(half_t);
+    const size_t smem = lds_halves(NJ) * sizeof(half_t);
 #define LG_FAST(E)                                                                                                  \
     do {                                                                                                            \
         static bool attr_set = false;                                                                               \
