@@ -76,8 +76,10 @@ template <> struct Vec16<half_t> {
 
 __device__ __forceinline__ float gelu_tanh(float x) {
     // 0.5 x (1 + tanh(0.79788456 (x + 0.044715 x^3)))   (reference cuda_kernels.cu:9-15)
+    // evaluated as x / (1 + exp(-2u)), the same function with one hardware exp2 and one reciprocal
     const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
-    return 0.5f * x * (1.0f + tanhf(u));
+    const float e = __builtin_amdgcn_exp2f(-2.0f * 1.4426950408889634f * u);  // inf for very negative x: result -0
+    return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

@@ -142,6 +142,7 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles
     constexpr int NMFMA = 8 * NJ;     // MFMAs per k-step
     constexpr int NLOAD = 4 + WCH;    // global -> LDS loads per k-tile and thread
     constexpr int DS_SPAN = NMFMA * 3 / 4;  // the reads of a phase are issued under its first 3/4 MFMAs
+    constexpr int LOAD_SPAN = NMFMA;        // the loads of a k-tile are issued under all MFMAs of the second k-step
     // One phase = the NMFMA MFMAs of one k-step (fragments ma, mb) with the LDS reads of the next k-step (into ra, rb)
     // and, if LOADS, the global -> LDS loads of a later k-tile placed between them in exactly this order: the
     // scheduling fence after every MFMA keeps the compiler from regrouping them.  Operands are swapped in the MFMA so
@@ -156,7 +157,7 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles
             acc[i][j] = mfma16(mb[j], ma[i], acc[i][j]);
             if (LOADS) {
 #pragma unroll
-                for (int l = m * NLOAD / NMFMA; l < (m + 1) * NLOAD / NMFMA; ++l) issue_one(l, xg, wg, lxs, lws);
+                for (int l = m * NLOAD / LOAD_SPAN; l < (m + 1) * NLOAD / LOAD_SPAN && l < NLOAD; ++l) issue_one(l, xg, wg, lxs, lws);
             }
 #pragma unroll
             for (int u = m * NDS / DS_SPAN; u < (m + 1) * NDS / DS_SPAN && u < NDS; ++u) read_unit(rxs, rws, rks, u, ra, rb);
@@ -197,11 +198,48 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the clamped refills of the last iterations
 
     // ---- epilogue: acc[i][j][r] = Y[m0 + wm*128 + i*16 + l16][n0 + wn*16*NJ + j*16 + 4*lk + r] -----------------------------
+    // Everything that depends only on the column (bias, head offset) or only on the row (batch / position split) is
+    // computed once, so the 8 x NJ stores of a lane are not separated by dependent loads or integer divisions.
+    float bias_v[NJ][4];
+    int64_t col_off[NJ];
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int j = 0; j < NJ; ++j) {
+        const int n = n0 + wn * (16 * NJ) + j * 16 + 4 * lk;
+        if (EPI != LG_EPI_NONE) {
+            const half4_t bv = *reinterpret_cast<const half4_t*>(g.epi.bias + n);
 #pragma unroll
-        for (int j = 0; j < NJ; ++j)
-            epilogue_store4<EPI>(g, g.Y, m0 + wm * 128 + i * 16 + l16, n0 + wn * (16 * NJ) + j * 16 + 4 * lk, acc[i][j], true);
+            for (int r = 0; r < 4; ++r) bias_v[j][r] = (float)bv[r];
+        }
+        // LG_EPI_BIAS_HEADS: [M = b*seq + s, N = head*d + e] -> [b, head, s, e] with ldy rows reserved per (b, head);
+        // n..n+3 stay inside one head (d % 4 == 0)
+        if (EPI == LG_EPI_BIAS_HEADS) col_off[j] = (int64_t)(n / g.epi.d) * g.ldy * g.epi.d + (n % g.epi.d);
+        else col_off[j] = n;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int m = m0 + wm * 128 + i * 16 + l16;
+        int64_t row_off;
+        if (EPI == LG_EPI_BIAS_HEADS) {
+            const int b = m / g.epi.seq, sq = m % g.epi.seq;
+            row_off = ((int64_t)b * g.epi.heads_total * g.ldy + sq) * (int64_t)g.epi.d;
+        } else {
+            row_off = (int64_t)m * g.ldy;
+        }
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            float v[4] = {acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
+            if (EPI != LG_EPI_NONE) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) v[r] += bias_v[j][r];
+            }
+            if (EPI == LG_EPI_BIAS_GELU) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) v[r] = gelu_tanh(v[r]);
+            }
+            const half4_t o = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+            *reinterpret_cast<half4_t*>(g.Y + row_off + col_off[j]) = o;
+        }
+    }
 }
 
 template <int WL, int NJ>
@@ -233,6 +271,7 @@ int launch_gemm_fast_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t 
     if (!aligned16(g.X) || !aligned16(g.W) || !aligned16(g.Y) || (g.ldx % 8) || (g.ldw % 8)) return LG_OK;
     if (g.ldx >= (1 << 22) || g.ldw >= (1 << 22)) return LG_OK;  // 256 rows x ld must fit the 31-bit tile offsets
     if (g.epi.kind == LG_EPI_BIAS_HEADS ? (g.epi.d % 4 != 0) : (g.ldy % 4 != 0)) return LG_OK;
+    if (g.epi.kind != LG_EPI_NONE && (reinterpret_cast<uintptr_t>(g.epi.bias) & 7u)) return LG_OK;  // 8-byte bias loads
     // tile width: the one that needs the least work-rounds on 256 CUs (rounds x tile width); ties go to the wider tile
     const int tiles_m = g.M / FB_M;
     int best_nj = 0;
