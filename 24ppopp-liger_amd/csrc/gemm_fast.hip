@@ -142,7 +142,8 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles
     constexpr int NMFMA = 8 * NJ;     // MFMAs per k-step
     constexpr int NLOAD = 4 + WCH;    // global -> LDS loads per k-tile and thread
     constexpr int DS_SPAN = NMFMA * 3 / 4;  // the reads of a phase are issued under its first 3/4 MFMAs
-    constexpr int LOAD_SPAN = NMFMA;        // the loads of a k-tile are issued under all MFMAs of the second k-step
+    constexpr int W_SPAN = NMFMA / 2;       // the W loads (needed first) go under the first half of the second k-step's
+                                            // MFMAs, the X loads under the second half
     // One phase = the NMFMA MFMAs of one k-step (fragments ma, mb) with the LDS reads of the next k-step (into ra, rb)
     // and, if LOADS, the global -> LDS loads of a later k-tile placed between them in exactly this order: the
     // scheduling fence after every MFMA keeps the compiler from regrouping them.  Operands are swapped in the MFMA so
@@ -157,7 +158,10 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles
             acc[i][j] = mfma16(mb[j], ma[i], acc[i][j]);
             if (LOADS) {
 #pragma unroll
-                for (int l = m * NLOAD / LOAD_SPAN; l < (m + 1) * NLOAD / LOAD_SPAN && l < NLOAD; ++l) issue_one(l, xg, wg, lxs, lws);
+                for (int l = 0; l < NLOAD; ++l) {
+                    const int at = l < WCH ? l * W_SPAN / WCH : W_SPAN + (l - WCH) * (NMFMA - W_SPAN) / 4;
+                    if (at == m) issue_one(l, xg, wg, lxs, lws);
+                }
             }
 #pragma unroll
             for (int u = m * NDS / DS_SPAN; u < (m + 1) * NDS / DS_SPAN && u < NDS; ++u) read_unit(rxs, rws, rks, u, ra, rb);
