@@ -6,7 +6,8 @@
 //   * a block = 4 waves x 32 output features; the grid is (N / 128) x S with S K-slices chosen so that >= ~1000 blocks
 //     keep >= 16 waves per CU streaming;
 //   * W fragments go from global memory straight into MFMA operand registers (a lane owns 8 consecutive k of one output
-//     feature: exactly the B operand of v_mfma_f32_16x16x32_f16), 16 independent 16-byte loads in flight per lane;
+//     feature: exactly the B operand of v_mfma_f32_16x16x32_f16) in a rolling pipeline that keeps 16 independent
+//     16-byte loads in flight per lane at all times;
 //   * the few X rows are staged once per 256-wide k-chunk in LDS (double buffered) and shared by the block's waves;
 //   * K-slices are summed in fp32 through a per-stream workspace and a small second kernel that also applies the
 //     epilogue (bias / GELU / head-transposed store), so results match the single-pass kernels' rounding.
@@ -30,20 +31,30 @@ __global__ __launch_bounds__(256) void gemm_skinny_nk_kernel(GemmArgs g, int ksl
     const int n0 = blockIdx.x * SK_BN + wave * 32;
     const int split = blockIdx.y;
     const int k_begin = split * kslice;
-    const int k_end = min(g.K, k_begin + kslice);
-    const int nchunks = (k_end - k_begin + SK_KC - 1) / SK_KC;
+    const int nchunks = (min(g.K, k_begin + kslice) - k_begin) / SK_KC;  // whole chunks only
 
-    // stage one X chunk [16*MT rows][256 k] into LDS buffer `buf` (rows >= M and k >= k_end are zero)
-    auto stage_x = [&](int chunk, int buf) {
-        const int kc0 = k_begin + chunk * SK_KC;
-        constexpr int VEC = 16 * MT * (SK_KC / 8);  // 16-byte vectors in the chunk
+    // The loop below is branch-free (the launcher guarantees K-slices made of whole 256-wide chunks): rows beyond M are
+    // read from row M-1 (they only feed accumulator rows that are never stored) and the chunk after the last one is the
+    // last one again, so that every load is unconditional and the compiler can count outstanding loads exactly.
+    // X chunk [16*MT rows][256 k]: global -> registers -> LDS buffer
+    constexpr int XV = 16 * MT * (SK_KC / 8) / 256;  // 16-byte vectors per thread and chunk
+    const half_t* xsrc[XV];
 #pragma unroll
-        for (int v = tid; v < VEC; v += 256) {
+    for (int u = 0; u < XV; ++u) {
+        const int v = tid + u * 256;
+        const int row = min(v / (SK_KC / 8), g.M - 1), c = v % (SK_KC / 8);
+        xsrc[u] = g.X + (int64_t)row * g.ldx + k_begin + c * 8;
+    }
+    auto load_x = [&](int chunk, half8_t (&xr)[XV]) {
+#pragma unroll
+        for (int u = 0; u < XV; ++u) xr[u] = *reinterpret_cast<const half8_t*>(xsrc[u] + chunk * SK_KC);
+    };
+    auto store_x = [&](int buf, const half8_t (&xr)[XV]) {
+#pragma unroll
+        for (int u = 0; u < XV; ++u) {
+            const int v = tid + u * 256;
             const int row = v / (SK_KC / 8), c = v % (SK_KC / 8);
-            const int k = kc0 + c * 8;
-            half8_t val = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-            if (row < g.M && k < k_end) val = *reinterpret_cast<const half8_t*>(g.X + (int64_t)row * g.ldx + k);
-            *reinterpret_cast<half8_t*>(&xs[buf][row * SK_XS + c * 8]) = val;
+            *reinterpret_cast<half8_t*>(&xs[buf][row * SK_XS + c * 8]) = xr[u];
         }
     };
 
@@ -53,28 +64,26 @@ __global__ __launch_bounds__(256) void gemm_skinny_nk_kernel(GemmArgs g, int ksl
 
     // this lane's two weight rows (output features n0 + l16 and n0 + 16 + l16); rows beyond N are clamped and never stored
     const int r0 = min(n0 + l16, g.N - 1), r1 = min(n0 + 16 + l16, g.N - 1);
-    const half_t* w0 = g.W + (int64_t)r0 * g.ldw + lk * 8;
-    const half_t* w1 = g.W + (int64_t)r1 * g.ldw + lk * 8;
+    const half_t* w0 = g.W + (int64_t)r0 * g.ldw + k_begin + lk * 8;
+    const half_t* w1 = g.W + (int64_t)r1 * g.ldw + k_begin + lk * 8;
 
-    stage_x(0, 0);
+    // Rolling pipeline: the 16 weight fragments of a chunk live in registers; as soon as fragment s of chunk ch has been
+    // multiplied its registers are reloaded with fragment s of chunk ch+1, so every lane keeps 16 loads in flight all the
+    // time.  The next X chunk is fetched at the start of a chunk (it queues behind weight loads that are consumed during
+    // the chunk anyway) and written to the other LDS buffer at its end.
+    half8_t b0[8], b1[8], xr[XV];
+    load_x(0, xr);
+    store_x(0, xr);
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+        b0[s] = *reinterpret_cast<const half8_t*>(w0 + s * 32);
+        b1[s] = *reinterpret_cast<const half8_t*>(w1 + s * 32);
+    }
     __syncthreads();
     for (int ch = 0; ch < nchunks; ++ch) {
         const int buf = ch & 1;
-        const int kc0 = k_begin + ch * SK_KC;
-        // all 16 weight fragments of the chunk are requested before anything is consumed
-        half8_t b0[8], b1[8];
-#pragma unroll
-        for (int s = 0; s < 8; ++s) {
-            const int k = kc0 + s * 32;  // k + lk*8 .. +8 for this lane; K % 8 == 0 so a vector is in or out as a whole
-            if (k + lk * 8 < k_end) {
-                b0[s] = *reinterpret_cast<const half8_t*>(w0 + k);
-                b1[s] = *reinterpret_cast<const half8_t*>(w1 + k);
-            } else {
-                b0[s] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-                b1[s] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-            }
-        }
-        if (ch + 1 < nchunks) stage_x(ch + 1, buf ^ 1);
+        const int next = min(ch + 1, nchunks - 1);
+        load_x(next, xr);
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
 #pragma unroll
@@ -84,7 +93,10 @@ __global__ __launch_bounds__(256) void gemm_skinny_nk_kernel(GemmArgs g, int ksl
                 acc[i][0] = mfma16(b0[s], a, acc[i][0]);
                 acc[i][1] = mfma16(b1[s], a, acc[i][1]);
             }
+            b0[s] = *reinterpret_cast<const half8_t*>(w0 + next * SK_KC + s * 32);
+            b1[s] = *reinterpret_cast<const half8_t*>(w1 + next * SK_KC + s * 32);
         }
+        store_x(buf ^ 1, xr);
         __syncthreads();
     }
 
@@ -148,7 +160,7 @@ static float* skinny_workspace(hipStream_t stream, size_t bytes) {
 int launch_gemm_skinny_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t stream, bool* handled) {
     *handled = false;
     if (batch != 1 || wlayout != W_NK) return LG_OK;
-    if (g.M <= 0 || g.M > 64 || g.N < 512 || g.K < 1024 || (g.K % 8) || (g.N % 4)) return LG_OK;
+    if (g.M <= 0 || g.M > 64 || g.N < 512 || g.K < 1024 || (g.K % SK_KC) || (g.N % 4)) return LG_OK;
     if (!aligned16(g.X) || !aligned16(g.W) || !aligned16(g.Y) || (g.ldx % 8) || (g.ldw % 8)) return LG_OK;
     if (g.epi.kind == LG_EPI_BIAS_HEADS ? (g.epi.d % 4 != 0) : (g.ldy % 4 != 0)) return LG_OK;
     const int nblk = (g.N + SK_BN - 1) / SK_BN;
