@@ -162,6 +162,16 @@ int lg_stream_create(void** stream) {
     *stream = (void*)s;
     return rc;
 }
+int lg_stream_create_cu_mask(void** stream, const unsigned* cu_mask, int mask_words) {
+    if (!stream || !cu_mask || mask_words <= 0) { set_error("lg_stream_create_cu_mask: bad arguments"); return LG_ERR_INVALID; }
+    bool any = false;
+    for (int w = 0; w < mask_words; ++w) any = any || cu_mask[w] != 0u;
+    if (!any) { set_error("lg_stream_create_cu_mask: empty mask"); return LG_ERR_INVALID; }
+    hipStream_t s = nullptr;
+    int rc = rt(hipExtStreamCreateWithCUMask(&s, (uint32_t)mask_words, cu_mask), "hipExtStreamCreateWithCUMask");
+    *stream = (void*)s;
+    return rc;
+}
 int lg_stream_destroy(void* stream) { return rt(hipStreamDestroy((hipStream_t)stream), "hipStreamDestroy"); }
 int lg_stream_synchronize(void* stream) { return rt(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize"); }
 int lg_stream_wait_event(void* stream, void* event) {

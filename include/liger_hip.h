@@ -48,6 +48,11 @@ int lg_memcpy_d2d_async(void* dst, const void* src, size_t bytes, void* stream);
 int lg_memset_async(void* dst, int value, size_t bytes, void* stream);
 int lg_device_synchronize(void);
 int lg_stream_create(void** stream);          /* non-blocking stream, default priority */
+/* Non-blocking stream whose kernels run only on the compute units whose bit is set in cu_mask (mask_words 32-bit
+ * words, bit i of word w = CU 32*w + i; at least one bit must be set).  Takes the place of the two stream priorities
+ * the reference gives its streams (context.h:28-29, schedule.h:54-55): on this platform the two streams of the scheduler
+ * are separated in space, not by priority. */
+int lg_stream_create_cu_mask(void** stream, const unsigned* cu_mask, int mask_words);
 int lg_stream_destroy(void* stream);
 int lg_stream_synchronize(void* stream);
 int lg_stream_wait_event(void* stream, void* event);
