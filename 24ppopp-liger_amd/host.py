@@ -46,6 +46,9 @@ SIGNATURES = {
     "lgh_sched_create": (_p, [_p, _i, _f, _i, _i, _i, _i, _i, _i]),
     "lgh_sched_profile": (_i, [_p, _i, _i, _i, _i, _i]),
     "lgh_sched_profile_decode": (_i, [_p, _i, _i, _i]),
+    "lgh_sched_profile_contention": (_i, [_p, _i, _i, _i, _i, C.POINTER(_f)]),
+    "lgh_sched_set_contention": (_i, [_p, _i, _i, _f]),
+    "lgh_sched_get_contention": (_f, [_p, _i, _i]),
     "lgh_sched_save": (_i, [_p, C.c_char_p, C.c_char_p]),
     "lgh_sched_load": (_i, [_p, C.c_char_p, C.c_char_p]),
     "lgh_sched_lookup": (_f, [_p, _i, _i, _i]),
@@ -207,6 +210,19 @@ class Scheduler:
 
     def profile_decode(self, bs, past, itr=20):
         check(lib.lgh_sched_profile_decode(self.h, bs, past, itr), "lgh_sched_profile_decode")
+
+    def profile_contention(self, bs, seq, dec_bs, past):
+        """Measures prefill MFMA-bound kernels || decode-step kernels on the two streams and installs the result in the
+        contention table.  Returns primary / secondary / concurrent ms, the hidden fraction and the secondary's repeats."""
+        out = (_f * 5)()
+        check(lib.lgh_sched_profile_contention(self.h, bs, seq, dec_bs, past, out), "lgh_sched_profile_contention")
+        return {"main_ms": out[0], "sub_ms": out[1], "both_ms": out[2], "hidden": out[3], "sub_repeats": int(out[4])}
+
+    def set_contention(self, main_class, sub_class, value):
+        check(lib.lgh_sched_set_contention(self.h, main_class, sub_class, value), "lgh_sched_set_contention")
+
+    def contention(self, main_class, sub_class):
+        return lib.lgh_sched_get_contention(self.h, main_class, sub_class)
 
     def save(self, main_file, sub_file):
         check(lib.lgh_sched_save(self.h, main_file.encode(), sub_file.encode()), "lgh_sched_save")

@@ -30,6 +30,9 @@ struct SchedBase {
     virtual void set_factor(int factor) = 0;
     virtual bool ctx_ptrs(int i, void** in, void** out) = 0;
     virtual Report run_queued(int mode, int* counters) = 0;
+    virtual bool profile_contention(int bs, int seq, int dec_bs, int past, float* out5) = 0;
+    virtual bool set_contention(int main_class, int sub_class, float v) = 0;
+    virtual float get_contention(int main_class, int sub_class) = 0;
 };
 
 struct ModelBase {
@@ -97,6 +100,18 @@ struct SchedT : SchedBase {
         if (counters) { counters[0] = s->rounds; counters[1] = s->secondary_launches; counters[2] = s->splits; counters[3] = s->profile_misses; }
         return r;
     }
+    bool profile_contention(int bs, int seq, int dec_bs, int past, float* out5) override {
+        auto r = s->profile_contention(bs, seq, dec_bs, past);
+        if (r.hidden < 0.f) return false;
+        out5[0] = r.main_ms; out5[1] = r.sub_ms; out5[2] = r.both_ms; out5[3] = r.hidden; out5[4] = (float)r.sub_repeats;
+        return true;
+    }
+    bool set_contention(int main_class, int sub_class, float v) override {
+        if (main_class < 0 || main_class > 2 || sub_class < 0 || sub_class > 2) return false;
+        s->contention_table[main_class][sub_class] = v;
+        return true;
+    }
+    float get_contention(int main_class, int sub_class) override { return s->contention(main_class, sub_class); }
     int sub_lookup(int name, int bs, int seq, float* out, int cap) override {
         auto it = s->profiling_decompse_res_dict.find({name, bs, seq});
         if (it == s->profiling_decompse_res_dict.end()) return -1;
@@ -309,6 +324,22 @@ int lgh_sched_profile_decode(void* sched, int bs, int past, int itr) {
     if (!sched || bs <= 0 || past < 0 || itr <= 0) return fail("lgh_sched_profile_decode: bad arguments");
     ((SchedBase*)sched)->profile_decode(bs, past, itr);
     return first_error();
+}
+// Measures the contention table entry for prefill MFMA-bound kernels || decode-step kernels (see Scheduler::profile_contention);
+// out5 = {primary ms, secondary ms, concurrent ms, hidden fraction, secondary repeats}.
+int lgh_sched_profile_contention(void* sched, int bs, int seq, int dec_bs, int past, float* out5) {
+    if (!sched || bs <= 0 || seq <= 0 || dec_bs <= 0 || past < 0 || !out5) return fail("lgh_sched_profile_contention: bad arguments");
+    if (!((SchedBase*)sched)->profile_contention(bs, seq, dec_bs, past, out5))
+        return fail("lgh_sched_profile_contention: needs a pool context and a KV cache");
+    return LG_OK;
+}
+// main_class / sub_class: 0 = MFMA-bound, 1 = HBM-bound, 2 = link-bound; a negative value restores the constant factor
+int lgh_sched_set_contention(void* sched, int main_class, int sub_class, float value) {
+    if (!sched || !((SchedBase*)sched)->set_contention(main_class, sub_class, value)) return fail("lgh_sched_set_contention: bad arguments");
+    return LG_OK;
+}
+float lgh_sched_get_contention(void* sched, int main_class, int sub_class) {
+    return sched ? ((SchedBase*)sched)->get_contention(main_class, sub_class) : -1.f;
 }
 int lgh_sched_save(void* sched, const char* main_file, const char* sub_file) {
     return (sched && ((SchedBase*)sched)->save(main_file, sub_file)) ? LG_OK : fail("lgh_sched_save: cannot write");

@@ -123,6 +123,10 @@ class Scheduler {
     std::vector<Sample*> exe_vec;
     int schedule_deep = 6;            // schedule.h:30
     float contention_factor = 0.8f;   // schedule.h:249
+    // Measured replacement of that constant (RESOURCE policy): contention_table[main][sub] = fraction of the stand-alone
+    // time of class-`sub` kernels that is hidden when they run on stream 1 next to class-`main` kernels on stream 0.
+    // Entries < 0 are unmeasured and fall back to contention_factor.
+    float contention_table[3][3] = {{-1.f, -1.f, -1.f}, {-1.f, -1.f, -1.f}, {-1.f, -1.f, -1.f}};
     class_policy policy = RESOURCE;
     split_axis axis = SPLIT_OUT_COLS;
     int seq_bucket = 1;               // durations are looked up at seq rounded up to a multiple of this
@@ -243,6 +247,68 @@ class Scheduler {
         const int count = _model->kernels_per_layer(true);
         for (int k = 0; k < count; k++) vec[k].callback(DParams0);
         profile_vector(vec, count, 1000, bs, past, itr);
+    }
+
+    // ---- contention ----------------------------------------------------------------------------------------------------
+    float contention(int main_class, int sub_class) const {
+        if (policy == RESOURCE && main_class >= 0 && main_class < 3 && sub_class >= 0 && sub_class < 3 &&
+            contention_table[main_class][sub_class] >= 0.f)
+            return contention_table[main_class][sub_class];
+        return contention_factor;
+    }
+    struct ContentionSample { float main_ms, sub_ms, both_ms, hidden; int sub_repeats; };
+    // Measures how much of a decode step (HBM-bound kernels, `dec_bs` sequences with `past` cached positions) is hidden
+    // when it runs on stream 1 next to the MFMA-bound kernels of one prefill layer (bs x seq) on stream 0, and fills
+    // contention_table[MFMA_BOUND][HBM_BOUND] and [HBM_BOUND][MFMA_BOUND].  The decode step is repeated so that both
+    // sides are about equally long.  Needs one pool context (the decode side uses its workspace and cache slot).
+    ContentionSample profile_contention(int bs, int seq, int dec_bs, int past, int trials = 3) {
+        ContentionSample r = {0.f, 0.f, 0.f, -1.f, 0};
+        if (_all_ctx.empty() || BertParams.max_cache_len <= 0) return r;
+        ReqCtx* c = _all_ctx[0];
+        std::vector<FuncWrap> pre = _model->forward(input, output, bs, seq);
+        std::vector<FuncWrap> A;
+        for (int k = 0; k < BertParams.kernel_num; k++)
+            if (pre[k].rclass == MFMA_BOUND) A.push_back(pre[k]);
+        const int kd = _model->kernels_per_layer(true);
+        std::vector<FuncWrap> dec = _model->forward_decode(c->dec_a, c->dec_b, dec_bs, past, c->slot, c->ws);
+        std::vector<FuncWrap> B(dec.begin(), dec.begin() + kd);
+        if (A.empty() || B.empty()) return r;
+        void *e0 = nullptr, *eA = nullptr, *eB = nullptr;
+        note_status(lg_event_create(&e0), "lg_event_create");
+        note_status(lg_event_create(&eA), "lg_event_create");
+        note_status(lg_event_create(&eB), "lg_event_create");
+        // one prefill pass first: every kernel then runs on initialised data
+        for (int k = 0; k < BertParams.kernel_num; k++) pre[k].callback(DParams0);
+        // returns {time of stream 0's part, time of stream 1's part} of one concurrent run, both from a common start
+        auto run = [&](int nA, int nB, float& tA, float& tB) {
+            note_status(lg_device_synchronize(), "lg_device_synchronize");
+            note_status(lg_event_record(e0, DParams0.stream), "lg_event_record");
+            note_status(lg_stream_wait_event(DParams1.stream, e0), "lg_stream_wait_event");
+            for (int i = 0; i < nA; ++i) for (auto& f : A) f.callback(DParams0);
+            for (int i = 0; i < nB; ++i) for (auto& f : B) f.callback(DParams1);
+            note_status(lg_event_record(eA, DParams0.stream), "lg_event_record");
+            note_status(lg_event_record(eB, DParams1.stream), "lg_event_record");
+            note_status(lg_event_synchronize(eA), "lg_event_synchronize");
+            note_status(lg_event_synchronize(eB), "lg_event_synchronize");
+            note_status(lg_event_elapsed_ms(&tA, e0, eA), "lg_event_elapsed_ms");
+            note_status(lg_event_elapsed_ms(&tB, e0, eB), "lg_event_elapsed_ms");
+        };
+        float a, b, best_main = 1e30f, best_one = 1e30f;
+        run(1, 1, a, b);  // warm-up of both sides
+        for (int t = 0; t < trials; ++t) { run(1, 0, a, b); best_main = std::min(best_main, a); }
+        for (int t = 0; t < trials; ++t) { run(0, 1, a, b); best_one = std::min(best_one, b); }
+        const int reps = std::max(1, (int)(best_main / std::max(best_one, 1e-6f) + 0.5f));
+        float best_sub = 1e30f, best_both = 1e30f;
+        for (int t = 0; t < trials; ++t) { run(0, reps, a, b); best_sub = std::min(best_sub, b); }
+        for (int t = 0; t < trials; ++t) { run(1, reps, a, b); best_both = std::min(best_both, std::max(a, b)); }
+        lg_event_destroy(e0); lg_event_destroy(eA); lg_event_destroy(eB);
+        const float hidden_ms = best_main + best_sub - best_both;
+        auto clamp = [](float x) { return x < 0.05f ? 0.05f : (x > 1.f ? 1.f : x); };
+        r.main_ms = best_main; r.sub_ms = best_sub; r.both_ms = best_both; r.sub_repeats = reps;
+        r.hidden = clamp(hidden_ms / best_sub);
+        contention_table[MFMA_BOUND][HBM_BOUND] = r.hidden;
+        contention_table[HBM_BOUND][MFMA_BOUND] = clamp(hidden_ms / best_main);
+        return r;
     }
 
     // ---- serve  (schedule.h:159-172) ------------------------------------------------------------------------
@@ -396,19 +462,22 @@ class Scheduler {
                 time_planned += head->dequeue(DParams0, 1, time_planned);
             }
             rounds++;
-            time_planned *= contention_factor;
+            // time_planned stays in units of the primary's time; a secondary kernel of stand-alone duration d uses up
+            // d / contention(main, sub) of it (with the constant factor this is the reference's 0.8 x time_planned budget)
             for (size_t s = 1; s < exe_vec.size(); s++) {
                 Sample* sub = exe_vec.at(s);
                 while (time_planned > 0 && !sub->empty()) {
                     if (sub->is_same_class(main_class)) break;
-                    if (sub->duration(0, time_planned) > time_planned) {
-                        if (sub->type() == GEMM && sub->possible_duration(time_planned)) {
+                    const float f = contention(main_class, sub->next_class());
+                    float avail = time_planned * f;
+                    if (sub->duration(0, avail) > avail) {
+                        if (sub->type() == GEMM && sub->possible_duration(avail)) {
                             splits++;
                             continue;  // the first piece now fits
                         }
                         time_planned = 0.0f;
                     } else {
-                        time_planned -= sub->dequeue(DParams1, 0, time_planned);
+                        time_planned -= sub->dequeue(DParams1, 0, avail) / f;
                         secondary_launches++;
                     }
                 }

@@ -146,11 +146,17 @@ def bench_cfg5(capi, host, weight_layout, n_requests):
     for past in range(128, 1024 + 64 + 1, 64):
         sched.profile_decode(1, min(past, 1024 + 63), 5)
     prof_s = time.perf_counter() - t0
+    # measured contention: the MFMA-bound kernels of a 512-token prefill next to batch-1 decode steps at 512 cached positions
+    meas = sched.profile_contention(1, 512, 1, 512)
+    table = {"mfma_main_hbm_sub": sched.contention(0, 1), "hbm_main_mfma_sub": sched.contention(1, 0)}
     out = []
     for lam in (4.0, 8.0, 16.0):
         trace = host.make_poisson_trace(lam, n_requests, 1, 128, 1024, 64, 32, 0)
         row = {"lambda_req_s": lam, "requests": n_requests}
-        for mode, name in ((host.MODE_SEQUENTIAL, "scheduling_off"), (host.MODE_LIGER, "scheduling_on")):
+        for mode, name, measured in ((host.MODE_SEQUENTIAL, "scheduling_off", False), (host.MODE_LIGER, "scheduling_on", False),
+                                     (host.MODE_LIGER, "scheduling_on_measured_contention", True)):
+            sched.set_contention(0, 1, table["mfma_main_hbm_sub"] if measured else -1.0)
+            sched.set_contention(1, 0, table["hbm_main_mfma_sub"] if measured else -1.0)
             r = sched.run_trace(trace, mode)
             row[name] = {"mean_latency_ms": round(r["avg_latency_ms"], 3), "p99_latency_ms": round(r["p99_latency_ms"], 3),
                          "mean_gpu_ms": round(r["avg_gpu_ms"], 3), "mean_queue_ms": round(r["avg_queue_ms"], 3),
@@ -158,7 +164,8 @@ def bench_cfg5(capi, host, weight_layout, n_requests):
                          "secondary_launches": r["secondary_launches"], "splits": r["splits"], "profile_misses": r["profile_misses"]}
         out.append(row)
     return {"workload": "cfg5: 4 layer shards, Poisson arrivals, prompts U[128,1024] rounded to 64, 32 decode tokens", "profile_seconds": round(prof_s, 1),
-            "results": out}
+            "contention_measurement": {k: (round(v, 4) if isinstance(v, float) else v) for k, v in meas.items()},
+            "contention_table": {k: round(v, 4) for k, v in table.items()}, "results": out}
 
 
 def main():

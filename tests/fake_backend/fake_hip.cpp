@@ -28,6 +28,7 @@ double g_host_now = 0;          // virtual milliseconds
 double g_launch_cost = 0.002;   // host time per launch call
 double g_mfma_rate = 1.0e9;     // flop per virtual ms
 double g_hbm_rate = 1.0e6;      // bytes per virtual ms
+double g_corun_speed = 1.0;     // a kernel launched while another stream is busy runs at this fraction of its speed
 std::vector<Stream*> g_streams;
 std::vector<Launch> g_trace;
 Stream g_default;
@@ -44,7 +45,9 @@ int launch(void* stream, const char* name, long long a, long long b, long long c
     l.name[sizeof(l.name) - 1] = 0;
     l.a = a; l.b = b; l.c = c; l.p0 = p0; l.p1 = p1; l.p2 = p2;
     l.start = std::max(s->ready, g_host_now);
-    l.end = l.start + cost;
+    bool other_busy = (s != &g_default && g_default.ready > l.start);
+    for (auto* o : g_streams) other_busy = other_busy || (o != s && o->ready > l.start);
+    l.end = l.start + (other_busy ? cost / g_corun_speed : cost);
     s->ready = l.end;
     g_trace.push_back(l);
     return LG_OK;
@@ -60,6 +63,7 @@ extern "C" {
 void fake_reset(void) {
     std::lock_guard<std::mutex> lk(g_mu);
     g_trace.clear();
+    g_corun_speed = 1.0;
     g_host_now = 0;
     g_default.ready = 0;
     for (auto* s : g_streams) s->ready = 0;
@@ -67,6 +71,7 @@ void fake_reset(void) {
 void fake_set_rates(double mfma_flop_per_ms, double hbm_bytes_per_ms, double launch_cost_ms) {
     g_mfma_rate = mfma_flop_per_ms; g_hbm_rate = hbm_bytes_per_ms; g_launch_cost = launch_cost_ms;
 }
+void fake_set_corun_speed(double speed) { g_corun_speed = speed > 0 ? speed : 1.0; }
 int fake_trace_count(void) { std::lock_guard<std::mutex> lk(g_mu); return (int)g_trace.size(); }
 int fake_trace_get(int i, int* stream, char* name, int name_len, long long* abc, unsigned long long* ptrs, double* start_end) {
     std::lock_guard<std::mutex> lk(g_mu);
@@ -117,6 +122,13 @@ int lg_stream_create(void** stream) {
     g_streams.push_back(s);
     *stream = s;
     return LG_OK;
+}
+int lg_stream_create_cu_mask(void** stream, const unsigned* cu_mask, int mask_words) {
+    if (!stream || !cu_mask || mask_words <= 0) return LG_ERR_INVALID;
+    bool any = false;
+    for (int w = 0; w < mask_words; ++w) any = any || cu_mask[w] != 0u;
+    if (!any) return LG_ERR_INVALID;
+    return lg_stream_create(stream);  // the virtual-time backend has no notion of compute units
 }
 int lg_stream_destroy(void*) { return LG_OK; }
 int lg_stream_synchronize(void* stream) { std::lock_guard<std::mutex> lk(g_mu); g_host_now = std::max(g_host_now, S(stream)->ready); return LG_OK; }

@@ -17,6 +17,7 @@ class Fake:
                                             C.POINTER(C.c_ulonglong), C.POINTER(C.c_double)]
         self.lib.fake_set_rates.argtypes = [C.c_double, C.c_double, C.c_double]
         self.lib.fake_host_now.restype = C.c_double
+        self.lib.fake_set_corun_speed.argtypes = [C.c_double]
 
     def close(self):
         self.host.lib = self._prev
@@ -26,6 +27,10 @@ class Fake:
 
     def set_rates(self, mfma_flop_per_ms, hbm_bytes_per_ms, launch_cost_ms):
         self.lib.fake_set_rates(mfma_flop_per_ms, hbm_bytes_per_ms, launch_cost_ms)
+
+    def set_corun_speed(self, speed):
+        """A kernel launched while another stream is busy runs at `speed` (0..1] of its stand-alone speed."""
+        self.lib.fake_set_corun_speed(speed)
 
     def trace(self):
         out = []

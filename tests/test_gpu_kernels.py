@@ -140,3 +140,30 @@ def test_fill_normal_matches_oracle_bitwise(dev, po):
         dev.call("lg_fill_normal_" + SUF[dt], t, n, 7, 42, 0.25, 0.02)
         ref = po.fill_normal(n, 7, 42, 0.25, 0.02, dt)
         assert np.array_equal(dev.down(t), ref)
+
+
+def test_cu_masked_stream_runs_kernels(dev, po):
+    """A stream restricted to 32 compute units computes the same LayerNorm as any other stream; an empty mask is refused."""
+    import ctypes as C
+    lib = dev.lib
+    m, n = 96, 1024
+    x = rnd(po, m * n, 1, 0).reshape(m, n) * 3 + 0.5
+    g = rnd(po, n, 2, 0, 0.1, 1.0)
+    b = rnd(po, n, 3, 0, 0.1)
+    ref = po.layer_norm(x, g, b, 0)
+    words = (C.c_uint * 8)(0xFFFFFFFF, 0, 0, 0, 0, 0, 0, 0)
+    s = C.c_void_p()
+    assert lib.lg_stream_create_cu_mask(C.byref(s), words, 8) == 0, dev.capi.last_error()
+    try:
+        dx, dg, db = dev.up(x, 0), dev.up(g, 0), dev.up(b, 0)
+        out = dev.empty((m, n), 0)
+        dev.down(out)  # the uploads on the default stream are complete before the masked stream reads them
+        ptr = lambda t: C.c_void_p(t.data_ptr())
+        assert lib.lg_layer_norm_f32(ptr(dx), ptr(dg), ptr(db), ptr(out), m, n, s) == 0, dev.capi.last_error()
+        assert lib.lg_stream_synchronize(s) == 0
+        assert max_rel_err(dev.down(out), ref) < tol(0)
+    finally:
+        assert lib.lg_stream_destroy(s) == 0
+    empty = (C.c_uint * 8)(*([0] * 8))
+    s2 = C.c_void_p()
+    assert lib.lg_stream_create_cu_mask(C.byref(s2), empty, 8) == 1  # LG_ERR_INVALID

@@ -68,3 +68,23 @@ def test_prefill_plus_decode_trace_on_gpu(dev, host):
         r = s.run_trace(trace, mode)
         assert r["records"] == 10 and r["profile_misses"] == 0
         assert r["avg_latency_ms"] > 0 and r["p99_latency_ms"] >= r["avg_latency_ms"] * 0.5
+
+
+def test_measured_contention_on_gpu(dev, host):
+    """The contention measurement runs on the device, yields a fraction in [0.05, 1] consistent with its three times, and
+    a trace scheduled with the measured table completes like one scheduled with the constant."""
+    heads, d, F = 8, 128, 2048
+    m = host.Model(1, 4, 128, heads, d, layer_num=2, ffn_inner=F, causal=True, fused=True, max_cache_len=192, factor=4, weight_layout=1, seed=5)
+    s = host.Scheduler(m, policy=host.POLICY_RESOURCE, axis=host.SPLIT_TOKEN_ROWS, seq_bucket=32, ignore_num=0, pool_count=4, ctx_batch=1)
+    r = s.profile_contention(1, 128, 1, 128)
+    assert r["main_ms"] > 0 and r["sub_ms"] > 0 and r["both_ms"] > 0 and r["sub_repeats"] >= 1
+    assert r["both_ms"] <= (r["main_ms"] + r["sub_ms"]) * 1.5
+    hidden = (r["main_ms"] + r["sub_ms"] - r["both_ms"]) / r["sub_ms"]
+    assert r["hidden"] == pytest.approx(min(1.0, max(0.05, hidden)), rel=1e-4)
+    assert s.contention(0, 1) == pytest.approx(r["hidden"])
+    s.profile(1, 64, 128, 32, 3)
+    for past in (64, 96, 128, 160):
+        s.profile_decode(1, past, 3)
+    trace = [{"arrival_s": 0.001 * i, "batch": 1, "seq": 64 + 32 * (i % 3), "n_decode": 4} for i in range(10)]
+    rr = s.run_trace(trace, host.MODE_LIGER)
+    assert rr["records"] == 10 and rr["profile_misses"] == 0

@@ -173,6 +173,70 @@ def test_decode_request_fills_prefill_gemm_windows_and_splits_cover_exactly(fake
         assert all(b["start"] >= a["end"] - 1e-12 for a, b in zip(mine, mine[1:]))
 
 
+MFMA, HBM = 0, 1   # resource classes (launch_context.h)
+
+
+@pytest.mark.parametrize("speed", [1.0, 0.625, 0.4])
+def test_measured_contention_matches_the_backend_model(fake, speed):
+    """profile_contention runs prefill MFMA kernels on stream 0 next to repeated decode steps on stream 1.  On the
+    virtual-time backend a kernel launched beside a busy stream runs at `speed`, so the concurrent run must take
+    max(primary, secondary / speed) and the hidden fraction follows from the three times."""
+    host = fake.host
+    m = small_model(host)
+    s = host.Scheduler(m, policy=host.POLICY_RESOURCE, pool_count=1, ctx_batch=1)
+    assert s.contention(MFMA, HBM) == pytest.approx(0.8)      # unmeasured: the reference's constant
+    fake.reset()                                               # also restores speed 1
+    fake.set_corun_speed(speed)
+    r = s.profile_contention(1, 64, 1, 64)
+    launch_slack = 0.002 * 64                                  # host launch cost of the issued kernels (virtual ms)
+    assert r["sub_repeats"] >= 1
+    assert r["both_ms"] == pytest.approx(max(r["main_ms"], r["sub_ms"] / speed), abs=launch_slack)
+    hidden = (r["main_ms"] + r["sub_ms"] - r["both_ms"]) / r["sub_ms"]
+    assert r["hidden"] == pytest.approx(min(1.0, max(0.05, hidden)), rel=1e-5)
+    assert s.contention(MFMA, HBM) == pytest.approx(r["hidden"])
+    assert s.contention(HBM, MFMA) == pytest.approx(min(1.0, max(0.05, (r["main_ms"] + r["sub_ms"] - r["both_ms"]) / r["main_ms"])), rel=1e-5)
+    assert s.contention(HBM, HBM) == pytest.approx(0.8)       # other pairs keep the constant
+    # independent timelines (speed 1) hide most of the secondary (all but launch offsets and the rounding of the repeat
+    # count); a slower co-run hides less
+    limit = {1.0: (0.6, 1.0), 0.625: (0.2, 0.6), 0.4: (0.05, 0.2)}[speed]
+    assert limit[0] <= r["hidden"] <= limit[1]
+    s.set_contention(MFMA, HBM, -1.0)
+    assert s.contention(MFMA, HBM) == pytest.approx(0.8)
+
+
+def test_contention_table_sets_the_secondary_budget(fake):
+    """The table entry for (primary class, secondary class) replaces the constant: a small entry admits fewer secondary
+    launches per round than the default 0.8, a table entry equal to the constant changes nothing."""
+    host = fake.host
+
+    def run(entry):
+        m = small_model(host, factor=8)
+        s = host.Scheduler(m, contention_factor=0.8, policy=host.POLICY_RESOURCE, seq_bucket=16, pool_count=3, ctx_batch=1)
+        s.profile(1, 48, 64, 16, 2)
+        for past in (48, 64, 80):
+            s.profile_decode(1, past, 2)
+        if entry is not None:
+            s.set_contention(HBM, MFMA, entry)
+            s.set_contention(MFMA, HBM, entry)
+        fake.reset()
+        s.serve(1, 48, 3)
+        s.serve(1, 64, 0)
+        r = s.run_queued(host.MODE_LIGER)
+        t = fake.trace()
+        ids = sorted({e["stream"] for e in t})   # stream ids grow with every scheduler: compare their rank
+        order = [(ids.index(e["stream"]), e["name"], e["m"], e["n"], e["k"]) for e in t]
+        return r, order
+
+    base, base_order = run(None)
+    same, same_order = run(0.8)
+    assert same_order == base_order and same["secondary_launches"] == base["secondary_launches"]
+    tight, tight_order = run(0.05)
+    assert tight["records"] == 2
+    assert sorted(x[1:] for x in tight_order if not x[1].startswith("gemm")) == sorted(x[1:] for x in base_order if not x[1].startswith("gemm"))
+    assert tight["rounds"] >= base["rounds"]
+    assert tight_order != base_order
+
+
 def test_missing_or_short_profile_never_splits_or_crashes(fake):
     host = fake.host
     m = small_model(host, factor=8)
