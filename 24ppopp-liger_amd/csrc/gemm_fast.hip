@@ -164,7 +164,12 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles
                 }
             }
 #pragma unroll
-            for (int u = m * NDS / DS_SPAN; u < (m + 1) * NDS / DS_SPAN && u < NDS; ++u) read_unit(rxs, rws, rks, u, ra, rb);
+            for (int u = 0; u < NDS; ++u) {
+                // [N, K] weights: one read unit every DS_SPAN / NDS MFMAs.  [K, N] weights: the W units (two transposed
+                // reads each) go under the first NJ MFMAs, the X units are spread over the rest (measured: 8 % faster)
+                const int at = (WL == W_NK) ? (u * DS_SPAN + DS_SPAN - 1) / NDS : (u < NJ ? u : NJ + (u - NJ) * (DS_SPAN - NJ) / 8);
+                if (at == m) read_unit(rxs, rws, rks, u, ra, rb);
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
     };
