@@ -1,7 +1,7 @@
 // gemm_fast.hip -- pipelined 256x256x64 fp16 GEMM for gfx950 (the prefill shapes of the launch vector).
 //
 //   Y[M, N] = X[M, K] * W,  W row-major [K, N] (the reference's layout) or [N, K];  fp32 accumulate, optional fused
-//   epilogue.  Requires M % 256 == 0, N % 256 == 0, K % 64 == 0 and 16-byte aligned operands; everything else goes to
+//   epilogue.  Requires M % 256 == 0, N % 128 == 0 (or % 192), K % 64 == 0 and 16-byte aligned operands; everything else goes to
 //   the generic kernel in gemm.hip.
 //
 // Structure (one workgroup = 8 waves = one 256x256 output tile, one workgroup per CU):
@@ -27,7 +27,7 @@ namespace lg {
 
 constexpr int FB_M = 256, FB_K = 64;
 constexpr int F_THREADS = 512;
-// The tile is 256 x (64 * NJ) outputs: NJ = 4 -> 256 x 256, NJ = 3 -> 256 x 192 (used when it needs fewer rounds of 256
+// The tile is 256 x (64 * NJ) outputs: NJ = 4 -> 256 x 256, NJ = 3 -> 256 x 192, NJ = 2 -> 256 x 128 (used when it needs fewer rounds of 256
 // workgroups, e.g. N = 6144: 512 tiles = 2 full rounds instead of 384 tiles = 1.5 rounds)
 // LDS: a ring of 3 X tiles and a ring of 2 W tiles (256-wide: 96 + 64 KiB = the whole 160 KiB of a CU)
 constexpr int X_STAGES = 3, W_STAGES = 2;
@@ -52,7 +52,7 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles
     constexpr int FB_N = 64 * NJ;
     constexpr int X_TILE = FB_M * FB_K, W_TILE = FB_K * FB_N;  // halves per ring slot
     constexpr int WCH = (FB_K * FB_N) / 512 / 8;  // 1 KiB chunks of the W tile per wave (= NJ)
-    static_assert(WL == W_NK || NJ == 4, "the [in, out] weight tile layout is written for 256-wide tiles");
+    static_assert(WL == W_NK || NJ == 4 || NJ == 2, "the [in, out] weight tile needs a power-of-two number of lanes per k-row");
     extern __shared__ __attribute__((aligned(16))) half_t smem[];  // X ring (3 tiles), then W ring (2 tiles)
     half_t* const xring = smem;
     half_t* const wring = smem + X_STAGES * X_TILE;
@@ -96,8 +96,9 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles
         if (WL == W_NK) {
             woff[i] = (unsigned)(row * (int)g.ldw + c * 8) * 2u;
         } else {
-            // W tile [64 k][256 n]: chunk q = k-rows 2q, 2q+1 (512 B each)
-            const int k = q * 2 + (lane >> 5), p = lane & 31;
+            // W tile [64 k][FB_N n]: a k-row is FB_N / 8 lanes wide, chunk q = 64 / (FB_N / 8) consecutive k-rows
+            constexpr int LPR = FB_N / 8;
+            const int k = q * (64 / LPR) + lane / LPR, p = lane % LPR;
             const int blk = swz_b(k, p >> 1);
             woff[i] = (unsigned)(k * (int)g.ldw + (blk * 2 + (p & 1)) * 8) * 2u;
         }
@@ -131,7 +132,7 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles
             const int row = wn * (16 * NJ) + u * 16 + l16;
             b[u] = *reinterpret_cast<const half8_t*>(&ws[row * FB_K + swz_a(row, ks * 4 + lk) * 8]);
         } else {
-            const int blk = wn * 4 + u;                      // 32-byte block = 16 output columns
+            const int blk = wn * NJ + u;                     // 32-byte block = 16 output columns
             const int k = ks * 32 + lk * 8 + (l16 >> 2);     // this lane's source row of the first 4x16 read
             const half4_t lo = lds_read_tr4(&ws[k * FB_N + swz_b(k, blk) * 16 + (l16 & 3) * 4]);
             const half4_t hi = lds_read_tr4(&ws[(k + 4) * FB_N + swz_b(k + 4, blk) * 16 + (l16 & 3) * 4]);
@@ -285,11 +286,12 @@ int launch_gemm_fast_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t 
     const int tiles_m = g.M / FB_M;
     int best_nj = 0;
     long best_cost = 0;
-    for (int nj = 4; nj >= 3; --nj) {
+    for (int nj = 4; nj >= 2; --nj) {
         if (g.N % (64 * nj)) continue;
         if (nj == 3 && wlayout != W_NK) continue;
         const long tiles = (long)tiles_m * (g.N / (64 * nj));
-        const long cost = ((tiles + 255) / 256) * nj;
+        // narrower tiles move more operand bytes per flop: about 3 % / 35 % more time per unit of width (measured)
+        const long cost = ((tiles + 255) / 256) * nj * (nj == 4 ? 100 : nj == 3 ? 103 : 135);
         if (!best_nj || cost < best_cost) { best_nj = nj; best_cost = cost; }
     }
     if (!best_nj) return LG_OK;
@@ -297,9 +299,11 @@ int launch_gemm_fast_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t 
     const int tiles_n = g.N / (64 * best_nj);
     if (wlayout == W_NK) {
         if (best_nj == 4) launch_fast_epi<W_NK, 4>(g, tiles_m, tiles_n, stream);
-        else launch_fast_epi<W_NK, 3>(g, tiles_m, tiles_n, stream);
+        else if (best_nj == 3) launch_fast_epi<W_NK, 3>(g, tiles_m, tiles_n, stream);
+        else launch_fast_epi<W_NK, 2>(g, tiles_m, tiles_n, stream);
     } else {
-        launch_fast_epi<W_KN, 4>(g, tiles_m, tiles_n, stream);
+        if (best_nj == 4) launch_fast_epi<W_KN, 4>(g, tiles_m, tiles_n, stream);
+        else launch_fast_epi<W_KN, 2>(g, tiles_m, tiles_n, stream);
     }
     return check_launch("gemm_f16_fast");
 }

@@ -17,8 +17,8 @@ SHAPES = [(64, 256, 256), (128, 128, 32), (130, 136, 72), (1, 8, 8), (33, 70, 19
           (512, 384, 160),
           # multiples of the 256 x 256 x 64 tile: the pipelined kernel
           (256, 256, 64), (512, 768, 256), (256, 512, 1024), (1024, 2048, 192), (2048, 256, 128),
-          # 256 x 192 tiles (weights stored [out, in]); the [in, out] layout takes the generic kernel here
-          (256, 384, 128), (512, 576, 192), (256, 1344, 64),
+          # 256 x 192 tiles (weights stored [out, in] only) and 256 x 128 tiles (both layouts)
+          (256, 384, 128), (512, 576, 192), (256, 1344, 64), (256, 640, 128), (512, 128, 192), (768, 1152, 320),
           # few tokens, many features: the weight-streaming split-K kernel (weights stored [out, in])
           (32, 1024, 2048), (1, 512, 1024), (17, 640, 4104), (64, 2048, 1536), (33, 516, 1032)]
 
