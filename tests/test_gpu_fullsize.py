@@ -1,0 +1,110 @@
+"""GPU parity at the full benchmark sizes (GLM-130B TP=2 shard: hidden 12288, 48 of 96 heads x 128, FFN 16384 of 32768,
+batch 8 x seq 512 prefill; batch 32 x 1024 cached positions decode).
+
+The CPU oracle needs ~20 s for one full prefill layer, so at these sizes the checks are
+  * size-independent properties that hold bit for bit (one-hot rows select weight rows, a batch element's result does
+    not depend on the rest of the batch), and
+  * the oracle on a slice of the problem (one sequence of the batch; the memory-bound kernels in full).
+Tolerance for fp16 against the oracle: max |gpu - oracle| / max |oracle| <= 1e-2 (the stated bar).
+"""
+import importlib
+
+import numpy as np
+import pytest
+import torch
+
+from tests.conftest import max_rel_err
+
+pytestmark = pytest.mark.gpu
+
+H, HL, F, D = 12288, 6144, 16384, 128
+B, S = 8, 512
+M = B * S
+
+
+@pytest.fixture(scope="module")
+def host(liger):
+    return importlib.import_module("24ppopp-liger_amd.host")
+
+
+@pytest.mark.parametrize("transa", [0, 1])
+@pytest.mark.parametrize("N,K", [(F, H), (H, F), (HL, H)])
+def test_full_size_gemm_one_hot_rows_select_weight_rows(dev, transa, N, K):
+    """Y = X W with X rows that hold a single 1 (or two) must reproduce rows of W exactly (sums of two rows: one fp16
+    rounding of the fp32 sum).  Every output tile of the full-size launch is checked, in both weight layouts."""
+    g = torch.Generator(device="cuda").manual_seed(7)
+    W = (torch.randn(K, N, device="cuda", dtype=torch.float32, generator=g) * 0.02).half()   # [in, out]
+    X = torch.zeros(M, K, device="cuda", dtype=torch.float16)
+    rows = torch.arange(M, device="cuda")
+    k1 = (rows * 7 + 3) % K
+    k2 = (rows * 13 + 5) % K
+    two = (rows % 3 == 0) & (k1 != k2)
+    X[rows, k1] = 1.0
+    X[rows[two], k2[two]] = 1.0
+    A = W.t().contiguous() if transa else W
+    Y = torch.empty(M, N, device="cuda", dtype=torch.float16)
+    torch.cuda.synchronize()
+    dev.call("lg_gemm_f16", transa, 0, N, M, K, A, K if transa else N, X, K, Y, N)
+    torch.cuda.synchronize()
+    expect = W[k1].float()
+    expect[two] += W[k2[two]].float()
+    assert torch.equal(Y, expect.half())
+
+
+def test_full_size_layer_batch_independence_and_oracle_slice(dev, po, host):
+    """The cfg2 prefill layer shard (fused assembly, causal) on the full batch: every sequence's result equals, bit for
+    bit, the result of running that sequence alone; one sequence is checked against the CPU oracle."""
+    m = host.Model(1, B, S, 96, D, layer_num=1, world_size=2, ffn_inner=2 * F, norm_mode=0, causal=True, fused=True,
+                   weight_layout=1, seed=0)
+    x = po.fill_normal(M * H, 0, 99, 0.0, 1.0, 1).reshape(M, H)
+    dx = dev.up(x, 1)
+    dy = dev.empty((M, H), 1)
+    m.run(dx.data_ptr(), dy.data_ptr(), B, S, None, dev.stream)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(dy).all())
+    one = dev.empty((S, H), 1)
+    for b in (0, 5, 7):
+        xb = dx[b * S:(b + 1) * S].contiguous()
+        m.run(xb.data_ptr(), one.data_ptr(), 1, S, None, dev.stream)
+        torch.cuda.synchronize()
+        assert torch.equal(one, dy[b * S:(b + 1) * S]), "sequence %d depends on its batch" % b
+    # oracle on sequence 5 (the weights are downloaded, so both sides see the same bits)
+    params = m.download_params()
+    w = {k[len("layer0."):]: v for k, v in params.items() if k.startswith("layer0.")}
+    shape = dict(batch=1, seq=S, hidden=H, head_num=48, size_per_head=D, ffn_inner=F, causal=1, norm_mode=0, dtype=1)
+    ref = po.encoder_forward(shape, w, x[5 * S:6 * S])
+    got = dy[5 * S:6 * S].float().cpu().numpy()
+    assert max_rel_err(got, ref) < 1e-2
+
+
+def test_full_size_layer_norm_against_oracle(dev, po):
+    x = po.fill_normal(M * H, 0, 1, 0.0, 1.0, 1).reshape(M, H) * 3 + 0.5
+    x = po.round_f16(x)
+    g = po.fill_normal(H, 0, 2, 1.0, 0.1, 1)
+    b = po.fill_normal(H, 0, 3, 0.0, 0.1, 1)
+    ref = po.layer_norm(x, g, b, 1)
+    out = dev.empty((M, H), 1)
+    dev.call("lg_layer_norm_f16", dev.up(x, 1), dev.up(g, 1), dev.up(b, 1), out, M, H)
+    assert max_rel_err(dev.down(out), ref) < 2e-3
+
+
+def test_full_size_decode_attention_against_oracle(dev, po):
+    """cfg3: 32 sequences x 48 heads, 1024 cached positions (805 MB of K/V), one new token each."""
+    Bd, h, L = 32, 48, 1024
+    q = po.fill_normal(Bd * h * D, 0, 50, 0.0, 1.0, 1).reshape(Bd, h, D)
+    kc = po.fill_normal(Bd * h * L * D, 0, 51, 0.0, 1.0, 1).reshape(Bd, h, L, D)
+    vc = po.fill_normal(Bd * h * L * D, 0, 52, 0.0, 1.0, 1).reshape(Bd, h, L, D)
+    scalar = 1.0 / np.sqrt(D)
+    ref = po.attn_decode(q, kc, vc, L, scalar, 1)
+    ws = dev.empty((max(1, dev.lib.lg_attn_decode_workspace_bytes(Bd, h, D, L) // 4),), 0)
+    out = dev.empty((Bd, h, D), 1)
+    dkc, dvc = dev.up(kc, 1), dev.up(vc, 1)
+    dev.call("lg_attn_decode_f16", dev.up(q, 1), dkc, dvc, out, ws, Bd, h, D, L, L, float(scalar))
+    got = dev.down(out)
+    assert max_rel_err(got, ref) < 1e-2
+    # permuting the cached positions (K and V together) must not change the result beyond rounding
+    perm = torch.randperm(L, device="cuda", generator=torch.Generator(device="cuda").manual_seed(3))
+    out2 = dev.empty((Bd, h, D), 1)
+    dev.call("lg_attn_decode_f16", dev.up(q, 1), dkc[:, :, perm].contiguous(), dvc[:, :, perm].contiguous(), out2, ws, Bd, h, D, L, L,
+             float(scalar))
+    assert max_rel_err(dev.down(out2), got) < 2e-3
