@@ -39,7 +39,7 @@ def gemm_flops_cfg2():
     return {"q": 2 * M * H * Hl, "k": 2 * M * H * Hl, "v": 2 * M * H * Hl, "out": 2 * M * Hl * H, "ffn1": 2 * M * H * F, "ffn2": 2 * M * F * H}
 
 
-def cpu_baseline(po, sample_batch=2, sample_seq=512):
+def cpu_baseline(po, sample_batch=4, sample_seq=512):
     """Times the CPU oracle (OpenMP C) on a bounded sample of the cfg2 layer: same shard shapes, M = sample rows,
     and scales linearly to M = 4096 (GEMM time is linear in M; attention at this size is < 1 % of the work)."""
     import numpy as np

@@ -84,12 +84,12 @@ def test_classic_policy_degenerates_to_sequential_without_communication(fake):
 
 def test_resource_policy_worked_example(fake):
     """Two identical prefill requests A (primary) and B.  Fused vector: [q k v attn out](MFMA) [ln](HBM) [ffn1 ffn2](MFMA) [ln](HBM).
-    Round 1: A launches q,k,v,attn,out; B's next is MFMA -> same class -> nothing on stream 1.
-    Round 2: A launches ln (0.0695 ms window, x0.8 = 0.0556).  B: q,k,v (0.0124 each), attn (0.0082) fit -> 0.0102 left;
+    Scheduling window 1: A launches q,k,v,attn,out; B's next is MFMA -> same class -> nothing on stream 1.
+    Scheduling window 2: A launches ln (0.0695 ms window, x0.8 = 0.0556).  B: q,k,v (0.0124 each), attn (0.0082) fit -> 0.0102 left;
              out_proj (0.0124) does not fit -> split with profiled fractions [0.0061, 0.0082, 0.0103] -> 2/4 fits ->
              first piece (128 of 256 output columns) goes to stream 1, remainder (128 columns) stays queued.
-    Round 3: A launches ffn1, ffn2 (MFMA); B's next (remainder of out_proj) is MFMA -> nothing.
-    Round 4: A launches its last ln; B's remainder fits the window and runs on stream 1; B's ln is HBM -> stop.
+    Scheduling window 3: A launches ffn1, ffn2 (MFMA); B's next (remainder of out_proj) is MFMA -> nothing.
+    Scheduling window 4: A launches its last ln; B's remainder fits the window and runs on stream 1; B's ln is HBM -> stop.
     Then B becomes primary and finishes alone on stream 0."""
     host = fake.host
     m = small_model(host, factor=4)
