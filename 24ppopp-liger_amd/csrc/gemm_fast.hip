@@ -1,7 +1,7 @@
 // gemm_fast.hip -- pipelined 256x256x64 fp16 GEMM for gfx950 (the prefill shapes of the launch vector).
 //
 //   Y[M, N] = X[M, K] * W,  W row-major [K, N] (the reference's layout) or [N, K];  fp32 accumulate, optional fused
-//   epilogue.  Requires M % 256 == 0, N % 128 == 0 (or % 192), K % 64 == 0 and 16-byte aligned operands; everything else goes to
+//   epilogue.  Requires N % 128 == 0 (or % 192), K % 64 == 0, M > 64 (any M; a partial last row of tiles is padded) and 16-byte aligned operands; everything else goes to
 //   the generic kernel in gemm.hip.
 //
 // Structure (one workgroup = 8 waves = one 256x256 output tile, one workgroup per CU):
@@ -48,7 +48,7 @@ __device__ __forceinline__ int swz_a(int row, int c) { return c ^ ((row >> 1) & 
 __device__ __forceinline__ int swz_b(int k, int blk) { return blk ^ ((k & 3) | ((k >> 1) & 4)); }
 
 template <int WL, int EPI, int NJ>
-__global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles_m, int tiles_n) {
+__global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles_m, int tiles_n, float* partial, int kt_per_split) {
     constexpr int FB_N = 64 * NJ;
     constexpr int X_TILE = FB_M * FB_K, W_TILE = FB_K * FB_N;  // halves per ring slot
     constexpr int WCH = (FB_K * FB_N) / 512 / 8;  // 1 KiB chunks of the W tile per wave (= NJ)
@@ -80,8 +80,12 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles
         }
     }
     const int m0 = tm * FB_M, n0 = tn * FB_N;
-    const half_t* X = g.X + (int64_t)m0 * g.ldx;
-    const half_t* W = (WL == W_KN) ? g.W + n0 : g.W + (int64_t)n0 * g.ldw;
+    // K-slice of this workgroup (blockIdx.y; the whole K when the launch is not split): k-tiles [kt0, kt0 + ktiles)
+    const int split = blockIdx.y;
+    const int kt0 = split * kt_per_split;
+    const int ktiles = min(g.K / FB_K - kt0, kt_per_split);
+    const half_t* X = g.X + (int64_t)m0 * g.ldx + (int64_t)kt0 * FB_K;
+    const half_t* W = (WL == W_KN) ? g.W + n0 + (int64_t)kt0 * FB_K * g.ldw : g.W + (int64_t)n0 * g.ldw + (int64_t)kt0 * FB_K;
 
     // ---- per-lane global offsets of the 8 direct-to-LDS loads of one k-tile ---------------------------------------------
     // X tile (and W tile when [N, K]): 32 chunks of 1 KiB = 8 rows x 128 B; wave w fills chunks w, w+8, w+16, w+24.
@@ -91,7 +95,9 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles
         const int q = i * 8 + wave;
         const int row = q * 8 + (lane >> 3), pos = lane & 7;
         const int c = swz_a(row, pos);  // XOR is an involution: the chunk stored at `pos` is logical chunk pos ^ f(row)
-        xoff[i] = (unsigned)(row * (int)g.ldx + c * 8) * 2u;
+        // token rows beyond M (last, partial row of tiles) are read from row M-1; their results are never stored
+        const int xrow = min(row, g.M - 1 - m0);
+        xoff[i] = (unsigned)(xrow * (int)g.ldx + c * 8) * 2u;
         if (i >= WCH) continue;
         if (WL == W_NK) {
             woff[i] = (unsigned)(row * (int)g.ldw + c * 8) * 2u;
@@ -107,7 +113,6 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles
 
     // tile index clamped to the last one: the loop body is branch-free, the extra loads of the last iterations
     // refill slots nobody reads any more
-    const int ktiles = g.K / FB_K;
     auto x_tile = [&](int kt) { return reinterpret_cast<const char*>(X + (int64_t)(kt < ktiles ? kt : ktiles - 1) * FB_K); };
     auto w_tile = [&](int kt) { return reinterpret_cast<const char*>(W + (int64_t)(kt < ktiles ? kt : ktiles - 1) * wstep); };
     // load l of a k-tile: l < WCH -> chunk l of the W tile, else chunk l - WCH of the X tile (W first: it is needed first)
@@ -210,12 +215,24 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles
     // ---- epilogue: acc[i][j][r] = Y[m0 + wm*128 + i*16 + l16][n0 + wn*16*NJ + j*16 + 4*lk + r] -----------------------------
     // Everything that depends only on the column (bias, head offset) or only on the row (batch / position split) is
     // computed once, so the 8 x NJ stores of a lane are not separated by dependent loads or integer divisions.
+    if (EPI == LG_EPI_PARTIAL) {
+        // split-K: the fp32 accumulators of this K-slice go to partial[split][M][N]; a second kernel sums the slices
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int m = m0 + wm * 128 + i * 16 + l16;
+            if (m >= g.M) continue;
+            float* prow = partial + ((int64_t)split * g.M + m) * g.N + n0 + wn * (16 * NJ) + 4 * lk;
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) *reinterpret_cast<float4_t*>(prow + j * 16) = acc[i][j];
+        }
+        return;
+    }
     float bias_v[NJ][4];
     int64_t col_off[NJ];
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
         const int n = n0 + wn * (16 * NJ) + j * 16 + 4 * lk;
-        if (EPI != LG_EPI_NONE) {
+        if (EPI != LG_EPI_NONE && EPI != LG_EPI_PARTIAL) {
             const half4_t bv = *reinterpret_cast<const half4_t*>(g.epi.bias + n);
 #pragma unroll
             for (int r = 0; r < 4; ++r) bias_v[j][r] = (float)bv[r];
@@ -228,6 +245,7 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         const int m = m0 + wm * 128 + i * 16 + l16;
+        if (m >= g.M) continue;
         int64_t row_off;
         if (EPI == LG_EPI_BIAS_HEADS) {
             const int b = m / g.epi.seq, sq = m % g.epi.seq;
@@ -253,8 +271,28 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles
 }
 
 template <int WL, int NJ>
-static void launch_fast_epi(const GemmArgs& g, int tiles_m, int tiles_n, hipStream_t stream) {
-    const dim3 grid(tiles_m * tiles_n), block(F_THREADS);
+static int launch_fast_epi(const GemmArgs& g, int tiles_m, int tiles_n, hipStream_t stream) {
+    const int tiles = tiles_m * tiles_n, ktiles = g.K / FB_K;
+    // At most 256 token rows (one row of tiles, the continuation of the weight-streaming kernel's regime): the time is set by
+    // how fast the weights stream in, so K is split over otherwise idle CUs (slices of >= 8 k-tiles, fp32 partials summed in
+    // slice order by a second kernel that applies the epilogue).  Larger M never splits K, so that a token row's result does
+    // not depend on how many other rows are in the batch (each output is one sequential sum over k).
+    int nsplit = 1;
+    if (tiles_m == 1 && tiles <= 128) {
+        nsplit = 256 / tiles;
+        if (nsplit > ktiles / 8) nsplit = ktiles / 8;
+        if (nsplit > 16) nsplit = 16;
+        if (nsplit < 1) nsplit = 1;
+    }
+    int kt_per_split = (ktiles + nsplit - 1) / nsplit;
+    nsplit = (ktiles + kt_per_split - 1) / kt_per_split;
+    float* partial = nullptr;
+    if (nsplit > 1) {
+        const size_t bytes = (size_t)nsplit * g.M * g.N * sizeof(float);
+        partial = splitk_workspace(stream, bytes);
+        if (!partial) { set_error("gemm_fast: cannot allocate the %zu-byte split-K workspace", bytes); return LG_ERR_LAUNCH; }
+    }
+    const dim3 grid(tiles, nsplit), block(F_THREADS);
     const size_t smem = lds_halves(NJ) * sizeof(half_t);
 #define LG_FAST(E)                                                                                                  \
     do {                                                                                                            \
@@ -263,27 +301,37 @@ static void launch_fast_epi(const GemmArgs& g, int tiles_m, int tiles_n, hipStre
             (void)hipFuncSetAttribute((const void*)gemm_f16_fast<WL, E, NJ>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
             attr_set = true;                                                                                        \
         }                                                                                                           \
-        hipLaunchKernelGGL((gemm_f16_fast<WL, E, NJ>), grid, block, smem, stream, g, tiles_m, tiles_n);             \
+        hipLaunchKernelGGL((gemm_f16_fast<WL, E, NJ>), grid, block, smem, stream, g, tiles_m, tiles_n, partial, kt_per_split); \
     } while (0)
-    switch (g.epi.kind) {
-        case LG_EPI_NONE: LG_FAST(LG_EPI_NONE); break;
-        case LG_EPI_BIAS: LG_FAST(LG_EPI_BIAS); break;
-        case LG_EPI_BIAS_GELU: LG_FAST(LG_EPI_BIAS_GELU); break;
-        default: LG_FAST(LG_EPI_BIAS_HEADS); break;
+    if (nsplit > 1) {
+        LG_FAST(LG_EPI_PARTIAL);
+        launch_splitk_reduce(g, partial, nsplit, stream);
+    } else {
+        switch (g.epi.kind) {
+            case LG_EPI_NONE: LG_FAST(LG_EPI_NONE); break;
+            case LG_EPI_BIAS: LG_FAST(LG_EPI_BIAS); break;
+            case LG_EPI_BIAS_GELU: LG_FAST(LG_EPI_BIAS_GELU); break;
+            default: LG_FAST(LG_EPI_BIAS_HEADS); break;
+        }
     }
 #undef LG_FAST
+    return LG_OK;
 }
 
 int launch_gemm_fast_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t stream, bool* handled) {
     *handled = false;
     if (batch != 1) return LG_OK;
-    if (g.M % FB_M || g.K % FB_K || g.M <= 0 || g.N <= 0 || g.K <= 0) return LG_OK;
+    if (g.K % FB_K || g.M <= 0 || g.N <= 0 || g.K <= 0) return LG_OK;
+    // A partial last row of tiles computes (and discards) up to 255 extra token rows.  Even so this kernel is the faster one
+    // for every token count the weight-streaming kernel does not take (M = 128: 182 us vs 331 us in the generic kernel for a
+    // 16384 x 12288 weight), because with few token rows the time is set by how fast the weights stream in.
+    if (g.M <= 64) return LG_OK;
     if (!aligned16(g.X) || !aligned16(g.W) || !aligned16(g.Y) || (g.ldx % 8) || (g.ldw % 8)) return LG_OK;
     if (g.ldx >= (1 << 22) || g.ldw >= (1 << 22)) return LG_OK;  // 256 rows x ld must fit the 31-bit tile offsets
     if (g.epi.kind == LG_EPI_BIAS_HEADS ? (g.epi.d % 4 != 0) : (g.ldy % 4 != 0)) return LG_OK;
     if (g.epi.kind != LG_EPI_NONE && (reinterpret_cast<uintptr_t>(g.epi.bias) & 7u)) return LG_OK;  // 8-byte bias loads
     // tile width: the one that needs the least work-rounds on 256 CUs (rounds x tile width); ties go to the wider tile
-    const int tiles_m = g.M / FB_M;
+    const int tiles_m = (g.M + FB_M - 1) / FB_M;
     int best_nj = 0;
     long best_cost = 0;
     for (int nj = 4; nj >= 2; --nj) {
@@ -297,15 +345,16 @@ int launch_gemm_fast_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t 
     if (!best_nj) return LG_OK;
     *handled = true;
     const int tiles_n = g.N / (64 * best_nj);
+    int rc;
     if (wlayout == W_NK) {
-        if (best_nj == 4) launch_fast_epi<W_NK, 4>(g, tiles_m, tiles_n, stream);
-        else if (best_nj == 3) launch_fast_epi<W_NK, 3>(g, tiles_m, tiles_n, stream);
-        else launch_fast_epi<W_NK, 2>(g, tiles_m, tiles_n, stream);
+        if (best_nj == 4) rc = launch_fast_epi<W_NK, 4>(g, tiles_m, tiles_n, stream);
+        else if (best_nj == 3) rc = launch_fast_epi<W_NK, 3>(g, tiles_m, tiles_n, stream);
+        else rc = launch_fast_epi<W_NK, 2>(g, tiles_m, tiles_n, stream);
     } else {
-        if (best_nj == 4) launch_fast_epi<W_KN, 4>(g, tiles_m, tiles_n, stream);
-        else launch_fast_epi<W_KN, 2>(g, tiles_m, tiles_n, stream);
+        if (best_nj == 4) rc = launch_fast_epi<W_KN, 4>(g, tiles_m, tiles_n, stream);
+        else rc = launch_fast_epi<W_KN, 2>(g, tiles_m, tiles_n, stream);
     }
-    return check_launch("gemm_f16_fast");
+    return rc != LG_OK ? rc : check_launch("gemm_f16_fast");
 }
 
 }  // namespace lg

@@ -143,7 +143,7 @@ struct SkinnyWs { float* ptr; size_t bytes; };
 static std::mutex g_ws_mu;
 static std::unordered_map<void*, SkinnyWs> g_ws;
 
-static float* skinny_workspace(hipStream_t stream, size_t bytes) {
+float* splitk_workspace(hipStream_t stream, size_t bytes) {
     std::lock_guard<std::mutex> lk(g_ws_mu);
     SkinnyWs& w = g_ws[(void*)stream];
     if (w.bytes < bytes) {
@@ -155,6 +155,19 @@ static float* skinny_workspace(hipStream_t stream, size_t bytes) {
         w.bytes = want;
     }
     return w.ptr;
+}
+
+void launch_splitk_reduce(const GemmArgs& g, const float* partial, int nsplit, hipStream_t stream) {
+    const dim3 block(256);
+    const int64_t quads = (int64_t)g.M * ((g.N + 3) / 4);
+    int rgrid = (int)((quads + 255) / 256);
+    if (rgrid > 4096) rgrid = 4096;
+    switch (g.epi.kind) {
+        case LG_EPI_NONE: hipLaunchKernelGGL((gemm_skinny_reduce_kernel<LG_EPI_NONE>), dim3(rgrid), block, 0, stream, g, partial, nsplit); break;
+        case LG_EPI_BIAS: hipLaunchKernelGGL((gemm_skinny_reduce_kernel<LG_EPI_BIAS>), dim3(rgrid), block, 0, stream, g, partial, nsplit); break;
+        case LG_EPI_BIAS_GELU: hipLaunchKernelGGL((gemm_skinny_reduce_kernel<LG_EPI_BIAS_GELU>), dim3(rgrid), block, 0, stream, g, partial, nsplit); break;
+        default: hipLaunchKernelGGL((gemm_skinny_reduce_kernel<LG_EPI_BIAS_HEADS>), dim3(rgrid), block, 0, stream, g, partial, nsplit); break;
+    }
 }
 
 int launch_gemm_skinny_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t stream, bool* handled) {
@@ -170,7 +183,7 @@ int launch_gemm_skinny_f16(const GemmArgs& g, int wlayout, int batch, hipStream_
     int kslice = ((g.K + nsplit - 1) / nsplit + SK_KC - 1) / SK_KC * SK_KC;
     nsplit = (g.K + kslice - 1) / kslice;
     const size_t bytes = (size_t)nsplit * g.M * g.N * sizeof(float);
-    float* ws = skinny_workspace(stream, bytes);
+    float* ws = splitk_workspace(stream, bytes);
     if (!ws) { set_error("gemm_skinny: cannot allocate the %zu-byte split-K workspace", bytes); *handled = true; return LG_ERR_LAUNCH; }
     *handled = true;
     const dim3 grid(nblk, nsplit), block(256);
@@ -181,15 +194,7 @@ int launch_gemm_skinny_f16(const GemmArgs& g, int wlayout, int batch, hipStream_
         case 3: hipLaunchKernelGGL((gemm_skinny_nk_kernel<3>), grid, block, 0, stream, g, kslice, ws, nsplit); break;
         default: hipLaunchKernelGGL((gemm_skinny_nk_kernel<4>), grid, block, 0, stream, g, kslice, ws, nsplit); break;
     }
-    const int64_t quads = (int64_t)g.M * ((g.N + 3) / 4);
-    int rgrid = (int)((quads + 255) / 256);
-    if (rgrid > 4096) rgrid = 4096;
-    switch (g.epi.kind) {
-        case LG_EPI_NONE: hipLaunchKernelGGL((gemm_skinny_reduce_kernel<LG_EPI_NONE>), dim3(rgrid), block, 0, stream, g, ws, nsplit); break;
-        case LG_EPI_BIAS: hipLaunchKernelGGL((gemm_skinny_reduce_kernel<LG_EPI_BIAS>), dim3(rgrid), block, 0, stream, g, ws, nsplit); break;
-        case LG_EPI_BIAS_GELU: hipLaunchKernelGGL((gemm_skinny_reduce_kernel<LG_EPI_BIAS_GELU>), dim3(rgrid), block, 0, stream, g, ws, nsplit); break;
-        default: hipLaunchKernelGGL((gemm_skinny_reduce_kernel<LG_EPI_BIAS_HEADS>), dim3(rgrid), block, 0, stream, g, ws, nsplit); break;
-    }
+    launch_splitk_reduce(g, ws, nsplit, stream);
     return check_launch("gemm_f16_skinny");
 }
 

@@ -24,10 +24,12 @@ def ctx_output(dev, sched, model, i, rows, H):
 
 @pytest.mark.parametrize("axis", [0, 1])
 @pytest.mark.parametrize("fused", [False, True])
-def test_interleaved_decomposed_requests_match_sequential_bitwise(dev, host, axis, fused):
+def test_interleaved_decomposed_requests_match_sequential(dev, host, axis, fused):
     """Two prefill requests under the resource-class policy with a hand-made profile that forces the second request's
     GEMMs to be split (and re-split) into the first one's LayerNorm windows.  Each request's output must equal a plain
-    in-order run of the same input bit for bit: pieces tile the GEMM outputs exactly and streams are ordered."""
+    in-order run of the same input: pieces tile the GEMM outputs exactly and streams are ordered.  A piece may take a
+    kernel that sums K in slices where the whole GEMM does not (or the other way round), so single outputs may differ by
+    the rounding of one fp32 summation order (and what that becomes two layers later), never by more."""
     B, S, heads, d, F = 2, 128, 8, 128, 2048
     H = heads * d
     m = host.Model(1, 2 * B, S, heads, d, layer_num=2, ffn_inner=F, causal=True, fused=fused, factor=8, seed=11)
@@ -51,7 +53,8 @@ def test_interleaved_decomposed_requests_match_sequential_bitwise(dev, host, axi
         ref = torch.empty_like(got)
         m.run(pin, ref.data_ptr(), B, S, None, dev.stream)
         torch.cuda.synchronize()
-        assert torch.equal(got, ref), "request %d differs from its sequential run" % i
+        diff = (got.float() - ref.float()).abs()
+        assert float(diff.max()) <= 4e-3 * float(ref.float().abs().max()), "request %d differs from its sequential run" % i
 
 
 def test_prefill_plus_decode_trace_on_gpu(dev, host):
