@@ -11,6 +11,7 @@ namespace lg {
 
 int launch_gemm_fast_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t stream, bool* handled);
 int launch_gemm_skinny_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t stream, bool* handled);
+int launch_gemv_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t stream, bool* handled);
 
 // ---------------------------------------------------------------------------------------------------
 // fp16 generic kernel
@@ -147,6 +148,8 @@ static int gemm_f16_dispatch(GemmArgs g, int wlayout, int batch, hipStream_t str
     if (g.K == 0) { set_error("gemm: k == 0 is not supported"); return LG_ERR_INVALID; }
     bool handled = false;
     int rc = launch_gemm_fast_f16(g, wlayout, batch, stream, &handled);
+    if (handled) return rc;
+    rc = launch_gemv_f16(g, wlayout, batch, stream, &handled);
     if (handled) return rc;
     rc = launch_gemm_skinny_f16(g, wlayout, batch, stream, &handled);
     if (handled) return rc;

@@ -22,7 +22,9 @@ SHAPES = [(64, 256, 256), (128, 128, 32), (130, 136, 72), (1, 8, 8), (33, 70, 19
           # token counts that are not a multiple of the tile: the pipelined kernel pads the last row of tiles
           (320, 256, 128), (448, 384, 192), (1000, 512, 256), (200, 256, 64), (161, 768, 128), (65, 256, 192), (100, 384, 64),
           # few tokens, many features: the weight-streaming split-K kernel (weights stored [out, in])
-          (32, 1024, 2048), (1, 512, 1024), (17, 640, 4104), (64, 2048, 1536), (33, 516, 1032)]
+          (32, 1024, 2048), (1, 512, 1024), (17, 640, 4104), (64, 2048, 1536), (33, 516, 1032),
+          # one to four token rows and K a multiple of 2048: the matrix-vector kernel (weights stored [out, in])
+          (1, 512, 2048), (2, 1024, 4096), (3, 256, 2048), (4, 644, 6144), (1, 6144, 12288)]
 
 
 @pytest.mark.parametrize("dt", [0, 1])
@@ -152,3 +154,28 @@ def test_gemm_fused_epilogues_on_the_pipelined_kernel(dev, po, transa):
     got = dev.down(out)
     assert max_rel_err(got[:, :, :S], ref_heads) < 2e-3
     assert np.all(got[:, :, S:] == 0)
+
+
+@pytest.mark.parametrize("M", [1, 2, 4])
+def test_gemm_fused_epilogues_on_the_matrix_vector_kernel(dev, po, M):
+    """Decode-shaped calls (a few token rows, weights [out, in]): bias + GELU and the head-transposed store into a
+    KV-cache-shaped destination with more rows per head than tokens."""
+    h, d, K = 6, 128, 4096
+    N = h * d
+    X = rnd(po, M * K, 43, 1).reshape(M, K)
+    W = rnd(po, K * N, 44, 1, 0.05).reshape(K, N)
+    bias = rnd(po, N, 45, 1, 0.3)
+    dA, dX, dB = dev.up(np.ascontiguousarray(W.T), 1), dev.up(X, 1), dev.up(bias, 1)
+    y = po.gemm(X, W, 1)
+    out = dev.empty((M, N), 1)
+    dev.call("lg_gemm_fused_f16", 1, N, M, K, dA, K, dX, K, out, N, dev.capi.EPI_BIAS_GELU, dB, 0, 0, 0)
+    assert max_rel_err(dev.down(out), po.add_bias_gelu(y.copy(), bias, 1)) < 4e-3
+    # one token per sequence (batch = M, seq = 1) written to row 0 of a [M, h, rows, d] destination
+    ref_heads, _, _ = po.add_qkv_bias_transpose(y, bias, y, bias, y, bias, M, 1, h, d, 1)
+    rows = 5
+    out = dev.empty((M, h, rows, d), 1)
+    out.zero_()
+    dev.call("lg_gemm_fused_f16", 1, N, M, K, dA, K, dX, K, out, rows, dev.capi.EPI_BIAS_HEADS, dB, 1, d, h)
+    got = dev.down(out)
+    assert max_rel_err(got[:, :, :1], ref_heads) < 2e-3
+    assert np.all(got[:, :, 1:] == 0)
