@@ -44,6 +44,7 @@ class Sample {
     class_policy _policy = CLASSIC;
     split_axis _axis = SPLIT_OUT_COLS;
     int _last_stream = -1;
+    void* _last_stream_handle = nullptr;
 
     bool _sub_empty() const { return _SubFuncWrapVec.size() == _sub_exe_num; }
     size_t _sub_size() const { return _SubFuncWrapVec.size() - _sub_exe_num; }
@@ -130,8 +131,12 @@ class Sample {
             record_gpu_start(DParams);
         }
         // a sample that changes stream must wait for its own kernels on the other stream
-        if (_last_stream >= 0 && _last_stream != DParams.stream_id)
+        // (the event is recorded on the old stream only now, at the switch: it then also covers whatever other requests
+        // have launched there since, which only orders more, and the common case of no switch costs no event at all)
+        if (_last_stream >= 0 && _last_stream != DParams.stream_id) {
+            note_status(lg_event_record(last_launch, _last_stream_handle), "lg_event_record");
             note_status(lg_stream_wait_event(DParams.stream, last_launch), "lg_stream_wait_event");
+        }
         const bool last = next_empty();
         if (!_sub_empty()) {
             if (_sub_exe_num == 0) exe_num++;  // the first piece consumes the parent GEMM
@@ -148,7 +153,7 @@ class Sample {
             exe_num++;
         }
         _last_stream = DParams.stream_id;
-        note_status(lg_event_record(last_launch, DParams.stream), "lg_event_record");
+        _last_stream_handle = DParams.stream;
         if (last) record_gpu_stop(DParams);
         return duration;
     }
