@@ -11,8 +11,8 @@
 //     store) applied in place;
 //   * the M token rows are staged once per block in LDS (M * K * 2 bytes) and shared by the 4 weight rows of every wave;
 //     the first weight loads are issued before that staging so that the stream starts at once.
-// Each output is one fixed-order fp32 sum (per-lane partial sums over k, then a butterfly), independent of N and of the
-// other token rows.
+// Each output is one fixed-order fp32 sum (per-lane partial sums over k in an order fixed by the output's position, then a
+// butterfly), independent of the other token rows.
 #include "gemm_common.cuh"
 
 namespace lg {
@@ -43,12 +43,17 @@ __global__ __launch_bounds__(256) void gemv_nk_kernel(GemmArgs g) {
 #pragma unroll
     for (int r = 0; r < GV_ROWS; ++r) wrow[r] = g.W + (int64_t)min(n0 + r, g.N - 1) * g.ldw + lane * 8;
 
+    // Every wave walks k in groups of GV_U k-steps, starting at its own group and wrapping around: with a power-of-two row
+    // pitch (K = 16384) rows that are walked in phase would all hit the same memory channels at the same time.
+    const int groups = ksteps / GV_U;
+    int grp = (blockIdx.x * 4 + wave) % groups;
+
     // the stream starts before X is staged
     half8_t wv[GV_U][GV_ROWS];
 #pragma unroll
     for (int u = 0; u < GV_U; ++u)
 #pragma unroll
-        for (int r = 0; r < GV_ROWS; ++r) wv[u][r] = *reinterpret_cast<const half8_t*>(wrow[r] + u * GV_KSTEP);
+        for (int r = 0; r < GV_ROWS; ++r) wv[u][r] = *reinterpret_cast<const half8_t*>(wrow[r] + (int64_t)(grp * GV_U + u) * GV_KSTEP);
 
     for (int v = tid; v < MR * (K / 8); v += 256) {
         const int row = v / (K / 8), c = v % (K / 8);
@@ -64,21 +69,22 @@ __global__ __launch_bounds__(256) void gemv_nk_kernel(GemmArgs g) {
 #pragma unroll
         for (int m = 0; m < MR; ++m) acc[r][m] = 0.f;
 
-    for (int ks = 0; ks < ksteps; ks += GV_U) {
+    for (int it = 0; it < groups; ++it) {
         // the group after the last one is the last one again: every load is unconditional
-        const int next = (ks + GV_U < ksteps) ? ks + GV_U : ks;
+        const int next = (it + 1 < groups) ? (grp + 1 == groups ? 0 : grp + 1) : grp;
 #pragma unroll
         for (int u = 0; u < GV_U; ++u) {
             half8_t xv[MR];
 #pragma unroll
-            for (int m = 0; m < MR; ++m) xv[m] = *reinterpret_cast<const half8_t*>(&xs[m * K + (ks + u) * GV_KSTEP + lane * 8]);
+            for (int m = 0; m < MR; ++m) xv[m] = *reinterpret_cast<const half8_t*>(&xs[m * K + (grp * GV_U + u) * GV_KSTEP + lane * 8]);
 #pragma unroll
             for (int r = 0; r < GV_ROWS; ++r) {
 #pragma unroll
                 for (int m = 0; m < MR; ++m) acc[r][m] = dot8(wv[u][r], xv[m], acc[r][m]);
-                wv[u][r] = *reinterpret_cast<const half8_t*>(wrow[r] + (int64_t)(next + u) * GV_KSTEP);
+                wv[u][r] = *reinterpret_cast<const half8_t*>(wrow[r] + (int64_t)(next * GV_U + u) * GV_KSTEP);
             }
         }
+        grp = next;
     }
 
 #pragma unroll
