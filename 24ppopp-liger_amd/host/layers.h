@@ -414,19 +414,37 @@ class Bert_MHA {
         const MhaBuffers<T> b = slice(ws, batch, 1);
         const int h = heads(), d = BertParams.size_per_head, Lmax = BertParams.max_cache_len;
         const float sc = scalar;
-        std::vector<FuncWrap> v = linear_q_col->forward(input, b.q, batch); v[0].label = "q_gemm(decode)"; v[0].rclass = HBM_BOUND;
-        FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
-        v = linear_k_col->forward(input, b.k, batch); v[0].label = "k_gemm(decode)"; v[0].rclass = HBM_BOUND;
-        FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
-        v = linear_v_col->forward(input, b.v, batch); v[0].label = "v_gemm(decode)"; v[0].rclass = HBM_BOUND;
-        FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
         T* kc = k_cache + (int64_t)cache_slot * h * Lmax * d;
         T* vc = v_cache + (int64_t)cache_slot * h * Lmax * d;
-        T *qbias = q_bias, *kbias = k_bias, *vbias = v_bias;
         void* dws = b.decode_ws;
-        FuncWrapVec.push_back(FuncWrap(0.05f, COMPUTATION, [=](const DynamicInitParam& D) {
-            note_status(lg_kv_append_f16(b.q_buf, kc, vc, b.q, qbias, b.k, kbias, b.v, vbias, batch, h, d, past, Lmax, D.stream), "lg_kv_append_f16");
-        }, "kv_append"));
+        std::vector<FuncWrap> v;
+        if (BertParams.fused) {
+            // the GEMM epilogues add the bias and write q as [B, h, d] and the new K/V rows straight into the cache at
+            // position `past` (one token per sequence: batch index = token index, row 0 of a slot shifted by `past` rows)
+            Linear_Col<T>* lin[3] = {linear_q_col, linear_k_col, linear_v_col};
+            T* dst[3] = {b.q_buf, kc + (int64_t)past * d, vc + (int64_t)past * d};
+            const T* bias[3] = {q_bias, k_bias, v_bias};
+            const char* lab[3] = {"q_gemm(decode)", "k_gemm(decode)", "v_gemm(decode)"};
+            for (int t = 0; t < 3; ++t) {
+                GemmDesc g = lin[t]->desc(input, dst[t], batch);
+                g.epilogue = LG_EPI_BIAS_HEADS;
+                g.bias = bias[t];
+                g.epi_seq = 1; g.epi_d = d; g.epi_heads_total = h;
+                g.ldc = (t == 0) ? 1 : Lmax;  // rows per (batch, head) slot of the destination
+                FuncWrapVec.push_back(FuncWrap(1.0f, GEMM, [g](const DynamicInitParam& D) { GemmEx(D, g); }, g, lab[t], HBM_BOUND));
+            }
+        } else {
+            v = linear_q_col->forward(input, b.q, batch); v[0].label = "q_gemm(decode)"; v[0].rclass = HBM_BOUND;
+            FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
+            v = linear_k_col->forward(input, b.k, batch); v[0].label = "k_gemm(decode)"; v[0].rclass = HBM_BOUND;
+            FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
+            v = linear_v_col->forward(input, b.v, batch); v[0].label = "v_gemm(decode)"; v[0].rclass = HBM_BOUND;
+            FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
+            T *qbias = q_bias, *kbias = k_bias, *vbias = v_bias;
+            FuncWrapVec.push_back(FuncWrap(0.05f, COMPUTATION, [=](const DynamicInitParam& D) {
+                note_status(lg_kv_append_f16(b.q_buf, kc, vc, b.q, qbias, b.k, kbias, b.v, vbias, batch, h, d, past, Lmax, D.stream), "lg_kv_append_f16");
+            }, "kv_append"));
+        }
         FuncWrapVec.push_back(FuncWrap(0.15f, COMPUTATION, [=](const DynamicInitParam& D) {
             note_status(lg_attn_decode_f16(b.q_buf, kc, vc, b.attn_out, dws, batch, h, d, past + 1, Lmax, sc, D.stream), "lg_attn_decode_f16");
         }, "attn_decode"));
@@ -556,7 +574,7 @@ class Bert_Model {
     // entries per layer of the vector forward() returns for this configuration
     int kernels_per_layer(bool decode = false) const {
         const bool fused = BertParams.fused && dtype_of<T>::value == LG_F16;
-        int mha = decode ? 6 : (fused ? 5 : 9);
+        int mha = decode ? (BertParams.fused ? 5 : 6) : (fused ? 5 : 9);
         int mlp = fused ? 2 : 3;
         return mha + mlp + 2 + (BertParams.norm_mode == PRE_LN_RESID ? 1 : 0);
     }
