@@ -48,6 +48,8 @@ SIGNATURES = {
     "lg_layer_norm_f16": (_i, [_p, _p, _p, _p, _i, _i, _p]),
     "lg_add_bias_act_f32": (_i, [_p, _p, _i, _i, _p]),
     "lg_add_bias_act_f16": (_i, [_p, _p, _i, _i, _p]),
+    "lg_add_bias_geglu_f32": (_i, [_p, _p, _p, _i, _i, _p]),
+    "lg_add_bias_geglu_f16": (_i, [_p, _p, _p, _i, _i, _p]),
     "lg_add_bias_input_layernorm_f32": (_i, [_p, _p, _p, _p, _p, _i, _i, _p]),
     "lg_add_bias_input_layernorm_f16": (_i, [_p, _p, _p, _p, _p, _i, _i, _p]),
     "lg_add_bias_input_layernorm_2_f32": (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _p]),

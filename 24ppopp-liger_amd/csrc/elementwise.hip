@@ -201,6 +201,55 @@ static int launch_bias_gelu(T* out, const T* bias, int m, int n, hipStream_t str
     return check_launch("add_bias_act");
 }
 
+// ---- GeGLU: out[m, f] = gelu_tanh(in[m, j] + bias[j]) * (in[m, f + j] + bias[f + j]),  in = [gate | up] ------------
+template <typename T>
+__global__ __launch_bounds__(256) void bias_geglu_vec_kernel(T* out, const T* __restrict__ in, const T* __restrict__ bias,
+                                                             int64_t total_vec, int nvec_row, int f) {
+    typedef Vec16<T> V;
+    for (int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; v < total_vec; v += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t row = v / nvec_row;
+        const int c = (int)(v % nvec_row);
+        const T* src = in + row * 2 * f + (int64_t)c * V::N;
+        V g = *reinterpret_cast<const V*>(src);
+        V u = *reinterpret_cast<const V*>(src + f);
+        V bg = *reinterpret_cast<const V*>(bias + (int64_t)c * V::N);
+        V bu = *reinterpret_cast<const V*>(bias + f + (int64_t)c * V::N);
+        V o;
+#pragma unroll
+        for (int j = 0; j < V::N; ++j) o.set(j, gelu_tanh(g.get(j) + bg.get(j)) * (u.get(j) + bu.get(j)));
+        *reinterpret_cast<V*>(out + v * V::N) = o;
+    }
+}
+template <typename T>
+__global__ __launch_bounds__(256) void bias_geglu_scalar_kernel(T* out, const T* in, const T* bias, int64_t total, int f) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t row = i / f;
+        const int j = (int)(i % f);
+        const T* src = in + row * 2 * f;
+        stf(out + i, gelu_tanh(ldf(src + j) + ldf(bias + j)) * (ldf(src + f + j) + ldf(bias + f + j)));
+    }
+}
+
+template <typename T>
+static int launch_bias_geglu(T* out, const T* in, const T* bias, int m, int f, hipStream_t stream) {
+    if (m < 0 || f <= 0) { set_error("add_bias_geglu: bad shape m=%d f=%d", m, f); return LG_ERR_INVALID; }
+    if (m == 0) return LG_OK;
+    if (!out || !in || !bias) { set_error("add_bias_geglu: null pointer"); return LG_ERR_INVALID; }
+    constexpr int VN = Vec16<T>::N;
+    const int64_t total = (int64_t)m * f;
+    if (f % VN == 0 && aligned16(out) && aligned16(in) && aligned16(bias)) {
+        const int64_t tv = total / VN;
+        int64_t grid = (tv + 255) / 256;
+        if (grid > 256 * 32) grid = 256 * 32;
+        hipLaunchKernelGGL((bias_geglu_vec_kernel<T>), dim3((int)grid), dim3(256), 0, stream, out, in, bias, tv, f / VN, f);
+    } else {
+        int64_t grid = (total + 255) / 256;
+        if (grid > 65536) grid = 65536;
+        hipLaunchKernelGGL((bias_geglu_scalar_kernel<T>), dim3((int)grid), dim3(256), 0, stream, out, in, bias, total, f);
+    }
+    return check_launch("add_bias_geglu");
+}
+
 // ---- output = output + input + bias -----------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void add_bias_input_vec_kernel(T* output, const T* __restrict__ input,
@@ -259,6 +308,12 @@ int lg_layer_norm_f16(const void* in, const void* gamma, const void* beta, void*
 }
 int lg_add_bias_act_f32(float* out, const float* bias, int m, int n, void* stream) {
     return launch_bias_gelu<float>(out, bias, m, n, (hipStream_t)stream);
+}
+int lg_add_bias_geglu_f32(float* out, const float* in, const float* bias, int m, int f, void* stream) {
+    return lg::launch_bias_geglu<float>(out, in, bias, m, f, (hipStream_t)stream);
+}
+int lg_add_bias_geglu_f16(void* out, const void* in, const void* bias, int m, int f, void* stream) {
+    return lg::launch_bias_geglu<lg::half_t>((lg::half_t*)out, (const lg::half_t*)in, (const lg::half_t*)bias, m, f, (hipStream_t)stream);
 }
 int lg_add_bias_act_f16(void* out, const void* bias, int m, int n, void* stream) {
     return launch_bias_gelu<half_t>((half_t*)out, (const half_t*)bias, m, n, (hipStream_t)stream);

@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(_PKG, "lib", "libliger_host.so")
 
 POST_NORESID, PRE_LN_RESID = 0, 1
 POLICY_CLASSIC, POLICY_RESOURCE = 0, 1
+FFN_GELU, FFN_GEGLU = 0, 1
 SPLIT_OUT_COLS, SPLIT_TOKEN_ROWS = 0, 1
 MODE_SEQUENTIAL, MODE_LIGER = 0, 1
 
@@ -33,6 +34,7 @@ SIGNATURES = {
     "lgh_first_error": (_i, [C.c_char_p, _i]),
     "lgh_clear_error": (None, []),
     "lgh_model_create": (_p, [_i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _u64]),
+    "lgh_model_create_ex": (_p, [_i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _u64]),
     "lgh_model_kernels_per_layer": (_i, [_p, _i]),
     "lgh_model_workspace_elems": (_i64, [_p, _i, _i]),
     "lgh_model_stream": (_p, [_p]),
@@ -120,10 +122,12 @@ class Model:
     """One tensor-parallel shard of a stack of encoder layers, assembled as launch vectors by the C++ runtime."""
 
     def __init__(self, dtype, max_batch, max_seq, head_num, size_per_head, layer_num=1, world_size=1, ffn_inner=0,
-                 norm_mode=POST_NORESID, causal=False, fused=False, max_cache_len=0, factor=8, weight_layout=0, seed=0):
+                 norm_mode=POST_NORESID, causal=False, fused=False, max_cache_len=0, factor=8, weight_layout=0, seed=0,
+                 ffn_act=FFN_GELU, packed_qkv=False):
         lib.lgh_clear_error()
-        self.h = lib.lgh_model_create(dtype, max_batch, max_seq, head_num, size_per_head, layer_num, world_size, ffn_inner,
-                                      norm_mode, int(causal), int(fused), max_cache_len, factor, weight_layout, seed)
+        self.h = lib.lgh_model_create_ex(dtype, max_batch, max_seq, head_num, size_per_head, layer_num, world_size, ffn_inner,
+                                         norm_mode, int(causal), int(fused), max_cache_len, factor, weight_layout, int(ffn_act),
+                                         int(packed_qkv), seed)
         if not self.h:
             check(1, "lgh_model_create")
         self.dtype = dtype

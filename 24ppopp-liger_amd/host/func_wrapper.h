@@ -88,6 +88,13 @@ void Add_bias_act_kernelLauncher(T* out, const T* bias, int m, int n, const Dyna
     else note_status(lg_add_bias_act_f32((float*)out, (const float*)bias, m, n, DParams.stream), "lg_add_bias_act_f32");
 }
 
+// GeGLU (no reference counterpart): in [m, 2f] = [gate | up] -> out [m, f]
+template <typename T>
+void Add_bias_geglu_kernelLauncher(T* out, const T* in, const T* bias, const int m, const int f, const DynamicInitParam& DParams) {
+    if (dtype_of<T>::value == LG_F16) note_status(lg_add_bias_geglu_f16(out, in, bias, m, f, DParams.stream), "lg_add_bias_geglu_f16");
+    else note_status(lg_add_bias_geglu_f32((float*)out, (const float*)in, (const float*)bias, m, f, DParams.stream), "lg_add_bias_geglu_f32");
+}
+
 template <typename T>
 void Add_bias_input_layernorm_kernelLauncher(T* out, const T* input_tensor, const T* bias, const T* gamma, const T* beta,
                                              int m, int n, const DynamicInitParam& DParams) {

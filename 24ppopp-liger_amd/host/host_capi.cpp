@@ -168,9 +168,20 @@ int lgh_first_error(char* buf, int len) {
 void lgh_clear_error(void) { clear_error(); }
 
 // dtype 0 = fp32, 1 = fp16.  head_num and ffn_inner are GLOBAL sizes; the model holds the 1/world_size shard.
+void* lgh_model_create_ex(int dtype, int max_batch, int max_seq, int head_num, int size_per_head, int layer_num, int world_size,
+                          int ffn_inner, int norm_mode, int causal, int fused, int max_cache_len, int factor, int weight_layout,
+                          int ffn_act, int packed_qkv, uint64_t seed);
 void* lgh_model_create(int dtype, int max_batch, int max_seq, int head_num, int size_per_head, int layer_num, int world_size,
                        int ffn_inner, int norm_mode, int causal, int fused, int max_cache_len, int factor, int weight_layout,
                        uint64_t seed) {
+    return lgh_model_create_ex(dtype, max_batch, max_seq, head_num, size_per_head, layer_num, world_size, ffn_inner, norm_mode, causal,
+                               fused, max_cache_len, factor, weight_layout, 0, 0, seed);
+}
+// ffn_act: 0 GELU, 1 GeGLU (FFN-1 is [H, 2F] = [gate | up]); packed_qkv: 1 = one [H, 3 Hl] projection + the fused
+// bias/transpose kernel (reference-shaped assembly without KV cache only)
+void* lgh_model_create_ex(int dtype, int max_batch, int max_seq, int head_num, int size_per_head, int layer_num, int world_size,
+                          int ffn_inner, int norm_mode, int causal, int fused, int max_cache_len, int factor, int weight_layout,
+                          int ffn_act, int packed_qkv, uint64_t seed) {
     if (max_batch <= 0 || max_seq <= 0 || head_num <= 0 || size_per_head <= 0 || layer_num <= 0 || world_size <= 0 ||
         head_num % world_size != 0 || (ffn_inner > 0 && ffn_inner % world_size != 0) || (dtype != 0 && dtype != 1)) {
         fail("lgh_model_create: bad configuration");
@@ -178,7 +189,10 @@ void* lgh_model_create(int dtype, int max_batch, int max_seq, int head_num, int 
     }
     if (fused && dtype != 1) { fail("lgh_model_create: the fused assembly is fp16 only"); return nullptr; }
     if (max_cache_len > 0 && !fused) { fail("lgh_model_create: the KV cache needs the fused assembly"); return nullptr; }
+    if (packed_qkv && (fused || max_cache_len > 0)) { fail("lgh_model_create: the packed QKV projection belongs to the reference-shaped assembly (fused = 0, no KV cache)"); return nullptr; }
+    if ((ffn_act != 0 && ffn_act != 1) || (packed_qkv != 0 && packed_qkv != 1)) { fail("lgh_model_create: bad ffn_act / packed_qkv"); return nullptr; }
     BertInitParam P(max_batch, max_seq, head_num, size_per_head, layer_num, 0, factor, 0);
+    P.ffn_act = ffn_act; P.packed_qkv = packed_qkv;
     P.ffn_inner = ffn_inner; P.norm_mode = norm_mode; P.causal = causal; P.fused = fused; P.max_cache_len = max_cache_len;
     P.weight_layout = weight_layout ? 1 : 0;
     StaticInitParam S(0, world_size, dtype);

@@ -76,6 +76,7 @@ class StaticInitParam {
 using StaticNvInitParam = StaticInitParam;
 
 enum norm_mode_t { POST_NORESID = 0, PRE_LN_RESID = 1 };
+enum ffn_act_t { FFN_GELU = 0, FFN_GEGLU = 1 };
 
 // ---- model / scheduler parameters  (context.h:59-85) --------------------------------------------------
 class BertInitParam {
@@ -96,6 +97,9 @@ class BertInitParam {
     int max_cache_len = 0;  // > 0 -> layers own a KV cache [max_batch, heads, max_cache_len, d] for decode steps
     int weight_layout = 0;  // 0: weights stored [in, out] (what the reference's (N,N) cuBLAS call implies);
                             // 1: stored [out, in] and multiplied with transa = T (both operands K-contiguous)
+    int ffn_act = 0;        // 0: FFN-1 -> bias + GELU -> FFN-2 (bert_layer.h:43-62); 1: GeGLU, FFN-1 is [H, 2F] = [gate | up]
+    int packed_qkv = 0;     // 1 (reference-shaped assembly only): one [H, 3 Hl] GEMM + add_fusedQKV_bias_transpose
+                            // (attention_kernels.cuh:23-34) instead of three GEMMs + add_QKV_bias_transpose
     BertInitParam() {}
     BertInitParam(int max_batch_size_, int max_seq_len_, int head_num_, int size_per_head_, int layer_num_,
                   int kernel_num_, int factor_, int rq_interval_)

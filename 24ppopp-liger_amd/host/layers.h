@@ -174,23 +174,30 @@ class Bert_MLP {
     Bert_MLP(const BertInitParam& BertParams_, const StaticInitParam& SParam_, const int& k_, const int& n_, T* workspace)
         : k(k_), n(n_), SParam(SParam_), BertParams(BertParams_), linear_row_output(workspace) {
         intermediate_size = BertParams.ffn_inner > 0 ? BertParams.ffn_inner : n * mlp_ratio;
-        linear_col = new Linear_Col<T>(SParam, k, intermediate_size, BertParams.weight_layout);
+        // GeGLU: FFN-1 produces [gate | up], 2 F local columns
+        linear_col = new Linear_Col<T>(SParam, k, intermediate_size * gate_mult(), BertParams.weight_layout);
         linear_row = new Linear_Row<T>(SParam, intermediate_size, k, BertParams.weight_layout);
-        bias = dev_alloc<T>(f_local());
+        bias = dev_alloc<T>(f_local() * gate_mult());
         bias2 = dev_alloc<T>(k);
-        dev_fill_const(bias, f_local(), 0.f);
+        dev_fill_const(bias, f_local() * gate_mult(), 0.f);
         dev_fill_const(bias2, k, 0.f);
     }
     int f_local() const { return intermediate_size / SParam.world_size; }
+    int gate_mult() const { return BertParams.ffn_act == FFN_GEGLU ? 2 : 1; }
+    // elements of the FFN-1 output buffer per token (GeGLU keeps [gate | up] and the product)
+    static int64_t inner_per_token(const BertInitParam& P, const StaticInitParam& S, int hidden) {
+        const int64_t F = (P.ffn_inner > 0 ? P.ffn_inner : 4 * hidden) / S.world_size;
+        return P.ffn_act == FFN_GEGLU ? 3 * F : F;
+    }
     void init_weights(uint64_t seed, uint64_t base) {
         linear_col->init_weights(seed, base + 0);
         linear_row->init_weights(seed, base + 1);
-        dev_fill_normal(bias, f_local(), seed, base + 2, 0.f, 0.02f);
+        dev_fill_normal(bias, f_local() * gate_mult(), seed, base + 2, 0.f, 0.02f);
         dev_fill_normal(bias2, k, seed, base + 3, 0.f, 0.02f);
     }
     void params(const std::string& prefix, std::vector<ParamRef>& out) {
         out.push_back(linear_col->param(prefix + "w1"));
-        out.push_back({prefix + "b1", bias, f_local(), 1, f_local(), 0});
+        out.push_back({prefix + "b1", bias, f_local() * gate_mult(), 1, f_local() * gate_mult(), 0});
         out.push_back(linear_row->param(prefix + "w2"));
         out.push_back({prefix + "b2", bias2, k, 1, k, 0});
     }
@@ -199,7 +206,17 @@ class Bert_MLP {
         FuncWrapVec.clear();
         if (!inner) inner = linear_row_output;
         const int F = f_local();
-        if (BertParams.fused && dtype_of<T>::value == LG_F16) {
+        if (BertParams.ffn_act == FFN_GEGLU) {
+            // inner holds [m, F] (the product) followed by [m, 2F] (gate | up)
+            T* gu = inner + (int64_t)m * F;
+            std::vector<FuncWrap> v = linear_col->forward(input, gu, m);
+            v[0].label = "ffn1(gate+up)";
+            FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
+            T* b = bias;
+            FuncWrapVec.push_back(FuncWrap(0.2f, COMPUTATION,
+                                           [=](const DynamicInitParam& D) { Add_bias_geglu_kernelLauncher<T>(inner, gu, b, m, F, D); },
+                                           "bias+geglu"));
+        } else if (BertParams.fused && dtype_of<T>::value == LG_F16) {
             GemmDesc g = linear_col->desc(input, inner, m);
             g.epilogue = LG_EPI_BIAS_GELU;
             g.bias = bias;
@@ -237,6 +254,8 @@ class Bert_MHA {
     Linear_Col<T>* linear_q_col;
     Linear_Col<T>* linear_k_col;
     Linear_Col<T>* linear_v_col;
+    Linear_Col<T>* linear_qkv_col = nullptr;  // packed_qkv: one [H, 3 Hl] projection, columns [q | k | v]
+    T* qkv_bias = nullptr;                    // packed_qkv: [3 Hl]
     Linear_Row<T>* linear_w_row;
     StaticInitParam SParam;
     BertInitParam BertParams;
@@ -257,6 +276,11 @@ class Bert_MHA {
         w_bias = dev_alloc<T>(n);
         dev_fill_const(q_bias, hl(), 0.f); dev_fill_const(k_bias, hl(), 0.f); dev_fill_const(v_bias, hl(), 0.f);
         dev_fill_const(w_bias, n, 0.f);
+        if (BertParams.packed_qkv) {
+            linear_qkv_col = new Linear_Col<T>(SParam, k, 3 * n, BertParams.weight_layout);
+            qkv_bias = dev_alloc<T>(3 * hl());
+            dev_fill_const(qkv_bias, 3 * hl(), 0.f);
+        }
         if (BertParams.max_cache_len > 0) {
             const size_t ce = (size_t)BertParams.max_batch_size * heads() * BertParams.max_cache_len * BertParams.size_per_head;
             k_cache = dev_alloc<T>(ce);
@@ -276,8 +300,20 @@ class Bert_MHA {
         dev_fill_normal(k_bias, hl(), seed, base + 5, 0.f, 0.02f);
         dev_fill_normal(v_bias, hl(), seed, base + 6, 0.f, 0.02f);
         dev_fill_normal(w_bias, n, seed, base + 7, 0.f, 0.02f);
+        if (linear_qkv_col) {
+            linear_qkv_col->init_weights(seed, base + 20);
+            dev_fill_normal(qkv_bias, 3 * hl(), seed, base + 21, 0.f, 0.02f);
+        }
     }
     void params(const std::string& prefix, std::vector<ParamRef>& out) {
+        if (linear_qkv_col) {
+            // the packed projection replaces wq / wk / wv and their biases
+            out.push_back(linear_qkv_col->param(prefix + "wqkv"));
+            out.push_back({prefix + "bqkv", qkv_bias, 3 * hl(), 1, 3 * hl(), 0});
+            out.push_back(linear_w_row->param(prefix + "wo"));
+            out.push_back({prefix + "bo", w_bias, n, 1, n, 0});
+            return;
+        }
         out.push_back(linear_q_col->param(prefix + "wq"));
         out.push_back(linear_k_col->param(prefix + "wk"));
         out.push_back(linear_v_col->param(prefix + "wv"));
@@ -368,18 +404,30 @@ class Bert_MHA {
             return FuncWrapVec;
         }
 
-        // qkv linear  (bert_layer.h:128-135)
-        std::vector<FuncWrap> v = linear_q_col->forward(input, b.q, M); v[0].label = "q_gemm";
-        FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
-        v = linear_k_col->forward(input, b.k, M); v[0].label = "k_gemm";
-        FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
-        v = linear_v_col->forward(input, b.v, M); v[0].label = "v_gemm";
-        FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
-        // bias + transpose  (:139-142)
-        T *qbias = q_bias, *kbias = k_bias, *vbias = v_bias;
-        FuncWrapVec.push_back(FuncWrap(0.2f, COMPUTATION, [=](const DynamicInitParam& D) {
-            Add_QKV_bias_transpose<T>(b.q_buf, b.k_buf, b.v_buf, b.q, qbias, b.k, kbias, b.v, vbias, batch_size, seq_len, h, d, D);
-        }, "qkv_bias_transpose"));
+        std::vector<FuncWrap> v;
+        if (linear_qkv_col) {
+            // packed projection: QKV [M, 3, Hl] in the (contiguous) q, k, v slices, then the reference's fused
+            // bias + transpose kernel (attention_kernels.cuh:23-34)
+            v = linear_qkv_col->forward(input, b.q, M); v[0].label = "qkv_gemm";
+            FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
+            T* qkvb = qkv_bias;
+            FuncWrapVec.push_back(FuncWrap(0.2f, COMPUTATION, [=](const DynamicInitParam& D) {
+                Add_fusedQKV_bias_transpose_kernelLauncher<T>(b.q_buf, b.k_buf, b.v_buf, b.q, qkvb, batch_size, seq_len, h, d, D);
+            }, "fused_qkv_bias_transpose"));
+        } else {
+            // qkv linear  (bert_layer.h:128-135)
+            v = linear_q_col->forward(input, b.q, M); v[0].label = "q_gemm";
+            FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
+            v = linear_k_col->forward(input, b.k, M); v[0].label = "k_gemm";
+            FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
+            v = linear_v_col->forward(input, b.v, M); v[0].label = "v_gemm";
+            FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
+            // bias + transpose  (:139-142)
+            T *qbias = q_bias, *kbias = k_bias, *vbias = v_bias;
+            FuncWrapVec.push_back(FuncWrap(0.2f, COMPUTATION, [=](const DynamicInitParam& D) {
+                Add_QKV_bias_transpose<T>(b.q_buf, b.k_buf, b.v_buf, b.q, qbias, b.k, kbias, b.v, vbias, batch_size, seq_len, h, d, D);
+            }, "qkv_bias_transpose"));
+        }
         // qk  (:145-150)
         FuncWrapVec.push_back(FuncWrap(0.3f, COMPUTATION, [=](const DynamicInitParam& D) {
             GemmStridedBatchedEx(D, dt, 1, 0, seq_len, seq_len, d, b.k_buf, d, (long long)seq_len * d, b.q_buf, d,
@@ -494,9 +542,9 @@ class Bert_Encoder {
     }
     static int64_t workspace_elems(const BertInitParam& P, const StaticInitParam& S, int batch, int seq) {
         const int hidden = P.head_num * P.size_per_head;
-        const int F = (P.ffn_inner > 0 ? P.ffn_inner : 4 * hidden) / S.world_size;
         const int64_t M = (int64_t)batch * seq;
-        return Bert_MHA<T>::workspace_elems(P, S, batch, seq) + align_up(M * F) + 4 * align_up(M * hidden);
+        return Bert_MHA<T>::workspace_elems(P, S, batch, seq) + align_up(M * Bert_MLP<T>::inner_per_token(P, S, hidden)) +
+               4 * align_up(M * hidden);
     }
 
     // bert.h:59-79: MHA -> LN -> MLP -> LN (POST_NORESID).  PRE_LN_RESID chains layer_norm -> MHA ->
@@ -510,7 +558,7 @@ class Bert_Encoder {
         const int M = batch_size * seq;
         T* attn_ws = ws;
         T* mlp_inner = attn_ws + Bert_MHA<T>::workspace_elems(BertParam, SParam, batch_size, seq);
-        T* mha_out = mlp_inner + align_up((int64_t)M * MLP->f_local());
+        T* mha_out = mlp_inner + align_up((int64_t)M * Bert_MLP<T>::inner_per_token(BertParam, SParam, k));
         T* ln_mha_out = mha_out + align_up((int64_t)M * n);
         T* mlp_out = ln_mha_out + align_up((int64_t)M * n);
         T* pre_ln_out = mlp_out + align_up((int64_t)M * n);
@@ -574,8 +622,8 @@ class Bert_Model {
     // entries per layer of the vector forward() returns for this configuration
     int kernels_per_layer(bool decode = false) const {
         const bool fused = BertParams.fused && dtype_of<T>::value == LG_F16;
-        int mha = decode ? (BertParams.fused ? 5 : 6) : (fused ? 5 : 9);
-        int mlp = fused ? 2 : 3;
+        int mha = decode ? (BertParams.fused ? 5 : 6) : (fused ? 5 : (BertParams.packed_qkv ? 7 : 9));
+        int mlp = (fused && BertParams.ffn_act != FFN_GEGLU) ? 2 : 3;
         return mha + mlp + 2 + (BertParams.norm_mode == PRE_LN_RESID ? 1 : 0);
     }
 

@@ -85,6 +85,11 @@ int lg_layer_norm_f16(const void* in, const void* gamma, const void* beta, void*
 /* add_bias_act_kernelLauncher<T> (GELU-tanh, in place)   cuda_kernels.cuh:23-24, cuda_kernels.cu:302-319 */
 int lg_add_bias_act_f32(float* out, const float* bias, int m, int n, void* stream);
 int lg_add_bias_act_f16(void* out, const void* bias, int m, int n, void* stream);
+/* GeGLU, the FFN activation of the GLM family; no reference counterpart (the reference's MLP is bias + GELU only,
+ * bert_layer.h:43-62).  in [m, 2f] = [gate | up], bias [2f]; out [m, f] = gelu_tanh(gate + b) * (up + b).  out must not
+ * overlap in. */
+int lg_add_bias_geglu_f32(float* out, const float* in, const float* bias, int m, int f, void* stream);
+int lg_add_bias_geglu_f16(void* out, const void* in, const void* bias, int m, int f, void* stream);
 /* add_bias_input_layernorm_kernelLauncher<T> (in place on out)   cuda_kernels.cuh:26-30.
  * Unlike the reference (n <= 1024 / 2048) any n is accepted. */
 int lg_add_bias_input_layernorm_f32(float* out, const float* input, const float* bias, const float* gamma,

@@ -229,25 +229,41 @@ void lo_gemm_strided_batched(int transa, int transb, int m, int n, int k, const 
 /* ------------------------------------------------------------------------------------------ */
 /* bias + GELU   cuda_kernels.cu:9-29 (gelu), :59-84 (add_bias_gelu)                           */
 /* ------------------------------------------------------------------------------------------ */
+/* gelu(x + b) with the rounding points of the instantiation */
+static float bias_gelu_one(float v, float b, int dtype) {
+    if (dtype == LO_F32) {
+        /* float instantiation, :9-15 */
+        float x = v + b;
+        float cdf = 0.5f * (1.0f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
+        return x * cdf;
+    }
+    /* half2 specialisation, :17-29,:72-84: add in half, cube in half (two rounded products), tanh in fp32,
+     * cdf rounded to half, product in half */
+    float x = lo_round_f16(v + b);
+    float x2 = lo_round_f16(x * x);
+    float x3 = lo_round_f16(x * x2);
+    float cdf = 0.5f * (1.0f + tanhf(0.7978845608028654f * (x + 0.044715f * x3)));
+    return lo_round_f16(x * lo_round_f16(cdf));
+}
+
 void lo_add_bias_gelu(float* out, const float* bias, int m, int n, int dtype) {
 #pragma omp parallel for schedule(static)
     for (int i = 0; i < m; ++i) {
         float* row = out + (int64_t)i * n;
-        for (int j = 0; j < n; ++j) {
-            if (dtype == LO_F32) {
-                /* float instantiation, :9-15 */
-                float x = row[j] + bias[j];
-                float cdf = 0.5f * (1.0f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
-                row[j] = x * cdf;
-            } else {
-                /* half2 specialisation, :17-29,:72-84: add in half, cube in half (two rounded
-                 * products), tanh in fp32, cdf rounded to half, product in half */
-                float x = lo_round_f16(row[j] + bias[j]);
-                float x2 = lo_round_f16(x * x);
-                float x3 = lo_round_f16(x * x2);
-                float cdf = 0.5f * (1.0f + tanhf(0.7978845608028654f * (x + 0.044715f * x3)));
-                row[j] = lo_round_f16(x * lo_round_f16(cdf));
-            }
+        for (int j = 0; j < n; ++j) row[j] = bias_gelu_one(row[j], bias[j], dtype);
+    }
+}
+
+/* GeGLU (no reference counterpart; the FFN of the GLM family): in [m, 2f] = [gate | up], bias [2f];
+ * out[i][j] = gelu(gate + b_gate) * (up + b_up), every operation rounded like the kernels above. */
+void lo_add_bias_geglu(float* out, const float* in, const float* bias, int m, int f, int dtype) {
+#pragma omp parallel for schedule(static)
+    for (int i = 0; i < m; ++i) {
+        const float* row = in + (int64_t)i * 2 * f;
+        for (int j = 0; j < f; ++j) {
+            const float g = bias_gelu_one(row[j], bias[j], dtype);
+            const float u = st(row[f + j] + bias[f + j], dtype);
+            out[(int64_t)i * f + j] = st(g * u, dtype);
         }
     }
 }
@@ -530,8 +546,15 @@ int lo_mlp_forward(const lo_layer_shape* sh, const lo_layer_weights* w, const fl
     if (!shape_ok(sh)) return -1;
     const int M = sh->batch * sh->seq, H = sh->hidden, F = sh->ffn_inner, dt = sh->dtype;
     float* t = falloc((int64_t)M * F);
-    lo_gemm(M, F, H, in, w->w1, t, dt);   /* idx 11 */
-    lo_add_bias_gelu(t, w->b1, M, F, dt); /* idx 12 */
+    if (sh->ffn_act == LO_FFN_GEGLU) {
+        float* t2 = falloc((int64_t)M * 2 * F);
+        lo_gemm(M, 2 * F, H, in, w->w1, t2, dt);
+        lo_add_bias_geglu(t, t2, w->b1, M, F, dt);
+        free(t2);
+    } else {
+        lo_gemm(M, F, H, in, w->w1, t, dt);   /* idx 11 */
+        lo_add_bias_gelu(t, w->b1, M, F, dt); /* idx 12 */
+    }
     lo_gemm(M, H, F, t, w->w2, out, dt);  /* idx 13 */
     free(t);
     return 0;
@@ -599,8 +622,15 @@ int lo_decoder_step(const lo_layer_shape* sh, const lo_layer_weights* w, const f
     } else {
         lo_add_bias_input_layernorm_2(x, w->ln2_g, w->ln2_b, w->bo ? w->bo : zb, a, l, B, H, dt);
     }
-    lo_gemm(B, F, H, l, w->w1, t, dt);
-    lo_add_bias_gelu(t, w->b1, B, F, dt);
+    if (sh->ffn_act == LO_FFN_GEGLU) {
+        float* t2 = falloc((int64_t)B * 2 * F);
+        lo_gemm(B, 2 * F, H, l, w->w1, t2, dt);
+        lo_add_bias_geglu(t, t2, w->b1, B, F, dt);
+        free(t2);
+    } else {
+        lo_gemm(B, F, H, l, w->w1, t, dt);
+        lo_add_bias_gelu(t, w->b1, B, F, dt);
+    }
     lo_gemm(B, H, F, t, w->w2, m, dt);
     if (sh->norm_mode == LO_POST_NORESID) {
         lo_layer_norm(m, w->ln2_g, w->ln2_b, out, B, H, dt);

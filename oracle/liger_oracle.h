@@ -19,7 +19,7 @@
  *                                             and one-hot operands; numpy matmul
  *     layer_norm family                       closed forms (constant row -> beta, two-point
  *                                             row), shift invariance, torch layer_norm
- *     add_bias_gelu                           tabulated tanh-GELU points, torch gelu(tanh)
+ *     add_bias_gelu / add_bias_geglu          tabulated tanh-GELU points, torch gelu(tanh) (x up)
  *     attn_softmax                            row-sum identity, uniform rows, mask zeroing,
  *                                             shift invariance, torch softmax
  *     qkv bias+transpose / transpose          exhaustive index check, round trip
@@ -46,6 +46,10 @@ extern "C" {
 /* norm_mode of the encoder layer */
 #define LO_POST_NORESID 0 /* exactly what src/layer/bert.h:59-79 assembles */
 #define LO_PRE_LN_RESID 1 /* pre-LN layer built from the reference's fused residual kernels */
+
+/* ffn_act of the encoder layer */
+#define LO_FFN_GELU 0  /* bert_layer.h:43-45: FFN-1 -> bias + GELU -> FFN-2 */
+#define LO_FFN_GEGLU 1 /* w1 is [H, 2F] = [gate | up], b1 [2F]: gelu(gate) * up feeds FFN-2 */
 
 /* ---- scalar helpers ---------------------------------------------------------------- */
 float lo_round_f16(float x);            /* nearest-even round trip through binary16 */
@@ -82,6 +86,9 @@ void lo_gemm_strided_batched(int transa, int transb, int m, int n, int k, const 
 
 /* ---- element-wise / normalisation kernels (src/cuda/cuda_kernels.cu) ------------------ */
 void lo_add_bias_gelu(float* out, const float* bias, int m, int n, int dtype);       /* :9-29,59-84 */
+/* GeGLU, the FFN activation of the GLM family (no reference counterpart): in [m, 2f] = [gate | up], bias [2f],
+ * out [m, f] = gelu(gate + b) * (up + b) */
+void lo_add_bias_geglu(float* out, const float* in, const float* bias, int m, int f, int dtype);
 void lo_layer_norm(const float* in, const float* gamma, const float* beta, float* out, int m,
                    int n, int dtype);                                                 /* :463-508 */
 void lo_add_bias_input_layernorm(float* out, const float* input, const float* bias,
@@ -140,6 +147,7 @@ typedef struct lo_layer_shape {
     int causal;    /* 0: use `mask` ([B,S,S] 0/1) if non-NULL else all ones; 1: lower-triangular */
     int norm_mode; /* LO_POST_NORESID / LO_PRE_LN_RESID */
     int dtype;
+    int ffn_act;   /* LO_FFN_GELU / LO_FFN_GEGLU */
 } lo_layer_shape;
 
 /* One encoder layer.  in/out: [B*S, H].  mask may be NULL.  Returns 0 or -1 on bad shapes. */

@@ -29,7 +29,7 @@ class LayerWeightsC(C.Structure):
 class LayerShapeC(C.Structure):
     _fields_ = [(n, C.c_int) for n in (
         "batch", "seq", "hidden", "head_num", "size_per_head", "ffn_inner", "causal", "norm_mode",
-        "dtype")]
+        "dtype", "ffn_act")]
 
 
 def build(force=False):
@@ -61,6 +61,7 @@ def lib():
         "lo_gemm_ex": (None, [i, i, i, i, i, _fp, i, _fp, i, _fp, i, i]),
         "lo_gemm_strided_batched": (None, [i, i, i, i, i, _fp, i, i64, _fp, i, i64, _fp, i, i64, i, i]),
         "lo_add_bias_gelu": (None, [_fp, _fp, i, i, i]),
+        "lo_add_bias_geglu": (None, [_fp, _fp, _fp, i, i, i]),
         "lo_layer_norm": (None, [_fp, _fp, _fp, _fp, i, i, i]),
         "lo_add_bias_input_layernorm": (None, [_fp, _fp, _fp, _fp, _fp, i, i, i]),
         "lo_add_bias_input_layernorm_2": (None, [_fp, _fp, _fp, _fp, _fp, _fp, i, i, i]),
@@ -140,6 +141,14 @@ def gemm_strided_batched(transa, transb, m, n, k, A, lda, sA, B, ldb, sB, C_, ld
 def add_bias_gelu(out, bias, dtype=F32):
     m, n = out.shape
     lib().lo_add_bias_gelu(_p(out), _p(bias), m, n, dtype)
+    return out
+
+
+def add_bias_geglu(x2, bias, dtype=F32):
+    """x2: [m, 2f] = [gate | up]; returns gelu(gate + b) * (up + b) as [m, f]."""
+    m, f2 = x2.shape
+    out = np.empty((m, f2 // 2), dtype=np.float32)
+    lib().lo_add_bias_geglu(_p(out), _p(x2), _p(bias), m, f2 // 2, dtype)
     return out
 
 

@@ -173,6 +173,8 @@ int lg_layer_norm_f32(const float* in, const float* g, const float*, float* out,
 int lg_layer_norm_f16(const void* in, const void* g, const void*, void* out, int m, int n, void* stream) { return EW("layer_norm", m, n, 2, 2, in, g, out); }
 int lg_add_bias_act_f32(float* out, const float* b, int m, int n, void* stream) { return EW("add_bias_act", m, n, 4, 2, out, b, out); }
 int lg_add_bias_act_f16(void* out, const void* b, int m, int n, void* stream) { return EW("add_bias_act", m, n, 2, 2, out, b, out); }
+int lg_add_bias_geglu_f32(float* out, const float* in, const float* b, int m, int f, void* stream) { return EW("add_bias_geglu", m, f, 4, 3, in, b, out); }
+int lg_add_bias_geglu_f16(void* out, const void* in, const void* b, int m, int f, void* stream) { return EW("add_bias_geglu", m, f, 2, 3, in, b, out); }
 int lg_add_bias_input_layernorm_f32(float* out, const float* in, const float*, const float*, const float*, int m, int n, void* stream) { return EW("add_bias_input_layernorm", m, n, 4, 3, in, nullptr, out); }
 int lg_add_bias_input_layernorm_f16(void* out, const void* in, const void*, const void*, const void*, int m, int n, void* stream) { return EW("add_bias_input_layernorm", m, n, 2, 3, in, nullptr, out); }
 int lg_add_bias_input_layernorm_2_f32(const float* in, const float*, const float*, const float*, float* o, float* no, int m, int n, void* stream) { return EW("add_bias_input_layernorm_2", m, n, 4, 4, in, o, no); }

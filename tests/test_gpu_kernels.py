@@ -50,6 +50,17 @@ def test_add_bias_gelu(dev, po, dt, m, n):
 
 
 @pytest.mark.parametrize("dt", [0, 1])
+@pytest.mark.parametrize("m,f", [(64, 1024), (4, 16384), (3, 100), (5, 7), (0, 64)])
+def test_add_bias_geglu(dev, po, dt, m, f):
+    x2 = rnd(po, m * 2 * f, 9, dt, 2.0).reshape(m, 2 * f)
+    bias = rnd(po, 2 * f, 10, dt, 0.5)
+    out = dev.empty((m, f), dt)
+    dev.call("lg_add_bias_geglu_" + SUF[dt], out, dev.up(x2, dt), dev.up(bias, dt), m, f)
+    if m:
+        assert max_rel_err(dev.down(out), po.add_bias_geglu(x2, bias, dt)) < (2e-5 if dt == 0 else 4e-3)
+
+
+@pytest.mark.parametrize("dt", [0, 1])
 @pytest.mark.parametrize("m,n", [(16, 256), (4, 12288), (3, 1001)])
 def test_add_bias_input_layernorm_family(dev, po, dt, m, n):
     out0 = rnd(po, m * n, 6, dt).reshape(m, n)

@@ -19,14 +19,22 @@ def host(liger):
 
 
 def oracle_weights(params, layer=0):
+    """Weights of one layer under the oracle's names; a packed QKV projection is split into its three column blocks."""
     pre = "layer%d." % layer
-    return {k[len(pre):]: v for k, v in params.items() if k.startswith(pre)}
+    w = {k[len(pre):]: v for k, v in params.items() if k.startswith(pre)}
+    if "wqkv" in w:
+        hl = w["wqkv"].shape[1] // 3
+        for i, n in enumerate("qkv"):
+            w["w" + n] = np.ascontiguousarray(w["wqkv"][:, i * hl:(i + 1) * hl])
+            w["b" + n] = np.ascontiguousarray(w["bqkv"][i * hl:(i + 1) * hl])
+    return w
 
 
-def run_layer_case(dev, po, host, dtype, B, S, heads, d, F, norm_mode, causal, fused, ws=1, layers=1, seed=0, weight_layout=0):
+def run_layer_case(dev, po, host, dtype, B, S, heads, d, F, norm_mode, causal, fused, ws=1, layers=1, seed=0, weight_layout=0,
+                   ffn_act=0, packed_qkv=False):
     H = heads * d
     m = host.Model(dtype, B, S, heads, d, layer_num=layers, world_size=ws, ffn_inner=F, norm_mode=norm_mode, causal=causal,
-                   fused=fused, weight_layout=weight_layout, seed=seed)
+                   fused=fused, weight_layout=weight_layout, seed=seed, ffn_act=ffn_act, packed_qkv=packed_qkv)
     params = m.download_params()
     x = po.fill_normal(B * S * H, seed, 99, 0.0, 1.0, dtype).reshape(B * S, H)
     dx = dev.up(x, dtype)
@@ -34,7 +42,7 @@ def run_layer_case(dev, po, host, dtype, B, S, heads, d, F, norm_mode, causal, f
     m.run(dx.data_ptr(), dy.data_ptr(), B, S, None, dev.stream)
     got = dev.down(dy)
     shape = dict(batch=B, seq=S, hidden=H, head_num=heads // ws, size_per_head=d, ffn_inner=(F or 4 * H) // ws,
-                 causal=int(causal), norm_mode=norm_mode, dtype=dtype)
+                 causal=int(causal), norm_mode=norm_mode, dtype=dtype, ffn_act=ffn_act)
     ref = x
     for l in range(layers):
         ref = po.encoder_forward(shape, oracle_weights(params, l), ref)
@@ -108,3 +116,24 @@ def test_decode_step_matches_oracle(dev, po, host):
         got = dev.down(dt_out)
         assert max_rel_err(got, ref) < 1e-2
         tok = po.round_f16(ref)
+
+
+@pytest.mark.parametrize("dtype,fused", [(0, False), (1, False), (1, True)])
+@pytest.mark.parametrize("norm_mode", [0, 1])
+def test_geglu_layer(dev, po, host, dtype, fused, norm_mode):
+    """GeGLU FFN (FFN-1 [H, 2F] = [gate | up] -> gelu(gate) * up -> FFN-2) behind the same launch vector."""
+    got, ref, m = run_layer_case(dev, po, host, dtype, 2, 96, 4, 64, 512, norm_mode, True, fused, ffn_act=1)
+    assert "bias+geglu" in [e["label"] for e in m.describe(2, 96)]
+    assert max_rel_err(got, ref) < (2e-5 if dtype == 0 else 1e-2)
+
+
+@pytest.mark.parametrize("dtype", [0, 1])
+@pytest.mark.parametrize("weight_layout", [0, 1])
+def test_packed_qkv_layer(dev, po, host, dtype, weight_layout):
+    """One [H, 3 Hl] projection + the reference's fused bias/transpose kernel instead of three GEMMs: 12 entries, same
+    result as the oracle run with the three column blocks of the packed weight."""
+    got, ref, m = run_layer_case(dev, po, host, dtype, 2, 80, 4, 64, 512, 0, True, False, ws=2, weight_layout=weight_layout,
+                                 packed_qkv=True)
+    labels = [e["label"] for e in m.describe(2, 80)]
+    assert labels[:2] == ["qkv_gemm", "fused_qkv_bias_transpose"] and m.kernels_per_layer() == 12
+    assert max_rel_err(got, ref) < (2e-5 if dtype == 0 else 1e-2)

@@ -120,6 +120,50 @@ def test_bias_gelu_tabulated_and_torch(po):
     assert np.abs(po.add_bias_gelu(xh.copy(), bh, 1) - th).max() < 8e-3
 
 
+def test_bias_geglu_composes_from_gelu_and_matches_torch(po):
+    """GeGLU = gelu(gate + b) * (up + b): closed forms (gate 0 -> 0; a large positive gate passes the up branch through
+    scaled by the gate), the exact composition from the pinned bias + GELU function, and torch."""
+    rng = np.random.default_rng(9)
+    m, f = 7, 24
+    x2 = rng.standard_normal((m, 2 * f)).astype(np.float32) * 2
+    bias = rng.standard_normal(2 * f).astype(np.float32) * 0.5
+    got = po.add_bias_geglu(x2, bias, 0)
+    t = torch.from_numpy(x2 + bias)
+    ref = (torch.nn.functional.gelu(t[:, :f], approximate="tanh") * t[:, f:]).numpy()
+    assert np.abs(got - ref).max() < 2e-6
+    # closed forms: zero gate, and gate = 10 (gelu(10) = 10 to fp32 precision) with zero bias
+    z = np.zeros((2, 8), np.float32); z[:, 4:] = 3.0
+    assert np.all(po.add_bias_geglu(z, np.zeros(8, np.float32), 0) == 0)
+    z[:, :4] = 10.0
+    assert np.allclose(po.add_bias_geglu(z, np.zeros(8, np.float32), 0), 30.0, rtol=1e-6)
+    # swapping the halves is not symmetric: the activation sits on the FIRST half
+    sw = np.concatenate([x2[:, f:], x2[:, :f]], axis=1)
+    assert np.abs(po.add_bias_geglu(sw, np.concatenate([bias[f:], bias[:f]]), 0) - got).max() > 1e-2
+    # fp16 semantics: every operation rounded; composes exactly from the bias + GELU kernel and two fp16 roundings
+    x16, b16 = po.round_f16(x2), po.round_f16(bias)
+    g = po.add_bias_gelu(x16[:, :f].copy(), b16[:f].copy(), 1)
+    u = po.round_f16(x16[:, f:] + b16[f:])
+    assert np.array_equal(po.add_bias_geglu(x16, b16, 1), po.round_f16(g * u))
+
+
+def test_geglu_mlp_is_the_composition_of_its_kernels(po):
+    """lo_mlp_forward with ffn_act = GeGLU: FFN-1 [H, 2F] -> bias + GeGLU -> FFN-2."""
+    rng = np.random.default_rng(10)
+    B, S, H, F = 2, 5, 16, 24
+    x = rng.standard_normal((B * S, H)).astype(np.float32)
+    w = {"w1": (rng.standard_normal((H, 2 * F)) * 0.2).astype(np.float32), "b1": (rng.standard_normal(2 * F) * 0.1).astype(np.float32),
+         "w2": (rng.standard_normal((F, H)) * 0.2).astype(np.float32)}
+    for dt in (0, 1):
+        xx = po.round_f16(x) if dt else x
+        ww = {k: (po.round_f16(v) if dt else v) for k, v in w.items()}
+        shape = dict(batch=B, seq=S, hidden=H, head_num=2, size_per_head=8, ffn_inner=F, causal=0, norm_mode=0, dtype=dt, ffn_act=1)
+        got = po.mlp_forward(shape, ww, xx)
+        ref = po.gemm(po.add_bias_geglu(po.gemm(xx, ww["w1"], dt), ww["b1"], dt), ww["w2"], dt)
+        assert np.array_equal(got, ref)
+        plain = po.mlp_forward(dict(shape, ffn_act=0), {"w1": ww["w1"][:, :F].copy(), "b1": ww["b1"][:F].copy(), "w2": ww["w2"]}, xx)
+        assert np.abs(plain - got).max() > 1e-3   # a different function from the GELU MLP on the gate half alone
+
+
 def test_softmax_identities_and_torch(po):
     B, h, S = 2, 3, 16
     scalar = 0.125

@@ -30,6 +30,13 @@ def small_model(host, fused=True, factor=4, layers=1, max_batch=4, cache=128):
                       max_cache_len=cache if fused else 0, factor=factor, seed=0)
 
 
+def fake_trace_of(fake, model, batch, seq):
+    """Launch records of one plain run of the model on the virtual-time backend."""
+    fake.reset()
+    model.run(0x10000, 0x20000000, batch, seq)   # the backend never dereferences "device" pointers
+    return fake.trace()
+
+
 def test_launch_vector_shapes_and_order(fake):
     host = fake.host
     m = small_model(host, fused=False, cache=0)
@@ -42,6 +49,15 @@ def test_launch_vector_shapes_and_order(fake):
     mf = small_model(host, fused=True)
     assert mf.kernels_per_layer() == 9 and mf.kernels_per_layer(decode=True) == 9   # K/V rows are appended by the GEMM epilogues
     assert all(e["class"] == "HBM_BOUND" for e in mf.describe(2, 1, decode_past=10))
+    mg = host.Model(1, 2, 32, 4, 64, ffn_inner=512, fused=True, ffn_act=host.FFN_GEGLU)
+    assert [e["label"] for e in mg.describe(2, 32)][-4:] == ["ffn1(gate+up)", "bias+geglu", "ffn2", "layer_norm"]
+    gate_up = [e for e in fake_trace_of(fake, mg, 2, 32) if e["name"].startswith("gemm")][-2]
+    assert (gate_up["m"], gate_up["n"], gate_up["k"]) == (1024, 64, 256)      # FFN-1 produces 2 F columns
+    mp = host.Model(0, 2, 32, 4, 64, packed_qkv=True)
+    assert [e["label"] for e in mp.describe(2, 32)][:3] == ["qkv_gemm", "fused_qkv_bias_transpose", "qk_gemm"]
+    assert mp.kernels_per_layer() == 12
+    with pytest.raises(host.capi.LigerError):
+        host.Model(1, 2, 32, 4, 64, fused=True, packed_qkv=True)   # packed QKV belongs to the reference-shaped assembly
     m2 = host.Model(0, 2, 32, 4, 64, layer_num=3, norm_mode=host.PRE_LN_RESID)
     assert len(m2.describe(2, 32)) == 3 * 15
     with pytest.raises(host.capi.LigerError):
