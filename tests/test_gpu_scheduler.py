@@ -91,3 +91,20 @@ def test_measured_contention_on_gpu(dev, host):
     trace = [{"arrival_s": 0.001 * i, "batch": 1, "seq": 64 + 32 * (i % 3), "n_decode": 4} for i in range(10)]
     rr = s.run_trace(trace, host.MODE_LIGER)
     assert rr["records"] == 10 and rr["profile_misses"] == 0
+
+
+def test_command_line_driver_runs_both_modes(tmp_path):
+    """The C++ driver (counterpart of the reference's main.cu): profile, serve the reference's own request generator with
+    interleaving and without, print the report.  Run as a child process in a scratch directory (it writes the two
+    profile JSON files there under the reference's file-name convention)."""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "24ppopp-liger_amd", "lib", "liger_main")
+    assert os.path.exists(exe), "liger_main is not built; run __graft_entry__.build()"
+    #            max_batch max_seq heads d layers factor rate world requests
+    args = [exe, "2", "64", "8", "128", "1", "4", "400", "1", "30"]
+    r = subprocess.run(args, cwd=str(tmp_path), capture_output=True, text=True, timeout=240)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert "---- run_stream_sync ----" in r.stdout and "---- run_sequential ----" in r.stdout
+    assert r.stdout.count("Average Latency") == 2 and r.stdout.count("Throughput") == 2
+    assert os.path.exists(tmp_path / "Main_1_128_8_2_64.json") and os.path.exists(tmp_path / "Sub_1_128_8_2_64.json")
