@@ -3,14 +3,16 @@
 //   Y[M, N] = X[M, K] * W^T with W stored [N, K] (both operands K-contiguous), M <= 64.
 // With a handful of token rows every weight byte is used for 2*M flops only, so the kernel is a pure HBM stream of W
 // (1.4 GB per GLM-130B TP=2 layer shard) and is organised like one:
-//   * a block = 4 waves x 32 output features; the grid is (N / 128) x S with S K-slices chosen so that >= ~1000 blocks
-//     keep >= 16 waves per CU streaming;
+//   * as few blocks as fill the chip (one block of 4 waves keeps 64 KiB of weight loads in flight, enough for one CU; more
+//     blocks mean more K-slices, fp32 partials and reduce work).  If N alone gives >= 192 blocks of 64 (or 32) features, a
+//     block walks the whole of K and applies the epilogue itself; otherwise a block = 4 waves x 32 features, the grid is
+//     (N / 128) x S with the fewest K-slices S that give >= 192 blocks, and a second kernel sums the slices;
 //   * W fragments go from global memory straight into MFMA operand registers (a lane owns 8 consecutive k of one output
 //     feature: exactly the B operand of v_mfma_f32_16x16x32_f16) in a rolling pipeline that keeps 16 independent
 //     16-byte loads in flight per lane at all times;
 //   * the few X rows are staged once per 256-wide k-chunk in LDS (double buffered) and shared by the block's waves;
-//   * K-slices are summed in fp32 through a per-stream workspace and a small second kernel that also applies the
-//     epilogue (bias / GELU / head-transposed store), so results match the single-pass kernels' rounding.
+//   * K-slices (when there are any) are summed in fp32 through a per-stream workspace and a small second kernel that also
+//     applies the epilogue (bias / GELU / head-transposed store), so results match the single-pass kernels' rounding.
 #include <mutex>
 #include <unordered_map>
 
@@ -32,6 +34,11 @@ __global__ __launch_bounds__(256) void gemm_skinny_nk_kernel(GemmArgs g, int ksl
     const int split = blockIdx.y;
     const int k_begin = split * kslice;
     const int nchunks = (min(g.K, k_begin + kslice) - k_begin) / SK_KC;  // whole chunks only
+    // Blocks walk their chunks in rotated order (block b starts at chunk b mod nchunks and wraps around): with a
+    // power-of-two row pitch (K = 16384) the blocks of a K-slice, which run in step, would otherwise all touch the same
+    // memory channels at the same time (12288 x 16384 weight, 32 token rows: 97 -> 84 us).
+    const int rot = blockIdx.x % nchunks;
+    auto chunk_at = [&](int i) { const int c = rot + i; return c >= nchunks ? c - nchunks : c; };
 
     // The loop below is branch-free (the launcher guarantees K-slices made of whole 256-wide chunks): rows beyond M are
     // read from row M-1 (they only feed accumulator rows that are never stored) and the chunk after the last one is the
@@ -72,17 +79,17 @@ __global__ __launch_bounds__(256) void gemm_skinny_nk_kernel(GemmArgs g, int ksl
     // time.  The next X chunk is fetched at the start of a chunk (it queues behind weight loads that are consumed during
     // the chunk anyway) and written to the other LDS buffer at its end.
     half8_t b0[8], b1[8], xr[XV];
-    load_x(0, xr);
+    load_x(rot, xr);
     store_x(0, xr);
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
-        b0[s] = *reinterpret_cast<const half8_t*>(w0 + s * 32);
-        b1[s] = *reinterpret_cast<const half8_t*>(w1 + s * 32);
+        b0[s] = *reinterpret_cast<const half8_t*>(w0 + rot * SK_KC + s * 32);
+        b1[s] = *reinterpret_cast<const half8_t*>(w1 + rot * SK_KC + s * 32);
     }
     __syncthreads();
     for (int ch = 0; ch < nchunks; ++ch) {
         const int buf = ch & 1;
-        const int next = min(ch + 1, nchunks - 1);
+        const int next = chunk_at(ch + 1 < nchunks ? ch + 1 : ch);
         load_x(next, xr);
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
@@ -116,6 +123,119 @@ __global__ __launch_bounds__(256) void gemm_skinny_nk_kernel(GemmArgs g, int ksl
             }
         }
     (void)nsplit;
+}
+
+// ---- whole K in one block ------------------------------------------------------------------------------------------------
+// When N alone gives enough blocks K is not sliced at all: a block = NWV waves x 16 output features walks the whole of K, the
+// epilogue is applied to the accumulators, and there are no fp32 partials and no second kernel.  A wave owns one 16-feature
+// MFMA tile (8 loads per chunk), so its rolling pipeline is DEPTH chunks deep: 4 waves x 2 chunks or 2 waves x 4 chunks
+// keep the same 64 KiB of weight loads in flight per block.
+template <int MT, int EPI, int NWV, int DEPTH>
+__global__ __launch_bounds__(64 * NWV) void gemm_skinny_direct_kernel(GemmArgs g) {
+    constexpr int THREADS = 64 * NWV;
+    __shared__ __attribute__((aligned(16))) half_t xs[2][16 * MT * SK_XS];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l16 = lane & 15, lk = lane >> 4;
+    const int n0 = blockIdx.x * (16 * NWV) + wave * 16;
+    const int nchunks = g.K / SK_KC;  // a multiple of DEPTH (the launcher checks)
+    const int rot = blockIdx.x % nchunks;  // rotated chunk order, see gemm_skinny_nk_kernel
+    auto chunk_at = [&](int i) { int c = rot + i; while (c >= nchunks) c -= nchunks; return c; };
+
+    constexpr int XV = 16 * MT * (SK_KC / 8) / THREADS;
+    const half_t* xsrc[XV];
+#pragma unroll
+    for (int u = 0; u < XV; ++u) {
+        const int v = tid + u * THREADS;
+        const int row = min(v / (SK_KC / 8), g.M - 1), c = v % (SK_KC / 8);
+        xsrc[u] = g.X + (int64_t)row * g.ldx + c * 8;
+    }
+    auto load_x = [&](int chunk, half8_t (&xr)[XV]) {
+#pragma unroll
+        for (int u = 0; u < XV; ++u) xr[u] = *reinterpret_cast<const half8_t*>(xsrc[u] + chunk * SK_KC);
+    };
+    auto store_x = [&](int buf, const half8_t (&xr)[XV]) {
+#pragma unroll
+        for (int u = 0; u < XV; ++u) {
+            const int v = tid + u * THREADS;
+            const int row = v / (SK_KC / 8), c = v % (SK_KC / 8);
+            *reinterpret_cast<half8_t*>(&xs[buf][row * SK_XS + c * 8]) = xr[u];
+        }
+    };
+
+    float4_t acc[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) acc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    const half_t* w0 = g.W + (int64_t)min(n0 + l16, g.N - 1) * g.ldw + lk * 8;  // rows beyond N are clamped, never stored
+
+    // bf[d]: the weight fragments of chunks d, d + DEPTH, ...; xq[p]: token rows on their way to LDS, fetched two chunks
+    // ahead (loads complete in order: waiting for rows fetched only one chunk ahead would also wait for all but the last 8
+    // weight loads, i.e. drain the pipeline at every chunk)
+    half8_t bf[DEPTH][8], xq[2][XV];
+    // the prologue issues its loads in the order the loop would have (W(c) DEPTH chunks and X(c) two chunks before chunk c),
+    // so that the compiler's count of outstanding loads at the loop head is exact
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+        if (d == DEPTH - 2) load_x(chunk_at(0), xq[0]);
+        if (d == DEPTH - 1) load_x(chunk_at(1), xq[1]);
+#pragma unroll
+        for (int s = 0; s < 8; ++s) bf[d][s] = *reinterpret_cast<const half8_t*>(w0 + chunk_at(d) * SK_KC + s * 32);
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    store_x(0, xq[0]);
+    __syncthreads();
+    // one chunk: multiply its 8 fragments (registers b) with the X chunk in LDS buffer `buf`, reloading each fragment's
+    // registers with the chunk DEPTH ahead as soon as it has been used; at its end the X chunk fetched one chunk ago goes
+    // to the other LDS buffer.  Chunks past the
+    // end wrap around to valid addresses and are never multiplied.
+    auto do_chunk = [&](int ch, int buf, half8_t (&b)[8]) {
+        load_x(chunk_at(ch + 2), xq[buf]);
+        const half_t* wn = w0 + chunk_at(ch + DEPTH) * SK_KC;
+        // compiler-only fences keep every load where it is written (left alone, the compiler moves the X loads to the end
+        // of the chunk, right in front of the LDS stores that wait for them)
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+                const half8_t a = *reinterpret_cast<const half8_t*>(&xs[buf][(i * 16 + l16) * SK_XS + s * 32 + lk * 8]);
+                acc[i] = mfma16(b[s], a, acc[i]);  // operands swapped: acc[i][r] = Y[16 i + l16][n0 + 4 lk + r]
+            }
+            b[s] = *reinterpret_cast<const half8_t*>(wn + s * 32);
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        store_x(buf ^ 1, xq[buf ^ 1]);
+        __syncthreads();
+    };
+    for (int ch = 0; ch < nchunks; ch += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) do_chunk(ch + d, d & 1, bf[d]);
+    }
+#pragma unroll
+    for (int i = 0; i < MT; ++i) epilogue_store4<EPI>(g, g.Y, i * 16 + l16, n0 + 4 * lk, acc[i], true);
+}
+
+template <int MT, int NWV, int DEPTH>
+static void launch_direct(const GemmArgs& g, hipStream_t stream) {
+    const dim3 grid((g.N + 16 * NWV - 1) / (16 * NWV)), block(64 * NWV);
+    switch (g.epi.kind) {
+        case LG_EPI_NONE: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_NONE, NWV, DEPTH>), grid, block, 0, stream, g); break;
+        case LG_EPI_BIAS: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_BIAS, NWV, DEPTH>), grid, block, 0, stream, g); break;
+        case LG_EPI_BIAS_GELU: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_BIAS_GELU, NWV, DEPTH>), grid, block, 0, stream, g); break;
+        default: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_BIAS_HEADS, NWV, DEPTH>), grid, block, 0, stream, g); break;
+    }
+}
+template <int NWV, int DEPTH>
+static void launch_direct_mt(const GemmArgs& g, hipStream_t stream) {
+    switch ((g.M + 15) / 16) {
+        case 1: launch_direct<1, NWV, DEPTH>(g, stream); break;
+        case 2: launch_direct<2, NWV, DEPTH>(g, stream); break;
+        case 3: launch_direct<3, NWV, DEPTH>(g, stream); break;
+        default: launch_direct<4, NWV, DEPTH>(g, stream); break;
+    }
 }
 
 // sums the K-slices and applies the epilogue; one thread per 4 consecutive output columns
@@ -176,10 +296,25 @@ int launch_gemm_skinny_f16(const GemmArgs& g, int wlayout, int batch, hipStream_
     if (g.M <= 0 || g.M > 64 || g.N < 512 || g.K < 1024 || (g.K % SK_KC) || (g.N % 4)) return LG_OK;
     if (!aligned16(g.X) || !aligned16(g.W) || !aligned16(g.Y) || (g.ldx % 8) || (g.ldw % 8)) return LG_OK;
     if (g.epi.kind == LG_EPI_BIAS_HEADS ? (g.epi.d % 4 != 0) : (g.ldy % 4 != 0)) return LG_OK;
+    const int mt = (g.M + 15) / 16;
+    // Enough blocks without slicing K (>= 192: see below)?  64 features per block, or 32 for up to 16 token rows (with more
+    // rows the 2-wave block's registers no longer hold its four-chunk pipeline).
+    if ((g.N + 63) / 64 >= 192 && g.K % (2 * SK_KC) == 0) {
+        *handled = true;
+        launch_direct_mt<4, 2>(g, stream);
+        return check_launch("gemm_f16_skinny");
+    }
+    if (mt == 1 && (g.N + 31) / 32 >= 192 && g.K % (4 * SK_KC) == 0) {
+        *handled = true;
+        launch_direct<1, 2, 4>(g, stream);
+        return check_launch("gemm_f16_skinny");
+    }
     const int nblk = (g.N + SK_BN - 1) / SK_BN;
-    // K-slices: enough blocks for ~4 per CU, slices are multiples of the 256-wide chunk
+    // K-slices: as few as fill the chip.  One block of 4 waves keeps 64 KiB of weight loads in flight, which is enough for one
+    // CU; more slices only add fp32 partials and reduce work (six GEMMs of a decode step at 32 token rows: 344 us with >= 1024
+    // blocks, 315 us with >= 256, 289 us with >= 192, 336 us with >= 128).  Slices are multiples of the 256-wide chunk.
     int nsplit = 1;
-    while (nblk * nsplit < 1024 && (g.K / (nsplit * 2)) >= 2 * SK_KC && nsplit < 32) nsplit *= 2;
+    while (nblk * nsplit < 192 && (g.K / (nsplit * 2)) >= 2 * SK_KC && nsplit < 32) nsplit *= 2;
     int kslice = ((g.K + nsplit - 1) / nsplit + SK_KC - 1) / SK_KC * SK_KC;
     nsplit = (g.K + kslice - 1) / kslice;
     const size_t bytes = (size_t)nsplit * g.M * g.N * sizeof(float);
@@ -187,7 +322,6 @@ int launch_gemm_skinny_f16(const GemmArgs& g, int wlayout, int batch, hipStream_
     if (!ws) { set_error("gemm_skinny: cannot allocate the %zu-byte split-K workspace", bytes); *handled = true; return LG_ERR_LAUNCH; }
     *handled = true;
     const dim3 grid(nblk, nsplit), block(256);
-    const int mt = (g.M + 15) / 16;
     switch (mt) {
         case 1: hipLaunchKernelGGL((gemm_skinny_nk_kernel<1>), grid, block, 0, stream, g, kslice, ws, nsplit); break;
         case 2: hipLaunchKernelGGL((gemm_skinny_nk_kernel<2>), grid, block, 0, stream, g, kslice, ws, nsplit); break;

@@ -23,6 +23,9 @@ SHAPES = [(64, 256, 256), (128, 128, 32), (130, 136, 72), (1, 8, 8), (33, 70, 19
           (320, 256, 128), (448, 384, 192), (1000, 512, 256), (200, 256, 64), (161, 768, 128), (65, 256, 192), (100, 384, 64),
           # few tokens, many features: the weight-streaming split-K kernel (weights stored [out, in])
           (32, 1024, 2048), (1, 512, 1024), (17, 640, 4104), (64, 2048, 1536), (33, 516, 1032),
+          # ... and enough features for unsliced blocks: 64 features per block (any M <= 64, K % 512 == 0), 32 per block
+          # (M <= 16, K % 1024 == 0); N not a multiple of the block width
+          (32, 12288, 1024), (48, 12292, 1536), (64, 12352, 512), (5, 12288, 512), (9, 6148, 2048), (16, 6144, 1024),
           # one to four token rows and K a multiple of 2048: the matrix-vector kernel (weights stored [out, in])
           (1, 512, 2048), (2, 1024, 4096), (3, 256, 2048), (4, 644, 6144), (1, 6144, 12288)]
 
@@ -179,3 +182,32 @@ def test_gemm_fused_epilogues_on_the_matrix_vector_kernel(dev, po, M):
     got = dev.down(out)
     assert max_rel_err(got[:, :, :1], ref_heads) < 2e-3
     assert np.all(got[:, :, 1:] == 0)
+
+
+@pytest.mark.parametrize("M,h", [(8, 96), (32, 96), (40, 16), (12, 48)])
+def test_gemm_fused_epilogues_on_the_weight_streaming_kernels(dev, po, M, h):
+    """5..64 token rows, weights [out, in]: h = 96 takes the blocks that walk the whole of K and apply the epilogue
+    themselves (64 features per block), h = 48 with <= 16 rows the 32-feature blocks, h = 16 the K-sliced kernel whose
+    second kernel applies it."""
+    d, K = 128, 1024
+    N = h * d
+    X = rnd(po, M * K, 46, 1).reshape(M, K)
+    W = rnd(po, K * N, 47, 1, 0.05).reshape(K, N)
+    bias = rnd(po, N, 48, 1, 0.3)
+    dA, dX, dB = dev.up(np.ascontiguousarray(W.T), 1), dev.up(X, 1), dev.up(bias, 1)
+    y = po.gemm(X, W, 1)
+    out = dev.empty((M, N), 1)
+    dev.call("lg_gemm_fused_f16", 1, N, M, K, dA, K, dX, K, out, N, dev.capi.EPI_BIAS_GELU, dB, 0, 0, 0)
+    assert max_rel_err(dev.down(out), po.add_bias_gelu(y.copy(), bias, 1)) < 4e-3
+    out = dev.empty((M, N), 1)
+    dev.call("lg_gemm_fused_f16", 1, N, M, K, dA, K, dX, K, out, N, dev.capi.EPI_BIAS, dB, 0, 0, 0)
+    assert max_rel_err(dev.down(out), po.round_f16(y + bias)) < 2e-3
+    # one token per sequence (batch = M, seq = 1) written to row 2 of a [M, h, rows, d] destination (a KV cache)
+    ref_heads, _, _ = po.add_qkv_bias_transpose(y, bias, y, bias, y, bias, M, 1, h, d, 1)
+    rows = 4
+    out = dev.empty((M, h, rows, d), 1)
+    out.zero_()
+    dev.call("lg_gemm_fused_f16", 1, N, M, K, dA, K, dX, K, out.data_ptr() + 2 * d * 2, rows, dev.capi.EPI_BIAS_HEADS, dB, 1, d, h)
+    got = dev.down(out)
+    assert max_rel_err(got[:, :, 2:3], ref_heads) < 2e-3
+    assert np.all(got[:, :, :2] == 0) and np.all(got[:, :, 3:] == 0)
