@@ -10,8 +10,8 @@
 namespace lg {
 
 int launch_gemm_fast_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t stream, bool* handled);
-int launch_gemm_skinny_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t stream, bool* handled);
-int launch_gemv_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t stream, bool* handled);
+int launch_gemm_skinny_f16(const GemmArgs& g, const GemmGroup& grp, int wlayout, int batch, hipStream_t stream, bool* handled);
+int launch_gemv_f16(const GemmArgs& g, const GemmGroup& grp, int wlayout, int batch, hipStream_t stream, bool* handled);
 
 // ---------------------------------------------------------------------------------------------------
 // fp16 generic kernel
@@ -149,9 +149,10 @@ static int gemm_f16_dispatch(GemmArgs g, int wlayout, int batch, hipStream_t str
     bool handled = false;
     int rc = launch_gemm_fast_f16(g, wlayout, batch, stream, &handled);
     if (handled) return rc;
-    rc = launch_gemv_f16(g, wlayout, batch, stream, &handled);
+    const GemmGroup one = single_group(g);
+    rc = launch_gemv_f16(g, one, wlayout, batch, stream, &handled);
     if (handled) return rc;
-    rc = launch_gemm_skinny_f16(g, wlayout, batch, stream, &handled);
+    rc = launch_gemm_skinny_f16(g, one, wlayout, batch, stream, &handled);
     if (handled) return rc;
     const bool aligned = aligned16(g.X) && aligned16(g.W) && aligned16(g.Y) && (g.ldx % 8 == 0) && (g.ldw % 8 == 0) &&
                          (g.strideX % 8 == 0) && (g.strideW % 8 == 0) && (g.strideY % 4 == 0) &&
@@ -305,6 +306,62 @@ int lg_gemm_fused_f16(int transa, int m, int n, int k, const void* A, int lda, c
     g.Y = (half_t*)C; g.ldy = ldc; g.strideY = 0;
     g.epi = Epilogue{epilogue, (const half_t*)bias, epi_arg0, epi_arg1, epi_arg2};
     return gemm_f16_dispatch(g, transa ? W_NK : W_KN, 1, (hipStream_t)stream);
+}
+
+int lg_gemm_fused_grouped_f16(int transa, int m, int n, int k, int count, const void* const* A, int lda, const void* B, int ldb,
+                              void* const* C, const int* ldc, int epilogue, const void* const* bias, int epi_arg0, int epi_arg1,
+                              int epi_arg2, void* stream) {
+    if (count < 1 || count > LG_MAX_GROUP || !A || !C || !ldc || (epilogue != LG_EPI_NONE && !bias)) {
+        set_error("gemm_fused_grouped_f16: count must be 1..%d and the pointer arrays non-null", LG_MAX_GROUP);
+        return LG_ERR_INVALID;
+    }
+    // the weight-streaming kernels run the whole group as one launch; every other case is `count` plain calls
+    GemmGroup grp{};
+    grp.count = count;
+    bool one_launch = transa == 1 && m > 0 && n > 0 && k > 0 && count > 1 && B != nullptr;
+    for (int i = 0; i < count; ++i) {
+        grp.W[i] = (const half_t*)A[i];
+        grp.Y[i] = (half_t*)C[i];
+        grp.bias[i] = epilogue != LG_EPI_NONE ? (const half_t*)bias[i] : nullptr;
+        grp.ldy[i] = ldc[i];
+        if (!A[i] || !C[i] || (epilogue != LG_EPI_NONE && !bias[i])) one_launch = false;  // the plain call reports it
+    }
+    if (one_launch) {
+        // same argument checks as the plain entry, member by member, before anything is launched
+        for (int i = 0; i < count; ++i) {
+            int rc = check_blas_args("gemm_fused_grouped_f16", transa, 0, m, n, k, A[i], lda, B, ldb, C[i],
+                                     epilogue == LG_EPI_BIAS_HEADS ? (m > 1 ? m : 1) : ldc[i], 1);
+            if (rc) return rc;
+        }
+        if (epilogue < LG_EPI_NONE || epilogue > LG_EPI_BIAS_HEADS) { set_error("gemm_fused_grouped_f16: unknown epilogue %d", epilogue); return LG_ERR_INVALID; }
+        int heads_total = epi_arg2;
+        bool ok = true;
+        if (epilogue == LG_EPI_BIAS_HEADS) {
+            const int seq = epi_arg0, d = epi_arg1;
+            ok = seq > 0 && d > 0 && m % d == 0 && n % seq == 0 && d % 4 == 0 && (epi_arg2 == 0 || epi_arg2 >= m / d);
+            for (int i = 0; i < count && ok; ++i) ok = ldc[i] >= seq;
+            if (ok && heads_total == 0) heads_total = m / d;
+        }
+        if (ok) {
+            GemmArgs g;
+            g.M = n; g.N = m; g.K = k;
+            g.X = (const half_t*)B; g.ldx = ldb; g.strideX = 0;
+            g.W = grp.W[0]; g.ldw = lda; g.strideW = 0;
+            g.Y = grp.Y[0]; g.ldy = grp.ldy[0]; g.strideY = 0;
+            g.epi = Epilogue{epilogue, grp.bias[0], epi_arg0, epi_arg1, heads_total};
+            bool handled = false;
+            int rc = launch_gemv_f16(g, grp, W_NK, 1, (hipStream_t)stream, &handled);
+            if (handled) return rc;
+            rc = launch_gemm_skinny_f16(g, grp, W_NK, 1, (hipStream_t)stream, &handled);
+            if (handled) return rc;
+        }
+    }
+    for (int i = 0; i < count; ++i) {
+        int rc = lg_gemm_fused_f16(transa, m, n, k, A[i], lda, B, ldb, C[i], ldc[i], epilogue, epilogue != LG_EPI_NONE ? bias[i] : nullptr,
+                                   epi_arg0, epi_arg1, epi_arg2, stream);
+        if (rc) return rc;
+    }
+    return LG_OK;
 }
 
 int lg_gemm_strided_batched_f32(int transa, int transb, int m, int n, int k, const float* A, int lda, int64_t strideA,

@@ -26,6 +26,42 @@ struct GemmArgs {
     Epilogue epi;
 };
 
+// Up to three problems that share X and the shape and differ in weight, bias and destination (the Q, K and V projections of a
+// decode step): the weight-streaming kernels run them as one launch, blockIdx.y selecting the problem.
+constexpr int LG_MAX_GROUP = 3;
+struct GemmGroup {
+    int count;  // 1 = plain launch (the GemmArgs' own W / Y / bias / ldy are used)
+    const half_t* W[LG_MAX_GROUP];
+    half_t* Y[LG_MAX_GROUP];
+    const half_t* bias[LG_MAX_GROUP];
+    int64_t ldy[LG_MAX_GROUP];
+};
+__device__ __forceinline__ void select_group(GemmArgs& g, const GemmGroup& grp) {
+    if (grp.count > 1) {
+        const int gi = blockIdx.y;
+        g.W = grp.W[gi];
+        g.Y = grp.Y[gi];
+        g.epi.bias = grp.bias[gi];
+        g.ldy = grp.ldy[gi];
+    }
+}
+
+// host side: a plain launch seen as a group of one
+inline GemmGroup single_group(const GemmArgs& g) {
+    GemmGroup grp{};
+    grp.count = 1;
+    grp.W[0] = g.W; grp.Y[0] = g.Y; grp.bias[0] = g.epi.bias; grp.ldy[0] = g.ldy;
+    return grp;
+}
+// what the vectorised loads and stores of the weight-streaming kernels need of every member of the group
+inline bool group_aligned(const GemmArgs& g, const GemmGroup& grp) {
+    for (int i = 0; i < grp.count; ++i) {
+        if (!aligned16(grp.W[i]) || !aligned16(grp.Y[i])) return false;
+        if (g.epi.kind == LG_EPI_BIAS_HEADS ? (g.epi.d % 4 != 0) : (grp.ldy[i] % 4 != 0)) return false;
+    }
+    return true;
+}
+
 __device__ __forceinline__ float4_t mfma16(half8_t a, half8_t b, float4_t c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
 }

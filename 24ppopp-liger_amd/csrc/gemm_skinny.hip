@@ -131,8 +131,9 @@ __global__ __launch_bounds__(256) void gemm_skinny_nk_kernel(GemmArgs g, int ksl
 // MFMA tile (8 loads per chunk), so its rolling pipeline is DEPTH chunks deep: 4 waves x 2 chunks or 2 waves x 4 chunks
 // keep the same 64 KiB of weight loads in flight per block.
 template <int MT, int EPI, int NWV, int DEPTH>
-__global__ __launch_bounds__(64 * NWV) void gemm_skinny_direct_kernel(GemmArgs g) {
+__global__ __launch_bounds__(64 * NWV) void gemm_skinny_direct_kernel(GemmArgs g, GemmGroup grp) {
     constexpr int THREADS = 64 * NWV;
+    select_group(g, grp);
     __shared__ __attribute__((aligned(16))) half_t xs[2][16 * MT * SK_XS];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l16 = lane & 15, lk = lane >> 4;
@@ -141,11 +142,14 @@ __global__ __launch_bounds__(64 * NWV) void gemm_skinny_direct_kernel(GemmArgs g
     const int rot = blockIdx.x % nchunks;  // rotated chunk order, see gemm_skinny_nk_kernel
     auto chunk_at = [&](int i) { int c = rot + i; while (c >= nchunks) c -= nchunks; return c; };
 
-    constexpr int XV = 16 * MT * (SK_KC / 8) / THREADS;
+    // X chunk = 16 MT rows x 32 vectors of 8 halves, spread over the block's threads; when that does not divide evenly (6
+    // waves) the last threads fetch and store the last vector once more, which keeps every load unconditional
+    constexpr int XTOT = 16 * MT * (SK_KC / 8);
+    constexpr int XV = (XTOT + THREADS - 1) / THREADS;
     const half_t* xsrc[XV];
 #pragma unroll
     for (int u = 0; u < XV; ++u) {
-        const int v = tid + u * THREADS;
+        const int v = min(tid + u * THREADS, XTOT - 1);
         const int row = min(v / (SK_KC / 8), g.M - 1), c = v % (SK_KC / 8);
         xsrc[u] = g.X + (int64_t)row * g.ldx + c * 8;
     }
@@ -156,7 +160,7 @@ __global__ __launch_bounds__(64 * NWV) void gemm_skinny_direct_kernel(GemmArgs g
     auto store_x = [&](int buf, const half8_t (&xr)[XV]) {
 #pragma unroll
         for (int u = 0; u < XV; ++u) {
-            const int v = tid + u * THREADS;
+            const int v = min(tid + u * THREADS, XTOT - 1);
             const int row = v / (SK_KC / 8), c = v % (SK_KC / 8);
             *reinterpret_cast<half8_t*>(&xs[buf][row * SK_XS + c * 8]) = xr[u];
         }
@@ -219,22 +223,22 @@ __global__ __launch_bounds__(64 * NWV) void gemm_skinny_direct_kernel(GemmArgs g
 }
 
 template <int MT, int NWV, int DEPTH>
-static void launch_direct(const GemmArgs& g, hipStream_t stream) {
-    const dim3 grid((g.N + 16 * NWV - 1) / (16 * NWV)), block(64 * NWV);
+static void launch_direct(const GemmArgs& g, const GemmGroup& grp, hipStream_t stream) {
+    const dim3 grid((g.N + 16 * NWV - 1) / (16 * NWV), grp.count), block(64 * NWV);
     switch (g.epi.kind) {
-        case LG_EPI_NONE: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_NONE, NWV, DEPTH>), grid, block, 0, stream, g); break;
-        case LG_EPI_BIAS: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_BIAS, NWV, DEPTH>), grid, block, 0, stream, g); break;
-        case LG_EPI_BIAS_GELU: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_BIAS_GELU, NWV, DEPTH>), grid, block, 0, stream, g); break;
-        default: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_BIAS_HEADS, NWV, DEPTH>), grid, block, 0, stream, g); break;
+        case LG_EPI_NONE: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_NONE, NWV, DEPTH>), grid, block, 0, stream, g, grp); break;
+        case LG_EPI_BIAS: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_BIAS, NWV, DEPTH>), grid, block, 0, stream, g, grp); break;
+        case LG_EPI_BIAS_GELU: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_BIAS_GELU, NWV, DEPTH>), grid, block, 0, stream, g, grp); break;
+        default: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_BIAS_HEADS, NWV, DEPTH>), grid, block, 0, stream, g, grp); break;
     }
 }
 template <int NWV, int DEPTH>
-static void launch_direct_mt(const GemmArgs& g, hipStream_t stream) {
+static void launch_direct_mt(const GemmArgs& g, const GemmGroup& grp, hipStream_t stream) {
     switch ((g.M + 15) / 16) {
-        case 1: launch_direct<1, NWV, DEPTH>(g, stream); break;
-        case 2: launch_direct<2, NWV, DEPTH>(g, stream); break;
-        case 3: launch_direct<3, NWV, DEPTH>(g, stream); break;
-        default: launch_direct<4, NWV, DEPTH>(g, stream); break;
+        case 1: launch_direct<1, NWV, DEPTH>(g, grp, stream); break;
+        case 2: launch_direct<2, NWV, DEPTH>(g, grp, stream); break;
+        case 3: launch_direct<3, NWV, DEPTH>(g, grp, stream); break;
+        default: launch_direct<4, NWV, DEPTH>(g, grp, stream); break;
     }
 }
 
@@ -290,25 +294,35 @@ void launch_splitk_reduce(const GemmArgs& g, const float* partial, int nsplit, h
     }
 }
 
-int launch_gemm_skinny_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t stream, bool* handled) {
+// grp.count > 1: handled only if the unsliced kernels apply (the caller then falls back to one launch per member)
+int launch_gemm_skinny_f16(const GemmArgs& g, const GemmGroup& grp, int wlayout, int batch, hipStream_t stream, bool* handled) {
     *handled = false;
     if (batch != 1 || wlayout != W_NK) return LG_OK;
     if (g.M <= 0 || g.M > 64 || g.N < 512 || g.K < 1024 || (g.K % SK_KC) || (g.N % 4)) return LG_OK;
-    if (!aligned16(g.X) || !aligned16(g.W) || !aligned16(g.Y) || (g.ldx % 8) || (g.ldw % 8)) return LG_OK;
-    if (g.epi.kind == LG_EPI_BIAS_HEADS ? (g.epi.d % 4 != 0) : (g.ldy % 4 != 0)) return LG_OK;
+    if (!aligned16(g.X) || (g.ldx % 8) || (g.ldw % 8) || !group_aligned(g, grp)) return LG_OK;
     const int mt = (g.M + 15) / 16;
-    // Enough blocks without slicing K (>= 192: see below)?  64 features per block, or 32 for up to 16 token rows (with more
-    // rows the 2-wave block's registers no longer hold its four-chunk pipeline).
-    if ((g.N + 63) / 64 >= 192 && g.K % (2 * SK_KC) == 0) {
-        *handled = true;
-        launch_direct_mt<4, 2>(g, stream);
-        return check_launch("gemm_f16_skinny");
+    // Unsliced blocks need a block width (128, 96, 64 or, up to 16 token rows, 32 features) that gives one round of blocks on
+    // the 256 CUs, 192..256 of them (fewer leave CUs idle; a few more than 256 double the time of the CUs that get two), or
+    // so many blocks that the last, partial round does not matter.  The widest such block re-reads the token rows least.
+    {
+        const int widths[4] = {128, 96, 64, 32};
+        for (int wi = 0; wi < 4; ++wi) {
+            const int w = widths[wi];
+            // whole pipeline depths of chunks; the 2-wave block's registers hold its four-chunk pipeline for one row tile only
+            if (w == 32 ? (mt != 1 || g.K % (4 * SK_KC) != 0) : (g.K % (2 * SK_KC) != 0)) continue;
+            const int blocks = (g.N + w - 1) / w * grp.count;
+            if (blocks < 192 || (blocks > 256 && blocks < 1024)) continue;
+            *handled = true;
+            switch (w) {
+                case 128: launch_direct_mt<8, 2>(g, grp, stream); break;
+                case 96: launch_direct_mt<6, 2>(g, grp, stream); break;
+                case 64: launch_direct_mt<4, 2>(g, grp, stream); break;
+                default: launch_direct<1, 2, 4>(g, grp, stream); break;
+            }
+            return check_launch("gemm_f16_skinny");
+        }
     }
-    if (mt == 1 && (g.N + 31) / 32 >= 192 && g.K % (4 * SK_KC) == 0) {
-        *handled = true;
-        launch_direct<1, 2, 4>(g, stream);
-        return check_launch("gemm_f16_skinny");
-    }
+    if (grp.count > 1) return LG_OK;
     const int nblk = (g.N + SK_BN - 1) / SK_BN;
     // K-slices: as few as fill the chip.  One block of 4 waves keeps 64 KiB of weight loads in flight, which is enough for one
     // CU; more slices only add fp32 partials and reduce work (six GEMMs of a decode step at 32 token rows: 344 us with >= 1024

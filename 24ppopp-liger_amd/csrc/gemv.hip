@@ -31,8 +31,9 @@ __device__ __forceinline__ float dot8(half8_t w, half8_t x, float acc) {
 
 // MR = staged token rows (1, 2 or 4; rows >= M are zero)
 template <int MR, int EPI>
-__global__ __launch_bounds__(256) void gemv_nk_kernel(GemmArgs g) {
+__global__ __launch_bounds__(256) void gemv_nk_kernel(GemmArgs g, GemmGroup members) {
     extern __shared__ __attribute__((aligned(16))) half_t xs[];  // [MR][K]
+    select_group(g, members);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n0 = (blockIdx.x * 4 + wave) * GV_ROWS;
     const int K = g.K;
@@ -89,24 +90,26 @@ __global__ __launch_bounds__(256) void gemv_nk_kernel(GemmArgs g) {
 
 #pragma unroll
     for (int m = 0; m < MR; ++m) {
-        float4_t out;
 #pragma unroll
-        for (int r = 0; r < GV_ROWS; ++r) out[r] = wave_sum(acc[r][m]);
-        if (lane == 0 && m < g.M) epilogue_store4<EPI>(g, g.Y, m, n0, out, true);
+        for (int q = 0; q < GV_ROWS / 4; ++q) {
+            float4_t out;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) out[r] = wave_sum(acc[q * 4 + r][m]);
+            if (lane == 0 && m < g.M) epilogue_store4<EPI>(g, g.Y, m, n0 + q * 4, out, true);
+        }
     }
 }
 
-int launch_gemv_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t stream, bool* handled) {
+int launch_gemv_f16(const GemmArgs& g, const GemmGroup& grp, int wlayout, int batch, hipStream_t stream, bool* handled) {
     *handled = false;
     if (batch != 1 || wlayout != W_NK) return LG_OK;
     if (g.M <= 0 || g.M > 4 || g.N < 256 || (g.N % 4) || g.K < GV_KSTEP * GV_U || (g.K % (GV_KSTEP * GV_U))) return LG_OK;
     const int mr = g.M == 1 ? 1 : (g.M == 2 ? 2 : 4);
     const size_t smem = (size_t)mr * g.K * sizeof(half_t);
     if (smem > (size_t)GV_MAX_LDS) return LG_OK;
-    if (!aligned16(g.X) || !aligned16(g.W) || !aligned16(g.Y) || (g.ldx % 8) || (g.ldw % 8)) return LG_OK;
-    if (g.epi.kind == LG_EPI_BIAS_HEADS ? (g.epi.d % 4 != 0) : (g.ldy % 4 != 0)) return LG_OK;
+    if (!aligned16(g.X) || (g.ldx % 8) || (g.ldw % 8) || !group_aligned(g, grp)) return LG_OK;
     *handled = true;
-    const dim3 grid((g.N + 4 * GV_ROWS - 1) / (4 * GV_ROWS)), block(256);
+    const dim3 grid((g.N + 4 * GV_ROWS - 1) / (4 * GV_ROWS), grp.count), block(256);
 #define LG_GV(MR_, E_)                                                                                              \
     do {                                                                                                            \
         static bool attr_set = false;                                                                               \
@@ -114,7 +117,7 @@ int launch_gemv_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t strea
             (void)hipFuncSetAttribute((const void*)gemv_nk_kernel<MR_, E_>, hipFuncAttributeMaxDynamicSharedMemorySize, GV_MAX_LDS); \
             attr_set = true;                                                                                        \
         }                                                                                                           \
-        hipLaunchKernelGGL((gemv_nk_kernel<MR_, E_>), grid, block, smem, stream, g);                                \
+        hipLaunchKernelGGL((gemv_nk_kernel<MR_, E_>), grid, block, smem, stream, g, grp);                              \
     } while (0)
 #define LG_GV_MR(E_)                                 \
     switch (mr) {                                    \

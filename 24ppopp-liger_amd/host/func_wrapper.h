@@ -21,6 +21,17 @@ inline void GemmEx(const DynamicInitParam& DParams, const GemmDesc& g) {
     }
 }
 
+// Q, K and V projections of a decode step as one call (bert_layer.h:127-137 issues them one after the other): the
+// descriptors share the activations, the shape and the epilogue arguments and differ in weight, bias and destination.
+inline void GemmExGrouped3(const DynamicInitParam& DParams, const GemmDesc& q, const GemmDesc& k, const GemmDesc& v) {
+    const void* A[3] = {q.A, k.A, v.A};
+    void* C[3] = {q.C, k.C, v.C};
+    const int ldc[3] = {q.ldc, k.ldc, v.ldc};
+    const void* bias[3] = {q.bias, k.bias, v.bias};
+    note_status(lg_gemm_fused_grouped_f16(q.transa, q.m, q.n, q.k, 3, A, q.lda, q.B, q.ldb, C, ldc, q.epilogue, bias, q.epi_seq,
+                                          q.epi_d, q.epi_heads_total, DParams.stream), "lg_gemm_fused_grouped_f16");
+}
+
 inline void GemmStridedBatchedEx(const DynamicInitParam& DParams, int dtype, int transa, int transb, int m, int n, int k,
                                  const void* A, int lda, long long strideA, const void* B, int ldb, long long strideB,
                                  void* C, int ldc, long long strideC, int batchCount) {

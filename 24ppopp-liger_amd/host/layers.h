@@ -14,6 +14,7 @@
 //   * optional assemblies: pre-LN with residuals built from the reference's fused residual kernels, a fused
 //     assembly (epilogue-fused GEMMs + one attention kernel) and a decode step over a KV cache.
 #pragma once
+#include <cstdlib>
 #include <cmath>
 #include <map>
 #include <memory>
@@ -472,15 +473,18 @@ class Bert_MHA {
             Linear_Col<T>* lin[3] = {linear_q_col, linear_k_col, linear_v_col};
             T* dst[3] = {b.q_buf, kc + (int64_t)past * d, vc + (int64_t)past * d};
             const T* bias[3] = {q_bias, k_bias, v_bias};
-            const char* lab[3] = {"q_gemm(decode)", "k_gemm(decode)", "v_gemm(decode)"};
+            GemmDesc g[3];
             for (int t = 0; t < 3; ++t) {
-                GemmDesc g = lin[t]->desc(input, dst[t], batch);
-                g.epilogue = LG_EPI_BIAS_HEADS;
-                g.bias = bias[t];
-                g.epi_seq = 1; g.epi_d = d; g.epi_heads_total = h;
-                g.ldc = (t == 0) ? 1 : Lmax;  // rows per (batch, head) slot of the destination
-                FuncWrapVec.push_back(FuncWrap(1.0f, GEMM, [g](const DynamicInitParam& D) { GemmEx(D, g); }, g, lab[t], HBM_BOUND));
+                g[t] = lin[t]->desc(input, dst[t], batch);
+                g[t].epilogue = LG_EPI_BIAS_HEADS;
+                g[t].bias = bias[t];
+                g[t].epi_seq = 1; g[t].epi_d = d; g[t].epi_heads_total = h;
+                g[t].ldc = (t == 0) ? 1 : Lmax;  // rows per (batch, head) slot of the destination
             }
+            // one launch for the three projections: they read the same token rows and nothing orders them among themselves
+            const GemmDesc gq = g[0], gk = g[1], gv = g[2];
+            FuncWrapVec.push_back(FuncWrap(1.0f, COMPUTATION, [gq, gk, gv](const DynamicInitParam& D) { GemmExGrouped3(D, gq, gk, gv); },
+                                           "qkv_gemm(decode)", HBM_BOUND));
         } else {
             v = linear_q_col->forward(input, b.q, batch); v[0].label = "q_gemm(decode)"; v[0].rclass = HBM_BOUND;
             FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
@@ -622,7 +626,7 @@ class Bert_Model {
     // entries per layer of the vector forward() returns for this configuration
     int kernels_per_layer(bool decode = false) const {
         const bool fused = BertParams.fused && dtype_of<T>::value == LG_F16;
-        int mha = decode ? (BertParams.fused ? 5 : 6) : (fused ? 5 : (BertParams.packed_qkv ? 7 : 9));
+        int mha = decode ? (BertParams.fused ? 3 : 6) : (fused ? 5 : (BertParams.packed_qkv ? 7 : 9));
         int mlp = (fused && BertParams.ffn_act != FFN_GEGLU) ? 2 : 3;
         return mha + mlp + 2 + (BertParams.norm_mode == PRE_LN_RESID ? 1 : 0);
     }

@@ -166,6 +166,15 @@ int lg_gemm_fused_f16(int transa, int m, int n, int k, const void* A, int lda, c
                       int ldc, int epilogue, const void* bias, int epi_arg0, int epi_arg1, int epi_arg2,
                       void* stream);
 
+/* `count` (1..3) lg_gemm_fused_f16 calls that share B (the token rows), the shape, lda and the epilogue arguments
+ * and differ in A[i], C[i], ldc[i] and bias[i]: the Q, K and V projections of a decode step (linear.h:99-101 issued
+ * three times by bert_layer.h:127-137).  Few-token problems with weights [out, in] run as ONE launch of the
+ * weight-streaming kernels; anything else is executed as `count` plain calls.  Results are those of the plain calls
+ * up to the order of the fp32 sum over k (the one launch may use another block width).  No reference counterpart. */
+int lg_gemm_fused_grouped_f16(int transa, int m, int n, int k, int count, const void* const* A, int lda, const void* B,
+                              int ldb, void* const* C, const int* ldc, int epilogue, const void* const* bias,
+                              int epi_arg0, int epi_arg1, int epi_arg2, void* stream);
+
 /* ---- attention kernels with no reference counterpart --------------------------------------------- */
 /* Fused prefill attention: out = softmax(q k^T * scalar + maskterm) v with the reference's softmax
  * semantics (-10000 additive mask, +1e-6 in the denominator); replaces launch-vector entries 4,5,6 (and 7

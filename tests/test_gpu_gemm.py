@@ -211,3 +211,55 @@ def test_gemm_fused_epilogues_on_the_weight_streaming_kernels(dev, po, M, h):
     got = dev.down(out)
     assert max_rel_err(got[:, :, 2:3], ref_heads) < 2e-3
     assert np.all(got[:, :, :2] == 0) and np.all(got[:, :, 3:] == 0)
+
+
+@pytest.mark.parametrize("M,transa", [(1, 1), (3, 1), (8, 1), (32, 1), (64, 1), (100, 1), (8, 0)])
+def test_grouped_qkv_gemm_equals_three_plain_calls(dev, po, M, transa):
+    """The grouped entry (Q, K and V projections of a decode step as one call) must return what three plain fused calls
+    return: one launch of the matrix-vector / weight-streaming kernels for few token rows and weights [out, in] (bit for
+    bit on the matrix-vector kernel; the weight-streaming kernel may choose another block width for the group and then
+    sums k in another order), three plain calls otherwise (bit for bit).  Q goes to [M, h, 1, d], K and V to row `past`
+    of cache-shaped buffers."""
+    import ctypes as C
+    h, d, K, rows, past = 48, 128, 2048, 6, 3
+    N = h * d
+    X = rnd(po, M * K, 50, 1).reshape(M, K)
+    dX = dev.up(X, 1)
+    Ws = [rnd(po, K * N, 51 + t, 1, 0.05).reshape(K, N) for t in range(3)]
+    bs = [rnd(po, N, 54 + t, 1, 0.3) for t in range(3)]
+    dA = [dev.up(np.ascontiguousarray(W.T) if transa else W, 1) for W in Ws]
+    dB = [dev.up(b, 1) for b in bs]
+    lda = K if transa else N
+    ldc = [1, rows, rows]
+
+    def outputs():
+        o = [dev.empty((M, h, 1, d), 1), dev.empty((M, h, rows, d), 1), dev.empty((M, h, rows, d), 1)]
+        for t in o:
+            t.zero_()
+        return o
+
+    def dst(o, t):
+        return o[t].data_ptr() + (past * d * 2 if t else 0)
+
+    plain = outputs()
+    for t in range(3):
+        dev.call("lg_gemm_fused_f16", transa, N, M, K, dA[t], lda, dX, K, dst(plain, t), ldc[t], dev.capi.EPI_BIAS_HEADS, dB[t], 1, d, h)
+    grouped = outputs()
+    arr = lambda ptrs: (C.c_void_p * 3)(*ptrs)
+    dev.call("lg_gemm_fused_grouped_f16", transa, N, M, K, 3, arr([a.data_ptr() for a in dA]), lda, dX, K,
+             arr([dst(grouped, t) for t in range(3)]), (C.c_int * 3)(*ldc), dev.capi.EPI_BIAS_HEADS,
+             arr([b.data_ptr() for b in dB]), 1, d, h)
+    for t in range(3):
+        if transa == 0 or M <= 4 or M > 64:
+            assert np.array_equal(dev.down(grouped[t]), dev.down(plain[t]))
+        else:
+            assert max_rel_err(dev.down(grouped[t]), dev.down(plain[t])) < 1e-3
+    y = po.gemm(X, Ws[1], 1)
+    ref, _, _ = po.add_qkv_bias_transpose(y, bs[1], y, bs[1], y, bs[1], M, 1, h, d, 1)
+    got = dev.down(grouped[1])
+    assert max_rel_err(got[:, :, past:past + 1], ref) < 2e-3
+    assert np.all(got[:, :, :past] == 0) and np.all(got[:, :, past + 1:] == 0)
+    # a null member is reported, nothing is launched
+    bad = arr([dA[0].data_ptr(), 0, dA[2].data_ptr()])
+    assert dev.call_rc("lg_gemm_fused_grouped_f16", transa, N, M, K, 3, bad, lda, dX, K, arr([dst(grouped, t) for t in range(3)]),
+                       (C.c_int * 3)(*ldc), dev.capi.EPI_BIAS_HEADS, arr([b.data_ptr() for b in dB]), 1, d, h) != 0

@@ -47,7 +47,8 @@ def test_launch_vector_shapes_and_order(fake):
     assert [e["type"] for e in d].count("GEMM") == 6
     assert m.kernels_per_layer() == 14
     mf = small_model(host, fused=True)
-    assert mf.kernels_per_layer() == 9 and mf.kernels_per_layer(decode=True) == 9   # K/V rows are appended by the GEMM epilogues
+    assert mf.kernels_per_layer() == 9 and mf.kernels_per_layer(decode=True) == 7   # one grouped Q/K/V launch whose epilogues append the K/V rows
+    assert [e["label"] for e in mf.describe(2, 1, decode_past=10)][:3] == ["qkv_gemm(decode)", "attn_decode", "out_proj(decode)"]
     assert all(e["class"] == "HBM_BOUND" for e in mf.describe(2, 1, decode_past=10))
     mg = host.Model(1, 2, 32, 4, 64, ffn_inner=512, fused=True, ffn_act=host.FFN_GEGLU)
     assert [e["label"] for e in mg.describe(2, 32)][-4:] == ["ffn1(gate+up)", "bias+geglu", "ffn2", "layer_norm"]
@@ -180,7 +181,7 @@ def test_decode_request_fills_prefill_gemm_windows_and_splits_cover_exactly(fake
         for (c0, m0), (c1, _) in zip(v, v[1:]):
             assert c1 - c0 == m0 * 2              # contiguous fp16 column ranges: no gap, no overlap
     assert (r["splits"] > 0) == expect_splits
-    # A's decode kernels: 3 steps x 9 entries, in order, attention lengths 49, 50, 51
+    # A's decode kernels: 3 steps x 7 entries, in order, attention lengths 49, 50, 51
     assert [e["n"] for e in t if e["name"] == "attn_decode"] == [49, 50, 51]
     assert r["secondary_launches"] > 0
     # per-request order in virtual time (n == tokens identifies the request for row-shaped kernels)
