@@ -29,6 +29,7 @@ SIGNATURES = {
     "lg_device_synchronize": (_i, []),
     "lg_stream_create": (_i, [C.POINTER(_p)]),
     "lg_stream_create_cu_mask": (_i, [C.POINTER(_p), C.POINTER(C.c_uint), _i]),
+    "lg_stream_create_concurrent": (_i, [_p, _p, _p]),
     "lg_stream_destroy": (_i, [_p]),
     "lg_stream_synchronize": (_i, [_p]),
     "lg_stream_wait_event": (_i, [_p, _p]),

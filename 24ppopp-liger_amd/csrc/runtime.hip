@@ -172,6 +172,69 @@ int lg_stream_create_cu_mask(void** stream, const unsigned* cu_mask, int mask_wo
     *stream = (void*)s;
     return rc;
 }
+// ---- a second stream that really runs next to the first ----------------------------------------------------------------------
+// HIP multiplexes streams onto a few hardware queues (4 per process by default) and hands a new stream the least used one,
+// so two streams of one process can land on the same hardware queue, where their kernels run strictly one after the other.
+// Whether that happened cannot be queried, but it can be measured: one wave spins for a fixed time on `other` while a
+// one-wave kernel is launched on the candidate; on separate queues the second finishes long before the first.
+__global__ void lg_probe_spin_kernel(long long ticks, int* sink) {
+    const long long t0 = wall_clock64();  // constant-rate counter: the loop ends after `ticks` whatever else happens
+    while (wall_clock64() - t0 < ticks) {}
+    if (sink && threadIdx.x == 1024) *sink = 1;  // never true: keeps the loop observable
+}
+__global__ void lg_probe_touch_kernel(int* sink) {
+    if (sink && threadIdx.x == 1024) *sink = 1;
+}
+static bool runs_concurrently(hipStream_t a, hipStream_t b, bool* ok) {
+    *ok = false;
+    int rate_khz = 0;
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    if (hipDeviceGetAttribute(&rate_khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess || rate_khz <= 0) rate_khz = 100000;
+    const double spin_ms = 0.4;
+    hipEvent_t ea = nullptr, eb = nullptr;
+    if (hipEventCreate(&ea) != hipSuccess || hipEventCreate(&eb) != hipSuccess) return false;
+    bool concurrent = false;
+    // warm both kernels up first (code upload), then the timed pair
+    for (int pass = 0; pass < 2; ++pass) {
+        hipLaunchKernelGGL(lg_probe_spin_kernel, dim3(1), dim3(64), 0, a, (long long)(pass ? spin_ms * rate_khz : 1), (int*)nullptr);
+        if (hipEventRecord(ea, a) != hipSuccess) break;
+        hipLaunchKernelGGL(lg_probe_touch_kernel, dim3(1), dim3(64), 0, b, (int*)nullptr);
+        if (hipEventRecord(eb, b) != hipSuccess) break;
+        if (hipStreamSynchronize(a) != hipSuccess || hipStreamSynchronize(b) != hipSuccess) break;
+        if (pass == 1) {
+            float ms = 0.f;  // from the end of the touch kernel on b to the end of the spin on a
+            if (hipEventElapsedTime(&ms, eb, ea) != hipSuccess) break;
+            concurrent = ms > 0.5f * (float)spin_ms;
+            *ok = true;
+        }
+    }
+    (void)hipEventDestroy(ea);
+    (void)hipEventDestroy(eb);
+    return concurrent;
+}
+int lg_stream_create_concurrent(void** stream, void* other, int* verified) {
+    if (!stream || !other) { set_error("lg_stream_create_concurrent: bad arguments"); return LG_ERR_INVALID; }
+    if (verified) *verified = 0;
+    constexpr int TRIES = 8;
+    hipStream_t cand[TRIES];
+    int n = 0, pick = -1;
+    for (; n < TRIES && pick < 0; ++n) {
+        // rejected candidates stay alive until the end, so that the next one is handed another hardware queue
+        if (rt(hipStreamCreateWithFlags(&cand[n], hipStreamNonBlocking), "hipStreamCreateWithFlags") != LG_OK) break;
+        bool ok = false;
+        const bool conc = runs_concurrently((hipStream_t)other, cand[n], &ok);
+        if (!ok) { ++n; set_error("lg_stream_create_concurrent: the concurrency probe failed"); break; }
+        if (conc) pick = n;
+    }
+    if (pick < 0 && n > 0) pick = 0;  // none verified: the caller still gets a working stream
+    else if (pick >= 0 && verified) *verified = 1;
+    for (int i = 0; i < n; ++i)
+        if (i != pick) (void)hipStreamDestroy(cand[i]);
+    if (pick < 0) return LG_ERR_LAUNCH;
+    *stream = (void*)cand[pick];
+    return LG_OK;
+}
 int lg_stream_destroy(void* stream) { return rt(hipStreamDestroy((hipStream_t)stream), "hipStreamDestroy"); }
 int lg_stream_synchronize(void* stream) { return rt(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize"); }
 int lg_stream_wait_event(void* stream, void* event) {

@@ -24,7 +24,7 @@ _i, _i64, _u64, _f, _d, _p = C.c_int, C.c_int64, C.c_uint64, C.c_float, C.c_doub
 class Report(C.Structure):
     _fields_ = [("records", _i), ("avg_latency_ms", _d), ("p99_latency_ms", _d), ("avg_gpu_ms", _d),
                 ("avg_queue_ms", _d), ("total_duration_ms", _d), ("throughput", _d), ("rounds", _i),
-                ("secondary_launches", _i), ("splits", _i), ("profile_misses", _i)]
+                ("secondary_launches", _i), ("splits", _i), ("profile_misses", _i), ("avg_e2e_ms", _d), ("p99_e2e_ms", _d)]
 
     def as_dict(self):
         return {n: getattr(self, n) for n, _ in self._fields_}
@@ -51,6 +51,8 @@ SIGNATURES = {
     "lgh_sched_profile_contention": (_i, [_p, _i, _i, _i, _i, C.POINTER(_f)]),
     "lgh_sched_set_contention": (_i, [_p, _i, _i, _f]),
     "lgh_sched_get_contention": (_f, [_p, _i, _i]),
+    "lgh_sched_streams_concurrent": (_i, [_p]),
+    "lgh_sched_set_merge_minor": (_i, [_p, _i]),
     "lgh_sched_save": (_i, [_p, C.c_char_p, C.c_char_p]),
     "lgh_sched_load": (_i, [_p, C.c_char_p, C.c_char_p]),
     "lgh_sched_lookup": (_f, [_p, _i, _i, _i]),
@@ -227,6 +229,15 @@ class Scheduler:
 
     def contention(self, main_class, sub_class):
         return lib.lgh_sched_get_contention(self.h, main_class, sub_class)
+
+    def set_merge_minor(self, on):
+        """Minor entries (LayerNorm, residual, cache append, row gather) take the scheduling class of the entry before them."""
+        check(lib.lgh_sched_set_merge_minor(self.h, int(bool(on))), "lgh_sched_set_merge_minor")
+
+    @property
+    def streams_concurrent(self):
+        """True when the second stream was verified (by measurement) to execute at the same time as the first."""
+        return bool(lib.lgh_sched_streams_concurrent(self.h))
 
     def save(self, main_file, sub_file):
         check(lib.lgh_sched_save(self.h, main_file.encode(), sub_file.encode()), "lgh_sched_save")

@@ -2,6 +2,7 @@
 //
 // A model handle owns a Bert_Model<T> (T = float or liger::half), its default workspace and two stream contexts.
 // Nothing here computes: vectors are built by the layer classes and launched entry by entry through FuncWrap.
+#include <cstdlib>
 #include <cstring>
 #include <memory>
 #include <string>
@@ -33,6 +34,8 @@ struct SchedBase {
     virtual bool profile_contention(int bs, int seq, int dec_bs, int past, float* out5) = 0;
     virtual bool set_contention(int main_class, int sub_class, float v) = 0;
     virtual float get_contention(int main_class, int sub_class) = 0;
+    virtual bool streams_concurrent() = 0;
+    virtual void set_merge_minor(bool on) = 0;
 };
 
 struct ModelBase {
@@ -74,7 +77,7 @@ struct SchedT : SchedBase {
         s->reset_run();
         s->serving(trace);
         if (mode == 0) s->run_sequential(); else s->run_stream_sync();
-        Report r = s->output_recording(false);
+        Report r = s->output_recording(getenv("LGH_PRINT_RECORDS") != nullptr);  // per-request lines as schedule.h:325-348 prints them
         if (counters) { counters[0] = s->rounds; counters[1] = s->secondary_launches; counters[2] = s->splits; counters[3] = s->profile_misses; }
         return r;
     }
@@ -119,6 +122,8 @@ struct SchedT : SchedBase {
         for (int i = 0; i < n && i < cap; ++i) out[i] = it->second[i];
         return n;
     }
+    bool streams_concurrent() override { return s->DParams1.concurrent; }
+    void set_merge_minor(bool on) override { s->merge_minor = on; }
 };
 
 template <typename T>
@@ -312,6 +317,7 @@ struct LghReport {
     int records;
     double avg_latency_ms, p99_latency_ms, avg_gpu_ms, avg_queue_ms, total_duration_ms, throughput;
     int rounds, secondary_launches, splits, profile_misses;
+    double avg_e2e_ms, p99_e2e_ms;  // arrival -> completion on one clock
 };
 
 // policy: 0 = classic (communication vs rest), 1 = resource classes (MFMA-bound vs HBM-bound)
@@ -352,6 +358,15 @@ int lgh_sched_set_contention(void* sched, int main_class, int sub_class, float v
     if (!sched || !((SchedBase*)sched)->set_contention(main_class, sub_class, value)) return fail("lgh_sched_set_contention: bad arguments");
     return LG_OK;
 }
+// Resource-class policy: minor entries (LayerNorm, residual, cache append, row gather) take the scheduling class of the entry
+// before them: a prefill's LayerNorms no longer cut it into runs and no longer stop it when it is interleaved.  Off by default.
+int lgh_sched_set_merge_minor(void* sched, int on) {
+    if (!sched) return fail("lgh_sched_set_merge_minor: null");
+    ((SchedBase*)sched)->set_merge_minor(on != 0);
+    return LG_OK;
+}
+// 1 when the scheduler's second stream was verified to execute at the same time as the first
+int lgh_sched_streams_concurrent(void* sched) { return (sched && ((SchedBase*)sched)->streams_concurrent()) ? 1 : 0; }
 float lgh_sched_get_contention(void* sched, int main_class, int sub_class) {
     return sched ? ((SchedBase*)sched)->get_contention(main_class, sub_class) : -1.f;
 }
@@ -376,6 +391,7 @@ int lgh_sched_run_trace(void* sched, int mode, const double* arrival_s, const in
     out->records = r.records; out->avg_latency_ms = r.avg_latency_ms; out->p99_latency_ms = r.p99_latency_ms;
     out->avg_gpu_ms = r.avg_gpu_ms; out->avg_queue_ms = r.avg_queue_ms; out->total_duration_ms = r.total_duration_ms;
     out->throughput = r.throughput; out->rounds = c[0]; out->secondary_launches = c[1]; out->splits = c[2]; out->profile_misses = c[3];
+    out->avg_e2e_ms = r.avg_e2e_ms; out->p99_e2e_ms = r.p99_e2e_ms;
     return first_error();
 }
 // Deterministic variant for tests: requests are queued up front with lgh_sched_serve (no request thread, no real-time
@@ -413,6 +429,7 @@ int lgh_sched_run_queued(void* sched, int mode, LghReport* out) {
     out->records = r.records; out->avg_latency_ms = r.avg_latency_ms; out->p99_latency_ms = r.p99_latency_ms;
     out->avg_gpu_ms = r.avg_gpu_ms; out->avg_queue_ms = r.avg_queue_ms; out->total_duration_ms = r.total_duration_ms;
     out->throughput = r.throughput; out->rounds = c[0]; out->secondary_launches = c[1]; out->splits = c[2]; out->profile_misses = c[3];
+    out->avg_e2e_ms = r.avg_e2e_ms; out->p99_e2e_ms = r.p99_e2e_ms;
     return first_error();
 }
 // the report arithmetic alone (known-answer tests against the reference's published logs)

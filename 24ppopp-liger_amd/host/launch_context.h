@@ -60,6 +60,14 @@ class DynamicInitParam {
     // the reference passes a CUDA stream priority here; priorities are deliberately not used on this platform
     explicit DynamicInitParam(int /*priority*/) { note_status(lg_stream_create(&stream), "lg_stream_create"); }
     DynamicInitParam(void* existing_stream, int id) : stream(existing_stream), stream_id(id) {}
+    // a stream that is verified to execute kernels at the same time as `first`'s (two streams of one process may share a
+    // hardware queue, on which they would run strictly in turn); `concurrent` tells whether the verification succeeded
+    bool concurrent = false;
+    DynamicInitParam(int /*priority*/, const DynamicInitParam& first) {
+        int verified = 0;
+        note_status(lg_stream_create_concurrent(&stream, first.stream, &verified), "lg_stream_create_concurrent");
+        concurrent = verified != 0;
+    }
 };
 using DynamicNvInitParam = DynamicInitParam;
 
@@ -134,6 +142,9 @@ class FuncWrap {
     std::function<void(const DynamicInitParam&)> callback;
     GemmDesc args_gemm;
     int name = -1;  // kernel index inside the layer (profile key)
+    // a small kernel between the big ones of its layer (normalisation, residual, cache append, row gather): a scheduler that
+    // is told to merge minor entries lets it take the scheduling class of the entry before it
+    bool minor = false;
     const char* label = "";
 
     FuncWrap() {}

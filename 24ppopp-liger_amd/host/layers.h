@@ -151,6 +151,7 @@ class LayerNorm {  // operator.h:16-41
         FuncWrapVec.push_back(FuncWrap(0.1f, COMPUTATION,
                                        [=](const DynamicInitParam& D) { Layer_Norm<T>(input, g, b, output, m, kk, D); },
                                        "layer_norm"));
+        FuncWrapVec.back().minor = true;
         return FuncWrapVec;
     }
 };
@@ -496,6 +497,7 @@ class Bert_MHA {
             FuncWrapVec.push_back(FuncWrap(0.05f, COMPUTATION, [=](const DynamicInitParam& D) {
                 note_status(lg_kv_append_f16(b.q_buf, kc, vc, b.q, qbias, b.k, kbias, b.v, vbias, batch, h, d, past, Lmax, D.stream), "lg_kv_append_f16");
             }, "kv_append"));
+            FuncWrapVec.back().minor = true;
         }
         FuncWrapVec.push_back(FuncWrap(0.15f, COMPUTATION, [=](const DynamicInitParam& D) {
             note_status(lg_attn_decode_f16(b.q_buf, kc, vc, b.attn_out, dws, batch, h, d, past + 1, Lmax, sc, D.stream), "lg_attn_decode_f16");
@@ -589,11 +591,13 @@ class Bert_Encoder {
             FuncWrapVec.push_back(FuncWrap(0.1f, COMPUTATION, [=](const DynamicInitParam& D) {
                 Add_bias_input_layernorm_2_kernelLauncher<T>(input, g, bt, wb, mha_out, ln_mha_out, M, nn, D);
             }, "residual+bias+layer_norm"));
+            FuncWrapVec.back().minor = true;
             append(mlp(ln_mha_out, output));
             T* b2 = MLP->bias2;
             FuncWrapVec.push_back(FuncWrap(0.1f, COMPUTATION, [=](const DynamicInitParam& D) {
                 Add_bias_input_kernelLauncher<T>(output, b2, mha_out, M, nn, D);
             }, "residual+bias"));
+            FuncWrapVec.back().minor = true;
         }
         return FuncWrapVec;
     }

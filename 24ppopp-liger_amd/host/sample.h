@@ -30,6 +30,7 @@ struct recorder {     // init.h:16-20
     void* start;      // events (lg_event_*)
     void* stop;
     int batch_size, seq_len;
+    std::chrono::steady_clock::time_point arrive;  // host clock at arrival (not in the reference: end-to-end latency)
 };
 
 class Sample {
@@ -53,6 +54,20 @@ class Sample {
         if (_policy == CLASSIC) return f.type == COMMUNICATION ? 0 : 1;
         return (int)f.rclass;
     }
+    // RESOURCE policy with merge_minor: a minor entry (FuncWrap::minor) is too small to matter as a resource user and takes the
+    // class of the nearest other entry before it (after it, at the head of the vector).  The LayerNorm of a prefill layer (tens
+    // of microseconds between milliseconds of GEMMs) then neither ends the primary's run of MFMA-bound launches nor stops a
+    // secondary request whose prefill is being interleaved into HBM-bound windows.
+    bool _neutral(const FuncWrap& f) const { return _policy == RESOURCE && merge_minor && f.minor && f.type != COMMUNICATION; }
+    int _class_at(size_t idx) const {
+        const FuncWrap& f = FuncWrapVec.at(idx);
+        if (!_neutral(f)) return _class_of(f);
+        for (size_t i = idx; i-- > 0;)
+            if (!_neutral(FuncWrapVec[i])) return _class_of(FuncWrapVec[i]);
+        for (size_t i = idx + 1; i < FuncWrapVec.size(); ++i)
+            if (!_neutral(FuncWrapVec[i])) return _class_of(FuncWrapVec[i]);
+        return _class_of(f);
+    }
     const std::vector<float>* _profile(const FuncWrap& f) const {
         if (!profiling_decompse_res_dict) return nullptr;
         auto it = profiling_decompse_res_dict->find({f.name, batch_size, seq_len});
@@ -69,6 +84,7 @@ class Sample {
     void *start = nullptr, *stop = nullptr, *last_launch = nullptr;
     int batch_size, seq_len;
     int id = 0;
+    bool merge_minor = false;  // see _neutral(); false = every entry keeps its own class (the reference's behaviour)
     void* user = nullptr;  // owner's per-request context (buffers), opaque here
 
     Sample(std::vector<FuncWrap>& vec, const SubDict& sub_dict, int batch_size_, int seq_len_, int factor,
@@ -102,16 +118,16 @@ class Sample {
     }
 
     // class of the next launch and of the one after it
-    int next_class() const { return _sub_empty() ? _class_of(FuncWrapVec.at(exe_num)) : _class_of(_SubFuncWrapVec[_sub_exe_num].func); }
+    int next_class() const { return _sub_empty() ? _class_at(exe_num) : _class_of(_SubFuncWrapVec[_sub_exe_num].func); }
     layer_type type() const { return _sub_empty() ? FuncWrapVec.at(exe_num).type : GEMM; }  // init.h:151-157
 
     // true when the next launch is the last of a run of same-class launches  (init.h:99-129)
     bool is_switch() const {
         if (next_empty()) return true;
-        if (_sub_empty()) return _class_of(FuncWrapVec.at(exe_num)) != _class_of(FuncWrapVec.at(exe_num + 1));
+        if (_sub_empty()) return _class_at(exe_num) != _class_at(exe_num + 1);
         if (_sub_size() >= 2) return false;  // next two launches are pieces of the same GEMM
         const size_t after = (_sub_exe_num > 0) ? exe_num : exe_num + 1;
-        return _class_of(_SubFuncWrapVec[_sub_exe_num].func) != _class_of(FuncWrapVec.at(after));
+        return _class_of(_SubFuncWrapVec[_sub_exe_num].func) != _class_at(after);
     }
 
     // may not co-run with a primary segment of class `cls`  (init.h:131-149)
@@ -158,7 +174,7 @@ class Sample {
         return duration;
     }
 
-    recorder get_recording() const { return recorder{time_cpu_elapsed(), start, stop, batch_size, seq_len}; }
+    recorder get_recording() const { return recorder{time_cpu_elapsed(), start, stop, batch_size, seq_len, sample_arrive}; }
 
     // profiled duration of the next launch  (init.h:200-215)
     float duration(int is_main, float& time_planned) const {

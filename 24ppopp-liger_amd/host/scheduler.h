@@ -13,6 +13,7 @@
 // in-flight requests); the class notion is a policy (see sample.h); requests may carry decode steps; the report
 // adds p99; the loop ends when stop has been requested AND all work has drained.
 #pragma once
+#include <cmath>
 #include <algorithm>
 #include <atomic>
 #include <condition_variable>
@@ -52,6 +53,10 @@ struct TraceRequest {
 struct Report {
     int records = 0;
     double avg_latency_ms = 0, p99_latency_ms = 0, avg_gpu_ms = 0, avg_queue_ms = 0, total_duration_ms = 0, throughput = 0;
+    // arrival -> completion on one clock (not in the reference's report): the stop event's distance from an epoch event whose
+    // host time is known, minus the arrival's.  cpu + gpu time under-counts when a request's start event, launched on the
+    // second stream, is held up on the device behind the first stream's work.
+    double avg_e2e_ms = 0, p99_e2e_ms = 0;
 };
 
 // Pure arithmetic of the reference's report (schedule.h:325-348): latency_i = cpu_ms[i] + gpu_ms[i];
@@ -128,6 +133,9 @@ class Scheduler {
     // Entries < 0 are unmeasured and fall back to contention_factor.
     float contention_table[3][3] = {{-1.f, -1.f, -1.f}, {-1.f, -1.f, -1.f}, {-1.f, -1.f, -1.f}};
     class_policy policy = RESOURCE;
+    // RESOURCE policy: minor entries (FuncWrap::minor: normalisation, residual, cache append, row gather) take the class of
+    // the entry before them, so that they neither cut a prefill into many runs nor stop an interleaved one
+    bool merge_minor = false;
     split_axis axis = SPLIT_OUT_COLS;
     int seq_bucket = 1;               // durations are looked up at seq rounded up to a multiple of this
     int ignore_num = 20;              // warm-up records dropped from the report (schedule.h:327)
@@ -145,7 +153,7 @@ class Scheduler {
 
     Scheduler(MODELTYPE* model, const BertInitParam& BertParams_, const StaticInitParam& SParams_, T* input_, T* output_,
               const std::string& main_filename = "", const std::string& sub_filename = "")
-        : _model(model), SParams(SParams_), DParams0(-4), DParams1(0), BertParams(BertParams_), input(input_), output(output_) {
+        : _model(model), SParams(SParams_), DParams0(-4), DParams1(0, DParams0), BertParams(BertParams_), input(input_), output(output_) {
         DParams0.stream_id = 0;
         DParams1.stream_id = 1;
         if (!main_filename.empty()) MainFileToDict(main_filename, profiling_res_dict);
@@ -341,6 +349,7 @@ class Scheduler {
                                                         (const char*)out + ((size_t)(b + 1) * seq_len - 1) * row_bytes, row_bytes,
                                                         D.stream), "lg_memcpy_d2d_async");
                 }, "gather_last_token");
+                g.minor = true;
                 g.name = 900;
                 g.duration = 0.005f;
                 vec.push_back(g);
@@ -359,6 +368,7 @@ class Scheduler {
         }
         Sample* sample = new Sample(vec, profiling_decompse_res_dict, batch_size, seq_len, BertParams.factor, policy, axis);
         sample->user = ctx;
+        sample->merge_minor = merge_minor;
         {
             std::lock_guard<std::mutex> lk(_q_mutex);
             sample->id = _next_id++;
@@ -389,6 +399,7 @@ class Scheduler {
         }
         Sample* sample = new Sample(vec, profiling_decompse_res_dict, batch_size, past, BertParams.factor, policy, axis);
         sample->user = ctx;
+        sample->merge_minor = merge_minor;
         {
             std::lock_guard<std::mutex> lk(_q_mutex);
             sample->id = _next_id++;
@@ -490,6 +501,12 @@ class Scheduler {
     void run_stop() { _stop.store(true); }
     void reset_run() {
         _stop.store(false);
+        // epoch of the run: an event whose host time is known (the stream is idle, so it completes as it is recorded)
+        if (!_epoch_event) note_status(lg_event_create(&_epoch_event), "lg_event_create");
+        note_status(lg_stream_synchronize(DParams0.stream), "lg_stream_synchronize");
+        note_status(lg_event_record(_epoch_event, DParams0.stream), "lg_event_record");
+        note_status(lg_event_synchronize(_epoch_event), "lg_event_synchronize");
+        _epoch_host = std::chrono::steady_clock::now();
         for (auto& r : recs) { lg_event_destroy(r.start); lg_event_destroy(r.stop); }
         recs.clear();
         rounds = secondary_launches = splits = 0;
@@ -537,9 +554,29 @@ class Scheduler {
             gpu.push_back(ms);
             if (print) printf("request: %zu, CPU_Time: %f ms, CUDA_Time: %f ms. \n", i - skip, cpu.back(), gpu.back());
         }
+        // first start -> last stop (schedule.h:340-343 takes the last record's stop; a request that ran on the second stream may
+        // finish before the one retired ahead of it, so the latest stop is looked for)
         float total = 0.f;
-        if (recs.size() > skip) note_status(lg_event_elapsed_ms(&total, recs[skip].start, recs.back().stop), "lg_event_elapsed_ms");
+        for (size_t i = skip; i < recs.size(); ++i) {
+            float ms = 0.f;
+            note_status(lg_event_elapsed_ms(&ms, recs[skip].start, recs[i].stop), "lg_event_elapsed_ms");
+            total = std::max(total, ms);
+        }
         Report r = summarize_records(cpu, gpu, total);
+        if (_epoch_event && recs.size() > skip) {
+            std::vector<double> e2e;
+            for (size_t i = skip; i < recs.size(); ++i) {
+                float done = 0.f;
+                note_status(lg_event_elapsed_ms(&done, _epoch_event, recs[i].stop), "lg_event_elapsed_ms");
+                e2e.push_back((double)done - std::chrono::duration<double, std::milli>(recs[i].arrive - _epoch_host).count());
+            }
+            double sum = 0;
+            for (double v : e2e) sum += v;
+            r.avg_e2e_ms = sum / (double)e2e.size();
+            std::sort(e2e.begin(), e2e.end());
+            size_t rank = (size_t)std::ceil(0.99 * (double)e2e.size());
+            r.p99_e2e_ms = e2e[std::min(e2e.size() - 1, rank ? rank - 1 : 0)];
+        }
         if (print) {
             printf("Total_Duration: %f ms. \n", r.total_duration_ms);
             printf("Throughput: %f samples/s. \n", r.throughput);
@@ -551,6 +588,8 @@ class Scheduler {
     }
 
   private:
+    void* _epoch_event = nullptr;
+    std::chrono::steady_clock::time_point _epoch_host;
     std::vector<Sample*> _retired;
     int _pool_total = 0;
     std::vector<ReqCtx*> _all_ctx;

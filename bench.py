@@ -117,7 +117,10 @@ def bench_cfg4(capi, host, weight_layout):
         sched.profile(4, 512, 512, 1, 10)
         sched.profile_decode(32, 1024, 10)
         res = {"factor": factor}
-        for mode, name in ((host.MODE_SEQUENTIAL, "sequential"), (host.MODE_LIGER, "interleaved")):
+        res["streams_verified_concurrent"] = sched.streams_concurrent
+        for mode, name, merge in ((host.MODE_SEQUENTIAL, "sequential", False), (host.MODE_LIGER, "interleaved", False),
+                                  (host.MODE_LIGER, "interleaved_minor_merged", True)):
+            sched.set_merge_minor(merge)
             best = None
             for _ in range(3):
                 sched.serve_decode(32, 1000, 8)
@@ -128,6 +131,7 @@ def bench_cfg4(capi, host, weight_layout):
             res[name] = {"makespan_ms": round(best["total_duration_ms"], 4), "secondary_launches": best["secondary_launches"],
                          "splits": best["splits"], "rounds": best["rounds"]}
         res["speedup"] = round(res["sequential"]["makespan_ms"] / res["interleaved"]["makespan_ms"], 4)
+        res["speedup_minor_merged"] = round(res["sequential"]["makespan_ms"] / res["interleaved_minor_merged"]["makespan_ms"], 4)
         out.append(res)
     return {"workload": "cfg4: prefill B4 S512 (split by token rows) || decode B32 L1024 x 8 steps, one layer shard", "results": out}
 
@@ -153,17 +157,23 @@ def bench_cfg5(capi, host, weight_layout, n_requests):
     for lam in (4.0, 8.0, 16.0):
         trace = host.make_poisson_trace(lam, n_requests, 1, 128, 1024, 64, 32, 0)
         row = {"lambda_req_s": lam, "requests": n_requests}
-        for mode, name, measured in ((host.MODE_SEQUENTIAL, "scheduling_off", False), (host.MODE_LIGER, "scheduling_on", False),
-                                     (host.MODE_LIGER, "scheduling_on_measured_contention", True)):
+        for mode, name, measured, merge_minor in ((host.MODE_SEQUENTIAL, "scheduling_off", False, False), (host.MODE_LIGER, "scheduling_on", False, False),
+                                                 (host.MODE_LIGER, "scheduling_on_measured_contention", True, False),
+                                                 (host.MODE_LIGER, "scheduling_on_minor_kernels_merged", False, True)):
             sched.set_contention(0, 1, table["mfma_main_hbm_sub"] if measured else -1.0)
             sched.set_contention(1, 0, table["hbm_main_mfma_sub"] if measured else -1.0)
+            sched.set_merge_minor(merge_minor)
             r = sched.run_trace(trace, mode)
-            row[name] = {"mean_latency_ms": round(r["avg_latency_ms"], 3), "p99_latency_ms": round(r["p99_latency_ms"], 3),
+            # latency = arrival -> completion on one clock; the reference's sum (first launch - arrival) + (start event -> stop
+            # event) is kept beside it: it under-counts when a start event is held up on the device
+            row[name] = {"mean_latency_ms": round(r["avg_e2e_ms"], 3), "p99_latency_ms": round(r["p99_e2e_ms"], 3),
+                         "mean_cpu_plus_gpu_ms": round(r["avg_latency_ms"], 3),
                          "mean_gpu_ms": round(r["avg_gpu_ms"], 3), "mean_queue_ms": round(r["avg_queue_ms"], 3),
                          "throughput_req_s": round(r["throughput"], 3), "records": r["records"],
                          "secondary_launches": r["secondary_launches"], "splits": r["splits"], "profile_misses": r["profile_misses"]}
         out.append(row)
     return {"workload": "cfg5: 4 layer shards, Poisson arrivals, prompts U[128,1024] rounded to 64, 32 decode tokens", "profile_seconds": round(prof_s, 1),
+            "streams_verified_concurrent": sched.streams_concurrent,
             "contention_measurement": {k: (round(v, 4) if isinstance(v, float) else v) for k, v in meas.items()},
             "contention_table": {k: round(v, 4) for k, v in table.items()}, "results": out}
 

@@ -53,6 +53,12 @@ int lg_stream_create(void** stream);          /* non-blocking stream, default pr
  * the reference gives its streams (context.h:28-29, schedule.h:54-55): on this platform the two streams of the scheduler
  * are separated in space, not by priority. */
 int lg_stream_create_cu_mask(void** stream, const unsigned* cu_mask, int mask_words);
+/* Non-blocking stream that is verified, by measurement, to run kernels at the same time as `other` (the scheduler's
+ * second stream, schedule.h:54-55).  HIP multiplexes a process's streams onto a few hardware queues and two streams
+ * that share one execute strictly in turn; candidates are created and probed (a 0.4 ms one-wave spin on `other` next
+ * to a one-wave kernel on the candidate) until one overlaps.  *verified = 1 if such a stream was found, 0 if the
+ * returned stream is an unverified fallback. */
+int lg_stream_create_concurrent(void** stream, void* other, int* verified);
 int lg_stream_destroy(void* stream);
 int lg_stream_synchronize(void* stream);
 int lg_stream_wait_event(void* stream, void* event);

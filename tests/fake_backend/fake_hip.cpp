@@ -123,6 +123,11 @@ int lg_stream_create(void** stream) {
     *stream = s;
     return LG_OK;
 }
+int lg_stream_create_concurrent(void** stream, void* other, int* verified) {
+    if (!stream || !other) return LG_ERR_INVALID;
+    if (verified) *verified = 1;  // virtual streams always overlap
+    return lg_stream_create(stream);
+}
 int lg_stream_create_cu_mask(void** stream, const unsigned* cu_mask, int mask_words) {
     if (!stream || !cu_mask || mask_words <= 0) return LG_ERR_INVALID;
     bool any = false;

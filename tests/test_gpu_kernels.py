@@ -178,3 +178,36 @@ def test_cu_masked_stream_runs_kernels(dev, po):
     empty = (C.c_uint * 8)(*([0] * 8))
     s2 = C.c_void_p()
     assert lib.lg_stream_create_cu_mask(C.byref(s2), empty, 8) == 1  # LG_ERR_INVALID
+
+
+def test_second_stream_is_verified_to_run_next_to_the_first(dev, po):
+    """lg_stream_create_concurrent hands out a stream whose kernels overlap with the given stream's (measured by the
+    library) even when the process already holds more streams than there are hardware queues; the stream computes like any
+    other; null arguments are refused."""
+    import ctypes as C
+    lib = dev.lib
+    crowd = []
+    for _ in range(6):  # more streams than the default four hardware queues of a process
+        s = C.c_void_p()
+        assert lib.lg_stream_create(C.byref(s)) == 0
+        crowd.append(s)
+    first, second, verified = crowd[2], C.c_void_p(), C.c_int(-1)
+    assert lib.lg_stream_create_concurrent(C.byref(second), first, C.byref(verified)) == 0, dev.capi.last_error()
+    try:
+        assert verified.value == 1
+        m, n = 64, 512
+        x = rnd(po, m * n, 4, 0).reshape(m, n)
+        g = rnd(po, n, 5, 0, 0.1, 1.0)
+        b = rnd(po, n, 6, 0, 0.1)
+        dx, dg, db = dev.up(x, 0), dev.up(g, 0), dev.up(b, 0)
+        out = dev.empty((m, n), 0)
+        dev.down(out)
+        ptr = lambda t: C.c_void_p(t.data_ptr())
+        assert lib.lg_layer_norm_f32(ptr(dx), ptr(dg), ptr(db), ptr(out), m, n, second) == 0, dev.capi.last_error()
+        assert lib.lg_stream_synchronize(second) == 0
+        assert max_rel_err(dev.down(out), po.layer_norm(x, g, b, 0)) < tol(0)
+    finally:
+        assert lib.lg_stream_destroy(second) == 0
+        for s in crowd:
+            assert lib.lg_stream_destroy(s) == 0
+    assert lib.lg_stream_create_concurrent(C.byref(second), None, C.byref(verified)) == 1  # LG_ERR_INVALID

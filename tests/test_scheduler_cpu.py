@@ -344,3 +344,42 @@ def test_realtime_trace_replay_drains(fake):
         r = s.run_trace(trace, mode)
         assert r["records"] == 12
         assert len([e for e in fake.trace() if e["name"] == "attn_prefill"]) == 12
+
+
+def test_merged_minor_kernels_keep_a_prefill_in_one_run(fake):
+    """RESOURCE policy with merge_minor: minor entries (the LayerNorms between a prefill's GEMMs, the row gather before the
+    decode steps) take the class of the entry before them.  A prefill is then one run of MFMA-bound launches instead of four
+    per layer, and a prefill that waits behind a request in its decode steps (HBM-bound) is interleaved past its first
+    LayerNorm.  Every entry is still launched exactly once and every request keeps its own order."""
+    host = fake.host
+    m = small_model(host, layers=2)
+
+    def run(merge, requests):
+        s = host.Scheduler(m, contention_factor=0.8, policy=host.POLICY_RESOURCE, seq_bucket=16, pool_count=3, ctx_batch=1)
+        s.profile(1, 48, 64, 16, 2)
+        for past in (48, 64, 80):
+            s.profile_decode(1, past, 2)
+        s.set_merge_minor(merge)
+        fake.reset()
+        for r in requests:
+            s.serve(*r)
+        rep = s.run_queued(host.MODE_LIGER)
+        return rep, fake.trace()
+
+    # one prefill-only request: 2 layers x (5 MFMA, LN, 2 MFMA, LN) = 8 runs; one run when the LayerNorms are merged
+    plain, t0 = run(False, [(1, 64, 0)])
+    merged, t1 = run(True, [(1, 64, 0)])
+    assert plain["rounds"] == 8 and merged["rounds"] == 1
+    assert [e["name"] for e in t0] == [e["name"] for e in t1] and len(t1) == 2 * 9
+    # A: prefill + 3 decode steps (one MFMA run, then one HBM run), B: prefill only, queued behind it
+    reqs = [(1, 48, 3), (1, 64, 0)]
+    plain, t0 = run(False, reqs)
+    merged, t1 = run(True, reqs)
+    assert plain["records"] == merged["records"] == 2
+    assert sorted(e["name"] for e in t0) == sorted(e["name"] for e in t1)     # the same launches, each exactly once
+    assert merged["rounds"] < plain["rounds"]
+    # without merging B's interleaving stops at its first LayerNorm at the latest (5 launches); with it B goes on past it
+    assert 0 < plain["secondary_launches"] <= 5
+    assert merged["secondary_launches"] > 5
+    b_rows = [e for e in t1 if (e["name"] in ("gemm", "gemm_fused") and e["n"] == 64) or (e["name"] == "layer_norm" and e["m"] == 64)]
+    assert all(y["start"] >= x["end"] - 1e-12 for x, y in zip(b_rows, b_rows[1:]))   # B's own order is kept
