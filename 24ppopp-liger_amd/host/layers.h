@@ -14,7 +14,6 @@
 //   * optional assemblies: pre-LN with residuals built from the reference's fused residual kernels, a fused
 //     assembly (epilogue-fused GEMMs + one attention kernel) and a decode step over a KV cache.
 #pragma once
-#include <cstdlib>
 #include <cmath>
 #include <map>
 #include <memory>
