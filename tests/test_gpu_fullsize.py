@@ -108,3 +108,34 @@ def test_full_size_decode_attention_against_oracle(dev, po):
     dev.call("lg_attn_decode_f16", dev.up(q, 1), dkc[:, :, perm].contiguous(), dvc[:, :, perm].contiguous(), out2, ws, Bd, h, D, L, L,
              float(scalar))
     assert max_rel_err(dev.down(out2), got) < 2e-3
+
+
+@pytest.mark.parametrize("batch", [2, 8])
+def test_full_size_decode_step_against_oracle(dev, po, host, batch):
+    """One decode step of the full-size layer shard (fused assembly) after a short prefill that fills the KV cache:
+    batch 2 takes the matrix-vector kernel, batch 8 the weight-streaming kernel with unsliced blocks, both with the
+    grouped Q/K/V launch whose epilogues append the new K/V rows to the cache.  The oracle repeats prefill projections
+    and the decoder step on the downloaded weights."""
+    S, Lmax = 64, 128
+    m = host.Model(1, batch, S, 96, D, layer_num=1, world_size=2, ffn_inner=2 * F, norm_mode=0, causal=True, fused=True,
+                   max_cache_len=Lmax, weight_layout=1, seed=1)
+    w = {k[len("layer0."):]: v for k, v in m.download_params().items() if k.startswith("layer0.")}
+    x = po.fill_normal(batch * S * H, 1, 99, 0.0, 1.0, 1).reshape(batch * S, H)
+    dx, dy = dev.up(x, 1), dev.empty((batch * S, H), 1)
+    m.run(dx.data_ptr(), dy.data_ptr(), batch, S, None, dev.stream, cache_slot=0)
+    # oracle-side cache from the same prefill input
+    k = po.gemm(x, w["wk"], 1)
+    v = po.gemm(x, w["wv"], 1)
+    _, kb, vb = po.add_qkv_bias_transpose(k, w["bk"], k, w["bk"], v, w["bv"], batch, S, 48, D, 1)
+    kc = np.zeros((batch, 48, Lmax, D), dtype=np.float32)
+    vc = np.zeros_like(kc)
+    kc[:, :, :S] = kb
+    vc[:, :, :S] = vb
+    shape = dict(batch=batch, seq=S, hidden=H, head_num=48, size_per_head=D, ffn_inner=F, causal=1, norm_mode=0, dtype=1)
+    tok = po.fill_normal(batch * H, 1, 100, 0.0, 1.0, 1).reshape(batch, H)
+    for step in range(2):
+        dt_in, dt_out = dev.up(tok, 1), dev.empty((batch, H), 1)
+        m.run_decode(dt_in.data_ptr(), dt_out.data_ptr(), batch, S + step, 0, None, dev.stream)
+        ref = po.decoder_step(shape, w, tok, kc, vc, S + step)   # also appends this step's K/V rows to kc / vc
+        assert max_rel_err(dev.down(dt_out), ref) < 1e-2
+        tok = po.round_f16(ref)
