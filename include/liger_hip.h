@@ -57,7 +57,7 @@ int lg_stream_create_cu_mask(void** stream, const unsigned* cu_mask, int mask_wo
  * second stream, schedule.h:54-55).  HIP multiplexes a process's streams onto a few hardware queues and two streams
  * that share one execute strictly in turn; candidates are created and probed (a 0.4 ms one-wave spin on `other` next
  * to a one-wave kernel on the candidate) until one overlaps.  *verified = 1 if such a stream was found, 0 if the
- * returned stream is an unverified fallback. */
+ * returned stream is an unverified fallback.  `other` must be a created stream (not the null stream). */
 int lg_stream_create_concurrent(void** stream, void* other, int* verified);
 int lg_stream_destroy(void* stream);
 int lg_stream_synchronize(void* stream);

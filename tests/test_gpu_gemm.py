@@ -263,3 +263,40 @@ def test_grouped_qkv_gemm_equals_three_plain_calls(dev, po, M, transa):
     bad = arr([dA[0].data_ptr(), 0, dA[2].data_ptr()])
     assert dev.call_rc("lg_gemm_fused_grouped_f16", transa, N, M, K, 3, bad, lda, dX, K, arr([dst(grouped, t) for t in range(3)]),
                        (C.c_int * 3)(*ldc), dev.capi.EPI_BIAS_HEADS, arr([b.data_ptr() for b in dB]), 1, d, h) != 0
+
+
+@pytest.mark.parametrize("M,count,epi", [(1, 2, "bias"), (4, 1, "gelu"), (16, 2, "bias"), (40, 3, "none"), (16, 3, "gelu")])
+def test_grouped_gemm_other_epilogues_and_counts(dev, po, M, count, epi):
+    """Groups of one, two and three problems with the plain, bias and bias + GELU epilogues and different leading
+    dimensions of the outputs: equal to the plain fused calls (up to the fp32 summation order on the weight-streaming
+    kernel) and to the oracle."""
+    import ctypes as C
+    N, K = 6144, 2048
+    kind = {"none": dev.capi.EPI_NONE, "bias": dev.capi.EPI_BIAS, "gelu": dev.capi.EPI_BIAS_GELU}[epi]
+    X = rnd(po, M * K, 60, 1).reshape(M, K)
+    dX = dev.up(X, 1)
+    Ws = [rnd(po, K * N, 61 + t, 1, 0.05).reshape(K, N) for t in range(count)]
+    bs = [rnd(po, N, 64 + t, 1, 0.3) for t in range(count)]
+    dA = [dev.up(np.ascontiguousarray(W.T), 1) for W in Ws]
+    dB = [dev.up(b, 1) for b in bs]
+    ldc = [N + 8 * t for t in range(count)]          # outputs with padded rows
+    plain = [dev.empty((M, ldc[t]), 1) for t in range(count)]
+    grouped = [dev.empty((M, ldc[t]), 1) for t in range(count)]
+    for t in plain + grouped:
+        t.zero_()
+    for t in range(count):
+        dev.call("lg_gemm_fused_f16", 1, N, M, K, dA[t], K, dX, K, plain[t], ldc[t], kind, dB[t] if epi != "none" else None, 0, 0, 0)
+    arr = lambda ptrs: (C.c_void_p * count)(*ptrs)
+    dev.call("lg_gemm_fused_grouped_f16", 1, N, M, K, count, arr([a.data_ptr() for a in dA]), K, dX, K,
+             arr([g.data_ptr() for g in grouped]), (C.c_int * count)(*ldc), kind,
+             arr([b.data_ptr() for b in dB]) if epi != "none" else None, 0, 0, 0)
+    for t in range(count):
+        got, ref_gpu = dev.down(grouped[t]), dev.down(plain[t])
+        assert np.all(got[:, N:] == 0)                                   # the padding is not written
+        if M <= 4:
+            assert np.array_equal(got, ref_gpu)
+        else:
+            assert max_rel_err(got, ref_gpu) < 1e-3
+        y = po.gemm(X, Ws[t], 1)
+        ref = y if epi == "none" else (po.round_f16(y + bs[t]) if epi == "bias" else po.add_bias_gelu(y.copy(), bs[t], 1))
+        assert max_rel_err(got[:, :N], ref) < 4e-3
