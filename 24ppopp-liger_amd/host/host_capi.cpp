@@ -67,11 +67,27 @@ struct SchedT : SchedBase {
         s->profile(bs, bs + 1, seq_lo, seq_hi + 1, "", "", seq_step, itr);
     }
     void profile_decode(int bs, int past, int itr) override { s->profile_decode(bs, past, itr); }
+    // The measured contention table travels in the main profile file inside the reference's record schema (utils.h:106-127):
+    // {"kernel_name": -1, "batch_size": primary class, "seq_len": secondary class, "duration": fraction}.
     bool save(const char* a, const char* b) override {
-        return MainDictToFile(s->profiling_res_dict, a) && SubDictToFile(s->profiling_decompse_res_dict, b);
+        auto dict = s->profiling_res_dict;
+        for (int m = 0; m < 3; ++m)
+            for (int c = 0; c < 3; ++c)
+                if (s->contention_table[m][c] >= 0.f) dict[{-1, m, c}] = s->contention_table[m][c];
+        return MainDictToFile(dict, a) && SubDictToFile(s->profiling_decompse_res_dict, b);
     }
     bool load(const char* a, const char* b) override {
-        return MainFileToDict(a, s->profiling_res_dict) && SubFileToDict(b, s->profiling_decompse_res_dict);
+        if (!MainFileToDict(a, s->profiling_res_dict) || !SubFileToDict(b, s->profiling_decompse_res_dict)) return false;
+        for (auto it = s->profiling_res_dict.begin(); it != s->profiling_res_dict.end();) {
+            if (it->first.kernel_name == -1) {
+                const int m = it->first.batch_size, c = it->first.seq_len;
+                if (m >= 0 && m < 3 && c >= 0 && c < 3) s->contention_table[m][c] = it->second;
+                it = s->profiling_res_dict.erase(it);
+            } else {
+                ++it;
+            }
+        }
+        return true;
     }
     Report run(int mode, const std::vector<TraceRequest>& trace, int* counters) override {
         s->reset_run();

@@ -290,6 +290,20 @@ def test_profile_json_roundtrip_and_failure_paths(fake, tmp_path):
     s2.load(a, b)
     for e in main:
         assert abs(s2.lookup(e["kernel_name"], e["batch_size"], e["seq_len"]) - e["duration"]) < 1e-6
+    # a measured contention table travels in the main file as records with kernel_name -1 (same schema) and comes back
+    s.set_contention(MFMA, HBM, 0.55)
+    s.set_contention(HBM, MFMA, 0.25)
+    s.save(a, b)
+    main2 = json.load(open(a))
+    extra = sorted((e["batch_size"], e["seq_len"], round(e["duration"], 6)) for e in main2 if e["kernel_name"] == -1)
+    assert extra == [(MFMA, HBM, 0.55), (HBM, MFMA, 0.25)] and len(main2) == len(main) + 2
+    s3 = host.Scheduler(m, contention_factor=0.8, pool_count=0)
+    assert s3.contention(MFMA, HBM) == pytest.approx(0.8)          # unmeasured: the constant factor
+    s3.load(a, b)
+    assert s3.contention(MFMA, HBM) == pytest.approx(0.55) and s3.contention(HBM, MFMA) == pytest.approx(0.25)
+    assert s3.lookup(-1, MFMA, HBM) == 0.0                         # not left behind as a kernel entry
+    s.set_contention(MFMA, HBM, -1.0)
+    s.set_contention(HBM, MFMA, -1.0)
     # a file in the reference's own writer format (trailing-comma-free, "duration": [ ... ] with a space)
     open(a, "w").write('[{"kernel_name":0,"batch_size":2,"seq_len":64,"duration":1.5},{"kernel_name":1,"batch_size":2,"seq_len":64,"duration":0.25}]')
     open(b, "w").write('[{"kernel_name":0,"batch_size":2,"seq_len":64,"duration": [0.2,0.4,0.6]}]')
