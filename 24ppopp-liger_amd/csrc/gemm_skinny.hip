@@ -128,8 +128,8 @@ __global__ __launch_bounds__(256) void gemm_skinny_nk_kernel(GemmArgs g, int ksl
 // ---- whole K in one block ------------------------------------------------------------------------------------------------
 // When N alone gives enough blocks K is not sliced at all: a block = NWV waves x 16 output features walks the whole of K, the
 // epilogue is applied to the accumulators, and there are no fp32 partials and no second kernel.  A wave owns one 16-feature
-// MFMA tile (8 loads per chunk), so its rolling pipeline is DEPTH chunks deep: 4 waves x 2 chunks or 2 waves x 4 chunks
-// keep the same 64 KiB of weight loads in flight per block.
+// MFMA tile (8 loads per chunk), so its rolling pipeline is DEPTH chunks deep: two chunks (16 loads per lane, as in the sliced
+// kernel) for blocks of 4, 6 or 8 waves, four chunks for the 2-wave block, which then keeps the 64 KiB of a 4-wave block in flight.
 template <int MT, int EPI, int NWV, int DEPTH>
 __global__ __launch_bounds__(64 * NWV) void gemm_skinny_direct_kernel(GemmArgs g, GemmGroup grp) {
     constexpr int THREADS = 64 * NWV;
