@@ -19,6 +19,8 @@ SHAPES = [(64, 256, 256), (128, 128, 32), (130, 136, 72), (1, 8, 8), (33, 70, 19
           (256, 256, 64), (512, 768, 256), (256, 512, 1024), (1024, 2048, 192), (2048, 256, 128),
           # 256 x 192 tiles (weights stored [out, in] only) and 256 x 128 tiles (both layouts)
           (256, 384, 128), (512, 576, 192), (256, 1344, 64), (256, 640, 128), (512, 128, 192), (768, 1152, 320),
+          # tile counts that take the region mappings of the workgroups: 8 x 32 tiles and 16 x 48 tiles
+          (2048, 8192, 64), (4096, 12288, 64),
           # token counts that are not a multiple of the tile: the pipelined kernel pads the last row of tiles
           (320, 256, 128), (448, 384, 192), (1000, 512, 256), (200, 256, 64), (161, 768, 128), (65, 256, 192), (100, 384, 64),
           # few tokens, many features: the weight-streaming split-K kernel (weights stored [out, in])
