@@ -17,63 +17,90 @@
 
 namespace lg {
 
-constexpr int DEC_UNROLL = 8;
+// Sequences of one launch that do not share a length or do not sit in consecutive cache slots (decode steps of different
+// requests batched into one launch): per-sequence cache slot and valid length, passed by value with the launch.
+constexpr int DEC_MAX_SEQS = LG_ATTN_DECODE_MAX_SEQS;
+struct DecodeSeqs {
+    int slot[DEC_MAX_SEQS];
+    int len[DEC_MAX_SEQS];
+};
 
 // partial result of one (b, head, split): max, sum, weighted V (fp32)
 //   workspace layout: [B*h][nsplit][2 + D] floats
-template <int D>
+// A key row of D halves is D/8 16-byte chunks; lane `sub` of an LPK-lane group holds chunks sub, sub + LPK, ... (CPL of
+// them), so one wave-wide load covers 64 / LPK keys with LPK * 16 contiguous bytes of each (D = 128: LPK 16, whole rows;
+// D = 64: LPK 8; D = 96: LPK 4 x 3 chunks).
+template <int D, int LPK, int UNROLL, bool VARLEN>
 __global__ __launch_bounds__(256) void attn_decode_kernel(const half_t* __restrict__ q, const half_t* __restrict__ kc,
                                                           const half_t* __restrict__ vc, half_t* out, float* ws,
-                                                          int len, int max_len, int nsplit, float scalar) {
-    constexpr int LPK = D / 8;        // lanes per key row
-    constexpr int KPL = 64 / LPK;     // keys per wave-wide load
+                                                          int len, int max_len, int nsplit, float scalar, int head_num,
+                                                          DecodeSeqs seqs) {
+    constexpr int CPL = D / (8 * LPK);  // 16-byte chunks per lane and key
+    constexpr int KPL = 64 / LPK;       // keys per wave-wide load
+    static_assert(CPL * LPK * 8 == D, "D must be LPK * CPL * 8");
     __shared__ float s_m[4 * KPL], s_l[4 * KPL];
     __shared__ float s_acc[4 * KPL][D];
 
     const int bh = blockIdx.x, split = blockIdx.y;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int grp = lane / LPK, sub = lane % LPK;
+    int64_t cache_row = bh;  // (cache slot, head) row of the caches
+    if (VARLEN) {
+        const int b = bh / head_num, head = bh % head_num;
+        len = seqs.len[b];
+        cache_row = (int64_t)seqs.slot[b] * head_num + head;
+    }
 
     // key range of this block, then of this wave (contiguous quarters)
     const int per_split = (len + nsplit - 1) / nsplit;
-    const int s_begin = split * per_split;
+    const int s_begin = min(len, split * per_split);
     const int s_end = min(len, s_begin + per_split);
     const int per_wave = (s_end - s_begin + 3) / 4;
-    const int w_begin = s_begin + wave * per_wave;
+    const int w_begin = min(s_end, s_begin + wave * per_wave);
     const int w_end = min(s_end, w_begin + per_wave);
 
-    float qf[8];
-    {
-        half8_t qv = *reinterpret_cast<const half8_t*>(q + (int64_t)bh * D + sub * 8);
+    float qf[CPL][8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) qf[j] = (float)qv[j] * scalar;
+    for (int c = 0; c < CPL; ++c) {
+        half8_t qv = *reinterpret_cast<const half8_t*>(q + (int64_t)bh * D + (c * LPK + sub) * 8);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) qf[c][j] = (float)qv[j] * scalar;
     }
-    const half_t* kbase = kc + (int64_t)bh * max_len * D + sub * 8;
-    const half_t* vbase = vc + (int64_t)bh * max_len * D + sub * 8;
+    const half_t* kbase = kc + cache_row * max_len * D + sub * 8;
+    const half_t* vbase = vc + cache_row * max_len * D + sub * 8;
 
     float m_run = -1e30f, l_run = 0.f;
-    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-
-    for (int base = w_begin; base < w_end; base += KPL * DEC_UNROLL) {
-        half8_t kv[DEC_UNROLL], vv[DEC_UNROLL];
+    float acc[CPL][8];
 #pragma unroll
-        for (int u = 0; u < DEC_UNROLL; ++u) {
+    for (int c = 0; c < CPL; ++c)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[c][j] = 0.f;
+
+    for (int base = w_begin; base < w_end; base += KPL * UNROLL) {
+        half8_t kv[UNROLL][CPL], vv[UNROLL][CPL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
             const int key = base + u * KPL + grp;
-            if (key < w_end) {
-                kv[u] = *reinterpret_cast<const half8_t*>(kbase + (int64_t)key * D);
-                vv[u] = *reinterpret_cast<const half8_t*>(vbase + (int64_t)key * D);
-            } else {
-                kv[u] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-                vv[u] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) {
+                if (key < w_end) {
+                    kv[u][c] = *reinterpret_cast<const half8_t*>(kbase + (int64_t)key * D + c * LPK * 8);
+                    vv[u][c] = *reinterpret_cast<const half8_t*>(vbase + (int64_t)key * D + c * LPK * 8);
+                } else {
+                    kv[u][c] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+                    vv[u][c] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+                }
             }
         }
-        float s[DEC_UNROLL];
+        float s[UNROLL];
         float m_new = m_run;
 #pragma unroll
-        for (int u = 0; u < DEC_UNROLL; ++u) {
+        for (int u = 0; u < UNROLL; ++u) {
             float p = 0.f;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) p = fmaf(qf[j], (float)kv[u][j], p);
+            for (int c = 0; c < CPL; ++c)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) p = fmaf(qf[c][j], (float)kv[u][c][j], p);
 #pragma unroll
             for (int o = LPK / 2; o > 0; o >>= 1) p += __shfl_xor(p, o, 64);
             const int key = base + u * KPL + grp;
@@ -83,14 +110,18 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const half_t* __restri
         const float corr = __expf(m_run - m_new);
         l_run *= corr;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[j] *= corr;
+        for (int c = 0; c < CPL; ++c)
 #pragma unroll
-        for (int u = 0; u < DEC_UNROLL; ++u) {
+            for (int j = 0; j < 8; ++j) acc[c][j] *= corr;
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
             const int key = base + u * KPL + grp;
             const float p = (key < w_end) ? __expf(s[u] - m_new) : 0.f;
             l_run += p;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) acc[j] = fmaf(p, (float)vv[u][j], acc[j]);
+            for (int c = 0; c < CPL; ++c)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc[c][j] = fmaf(p, (float)vv[u][c][j], acc[c][j]);
         }
         m_run = m_new;
     }
@@ -99,7 +130,9 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const half_t* __restri
     const int slot = wave * KPL + grp;
     if (sub == 0) { s_m[slot] = m_run; s_l[slot] = l_run; }
 #pragma unroll
-    for (int j = 0; j < 8; ++j) s_acc[slot][sub * 8 + j] = acc[j];
+    for (int c = 0; c < CPL; ++c)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s_acc[slot][(c * LPK + sub) * 8 + j] = acc[c][j];
     __syncthreads();
     if (threadIdx.x < D) {
         float m = -1e30f;
@@ -135,6 +168,11 @@ __global__ void attn_decode_merge_kernel(const float* __restrict__ ws, half_t* o
     out[(int64_t)bh * D + t] = (half_t)(o / (l + 1e-6f));
 }
 
+// Split-KV partial slots (b, head, split) any launch can need.  decode_nsplit only doubles the split count while
+// bh * ns < 1024, so whenever partials are used at all (ns > 1) there are fewer than 2048 of them -- whatever the batch.
+constexpr int DEC_MAX_SLOTS = 2048;
+constexpr int DEC_MAX_D = 128;
+
 static int decode_nsplit(int bh, int len) {
     // aim for >= 1024 blocks (4 per CU on 256 CUs) while keeping >= 128 keys per block
     int ns = 1;
@@ -142,18 +180,59 @@ static int decode_nsplit(int bh, int len) {
     return ns;
 }
 
-// q_out[b,head,:] = Q[b, head*d ..] + bq;  caches[b,head,pos,:] = K/V + bias
+template <int D, int LPK, int UNROLL>
+static void launch_decode(const half_t* q, const half_t* kc, const half_t* vc, half_t* out, float* ws, int bh, int head_num,
+                          int len, int max_len, int ns, float scalar, const DecodeSeqs* seqs, hipStream_t st) {
+    const dim3 grid(bh, ns);
+    if (seqs)
+        hipLaunchKernelGGL((attn_decode_kernel<D, LPK, UNROLL, true>), grid, dim3(256), 0, st, q, kc, vc, out, ws, len, max_len, ns, scalar, head_num, *seqs);
+    else
+        hipLaunchKernelGGL((attn_decode_kernel<D, LPK, UNROLL, false>), grid, dim3(256), 0, st, q, kc, vc, out, ws, len, max_len, ns, scalar, head_num, DecodeSeqs{});
+    if (ns > 1) hipLaunchKernelGGL((attn_decode_merge_kernel<D>), dim3(bh), dim3(D), 0, st, (const float*)ws, out, ns);
+}
+
+// Argument checks and launch shared by the entry points.  `seqs` = per-sequence slots and lengths or nullptr (all
+// sequences `len` long, sequence b in cache slot b); ws_capacity_slots = partial slots the workspace holds.
+static int attn_decode_common(const char* what, const void* q, const void* k_cache, const void* v_cache, void* out, float* ws,
+                              int64_t ws_capacity_slots, int batch, int head_num, int size_per_head, int len, int max_len,
+                              float scalar, const DecodeSeqs* seqs, hipStream_t st) {
+    if (batch < 0 || head_num <= 0 || len <= 0 || max_len < len) { set_error("%s: bad shape (len=%d max_len=%d)", what, len, max_len); return LG_ERR_INVALID; }
+    if (size_per_head != 64 && size_per_head != 96 && size_per_head != 128) { set_error("%s: size_per_head must be 64, 96 or 128", what); return LG_ERR_INVALID; }
+    if (batch == 0) return LG_OK;
+    if (!q || !k_cache || !v_cache || !out) { set_error("%s: null pointer", what); return LG_ERR_INVALID; }
+    if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache)) { set_error("%s: pointers must be 16-byte aligned", what); return LG_ERR_INVALID; }
+    if ((int64_t)batch * head_num > 0x7fffffff) { set_error("%s: batch * head_num too large", what); return LG_ERR_INVALID; }
+    const int bh = batch * head_num;
+    const int ns = decode_nsplit(bh, len);
+    if (ns > 1 && !ws) { set_error("%s: workspace required", what); return LG_ERR_INVALID; }
+    if (ns > 1 && (int64_t)bh * ns > ws_capacity_slots) {
+        set_error("%s: %d x %d split-KV partials exceed the workspace's %lld slots", what, bh, ns, (long long)ws_capacity_slots);
+        return LG_ERR_INVALID;
+    }
+    scalar = (float)(half_t)scalar;
+    const half_t *qh = (const half_t*)q, *kh = (const half_t*)k_cache, *vh = (const half_t*)v_cache;
+    if (size_per_head == 128) launch_decode<128, 16, 8>(qh, kh, vh, (half_t*)out, ws, bh, head_num, len, max_len, ns, scalar, seqs, st);
+    else if (size_per_head == 96) launch_decode<96, 4, 4>(qh, kh, vh, (half_t*)out, ws, bh, head_num, len, max_len, ns, scalar, seqs, st);
+    else launch_decode<64, 8, 8>(qh, kh, vh, (half_t*)out, ws, bh, head_num, len, max_len, ns, scalar, seqs, st);
+    return check_launch(what);
+}
+
+// q_out[b,head,:] = Q[b, head*d ..] + bq;  caches[slot_b,head,pos_b,:] = K/V + bias.  VARLEN: slot_b, pos_b come per sequence
+// (seqs.slot / seqs.len), otherwise slot_b = b and pos_b = pos.
+template <bool VARLEN>
 __global__ __launch_bounds__(256) void kv_append_kernel(half_t* q_out, half_t* kc, half_t* vc, const half_t* __restrict__ Q,
                                                         const half_t* __restrict__ bq, const half_t* __restrict__ K,
                                                         const half_t* __restrict__ bk, const half_t* __restrict__ V,
                                                         const half_t* __restrict__ bv, int head_num, int d, int pos,
-                                                        int max_len, int64_t total_vec) {
+                                                        int max_len, int64_t total_vec, DecodeSeqs seqs) {
     const int dv = d / 8, nv = head_num * dv;
     for (int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; v < total_vec; v += (int64_t)gridDim.x * blockDim.x) {
         const int64_t b = v / nv;
         const int c = (int)(v % nv), head = c / dv, e = c % dv;
         const int64_t si = b * (int64_t)head_num * d + (int64_t)c * 8;
-        const int64_t ci = ((b * head_num + head) * (int64_t)max_len + pos) * d + (int64_t)e * 8;
+        const int64_t row = VARLEN ? seqs.slot[b] : b;
+        const int p = VARLEN ? seqs.len[b] : pos;
+        const int64_t ci = ((row * head_num + head) * (int64_t)max_len + p) * d + (int64_t)e * 8;
         typedef Vec16<half_t> Vh;
         Vh a, bb, o;
         a = *reinterpret_cast<const Vh*>(Q + si); bb = *reinterpret_cast<const Vh*>(bq + (int64_t)c * 8);
@@ -171,6 +250,31 @@ __global__ __launch_bounds__(256) void kv_append_kernel(half_t* q_out, half_t* k
     }
 }
 
+static int kv_append_common(const char* what, void* q_out, void* k_cache, void* v_cache, const void* Q, const void* bias_Q,
+                            const void* K, const void* bias_K, const void* V, const void* bias_V, int batch, int head_num,
+                            int size_per_head, int pos, int max_len, const DecodeSeqs* seqs, hipStream_t st) {
+    if (batch < 0 || head_num <= 0 || size_per_head <= 0 || size_per_head % 8 != 0 || pos < 0 || pos >= max_len) {
+        set_error("%s: bad shape (pos=%d max_len=%d d=%d)", what, pos, max_len, size_per_head);
+        return LG_ERR_INVALID;
+    }
+    if (batch == 0) return LG_OK;
+    const void* ptrs[9] = {q_out, k_cache, v_cache, Q, bias_Q, K, bias_K, V, bias_V};
+    for (const void* p : ptrs)
+        if (!p || !aligned16(p)) { set_error("%s: null or unaligned pointer", what); return LG_ERR_INVALID; }
+    const int64_t total = (int64_t)batch * head_num * size_per_head / 8;
+    int64_t grid = (total + 255) / 256;
+    if (grid > 4096) grid = 4096;
+    if (seqs)
+        hipLaunchKernelGGL(kv_append_kernel<true>, dim3((int)grid), dim3(256), 0, st, (half_t*)q_out, (half_t*)k_cache,
+                           (half_t*)v_cache, (const half_t*)Q, (const half_t*)bias_Q, (const half_t*)K, (const half_t*)bias_K,
+                           (const half_t*)V, (const half_t*)bias_V, head_num, size_per_head, pos, max_len, total, *seqs);
+    else
+        hipLaunchKernelGGL(kv_append_kernel<false>, dim3((int)grid), dim3(256), 0, st, (half_t*)q_out, (half_t*)k_cache,
+                           (half_t*)v_cache, (const half_t*)Q, (const half_t*)bias_Q, (const half_t*)K, (const half_t*)bias_K,
+                           (const half_t*)V, (const half_t*)bias_V, head_num, size_per_head, pos, max_len, total, DecodeSeqs{});
+    return check_launch(what);
+}
+
 }  // namespace lg
 
 using namespace lg;
@@ -179,53 +283,55 @@ extern "C" {
 
 size_t lg_attn_decode_workspace_bytes(int batch, int head_num, int size_per_head, int max_len) {
     if (batch <= 0 || head_num <= 0 || size_per_head <= 0 || max_len <= 0) return 0;
-    const int bh = batch * head_num;
-    return (size_t)bh * decode_nsplit(bh, max_len) * (2 + (size_t)size_per_head) * sizeof(float);
+    // an upper bound for every batch and length (a smaller batch may split its keys further than a larger one)
+    return (size_t)DEC_MAX_SLOTS * (2 + (size_t)size_per_head) * sizeof(float);
 }
 
 int lg_attn_decode_f16(const void* q, const void* k_cache, const void* v_cache, void* out, void* workspace, int batch,
                        int head_num, int size_per_head, int len, int max_len, float scalar, void* stream) {
-    if (batch < 0 || head_num <= 0 || len <= 0 || max_len < len) { set_error("attn_decode: bad shape (len=%d max_len=%d)", len, max_len); return LG_ERR_INVALID; }
-    if (size_per_head != 64 && size_per_head != 128) { set_error("attn_decode: size_per_head must be 64 or 128"); return LG_ERR_INVALID; }
+    return attn_decode_common("attn_decode", q, k_cache, v_cache, out, (float*)workspace, DEC_MAX_SLOTS, batch, head_num,
+                              size_per_head, len, max_len, scalar, nullptr, (hipStream_t)stream);
+}
+
+int lg_attn_decode_varlen_f16(const void* q, const void* k_cache, const void* v_cache, void* out, void* workspace, int batch,
+                              int head_num, int size_per_head, const int* slot, const int* len, int max_len, float scalar,
+                              void* stream) {
+    if (batch < 0 || batch > DEC_MAX_SEQS) { set_error("attn_decode_varlen: batch must be 0..%d", DEC_MAX_SEQS); return LG_ERR_INVALID; }
     if (batch == 0) return LG_OK;
-    if (!q || !k_cache || !v_cache || !out) { set_error("attn_decode: null pointer"); return LG_ERR_INVALID; }
-    if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache)) { set_error("attn_decode: pointers must be 16-byte aligned"); return LG_ERR_INVALID; }
-    const int bh = batch * head_num;
-    const int ns = decode_nsplit(bh, len);
-    if (ns > 1 && !workspace) { set_error("attn_decode: workspace required"); return LG_ERR_INVALID; }
-    scalar = (float)(half_t)scalar;
-    hipStream_t st = (hipStream_t)stream;
-    dim3 grid(bh, ns);
-    if (size_per_head == 128) {
-        hipLaunchKernelGGL((attn_decode_kernel<128>), grid, dim3(256), 0, st, (const half_t*)q, (const half_t*)k_cache,
-                           (const half_t*)v_cache, (half_t*)out, (float*)workspace, len, max_len, ns, scalar);
-        if (ns > 1) hipLaunchKernelGGL((attn_decode_merge_kernel<128>), dim3(bh), dim3(128), 0, st, (const float*)workspace, (half_t*)out, ns);
-    } else {
-        hipLaunchKernelGGL((attn_decode_kernel<64>), grid, dim3(256), 0, st, (const half_t*)q, (const half_t*)k_cache,
-                           (const half_t*)v_cache, (half_t*)out, (float*)workspace, len, max_len, ns, scalar);
-        if (ns > 1) hipLaunchKernelGGL((attn_decode_merge_kernel<64>), dim3(bh), dim3(64), 0, st, (const float*)workspace, (half_t*)out, ns);
+    if (!slot || !len) { set_error("attn_decode_varlen: null slot / len array"); return LG_ERR_INVALID; }
+    DecodeSeqs seqs{};
+    int longest = 0;
+    for (int b = 0; b < batch; ++b) {
+        if (slot[b] < 0 || len[b] <= 0 || len[b] > max_len) { set_error("attn_decode_varlen: sequence %d: slot %d, len %d (max_len %d)", b, slot[b], len[b], max_len); return LG_ERR_INVALID; }
+        seqs.slot[b] = slot[b];
+        seqs.len[b] = len[b];
+        longest = len[b] > longest ? len[b] : longest;
     }
-    return check_launch("attn_decode");
+    return attn_decode_common("attn_decode_varlen", q, k_cache, v_cache, out, (float*)workspace, DEC_MAX_SLOTS, batch, head_num,
+                              size_per_head, longest, max_len, scalar, &seqs, (hipStream_t)stream);
 }
 
 int lg_kv_append_f16(void* q_out, void* k_cache, void* v_cache, const void* Q, const void* bias_Q, const void* K,
                      const void* bias_K, const void* V, const void* bias_V, int batch, int head_num, int size_per_head,
                      int pos, int max_len, void* stream) {
-    if (batch < 0 || head_num <= 0 || size_per_head <= 0 || size_per_head % 8 != 0 || pos < 0 || pos >= max_len) {
-        set_error("kv_append: bad shape (pos=%d max_len=%d d=%d)", pos, max_len, size_per_head);
-        return LG_ERR_INVALID;
-    }
+    return kv_append_common("kv_append", q_out, k_cache, v_cache, Q, bias_Q, K, bias_K, V, bias_V, batch, head_num, size_per_head,
+                            pos, max_len, nullptr, (hipStream_t)stream);
+}
+
+int lg_kv_append_varlen_f16(void* q_out, void* k_cache, void* v_cache, const void* Q, const void* bias_Q, const void* K,
+                            const void* bias_K, const void* V, const void* bias_V, int batch, int head_num, int size_per_head,
+                            const int* slot, const int* pos, int max_len, void* stream) {
+    if (batch < 0 || batch > DEC_MAX_SEQS) { set_error("kv_append_varlen: batch must be 0..%d", DEC_MAX_SEQS); return LG_ERR_INVALID; }
     if (batch == 0) return LG_OK;
-    const void* ptrs[9] = {q_out, k_cache, v_cache, Q, bias_Q, K, bias_K, V, bias_V};
-    for (const void* p : ptrs)
-        if (!p || !aligned16(p)) { set_error("kv_append: null or unaligned pointer"); return LG_ERR_INVALID; }
-    const int64_t total = (int64_t)batch * head_num * size_per_head / 8;
-    int64_t grid = (total + 255) / 256;
-    if (grid > 4096) grid = 4096;
-    hipLaunchKernelGGL(kv_append_kernel, dim3((int)grid), dim3(256), 0, (hipStream_t)stream, (half_t*)q_out, (half_t*)k_cache,
-                       (half_t*)v_cache, (const half_t*)Q, (const half_t*)bias_Q, (const half_t*)K, (const half_t*)bias_K,
-                       (const half_t*)V, (const half_t*)bias_V, head_num, size_per_head, pos, max_len, total);
-    return check_launch("kv_append");
+    if (!slot || !pos) { set_error("kv_append_varlen: null slot / pos array"); return LG_ERR_INVALID; }
+    DecodeSeqs seqs{};
+    for (int b = 0; b < batch; ++b) {
+        if (slot[b] < 0 || pos[b] < 0 || pos[b] >= max_len) { set_error("kv_append_varlen: sequence %d: slot %d, pos %d (max_len %d)", b, slot[b], pos[b], max_len); return LG_ERR_INVALID; }
+        seqs.slot[b] = slot[b];
+        seqs.len[b] = pos[b];
+    }
+    return kv_append_common("kv_append_varlen", q_out, k_cache, v_cache, Q, bias_Q, K, bias_K, V, bias_V, batch, head_num,
+                            size_per_head, 0, max_len, &seqs, (hipStream_t)stream);
 }
 
 }  // extern "C"

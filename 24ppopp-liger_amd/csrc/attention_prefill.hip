@@ -207,7 +207,7 @@ extern "C" int lg_attn_prefill_f16(const void* q_buf, const void* k_buf, const v
         set_error("attn_prefill: bad shape (seq=%d kv_rows=%d)", seq, kv_rows);
         return LG_ERR_INVALID;
     }
-    if (size_per_head != 64 && size_per_head != 128) { set_error("attn_prefill: size_per_head must be 64 or 128"); return LG_ERR_INVALID; }
+    if (size_per_head != 64 && size_per_head != 96 && size_per_head != 128) { set_error("attn_prefill: size_per_head must be 64, 96 or 128"); return LG_ERR_INVALID; }
     if (batch == 0 || seq == 0) return LG_OK;
     if (!q_buf || !k_buf || !v_buf || !out) { set_error("attn_prefill: null pointer"); return LG_ERR_INVALID; }
     if (!aligned16(q_buf) || !aligned16(k_buf) || !aligned16(v_buf) || !aligned16(out)) {
@@ -219,6 +219,9 @@ extern "C" int lg_attn_prefill_f16(const void* q_buf, const void* k_buf, const v
     if (size_per_head == 128)
         launch_prefill<128>((const half_t*)q_buf, (const half_t*)k_buf, (const half_t*)v_buf, (const half_t*)attr_mask,
                             (half_t*)out, batch, seq, head_num, kv_rows, scalar, causal, out_layout, (hipStream_t)stream);
+    else if (size_per_head == 96)
+        launch_prefill<96>((const half_t*)q_buf, (const half_t*)k_buf, (const half_t*)v_buf, (const half_t*)attr_mask,
+                           (half_t*)out, batch, seq, head_num, kv_rows, scalar, causal, out_layout, (hipStream_t)stream);
     else
         launch_prefill<64>((const half_t*)q_buf, (const half_t*)k_buf, (const half_t*)v_buf, (const half_t*)attr_mask,
                            (half_t*)out, batch, seq, head_num, kv_rows, scalar, causal, out_layout, (hipStream_t)stream);

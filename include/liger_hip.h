@@ -187,21 +187,35 @@ int lg_gemm_fused_grouped_f16(int transa, int m, int n, int k, int count, const 
  * when out_layout = 1).  q_buf [B,h,S,d]; k_buf, v_buf [B,h,kv_rows,d] with the S valid rows first
  * (kv_rows = S for plain buffers, = max_len when they are a KV cache).  causal != 0: implicit
  * lower-triangular mask (attr_mask ignored, may be NULL); causal == 0: attr_mask [B,S,S] of 0/1 or NULL
- * for all ones.  out_layout 0: [B,h,S,d]; 1: [B,S,h,d] (= transpose-back fused).  size_per_head: 64 or 128. */
+ * for all ones.  out_layout 0: [B,h,S,d]; 1: [B,S,h,d] (= transpose-back fused).  size_per_head: 64, 96 or 128. */
 int lg_attn_prefill_f16(const void* q_buf, const void* k_buf, const void* v_buf, const void* attr_mask,
                         void* out, int batch, int seq, int head_num, int size_per_head, int kv_rows,
                         float scalar, int causal, int out_layout, void* stream);
 /* Decode attention: q [B,h,d]; k_cache, v_cache [B,h,max_len,d] with `len` valid positions; out [B,h,d].
- * workspace: float buffer of lg_attn_decode_workspace_bytes(...) bytes (split-KV partials), caller-owned. */
+ * size_per_head: 64, 96 or 128.  workspace: float buffer of lg_attn_decode_workspace_bytes(...) bytes (split-KV partials),
+ * caller-owned; that size is an upper bound for every batch and every len <= max_len, so a buffer sized once for the
+ * largest batch serves all smaller ones. */
 size_t lg_attn_decode_workspace_bytes(int batch, int head_num, int size_per_head, int max_len);
 int lg_attn_decode_f16(const void* q, const void* k_cache, const void* v_cache, void* out, void* workspace,
                        int batch, int head_num, int size_per_head, int len, int max_len, float scalar,
                        void* stream);
+/* The same over sequences that differ in length and sit in arbitrary cache slots (decode steps of different requests
+ * batched into one launch): sequence b reads slot[b] of the caches [slots,h,max_len,d] and attends to its first len[b]
+ * positions.  slot and len are HOST arrays of `batch` ints, copied into the launch (batch <= LG_ATTN_DECODE_MAX_SEQS). */
+#define LG_ATTN_DECODE_MAX_SEQS 64
+int lg_attn_decode_varlen_f16(const void* q, const void* k_cache, const void* v_cache, void* out, void* workspace,
+                              int batch, int head_num, int size_per_head, const int* slot, const int* len, int max_len,
+                              float scalar, void* stream);
 /* Adds the Q/K/V biases to one new token per sequence ([B, h*d] rows straight from the QKV GEMMs), writes
  * q -> q_out [B,h,d] and appends k, v at position `pos` of the caches [B,h,max_len,d]. */
 int lg_kv_append_f16(void* q_out, void* k_cache, void* v_cache, const void* Q, const void* bias_Q, const void* K,
                      const void* bias_K, const void* V, const void* bias_V, int batch, int head_num,
                      int size_per_head, int pos, int max_len, void* stream);
+/* The same with a cache slot and a position per sequence (HOST arrays of `batch` ints, batch <= LG_ATTN_DECODE_MAX_SEQS):
+ * sequence b's k, v go to position pos[b] of slot[b] of the caches [slots,h,max_len,d]. */
+int lg_kv_append_varlen_f16(void* q_out, void* k_cache, void* v_cache, const void* Q, const void* bias_Q, const void* K,
+                            const void* bias_K, const void* V, const void* bias_V, int batch, int head_num,
+                            int size_per_head, const int* slot, const int* pos, int max_len, void* stream);
 
 #ifdef __cplusplus
 }

@@ -35,4 +35,4 @@ def test_version_and_error_text_without_a_gpu(liger):
     assert liger.capi.lib.lg_layer_norm_f32(None, None, None, None, 4, 0, None) == liger.capi.ERR_INVALID
     assert "bad shape" in liger.capi.last_error()
     assert liger.capi.lib.lg_gemm_f16(0, 1, 4, 4, 4, None, 4, None, 4, None, 4, None) == liger.capi.ERR_INVALID
-    assert liger.capi.lib.lg_attn_decode_f16(None, None, None, None, None, 1, 1, 96, 8, 8, 1.0, None) == liger.capi.ERR_INVALID
+    assert liger.capi.lib.lg_attn_decode_f16(None, None, None, None, None, 1, 1, 80, 8, 8, 1.0, None) == liger.capi.ERR_INVALID
