@@ -75,6 +75,7 @@ SIGNATURES = {
     "lg_attn_decode_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "lg_attn_decode_f16": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _f, _p]),
     "lg_attn_decode_varlen_f16": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, C.POINTER(_i), C.POINTER(_i), _i, _f, _p]),
+    "lg_attn_decode_static_f16": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _f, _p]),
     "lg_kv_append_f16": (_i, [_p] * 9 + [_i, _i, _i, _i, _i, _p]),
     "lg_kv_append_varlen_f16": (_i, [_p] * 9 + [_i, _i, _i, C.POINTER(_i), C.POINTER(_i), _i, _p]),
 }

@@ -13,6 +13,8 @@
 //     independent 1 KiB loads in flight.
 // Softmax semantics are the reference's (attention_kernels.cu:480-519): p = exp(t - max t) / (sum + 1e-6),
 // t = q.k * scalar, all positions < len unmasked.
+#include <mutex>
+
 #include "common.cuh"
 
 namespace lg {
@@ -191,7 +193,7 @@ static void launch_decode(const half_t* q, const half_t* kc, const half_t* vc, h
     if (ns > 1) hipLaunchKernelGGL((attn_decode_merge_kernel<D>), dim3(bh), dim3(D), 0, st, (const float*)ws, out, ns);
 }
 
-// Argument checks and launch shared by the entry points.  `seqs` = per-sequence slots and lengths or nullptr (all
+// Argument checks and launch shared by the three entry points.  `seqs` = per-sequence slots and lengths or nullptr (all
 // sequences `len` long, sequence b in cache slot b); ws_capacity_slots = partial slots the workspace holds.
 static int attn_decode_common(const char* what, const void* q, const void* k_cache, const void* v_cache, void* out, float* ws,
                               int64_t ws_capacity_slots, int batch, int head_num, int size_per_head, int len, int max_len,
@@ -215,6 +217,31 @@ static int attn_decode_common(const char* what, const void* q, const void* k_cac
     else if (size_per_head == 96) launch_decode<96, 4, 4>(qh, kh, vh, (half_t*)out, ws, bh, head_num, len, max_len, ns, scalar, seqs, st);
     else launch_decode<64, 8, 8>(qh, kh, vh, (half_t*)out, ws, bh, head_num, len, max_len, ns, scalar, seqs, st);
     return check_launch(what);
+}
+
+// ---- split-KV partials in device memory that belongs to the library (lg_attn_decode_static_f16) ---------------------------
+// One array per GPU, held until the process ends; every call on a GPU uses that GPU's array.
+static __device__ __align__(256) float scratch[DEC_MAX_SLOTS * (2 + DEC_MAX_D)];
+constexpr int DEC_MAX_DEVICES = 64;
+static std::mutex g_scratch_mu;
+static float* g_scratch_ptr[DEC_MAX_DEVICES] = {};
+
+// Device address of this GPU's `scratch` (the array's name is only a host-side stand-in for it): looked up once per device,
+// with that device current.
+static int scratch_address(float** ptr) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) { set_error("attn_decode_static: hipGetDevice: %s", hipGetErrorString(e)); return LG_ERR_LAUNCH; }
+    if (dev < 0 || dev >= DEC_MAX_DEVICES) { set_error("attn_decode_static: device %d not supported", dev); return LG_ERR_INVALID; }
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) { set_error("attn_decode_static: hipGetSymbolAddress: %s", hipGetErrorString(e)); return LG_ERR_LAUNCH; }
+        g_scratch_ptr[dev] = (float*)p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return LG_OK;
 }
 
 // q_out[b,head,:] = Q[b, head*d ..] + bq;  caches[slot_b,head,pos_b,:] = K/V + bias.  VARLEN: slot_b, pos_b come per sequence
@@ -309,6 +336,16 @@ int lg_attn_decode_varlen_f16(const void* q, const void* k_cache, const void* v_
     }
     return attn_decode_common("attn_decode_varlen", q, k_cache, v_cache, out, (float*)workspace, DEC_MAX_SLOTS, batch, head_num,
                               size_per_head, longest, max_len, scalar, &seqs, (hipStream_t)stream);
+}
+
+int lg_attn_decode_static_f16(const void* q, const void* k_cache, const void* v_cache, void* out, int batch, int head_num,
+                              int size_per_head, int len, int max_len, float scalar, void* stream) {
+    if (size_per_head > DEC_MAX_D) { set_error("attn_decode_static: size_per_head %d exceeds the maximum %d", size_per_head, DEC_MAX_D); return LG_ERR_INVALID; }
+    float* ws = nullptr;
+    const int rc = scratch_address(&ws);
+    if (rc != LG_OK) return rc;
+    return attn_decode_common("attn_decode_static", q, k_cache, v_cache, out, ws, DEC_MAX_SLOTS, batch, head_num, size_per_head, len,
+                              max_len, scalar, nullptr, (hipStream_t)stream);
 }
 
 int lg_kv_append_f16(void* q_out, void* k_cache, void* v_cache, const void* Q, const void* bias_Q, const void* K,

@@ -206,6 +206,14 @@ int lg_attn_decode_f16(const void* q, const void* k_cache, const void* v_cache, 
 int lg_attn_decode_varlen_f16(const void* q, const void* k_cache, const void* v_cache, void* out, void* workspace,
                               int batch, int head_num, int size_per_head, const int* slot, const int* len, int max_len,
                               float scalar, void* stream);
+/* lg_attn_decode_f16 for callers that cannot allocate device memory or pass a workspace (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc); no counterpart in the reference.  The split-KV partials live in
+ * a fixed array inside the library's device image (2048 partial slots x (2 + 128) floats = 1.02 MiB per GPU, held until
+ * the process ends); this call allocates nothing.  Same results as lg_attn_decode_f16, bit for bit.  size_per_head > 128
+ * is rejected.  Every call on a GPU uses that GPU's one array: calls that overlap in time on one GPU (two streams)
+ * race; calls on one stream are ordered and safe. */
+int lg_attn_decode_static_f16(const void* q, const void* k_cache, const void* v_cache, void* out, int batch, int head_num,
+                              int size_per_head, int len, int max_len, float scalar, void* stream);
 /* Adds the Q/K/V biases to one new token per sequence ([B, h*d] rows straight from the QKV GEMMs), writes
  * q -> q_out [B,h,d] and appends k, v at position `pos` of the caches [B,h,max_len,d]. */
 int lg_kv_append_f16(void* q_out, void* k_cache, void* v_cache, const void* Q, const void* bias_Q, const void* K,
