@@ -28,6 +28,9 @@ SIGNATURES = {
     "lg_memset_async": (_i, [_p, _i, _sz, _p]),
     "lg_device_synchronize": (_i, []),
     "lg_stream_create": (_i, [C.POINTER(_p)]),
+    "lg_stream_attach": (_i, [_p, _i]),
+    "lg_stream_detach": (_i, [_p]),
+    "lg_stream_cu_count": (_i, [_p]),
     "lg_stream_create_cu_mask": (_i, [C.POINTER(_p), C.POINTER(C.c_uint), _i]),
     "lg_stream_create_concurrent": (_i, [_p, _p, _p]),
     "lg_stream_destroy": (_i, [_p]),

@@ -21,6 +21,17 @@ constexpr int kWave = 64;
 void set_error(const char* fmt, ...);
 int check_launch(const char* what);
 
+// What is known about a stream (runtime.hip): the compute units its kernels may run on (fewer than the device for a CU-masked
+// stream) and its split-K workspace (nullptr for a stream the library neither created nor was told about with lg_stream_attach).
+constexpr size_t LG_SPLITK_WORKSPACE_BYTES = (size_t)64 << 20;
+struct StreamInfo {
+    int cus;
+    float* ws;
+    size_t ws_bytes;
+};
+StreamInfo stream_info(hipStream_t stream);
+int device_cu_count();
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);

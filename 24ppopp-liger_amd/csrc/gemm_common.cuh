@@ -112,8 +112,8 @@ __device__ __forceinline__ void epilogue_store4(const GemmArgs& g, half_t* Yb, i
 
 // ---- split-K support shared by the weight-streaming and the pipelined kernel (gemm_skinny.hip) --------------------------
 constexpr int LG_EPI_PARTIAL = 100;  // kernel-internal: store the fp32 accumulators of K-slice `split` to partial[split][M][N]
-// per-stream fp32 workspace (grows on demand, kept until the process ends); nullptr if the allocation fails
-float* splitk_workspace(hipStream_t stream, size_t bytes);
+// The fp32 partials live in the stream's workspace (StreamInfo::ws, allocated when the stream was created or attached); a
+// launcher never allocates: with no workspace, or one that is too small, it slices K less or not at all.
 // Y = epilogue(sum over the nsplit K-slices in slice order) of the fp32 partials [nsplit][M][N]
 void launch_splitk_reduce(const GemmArgs& g, const float* partial, int nsplit, hipStream_t stream);
 

@@ -48,7 +48,7 @@ __device__ __forceinline__ int swz_a(int row, int c) { return c ^ ((row >> 1) & 
 __device__ __forceinline__ int swz_b(int k, int blk) { return blk ^ ((k & 3) | ((k >> 1) & 4)); }
 
 template <int WL, int EPI, int NJ>
-__global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles_m, int tiles_n, float* partial, int kt_per_split) {
+__global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles_m, int tiles_n, float* partial, int kt_per_split, int cus) {
     constexpr int FB_N = 64 * NJ;
     constexpr int X_TILE = FB_M * FB_K, W_TILE = FB_K * FB_N;  // halves per ring slot
     constexpr int WCH = (FB_K * FB_N) / 512 / 8;  // 1 KiB chunks of the W tile per wave (= NJ)
@@ -67,27 +67,31 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles
     {
         const int bid = blockIdx.x;
         const int ntiles = tiles_m * tiles_n;
-        // The 256 workgroups that run at the same time ("a round") cover an RM x RN region of tiles, each XCD a compact 4 x 8
-        // block of it (its L2 then serves 4 + 8 operand panels to 32 tiles).  A round reads RM X panels and RN W panels from
-        // memory, so the region is made as square as the tile counts allow: 16 x 16 (32 panels; FFN-1 1346 -> 1412 TFLOP/s
-        // against rounds of 4 x 64), else 8 x 32.
+        // The workgroups that run at the same time ("a round": one per compute unit of the stream, P = cus / 8 on each XCD; 256
+        // and 32 on the whole chip) cover an RM x RN region of tiles, each XCD a compact 4 x P/4 block of it (its L2 then serves
+        // 4 + P/4 operand panels to P tiles).  A round reads RM X panels and RN W panels from memory, so the region is made as
+        // square as the tile counts allow: on the whole chip 16 x 16 (32 panels; FFN-1 1346 -> 1412 TFLOP/s against rounds of
+        // 4 x 64), else 8 x 32.
+        const int P = cus >> 3, pw = P >> 2;  // pw: width of an XCD's block in tiles
         int RM = 0;
-        if ((tiles_m % 16 == 0) && (tiles_n % 16 == 0) && tiles_n >= 48) RM = 16;
-        else if ((tiles_m % 8 == 0) && (tiles_n % 32 == 0)) RM = 8;
+        if (pw >= 1 && (P & 3) == 0) {
+            if ((tiles_m % 16 == 0) && (tiles_n % (2 * pw) == 0) && tiles_n >= 6 * pw) RM = 16;
+            else if ((tiles_m % 8 == 0) && (tiles_n % (4 * pw) == 0)) RM = 8;
+        }
         if (RM) {
-            const int RN = 256 / RM, xcols = RN >> 3;          // XCD blocks per region row
+            const int RN = (8 * P) / RM, xcols = RN / pw;      // XCD blocks per region row
             const int xcd = bid & 7, slot = bid >> 3;          // slot: order of arrival on this XCD
-            const int round = slot >> 5, in = slot & 31;
+            const int round = slot / P, in = slot % P;
             const int regions_n = tiles_n / RN;
             tm = (round / regions_n) * RM + (xcd / xcols) * 4 + (in & 3);
-            tn = (round % regions_n) * RN + (xcd % xcols) * 8 + (in >> 2);
-        } else if ((tiles_m % 4 == 0) && (tiles_n % 8 == 0) && (ntiles % 256 == 0)) {
+            tn = (round % regions_n) * RN + (xcd % xcols) * pw + (in >> 2);
+        } else if (pw >= 1 && (P & 3) == 0 && (tiles_m % 4 == 0) && (tiles_n % pw == 0) && (ntiles % (8 * P) == 0)) {
             const int xcd = bid & 7, slot = bid >> 3;
-            const int chunk = (slot >> 5) * 8 + xcd;          // blocks of 32 tiles (4 x 8)
-            const int in = slot & 31;
-            const int chunks_n = tiles_n >> 3;
+            const int chunk = (slot / P) * 8 + xcd;           // blocks of P tiles (4 x P/4)
+            const int in = slot % P;
+            const int chunks_n = tiles_n / pw;
             tm = (chunk / chunks_n) * 4 + (in & 3);
-            tn = (chunk % chunks_n) * 8 + (in >> 2);
+            tn = (chunk % chunks_n) * pw + (in >> 2);
         } else {
             tm = bid % tiles_m;
             tn = bid / tiles_m;
@@ -285,37 +289,34 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles
 }
 
 template <int WL, int NJ>
-static int launch_fast_epi(const GemmArgs& g, int tiles_m, int tiles_n, hipStream_t stream) {
+static int launch_fast_epi(const GemmArgs& g, int tiles_m, int tiles_n, const StreamInfo& si, hipStream_t stream) {
     const int tiles = tiles_m * tiles_n, ktiles = g.K / FB_K;
+    const int cus = si.cus;
     // At most 256 token rows (one row of tiles, the continuation of the weight-streaming kernel's regime): the time is set by
-    // how fast the weights stream in, so K is split over otherwise idle CUs (slices of >= 8 k-tiles, fp32 partials summed in
-    // slice order by a second kernel that applies the epilogue).  Larger M never splits K, so that a token row's result does
-    // not depend on how many other rows are in the batch (each output is one sequential sum over k).
+    // how fast the weights stream in, so K is split over otherwise idle CUs (slices of >= 8 k-tiles, fp32 partials in the
+    // stream's workspace, summed in slice order by a second kernel that applies the epilogue; no more slices than the workspace
+    // holds, none on a stream without one).  Larger M never splits K, so that a token row's result does not depend on how many
+    // other rows are in the batch (each output is one sequential sum over k).
     int nsplit = 1;
-    if (tiles_m == 1 && tiles <= 128) {
-        nsplit = 256 / tiles;
+    if (tiles_m == 1 && tiles <= cus / 2 && si.ws) {
+        nsplit = cus / tiles;
         if (nsplit > ktiles / 8) nsplit = ktiles / 8;
         if (nsplit > 16) nsplit = 16;
+        const size_t slice_bytes = (size_t)g.M * g.N * sizeof(float);
+        if ((size_t)nsplit * slice_bytes > si.ws_bytes) nsplit = (int)(si.ws_bytes / slice_bytes);
         if (nsplit < 1) nsplit = 1;
     }
     int kt_per_split = (ktiles + nsplit - 1) / nsplit;
     nsplit = (ktiles + kt_per_split - 1) / kt_per_split;
-    float* partial = nullptr;
-    if (nsplit > 1) {
-        const size_t bytes = (size_t)nsplit * g.M * g.N * sizeof(float);
-        partial = splitk_workspace(stream, bytes);
-        if (!partial) { set_error("gemm_fast: cannot allocate the %zu-byte split-K workspace", bytes); return LG_ERR_LAUNCH; }
-    }
+    float* partial = nsplit > 1 ? si.ws : nullptr;
     const dim3 grid(tiles, nsplit), block(F_THREADS);
     const size_t smem = lds_halves(NJ) * sizeof(half_t);
 #define LG_FAST(E)                                                                                                  \
     do {                                                                                                            \
-        static bool attr_set = false;                                                                               \
-        if (!attr_set) {                                                                                            \
-            (void)hipFuncSetAttribute((const void*)gemm_f16_fast<WL, E, NJ>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
-            attr_set = true;                                                                                        \
-        }                                                                                                           \
-        hipLaunchKernelGGL((gemm_f16_fast<WL, E, NJ>), grid, block, smem, stream, g, tiles_m, tiles_n, partial, kt_per_split); \
+        /* set once per instantiation; the initialisation of a function-local static is thread-safe */              \
+        static const hipError_t attr_rc = hipFuncSetAttribute((const void*)gemm_f16_fast<WL, E, NJ>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
+        (void)attr_rc;                                                                                              \
+        hipLaunchKernelGGL((gemm_f16_fast<WL, E, NJ>), grid, block, smem, stream, g, tiles_m, tiles_n, partial, kt_per_split, cus); \
     } while (0)
     if (nsplit > 1) {
         LG_FAST(LG_EPI_PARTIAL);
@@ -344,7 +345,8 @@ int launch_gemm_fast_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t 
     if (g.ldx >= (1 << 22) || g.ldw >= (1 << 22)) return LG_OK;  // 256 rows x ld must fit the 31-bit tile offsets
     if (g.epi.kind == LG_EPI_BIAS_HEADS ? (g.epi.d % 4 != 0) : (g.ldy % 4 != 0)) return LG_OK;
     if (g.epi.kind != LG_EPI_NONE && (reinterpret_cast<uintptr_t>(g.epi.bias) & 7u)) return LG_OK;  // 8-byte bias loads
-    // tile width: the one that needs the least work-rounds on 256 CUs (rounds x tile width); ties go to the wider tile
+    // tile width: the one that needs the least work-rounds on the stream's CUs (rounds x tile width); ties go to the wider tile
+    const StreamInfo si = stream_info(stream);
     const int tiles_m = (g.M + FB_M - 1) / FB_M;
     int best_nj = 0;
     long best_cost = 0;
@@ -353,7 +355,7 @@ int launch_gemm_fast_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t 
         if (nj == 3 && wlayout != W_NK) continue;
         const long tiles = (long)tiles_m * (g.N / (64 * nj));
         // narrower tiles move more operand bytes per flop: about 3 % / 35 % more time per unit of width (measured)
-        const long cost = ((tiles + 255) / 256) * nj * (nj == 4 ? 100 : nj == 3 ? 103 : 135);
+        const long cost = ((tiles + si.cus - 1) / si.cus) * nj * (nj == 4 ? 100 : nj == 3 ? 103 : 135);
         if (!best_nj || cost < best_cost) { best_nj = nj; best_cost = cost; }
     }
     if (!best_nj) return LG_OK;
@@ -361,12 +363,12 @@ int launch_gemm_fast_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t 
     const int tiles_n = g.N / (64 * best_nj);
     int rc;
     if (wlayout == W_NK) {
-        if (best_nj == 4) rc = launch_fast_epi<W_NK, 4>(g, tiles_m, tiles_n, stream);
-        else if (best_nj == 3) rc = launch_fast_epi<W_NK, 3>(g, tiles_m, tiles_n, stream);
-        else rc = launch_fast_epi<W_NK, 2>(g, tiles_m, tiles_n, stream);
+        if (best_nj == 4) rc = launch_fast_epi<W_NK, 4>(g, tiles_m, tiles_n, si, stream);
+        else if (best_nj == 3) rc = launch_fast_epi<W_NK, 3>(g, tiles_m, tiles_n, si, stream);
+        else rc = launch_fast_epi<W_NK, 2>(g, tiles_m, tiles_n, si, stream);
     } else {
-        if (best_nj == 4) rc = launch_fast_epi<W_KN, 4>(g, tiles_m, tiles_n, stream);
-        else rc = launch_fast_epi<W_KN, 2>(g, tiles_m, tiles_n, stream);
+        if (best_nj == 4) rc = launch_fast_epi<W_KN, 4>(g, tiles_m, tiles_n, si, stream);
+        else rc = launch_fast_epi<W_KN, 2>(g, tiles_m, tiles_n, si, stream);
     }
     return rc != LG_OK ? rc : check_launch("gemm_f16_fast");
 }

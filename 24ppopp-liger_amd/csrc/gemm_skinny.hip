@@ -11,11 +11,8 @@
 //     feature: exactly the B operand of v_mfma_f32_16x16x32_f16) in a rolling pipeline that keeps 16 independent
 //     16-byte loads in flight per lane at all times;
 //   * the few X rows are staged once per 256-wide k-chunk in LDS (double buffered) and shared by the block's waves;
-//   * K-slices (when there are any) are summed in fp32 through a per-stream workspace and a small second kernel that also
+//   * K-slices (when there are any) are summed in fp32 through the stream's workspace and a small second kernel that also
 //     applies the epilogue (bias / GELU / head-transposed store), so results match the single-pass kernels' rounding.
-#include <mutex>
-#include <unordered_map>
-
 #include "gemm_common.cuh"
 
 namespace lg {
@@ -262,25 +259,6 @@ __global__ __launch_bounds__(256) void gemm_skinny_reduce_kernel(GemmArgs g, con
     }
 }
 
-// ---- per-stream workspace (the counterpart of a cuBLAS handle's workspace: context.h:20-29 binds one handle per stream) ----
-struct SkinnyWs { float* ptr; size_t bytes; };
-static std::mutex g_ws_mu;
-static std::unordered_map<void*, SkinnyWs> g_ws;
-
-float* splitk_workspace(hipStream_t stream, size_t bytes) {
-    std::lock_guard<std::mutex> lk(g_ws_mu);
-    SkinnyWs& w = g_ws[(void*)stream];
-    if (w.bytes < bytes) {
-        // grows only; the old block is kept alive because earlier launches on this stream may still read it
-        float* p = nullptr;
-        size_t want = bytes < ((size_t)32 << 20) ? ((size_t)32 << 20) : bytes;
-        if (hipMalloc((void**)&p, want) != hipSuccess) return nullptr;
-        w.ptr = p;
-        w.bytes = want;
-    }
-    return w.ptr;
-}
-
 void launch_splitk_reduce(const GemmArgs& g, const float* partial, int nsplit, hipStream_t stream) {
     const dim3 block(256);
     const int64_t quads = (int64_t)g.M * ((g.N + 3) / 4);
@@ -301,9 +279,12 @@ int launch_gemm_skinny_f16(const GemmArgs& g, const GemmGroup& grp, int wlayout,
     if (g.M <= 0 || g.M > 64 || g.N < 512 || g.K < 1024 || (g.K % SK_KC) || (g.N % 4)) return LG_OK;
     if (!aligned16(g.X) || (g.ldx % 8) || (g.ldw % 8) || !group_aligned(g, grp)) return LG_OK;
     const int mt = (g.M + 15) / 16;
+    const StreamInfo si = stream_info(stream);
+    const int cus = si.cus;  // compute units this stream's kernels run on: "one round of blocks" means this many
     // Unsliced blocks need a block width (128, 96, 64 or, up to 16 token rows, 32 features) that gives one round of blocks on
-    // the 256 CUs, 192..256 of them (fewer leave CUs idle; a few more than 256 double the time of the CUs that get two), or
-    // so many blocks that the last, partial round does not matter.  The widest such block re-reads the token rows least.
+    // the stream's CUs, 3/4 of them to all of them (fewer leave CUs idle; a few more than a round double the time of the CUs
+    // that get two), or so many blocks that the last, partial round does not matter.  The widest such block re-reads the token
+    // rows least.
     {
         const int widths[4] = {128, 96, 64, 32};
         for (int wi = 0; wi < 4; ++wi) {
@@ -311,7 +292,7 @@ int launch_gemm_skinny_f16(const GemmArgs& g, const GemmGroup& grp, int wlayout,
             // whole pipeline depths of chunks; the 2-wave block's registers hold its four-chunk pipeline for one row tile only
             if (w == 32 ? (mt != 1 || g.K % (4 * SK_KC) != 0) : (g.K % (2 * SK_KC) != 0)) continue;
             const int blocks = (g.N + w - 1) / w * grp.count;
-            if (blocks < 192 || (blocks > 256 && blocks < 1024)) continue;
+            if (blocks < cus * 3 / 4 || (blocks > cus && blocks < 4 * cus)) continue;
             *handled = true;
             switch (w) {
                 case 128: launch_direct_mt<8, 2>(g, grp, stream); break;
@@ -325,15 +306,18 @@ int launch_gemm_skinny_f16(const GemmArgs& g, const GemmGroup& grp, int wlayout,
     if (grp.count > 1) return LG_OK;
     const int nblk = (g.N + SK_BN - 1) / SK_BN;
     // K-slices: as few as fill the chip.  One block of 4 waves keeps 64 KiB of weight loads in flight, which is enough for one
-    // CU; more slices only add fp32 partials and reduce work (six GEMMs of a decode step at 32 token rows: 344 us with >= 1024
-    // blocks, 315 us with >= 256, 289 us with >= 192, 336 us with >= 128).  Slices are multiples of the 256-wide chunk.
+    // CU; more slices only add fp32 partials and reduce work (six GEMMs of a decode step at 32 token rows on 256 CUs: 344 us
+    // with >= 1024 blocks, 315 us with >= 256, 289 us with >= 192, 336 us with >= 128).  Slices are multiples of the 256-wide
+    // chunk, and no more than the stream's workspace holds; a stream without a workspace leaves the problem to the generic kernel.
+    if (!si.ws) return LG_OK;
     int nsplit = 1;
-    while (nblk * nsplit < 192 && (g.K / (nsplit * 2)) >= 2 * SK_KC && nsplit < 32) nsplit *= 2;
+    while (nblk * nsplit < cus * 3 / 4 && (g.K / (nsplit * 2)) >= 2 * SK_KC && nsplit < 32) nsplit *= 2;
+    const size_t slice_bytes = (size_t)g.M * g.N * sizeof(float);
+    while (nsplit > 1 && (size_t)nsplit * slice_bytes > si.ws_bytes) nsplit /= 2;
+    if (slice_bytes > si.ws_bytes) return LG_OK;
     int kslice = ((g.K + nsplit - 1) / nsplit + SK_KC - 1) / SK_KC * SK_KC;
     nsplit = (g.K + kslice - 1) / kslice;
-    const size_t bytes = (size_t)nsplit * g.M * g.N * sizeof(float);
-    float* ws = splitk_workspace(stream, bytes);
-    if (!ws) { set_error("gemm_skinny: cannot allocate the %zu-byte split-K workspace", bytes); *handled = true; return LG_ERR_LAUNCH; }
+    float* ws = si.ws;
     *handled = true;
     const dim3 grid(nblk, nsplit), block(256);
     switch (mt) {

@@ -112,11 +112,9 @@ int launch_gemv_f16(const GemmArgs& g, const GemmGroup& grp, int wlayout, int ba
     const dim3 grid((g.N + 4 * GV_ROWS - 1) / (4 * GV_ROWS), grp.count), block(256);
 #define LG_GV(MR_, E_)                                                                                              \
     do {                                                                                                            \
-        static bool attr_set = false;                                                                               \
-        if (!attr_set) {                                                                                            \
-            (void)hipFuncSetAttribute((const void*)gemv_nk_kernel<MR_, E_>, hipFuncAttributeMaxDynamicSharedMemorySize, GV_MAX_LDS); \
-            attr_set = true;                                                                                        \
-        }                                                                                                           \
+        /* set once per instantiation; the initialisation of a function-local static is thread-safe */              \
+        static const hipError_t attr_rc = hipFuncSetAttribute((const void*)gemv_nk_kernel<MR_, E_>, hipFuncAttributeMaxDynamicSharedMemorySize, GV_MAX_LDS); \
+        (void)attr_rc;                                                                                              \
         hipLaunchKernelGGL((gemv_nk_kernel<MR_, E_>), grid, block, smem, stream, g, grp);                              \
     } while (0)
 #define LG_GV_MR(E_)                                 \

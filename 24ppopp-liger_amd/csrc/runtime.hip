@@ -2,6 +2,8 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
+#include <unordered_map>
 
 #include "common.cuh"
 
@@ -29,6 +31,68 @@ static int rt(hipError_t e, const char* what) {
     if (e == hipSuccess) return LG_OK;
     set_error("%s: %s", what, hipGetErrorString(e));
     return LG_ERR_LAUNCH;
+}
+
+// ---- stream registry -----------------------------------------------------------------------------------------------------------
+// What the launchers need to know about the stream they are handed: how many compute units its kernels may run on (a CU-masked
+// stream has fewer than the device, and grids are sized for what is there) and where its split-K workspace is.  The workspace is
+// allocated when a stream is created or attached, never on the launch path (the counterpart of the workspace a cuBLAS handle
+// owns: context.h:20-29 binds one handle per stream).
+static std::mutex g_streams_mu;
+static std::unordered_map<void*, StreamInfo> g_streams;
+
+int device_cu_count() {
+    static int cached = 0;
+    if (cached > 0) return cached;
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+        cached = n;
+    return cached > 0 ? cached : 256;
+}
+
+StreamInfo stream_info(hipStream_t stream) {
+    {
+        std::lock_guard<std::mutex> lk(g_streams_mu);
+        auto it = g_streams.find((void*)stream);
+        if (it != g_streams.end()) return it->second;
+    }
+    return StreamInfo{device_cu_count(), nullptr, 0};
+}
+
+static int register_stream(void* stream, int cus) {
+    StreamInfo info{cus > 0 ? cus : device_cu_count(), nullptr, 0};
+    {
+        std::lock_guard<std::mutex> lk(g_streams_mu);
+        auto it = g_streams.find(stream);
+        if (it != g_streams.end()) {  // already known: only an explicit CU count changes anything
+            if (cus > 0) it->second.cus = cus;
+            return LG_OK;
+        }
+    }
+    void* p = nullptr;
+    const int rc = rt(hipMalloc(&p, LG_SPLITK_WORKSPACE_BYTES), "hipMalloc (split-K workspace)");
+    if (rc) return rc;
+    info.ws = (float*)p;
+    info.ws_bytes = LG_SPLITK_WORKSPACE_BYTES;
+    std::lock_guard<std::mutex> lk(g_streams_mu);
+    g_streams[stream] = info;
+    return LG_OK;
+}
+
+static int unregister_stream(void* stream) {
+    StreamInfo info{0, nullptr, 0};
+    {
+        std::lock_guard<std::mutex> lk(g_streams_mu);
+        auto it = g_streams.find(stream);
+        if (it == g_streams.end()) return LG_OK;
+        info = it->second;
+        g_streams.erase(it);
+    }
+    if (!info.ws) return LG_OK;
+    // launches on the stream may still read the workspace
+    int rc = rt(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize");
+    const int rc2 = rt(hipFree(info.ws), "hipFree (split-K workspace)");
+    return rc ? rc : rc2;
 }
 
 // ---- counter-based Irwin-Hall(8) generator; integer work + two rounded fp32 ops --------------------
@@ -157,20 +221,33 @@ int lg_memset_async(void* dst, int value, size_t bytes, void* stream) {
 }
 int lg_device_synchronize(void) { return rt(hipDeviceSynchronize(), "hipDeviceSynchronize"); }
 int lg_stream_create(void** stream) {
+    if (!stream) { set_error("lg_stream_create: null argument"); return LG_ERR_INVALID; }
     hipStream_t s = nullptr;
     int rc = rt(hipStreamCreateWithFlags(&s, hipStreamNonBlocking), "hipStreamCreateWithFlags");
     *stream = (void*)s;
-    return rc;
+    return rc ? rc : register_stream((void*)s, 0);
 }
+int lg_stream_attach(void* stream, int cu_count) {
+    if (cu_count < 0) { set_error("lg_stream_attach: negative CU count"); return LG_ERR_INVALID; }
+    return register_stream(stream, cu_count);
+}
+int lg_stream_detach(void* stream) { return unregister_stream(stream); }
+int lg_stream_cu_count(void* stream) { return stream_info((hipStream_t)stream).cus; }
 int lg_stream_create_cu_mask(void** stream, const unsigned* cu_mask, int mask_words) {
     if (!stream || !cu_mask || mask_words <= 0) { set_error("lg_stream_create_cu_mask: bad arguments"); return LG_ERR_INVALID; }
-    bool any = false;
-    for (int w = 0; w < mask_words; ++w) any = any || cu_mask[w] != 0u;
-    if (!any) { set_error("lg_stream_create_cu_mask: empty mask"); return LG_ERR_INVALID; }
+    // Bit i of the mask selects a compute unit of accelerator die i mod 8 (the dies take the bits in turn).  A mask that leaves
+    // a die without any unit is refused: the runtime fails on the host for such a stream.
+    const int total = device_cu_count();
+    const int dies = total >= 64 ? 8 : 1;
+    int cus = 0, per_die[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int b = 0; b < mask_words * 32 && b < total; ++b)
+        if (cu_mask[b >> 5] & (1u << (b & 31))) { ++cus; ++per_die[b % dies]; }
+    for (int x = 0; x < dies; ++x)
+        if (per_die[x] == 0) { set_error("lg_stream_create_cu_mask: the mask selects no compute unit on die %d (bit i belongs to die i mod %d)", x, dies); return LG_ERR_INVALID; }
     hipStream_t s = nullptr;
     int rc = rt(hipExtStreamCreateWithCUMask(&s, (uint32_t)mask_words, cu_mask), "hipExtStreamCreateWithCUMask");
     *stream = (void*)s;
-    return rc;
+    return rc ? rc : register_stream((void*)s, cus);
 }
 // ---- a second stream that really runs next to the first ----------------------------------------------------------------------
 // HIP multiplexes streams onto a few hardware queues (4 per process by default) and hands a new stream the least used one,
@@ -233,9 +310,13 @@ int lg_stream_create_concurrent(void** stream, void* other, int* verified) {
         if (i != pick) (void)hipStreamDestroy(cand[i]);
     if (pick < 0) return LG_ERR_LAUNCH;
     *stream = (void*)cand[pick];
-    return LG_OK;
+    return register_stream(*stream, 0);
 }
-int lg_stream_destroy(void* stream) { return rt(hipStreamDestroy((hipStream_t)stream), "hipStreamDestroy"); }
+int lg_stream_destroy(void* stream) {
+    const int rc = unregister_stream(stream);
+    const int rc2 = rt(hipStreamDestroy((hipStream_t)stream), "hipStreamDestroy");
+    return rc ? rc : rc2;
+}
 int lg_stream_synchronize(void* stream) { return rt(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize"); }
 int lg_stream_wait_event(void* stream, void* event) {
     return rt(hipStreamWaitEvent((hipStream_t)stream, (hipEvent_t)event, 0), "hipStreamWaitEvent");

@@ -24,7 +24,8 @@ _i, _i64, _u64, _f, _d, _p = C.c_int, C.c_int64, C.c_uint64, C.c_float, C.c_doub
 class Report(C.Structure):
     _fields_ = [("records", _i), ("avg_latency_ms", _d), ("p99_latency_ms", _d), ("avg_gpu_ms", _d),
                 ("avg_queue_ms", _d), ("total_duration_ms", _d), ("throughput", _d), ("rounds", _i),
-                ("secondary_launches", _i), ("splits", _i), ("profile_misses", _i), ("avg_e2e_ms", _d), ("p99_e2e_ms", _d)]
+                ("secondary_launches", _i), ("splits", _i), ("profile_misses", _i), ("avg_e2e_ms", _d), ("p99_e2e_ms", _d),
+                ("partition_rounds", _i), ("sub_profile_misses", _i)]
 
     def as_dict(self):
         return {n: getattr(self, n) for n, _ in self._fields_}
@@ -50,6 +51,10 @@ SIGNATURES = {
     "lgh_sched_profile_decode": (_i, [_p, _i, _i, _i]),
     "lgh_sched_profile_contention": (_i, [_p, _i, _i, _i, _i, C.POINTER(_f)]),
     "lgh_sched_set_contention": (_i, [_p, _i, _i, _f]),
+    "lgh_sched_enable_partition": (_i, [_p, _i]),
+    "lgh_sched_profile_partition": (_i, [_p, _i, _i, _i, _i, C.POINTER(_f)]),
+    "lgh_sched_set_partition_factor": (_i, [_p, _i, _i, _f]),
+    "lgh_sched_get_partition_factor": (_f, [_p, _i, _i]),
     "lgh_sched_get_contention": (_f, [_p, _i, _i]),
     "lgh_sched_streams_concurrent": (_i, [_p]),
     "lgh_sched_set_merge_minor": (_i, [_p, _i]),
@@ -223,6 +228,24 @@ class Scheduler:
         out = (_f * 5)()
         check(lib.lgh_sched_profile_contention(self.h, bs, seq, dec_bs, past, out), "lgh_sched_profile_contention")
         return {"main_ms": out[0], "sub_ms": out[1], "both_ms": out[2], "hidden": out[3], "sub_repeats": int(out[4])}
+
+    def enable_partition(self, hbm_cus):
+        """Co-running rounds give the HBM-bound side `hbm_cus` compute units and the MFMA-bound side the rest (0 = off)."""
+        check(lib.lgh_sched_enable_partition(self.h, hbm_cus), "lgh_sched_enable_partition")
+
+    def profile_partition(self, bs, seq, dec_bs, past):
+        """Measures a partitioned co-run (prefill MFMA-bound kernels || decode steps) and installs the budget factors when
+        it beats back-to-back execution on the whole chip."""
+        out = (_f * 7)()
+        check(lib.lgh_sched_profile_partition(self.h, bs, seq, dec_bs, past, out), "lgh_sched_profile_partition")
+        return {"main_ms": out[0], "sub_ms": out[1], "main_part_ms": out[2], "sub_part_ms": out[3], "factor": out[4],
+                "gain": out[5], "sub_repeats": int(out[6])}
+
+    def set_partition_factor(self, main_class, sub_class, value):
+        check(lib.lgh_sched_set_partition_factor(self.h, main_class, sub_class, value), "lgh_sched_set_partition_factor")
+
+    def partition_factor(self, main_class, sub_class):
+        return lib.lgh_sched_get_partition_factor(self.h, main_class, sub_class)
 
     def set_contention(self, main_class, sub_class, value):
         check(lib.lgh_sched_set_contention(self.h, main_class, sub_class, value), "lgh_sched_set_contention")

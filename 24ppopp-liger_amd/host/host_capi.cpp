@@ -26,8 +26,13 @@ struct SchedBase {
     virtual float lookup(int name, int bs, int seq) = 0;
     virtual int sub_lookup(int name, int bs, int seq, float* out, int cap) = 0;
     virtual void set_profile(int name, int bs, int seq, float ms, const float* sub, int nsub) = 0;
-    virtual void serve(int bs, int seq, int n_decode) = 0;
-    virtual void serve_decode(int bs, int past, int n_steps) = 0;
+    virtual bool serve(int bs, int seq, int n_decode) = 0;
+    virtual bool serve_decode(int bs, int past, int n_steps) = 0;
+    virtual bool enable_partition(int hbm_cus) = 0;
+    virtual bool profile_partition(int bs, int seq, int dec_bs, int past, float* out7) = 0;
+    virtual bool set_partition_factor(int main_class, int sub_class, float v) = 0;
+    virtual float get_partition_factor(int main_class, int sub_class) = 0;
+    virtual void extra_counters(int* out2) = 0;
     virtual void set_factor(int factor) = 0;
     virtual bool ctx_ptrs(int i, void** in, void** out) = 0;
     virtual Report run_queued(int mode, int* counters) = 0;
@@ -102,8 +107,28 @@ struct SchedT : SchedBase {
         s->profiling_res_dict[{name, bs, seq}] = ms;
         if (sub && nsub > 0) s->profiling_decompse_res_dict[{name, bs, seq}] = std::vector<float>(sub, sub + nsub);
     }
-    void serve(int bs, int seq, int n_decode) override { s->serve(bs, seq, n_decode); }
-    void serve_decode(int bs, int past, int n_steps) override { s->serve_decode(bs, past, n_steps); }
+    bool serve(int bs, int seq, int n_decode) override { return s->serve(bs, seq, n_decode); }
+    bool serve_decode(int bs, int past, int n_steps) override { return s->serve_decode(bs, past, n_steps); }
+    bool enable_partition(int hbm_cus) override {
+        if (hbm_cus == 0) { s->disable_partition(); return true; }
+        return s->enable_partition(hbm_cus, lg_stream_cu_count(s->DParams0.stream));
+    }
+    bool profile_partition(int bs, int seq, int dec_bs, int past, float* out7) override {
+        auto r = s->profile_partition(bs, seq, dec_bs, past);
+        if (r.factor < 0.f) return false;
+        out7[0] = r.main_ms; out7[1] = r.sub_ms; out7[2] = r.main_part_ms; out7[3] = r.sub_part_ms; out7[4] = r.factor; out7[5] = r.gain;
+        out7[6] = (float)r.sub_repeats;
+        return true;
+    }
+    bool set_partition_factor(int main_class, int sub_class, float v) override {
+        if (main_class < 0 || main_class > 2 || sub_class < 0 || sub_class > 2) return false;
+        s->partition_table[main_class][sub_class] = v;
+        return true;
+    }
+    float get_partition_factor(int main_class, int sub_class) override {
+        return (main_class < 0 || main_class > 2 || sub_class < 0 || sub_class > 2) ? -1.f : s->partition_table[main_class][sub_class];
+    }
+    void extra_counters(int* out2) override { out2[0] = s->partition_rounds; out2[1] = s->sub_profile_misses; }
     void set_factor(int factor) override { s->BertParams.factor = factor; }
     bool ctx_ptrs(int i, void** in, void** out) override {
         auto* c = s->context(i);
@@ -164,15 +189,22 @@ struct ModelT : ModelBase {
 };
 
 int fail(const char* msg) {
-    if (error_state().code == 0) {
-        error_state().code = LG_ERR_INVALID;
-        error_state().text = msg;
-    }
+    set_error_state(LG_ERR_INVALID, msg);
     return LG_ERR_INVALID;
 }
 
 bool shape_ok(ModelBase* mb, int batch, int seq) {
     return mb && batch > 0 && seq > 0 && batch <= mb->P.max_batch_size && seq <= mb->P.max_seq_len;
+}
+
+// what a prefill (decode_past < 0) or decode-step launch vector may touch: the model's default buffers are sized for
+// (max_batch, max_seq), the KV cache for max_batch slots of max_cache_len rows
+bool launch_shape_ok(ModelBase* mb, int batch, int seq, int decode_past, int cache_slot) {
+    if (!mb || batch <= 0 || batch > mb->P.max_batch_size) return false;
+    if (decode_past >= 0)
+        return mb->P.max_cache_len > 0 && decode_past < mb->P.max_cache_len && cache_slot >= 0 && cache_slot + batch <= mb->P.max_batch_size;
+    if (seq <= 0 || seq > mb->P.max_seq_len) return false;
+    return cache_slot < 0 || (mb->P.max_cache_len > 0 && seq <= mb->P.max_cache_len && cache_slot + batch <= mb->P.max_batch_size);
 }
 
 }  // namespace
@@ -181,7 +213,7 @@ extern "C" {
 
 int lgh_first_error(char* buf, int len) {
     if (buf && len > 0) {
-        strncpy(buf, error_state().text.c_str(), (size_t)len - 1);
+        strncpy(buf, error_text().c_str(), (size_t)len - 1);
         buf[len - 1] = 0;
     }
     return first_error();
@@ -289,6 +321,8 @@ int lgh_model_describe(void* model, int batch, int seq, int decode_past, char* b
 int lgh_model_run(void* model, void* input, void* output, int batch, int seq, void* workspace, void* stream, int cache_slot) {
     ModelBase* mb = (ModelBase*)model;
     if (!shape_ok(mb, batch, seq) || !input || !output) return fail("lgh_model_run: bad arguments");
+    if (cache_slot >= 0 && (mb->P.max_cache_len <= 0 || seq > mb->P.max_cache_len || cache_slot + batch > mb->P.max_batch_size))
+        return fail("lgh_model_run: sequence or cache slot outside the KV cache");
     DynamicInitParam D(stream ? stream : mb->stream0->stream, 0);
     for (auto& f : mb->build(input, output, batch, seq, workspace, cache_slot)) f.callback(D);
     return first_error();
@@ -310,10 +344,11 @@ int lgh_model_run_decode(void* model, void* input, void* output, int batch, int 
 int lgh_model_time_kernels(void* model, void* input, void* output, int batch, int seq, int decode_past, int cache_slot,
                            int iters, int trials, float* ms_out, int ms_cap) {
     ModelBase* mb = (ModelBase*)model;
-    if (!mb || !input || !output || iters <= 0 || trials <= 0) return fail("lgh_model_time_kernels: bad arguments");
+    if (!mb || !input || !output || iters <= 0 || trials <= 0) { fail("lgh_model_time_kernels: bad arguments"); return -1; }
+    if (!launch_shape_ok(mb, batch, seq, decode_past, cache_slot)) { fail("lgh_model_time_kernels: shape, position or cache slot outside the model's buffers"); return -1; }
     std::vector<FuncWrap> v = decode_past >= 0 ? mb->build_decode(input, output, batch, decode_past, cache_slot, nullptr)
                                                : mb->build(input, output, batch, seq, nullptr, cache_slot);
-    if ((int)v.size() > ms_cap) return fail("lgh_model_time_kernels: output array too small");
+    if ((int)v.size() > ms_cap) { fail("lgh_model_time_kernels: output array too small"); return -1; }
     DynamicInitParam& D = *mb->stream0;
     void *e0 = nullptr, *e1 = nullptr;
     note_status(lg_event_create(&e0), "lg_event_create");
@@ -334,6 +369,7 @@ struct LghReport {
     double avg_latency_ms, p99_latency_ms, avg_gpu_ms, avg_queue_ms, total_duration_ms, throughput;
     int rounds, secondary_launches, splits, profile_misses;
     double avg_e2e_ms, p99_e2e_ms;  // arrival -> completion on one clock
+    int partition_rounds, sub_profile_misses;
 };
 
 // policy: 0 = classic (communication vs rest), 1 = resource classes (MFMA-bound vs HBM-bound)
@@ -368,6 +404,27 @@ int lgh_sched_profile_contention(void* sched, int bs, int seq, int dec_bs, int p
     if (!((SchedBase*)sched)->profile_contention(bs, seq, dec_bs, past, out5))
         return fail("lgh_sched_profile_contention: needs a pool context and a KV cache");
     return LG_OK;
+}
+// Spatial partition of co-running rounds: hbm_cus compute units (a multiple of 8; 0 switches partitioning off) for the HBM-bound
+// side, the rest for the MFMA-bound side (Scheduler::enable_partition).
+int lgh_sched_enable_partition(void* sched, int hbm_cus) {
+    if (!sched || hbm_cus < 0 || !((SchedBase*)sched)->enable_partition(hbm_cus)) return fail("lgh_sched_enable_partition: bad CU count (a multiple of 8 below the device's) or stream creation failed");
+    return LG_OK;
+}
+// out7 = {prefill kernels alone ms, one decode step alone ms (both on the whole chip), prefill side ms and decode side ms of the
+// partitioned co-run, factor, gain, decode steps co-run}; see Scheduler::profile_partition.
+int lgh_sched_profile_partition(void* sched, int bs, int seq, int dec_bs, int past, float* out7) {
+    if (!sched || bs <= 0 || seq <= 0 || dec_bs <= 0 || past < 0 || !out7) return fail("lgh_sched_profile_partition: bad arguments");
+    if (!((SchedBase*)sched)->profile_partition(bs, seq, dec_bs, past, out7))
+        return fail("lgh_sched_profile_partition: needs lgh_sched_enable_partition, a pool context, a KV cache and shapes inside them");
+    return LG_OK;
+}
+int lgh_sched_set_partition_factor(void* sched, int main_class, int sub_class, float value) {
+    if (!sched || !((SchedBase*)sched)->set_partition_factor(main_class, sub_class, value)) return fail("lgh_sched_set_partition_factor: bad arguments");
+    return LG_OK;
+}
+float lgh_sched_get_partition_factor(void* sched, int main_class, int sub_class) {
+    return sched ? ((SchedBase*)sched)->get_partition_factor(main_class, sub_class) : -1.f;
 }
 // main_class / sub_class: 0 = MFMA-bound, 1 = HBM-bound, 2 = link-bound; a negative value restores the constant factor
 int lgh_sched_set_contention(void* sched, int main_class, int sub_class, float value) {
@@ -408,6 +465,7 @@ int lgh_sched_run_trace(void* sched, int mode, const double* arrival_s, const in
     out->avg_gpu_ms = r.avg_gpu_ms; out->avg_queue_ms = r.avg_queue_ms; out->total_duration_ms = r.total_duration_ms;
     out->throughput = r.throughput; out->rounds = c[0]; out->secondary_launches = c[1]; out->splits = c[2]; out->profile_misses = c[3];
     out->avg_e2e_ms = r.avg_e2e_ms; out->p99_e2e_ms = r.p99_e2e_ms;
+    { int x[2] = {0, 0}; ((SchedBase*)sched)->extra_counters(x); out->partition_rounds = x[0]; out->sub_profile_misses = x[1]; }
     return first_error();
 }
 // Deterministic variant for tests: requests are queued up front with lgh_sched_serve (no request thread, no real-time
@@ -419,12 +477,12 @@ int lgh_sched_set_profile(void* sched, int name, int bs, int seq, float ms, cons
 }
 int lgh_sched_serve(void* sched, int bs, int seq, int n_decode) {
     if (!sched || bs <= 0 || seq <= 0 || n_decode < 0) return fail("lgh_sched_serve: bad arguments");
-    ((SchedBase*)sched)->serve(bs, seq, n_decode);
+    if (!((SchedBase*)sched)->serve(bs, seq, n_decode)) return fail("lgh_sched_serve: request refused");
     return first_error();
 }
 int lgh_sched_serve_decode(void* sched, int bs, int past, int n_steps) {
     if (!sched || bs <= 0 || past < 0 || n_steps <= 0) return fail("lgh_sched_serve_decode: bad arguments");
-    ((SchedBase*)sched)->serve_decode(bs, past, n_steps);
+    if (!((SchedBase*)sched)->serve_decode(bs, past, n_steps)) return fail("lgh_sched_serve_decode: request refused");
     return first_error();
 }
 // decomposition factor used by profile() and by the samples queued afterwards
@@ -446,6 +504,7 @@ int lgh_sched_run_queued(void* sched, int mode, LghReport* out) {
     out->avg_gpu_ms = r.avg_gpu_ms; out->avg_queue_ms = r.avg_queue_ms; out->total_duration_ms = r.total_duration_ms;
     out->throughput = r.throughput; out->rounds = c[0]; out->secondary_launches = c[1]; out->splits = c[2]; out->profile_misses = c[3];
     out->avg_e2e_ms = r.avg_e2e_ms; out->p99_e2e_ms = r.p99_e2e_ms;
+    { int x[2] = {0, 0}; ((SchedBase*)sched)->extra_counters(x); out->partition_rounds = x[0]; out->sub_profile_misses = x[1]; }
     return first_error();
 }
 // the report arithmetic alone (known-answer tests against the reference's published logs)
@@ -455,6 +514,7 @@ int lgh_summarize(const double* cpu_ms, const double* gpu_ms, int n, double tota
     out->records = r.records; out->avg_latency_ms = r.avg_latency_ms; out->p99_latency_ms = r.p99_latency_ms;
     out->avg_gpu_ms = r.avg_gpu_ms; out->avg_queue_ms = r.avg_queue_ms; out->total_duration_ms = r.total_duration_ms;
     out->throughput = r.throughput; out->rounds = out->secondary_launches = out->splits = out->profile_misses = 0;
+    out->avg_e2e_ms = out->p99_e2e_ms = 0; out->partition_rounds = out->sub_profile_misses = 0;
     return LG_OK;
 }
 int lgh_make_poisson_trace(double lambda, int n, int batch, int seq_lo, int seq_hi, int seq_round, int n_decode, uint64_t seed,
@@ -472,6 +532,7 @@ float lgh_model_time_one(void* model, void* input, void* output, int batch, int 
                          int iters) {
     ModelBase* mb = (ModelBase*)model;
     if (!mb || !input || !output || iters <= 0) { fail("lgh_model_time_one: bad arguments"); return -1.f; }
+    if (!launch_shape_ok(mb, batch, seq, decode_past, cache_slot)) { fail("lgh_model_time_one: shape, position or cache slot outside the model's buffers"); return -1.f; }
     std::vector<FuncWrap> v = decode_past >= 0 ? mb->build_decode(input, output, batch, decode_past, cache_slot, nullptr)
                                                : mb->build(input, output, batch, seq, nullptr, cache_slot);
     if (index < 0 || index >= (int)v.size()) { fail("lgh_model_time_one: index out of range"); return -1.f; }

@@ -15,6 +15,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <functional>
+#include <mutex>
 #include <string>
 #include <tuple>
 #include <unordered_map>
@@ -34,22 +35,41 @@ template <> struct dtype_of<float> { static constexpr int value = LG_F32; };
 template <> struct dtype_of<half> { static constexpr int value = LG_F16; };
 
 // ---- error capture ---------------------------------------------------------------------------------
+// The first failing status of the process, written by whichever thread sees it first (the request thread builds vectors, the
+// scheduler thread launches them), hence the lock.
 struct ErrorState {
     int code = 0;
     std::string text;
 };
-inline ErrorState& error_state() {
+inline std::mutex& error_mutex() {
+    static std::mutex m;
+    return m;
+}
+inline ErrorState& error_state_unlocked() {
     static ErrorState s;
     return s;
 }
-inline void note_status(int rc, const char* what) {
-    if (rc != LG_OK && error_state().code == 0) {
-        error_state().code = rc;
-        error_state().text = std::string(what) + ": " + lg_last_error();
-    }
+inline void set_error_state(int code, const std::string& text) {
+    std::lock_guard<std::mutex> lk(error_mutex());
+    ErrorState& e = error_state_unlocked();
+    if (e.code == 0) { e.code = code; e.text = text; }
 }
-inline int first_error() { return error_state().code; }
-inline void clear_error() { error_state() = ErrorState(); }
+inline void note_status(int rc, const char* what) {
+    if (rc != LG_OK) set_error_state(rc, std::string(what) + ": " + lg_last_error());
+}
+inline int error_code() {
+    std::lock_guard<std::mutex> lk(error_mutex());
+    return error_state_unlocked().code;
+}
+inline std::string error_text() {
+    std::lock_guard<std::mutex> lk(error_mutex());
+    return error_state_unlocked().text;
+}
+inline int first_error() { return error_code(); }
+inline void clear_error() {
+    std::lock_guard<std::mutex> lk(error_mutex());
+    error_state_unlocked() = ErrorState();
+}
 
 // ---- per-stream context  (context.h:14-31) ------------------------------------------------------------
 class DynamicInitParam {
@@ -59,7 +79,14 @@ class DynamicInitParam {
     DynamicInitParam() { note_status(lg_stream_create(&stream), "lg_stream_create"); }
     // the reference passes a CUDA stream priority here; priorities are deliberately not used on this platform
     explicit DynamicInitParam(int /*priority*/) { note_status(lg_stream_create(&stream), "lg_stream_create"); }
-    DynamicInitParam(void* existing_stream, int id) : stream(existing_stream), stream_id(id) {}
+    // a stream created elsewhere: the device library is told about it (it then owns a split-K workspace for it)
+    DynamicInitParam(void* existing_stream, int id) : stream(existing_stream), stream_id(id) {
+        note_status(lg_stream_attach(existing_stream, 0), "lg_stream_attach");
+    }
+    // a stream whose kernels run on the compute units selected by the mask only (see lg_stream_create_cu_mask)
+    DynamicInitParam(const unsigned* cu_mask, int mask_words, int id) : stream_id(id) {
+        note_status(lg_stream_create_cu_mask(&stream, cu_mask, mask_words), "lg_stream_create_cu_mask");
+    }
     // a stream that is verified to execute kernels at the same time as `first`'s (two streams of one process may share a
     // hardware queue, on which they would run strictly in turn); `concurrent` tells whether the verification succeeded
     bool concurrent = false;

@@ -244,6 +244,7 @@ class Bert_MLP {
 template <typename T>
 struct MhaBuffers {  // per-request slices, all in elements of T
     T *q, *k, *v, *q_buf, *k_buf, *v_buf, *qk_buf, *attn_trans_out, *attn_out;
+    T* mask;          // attr_mask [batch, seq, seq] of the reference-shaped assembly
     void* decode_ws;  // split-KV partials of the decode attention
 };
 
@@ -262,7 +263,6 @@ class Bert_MHA {
     BertInitParam BertParams;
     T *q_bias, *k_bias, *v_bias, *w_bias;
     T* workspace;
-    std::map<int, T*> masks;  // seq -> attr_mask [max_batch, seq, seq] (all ones, or lower-triangular if causal)
     T *k_cache = nullptr, *v_cache = nullptr;  // [max_batch, heads, max_cache_len, d] when max_cache_len > 0
     std::vector<FuncWrap> FuncWrapVec;
 
@@ -333,9 +333,15 @@ class Bert_MHA {
         const size_t bytes = lg_attn_decode_workspace_bytes(batch, P.head_num / S.world_size, P.size_per_head, P.max_cache_len);
         return align_up((int64_t)((bytes + sizeof(T) - 1) / sizeof(T)));
     }
+    // attr_mask [batch, seq, seq] lives in the request's workspace (reference-shaped assembly only; bert_layer.h:118 keeps one
+    // buffer in the layer, which requests of different lengths in flight at the same time could not share)
+    static int64_t mask_elems(const BertInitParam& P, int batch, int seq) {
+        const bool fused = P.fused && dtype_of<T>::value == LG_F16;
+        return fused ? 0 : align_up((int64_t)batch * seq * seq);
+    }
     static int64_t workspace_elems(const BertInitParam& P, const StaticInitParam& S, int batch, int seq) {
         const int64_t M = (int64_t)batch * seq, hl_ = (int64_t)(P.head_num / S.world_size) * P.size_per_head;
-        return 8 * align_up(M * hl_) + score_elems(P, S, batch, seq) + decode_ws_elems(P, S, batch);
+        return 8 * align_up(M * hl_) + score_elems(P, S, batch, seq) + mask_elems(P, batch, seq) + decode_ws_elems(P, S, batch);
     }
     MhaBuffers<T> slice(T* ws, int batch, int seq) const {
         const int64_t M = (int64_t)batch * seq, a = align_up(M * hl());
@@ -344,25 +350,10 @@ class Bert_MHA {
         b.q_buf = b.v + a; b.k_buf = b.q_buf + a; b.v_buf = b.k_buf + a;
         b.attn_trans_out = b.v_buf + a; b.attn_out = b.attn_trans_out + a;
         b.qk_buf = b.attn_out + a;
-        b.decode_ws = b.qk_buf + score_elems(BertParams, SParam, batch, seq);
+        b.mask = b.qk_buf + score_elems(BertParams, SParam, batch, seq);
+        b.decode_ws = b.mask + mask_elems(BertParams, batch, seq);
         return b;
     }
-    T* mask_for(int seq) {
-        auto it = masks.find(seq);
-        if (it != masks.end()) return it->second;
-        const int64_t e = (int64_t)BertParams.max_batch_size * seq * seq;
-        T* m = dev_alloc<T>(e);
-        if (BertParams.causal) {
-            if (dtype_of<T>::value == LG_F16) note_status(lg_fill_causal_mask_f16(m, BertParams.max_batch_size, seq, nullptr), "lg_fill_causal_mask_f16");
-            else note_status(lg_fill_causal_mask_f32((float*)m, BertParams.max_batch_size, seq, nullptr), "lg_fill_causal_mask_f32");
-        } else {
-            dev_fill_const(m, e, 1.0f);
-        }
-        note_status(lg_device_synchronize(), "lg_device_synchronize");
-        masks[seq] = m;
-        return m;
-    }
-
     // idx 0..8 of the launch vector (9 entries); fused assembly: 5 entries.
     // cache_slot >= 0 (fused only): K/V are written straight into the KV cache rows [cache_slot, cache_slot+batch).
     std::vector<FuncWrap> forward(T* input, T* output, int batch_size, int seq_len, T* ws = nullptr, int cache_slot = -1) {
@@ -372,6 +363,10 @@ class Bert_MHA {
         const int M = batch_size * seq_len, h = heads(), d = BertParams.size_per_head;
         const int dt = dtype_of<T>::value;
         const float sc = scalar;
+        if (cache_slot >= 0 && k_cache && (seq_len > BertParams.max_cache_len || cache_slot + batch_size > BertParams.max_batch_size)) {
+            set_error_state(LG_ERR_INVALID, "Bert_MHA::forward: sequence or cache slot outside the KV cache");
+            return FuncWrapVec;
+        }
         if (BertParams.fused && dt == LG_F16) {
             T* kdst = b.k_buf;
             T* vdst = b.v_buf;
@@ -434,10 +429,18 @@ class Bert_MHA {
             GemmStridedBatchedEx(D, dt, 1, 0, seq_len, seq_len, d, b.k_buf, d, (long long)seq_len * d, b.q_buf, d,
                                  (long long)seq_len * d, b.qk_buf, seq_len, (long long)seq_len * seq_len, batch_size * h);
         }, "qk_gemm", MFMA_BOUND));
-        // softmax  (:153-155)
-        T* mask = mask_for(seq_len);
+        // softmax  (:153-155).  The mask (all ones, or lower-triangular) is written into the request's workspace by the same
+        // entry, on the launch stream: building the vector neither allocates nor synchronises.
+        const int causal_mask = BertParams.causal;
         FuncWrapVec.push_back(FuncWrap(0.2f, COMPUTATION, [=](const DynamicInitParam& D) {
-            Attn_softmax_kernel<T>(b.qk_buf, mask, batch_size, seq_len, h, sc, D);
+            if (dt == LG_F16) {
+                if (causal_mask) note_status(lg_fill_causal_mask_f16(b.mask, batch_size, seq_len, D.stream), "lg_fill_causal_mask_f16");
+                else note_status(lg_fill_const_f16(b.mask, (int64_t)batch_size * seq_len * seq_len, 1.0f, D.stream), "lg_fill_const_f16");
+            } else {
+                if (causal_mask) note_status(lg_fill_causal_mask_f32((float*)b.mask, batch_size, seq_len, D.stream), "lg_fill_causal_mask_f32");
+                else note_status(lg_fill_const_f32((float*)b.mask, (int64_t)batch_size * seq_len * seq_len, 1.0f, D.stream), "lg_fill_const_f32");
+            }
+            Attn_softmax_kernel<T>(b.qk_buf, b.mask, batch_size, seq_len, h, sc, D);
         }, "softmax"));
         // qkv  (:158-163)
         FuncWrapVec.push_back(FuncWrap(0.3f, COMPUTATION, [=](const DynamicInitParam& D) {
@@ -462,6 +465,11 @@ class Bert_MHA {
         if (!ws) ws = workspace;
         const MhaBuffers<T> b = slice(ws, batch, 1);
         const int h = heads(), d = BertParams.size_per_head, Lmax = BertParams.max_cache_len;
+        // the K/V epilogues write cache row `past` of slots [cache_slot, cache_slot + batch): outside the cache nothing is built
+        if (!k_cache || past < 0 || past >= Lmax || cache_slot < 0 || cache_slot + batch > BertParams.max_batch_size) {
+            set_error_state(LG_ERR_INVALID, "Bert_MHA::forward_decode: position or cache slot outside the KV cache");
+            return FuncWrapVec;
+        }
         const float sc = scalar;
         T* kc = k_cache + (int64_t)cache_slot * h * Lmax * d;
         T* vc = v_cache + (int64_t)cache_slot * h * Lmax * d;

@@ -52,7 +52,7 @@ int main(int argc, char** argv) {
         sched.output_recording();
     }
     if (first_error()) {
-        fprintf(stderr, "error: %s\n", error_state().text.c_str());
+        fprintf(stderr, "error: %s\n", error_text().c_str());
         return 1;
     }
     return 0;

@@ -68,10 +68,13 @@ class Sample {
             if (!_neutral(FuncWrapVec[i])) return _class_of(FuncWrapVec[i]);
         return _class_of(f);
     }
-    const std::vector<float>* _profile(const FuncWrap& f) const {
+    // The decomposition table is looked up with the key the scheduler used for the durations: seq rounded up to the
+    // profile grid (key_seq), so a request whose length is not itself a profiled key can still be split.
+    const std::vector<float>* _profile(const FuncWrap& f) {
         if (!profiling_decompse_res_dict) return nullptr;
-        auto it = profiling_decompse_res_dict->find({f.name, batch_size, seq_len});
-        if (it == profiling_decompse_res_dict->end() || (int)it->second.size() < _factor - 1) return nullptr;
+        auto it = profiling_decompse_res_dict->find({f.name, batch_size, key_seq});
+        if (it == profiling_decompse_res_dict->end() && key_seq != seq_len) it = profiling_decompse_res_dict->find({f.name, batch_size, seq_len});
+        if (it == profiling_decompse_res_dict->end() || (int)it->second.size() < _factor - 1) { sub_profile_misses++; return nullptr; }
         return &it->second;
     }
 
@@ -83,6 +86,8 @@ class Sample {
     size_t exe_num = 0;
     void *start = nullptr, *stop = nullptr, *last_launch = nullptr;
     int batch_size, seq_len;
+    int key_seq = 0;            // seq_len on the profile grid (set by the scheduler; seq_len when there is no grid)
+    int sub_profile_misses = 0; // GEMMs that could not be split because the decomposition table has no entry for them
     int id = 0;
     bool merge_minor = false;  // see _neutral(); false = every entry keeps its own class (the reference's behaviour)
     void* user = nullptr;  // owner's per-request context (buffers), opaque here
@@ -90,7 +95,7 @@ class Sample {
     Sample(std::vector<FuncWrap>& vec, const SubDict& sub_dict, int batch_size_, int seq_len_, int factor,
            class_policy policy = CLASSIC, split_axis axis = SPLIT_OUT_COLS)
         : _factor(factor), _policy(policy), _axis(axis), FuncWrapVec(vec), profiling_decompse_res_dict(&sub_dict),
-          batch_size(batch_size_), seq_len(seq_len_) {
+          batch_size(batch_size_), seq_len(seq_len_), key_seq(seq_len_) {
         note_status(lg_event_create(&start), "lg_event_create");
         note_status(lg_event_create(&stop), "lg_event_create");
         note_status(lg_event_create(&last_launch), "lg_event_create");
@@ -128,6 +133,22 @@ class Sample {
         if (_sub_size() >= 2) return false;  // next two launches are pieces of the same GEMM
         const size_t after = (_sub_exe_num > 0) ? exe_num : exe_num + 1;
         return _class_of(_SubFuncWrapVec[_sub_exe_num].func) != _class_at(after);
+    }
+
+    // Stand-alone milliseconds of the launches at the head of this request that may run next to a primary segment of class
+    // `cls`: everything up to the next entry of that class (at most `limit` entries are looked at).
+    float run_ahead_duration(int cls, int limit = 256) const {
+        float t = 0.f;
+        for (size_t i = _sub_exe_num; i < _SubFuncWrapVec.size(); ++i) {
+            if (_class_of(_SubFuncWrapVec[i].func) == cls) return t;
+            t += _SubFuncWrapVec[i].func.duration;
+        }
+        const size_t first = exe_num + ((!_sub_empty() && _sub_exe_num == 0) ? 1 : 0);  // pending pieces stand for their parent
+        for (size_t i = first; i < FuncWrapVec.size() && (int)(i - first) < limit; ++i) {
+            if (_class_at(i) == cls) break;
+            t += FuncWrapVec[i].duration;
+        }
+        return t;
     }
 
     // may not co-run with a primary segment of class `cls`  (init.h:131-149)

@@ -139,8 +139,19 @@ class Scheduler {
     split_axis axis = SPLIT_OUT_COLS;
     int seq_bucket = 1;               // durations are looked up at seq rounded up to a multiple of this
     int ignore_num = 20;              // warm-up records dropped from the report (schedule.h:327)
-    int profile_misses = 0;
-    int rounds = 0, secondary_launches = 0, splits = 0;
+    int profile_misses = 0, sub_profile_misses = 0;
+    int rounds = 0, secondary_launches = 0, splits = 0, partition_rounds = 0;
+    // ---- spatial partition of the two streams (enable_partition) ---------------------------------------------------------
+    // The reference keeps its two streams apart with stream priorities and a cap on hardware queues (schedule.h:54-55,
+    // context.h:27); here a co-running round gives each class its own compute units instead: the HBM-bound side runs on
+    // partition_hbm_cus of them, the MFMA-bound side on the rest, on CU-masked streams, and every kernel sizes its grid for
+    // its share.  A round is partitioned only while a waiting request has work of the other class, and only for as long as
+    // that work lasts; all other rounds run on the whole chip.  partition_table[main][sub] = stand-alone milliseconds of
+    // class-`sub` work that complete per stand-alone millisecond of the class-`main` primary in a partitioned round
+    // (measured by profile_partition; <= 0: partitioning that pair does not pay and is not done).
+    int partition_hbm_cus = 0;
+    float partition_table[3][3] = {{-1.f, -1.f, -1.f}, {-1.f, -1.f, -1.f}, {-1.f, -1.f, -1.f}};
+    float partition_min_ms = 0.05f;   // less waiting work than this is not worth a partitioned round
     StaticInitParam SParams;
     DynamicInitParam DParams0;
     DynamicInitParam DParams1;
@@ -165,6 +176,27 @@ class Scheduler {
         if (_thread.joinable()) _thread.join();
     }
 
+    // Creates the four CU-masked streams of partitioned rounds: [role: primary, secondary] x [class: MFMA-bound, HBM-bound].
+    // hbm_cus compute units (a multiple of 8, spread evenly over the 8 dies: mask bits 0 .. hbm_cus-1) go to the HBM-bound
+    // side, the rest to the MFMA-bound side.  Returns false (and leaves partitioning off) on bad arguments.
+    bool enable_partition(int hbm_cus, int total_cus = 256) {
+        if (hbm_cus <= 0 || hbm_cus % 8 != 0 || hbm_cus >= total_cus || total_cus > 256 || total_cus % 8 != 0) return false;
+        if (partition_hbm_cus == hbm_cus) return true;
+        unsigned hbm_mask[8] = {0}, mfma_mask[8] = {0};
+        for (int b = 0; b < total_cus; ++b) (b < hbm_cus ? hbm_mask : mfma_mask)[b >> 5] |= 1u << (b & 31);
+        for (int role = 0; role < 2; ++role) {
+            _part[role][MFMA_BOUND].reset(new DynamicInitParam(mfma_mask, 8, 2 + 2 * role + MFMA_BOUND));
+            _part[role][HBM_BOUND].reset(new DynamicInitParam(hbm_mask, 8, 2 + 2 * role + HBM_BOUND));
+        }
+        if (first_error()) { partition_hbm_cus = 0; return false; }
+        partition_hbm_cus = hbm_cus;
+        return true;
+    }
+    void disable_partition() { partition_hbm_cus = 0; }
+    const DynamicInitParam* partition_stream(int role, int cls) const {
+        return (partition_hbm_cus > 0 && (cls == MFMA_BOUND || cls == HBM_BOUND)) ? _part[role][cls].get() : nullptr;
+    }
+
     // ---- per-request contexts ------------------------------------------------------------------------------
     // Allocates `count` contexts sized for (max_batch_size, max_seq_len); serve() blocks when all are in flight.
     void make_pool(int count, int ctx_batch) {
@@ -184,13 +216,39 @@ class Scheduler {
             _all_ctx.push_back(c);
             _pool_total++;
         }
+        _ctx_batch = ctx_batch;
         note_status(lg_device_synchronize(), "lg_device_synchronize");
+    }
+    // Shapes a request may have: they decide how far the launch vector writes into the request's buffers, its workspace and
+    // its KV-cache slots, so they are checked once here, on the host, before anything is built or launched.
+    bool request_fits(int batch_size, int seq_len, int n_decode, const char* who) {
+        const int max_b = _pool_total ? _ctx_batch : BertParams.max_batch_size;
+        const bool ok = batch_size > 0 && seq_len > 0 && n_decode >= 0 && batch_size <= max_b && seq_len <= BertParams.max_seq_len &&
+                        (n_decode == 0 || (BertParams.max_cache_len > 0 && seq_len + n_decode <= BertParams.max_cache_len));
+        if (!ok && error_code() == 0)
+            set_error_state(LG_ERR_INVALID, std::string(who) + ": request (batch " + std::to_string(batch_size) + ", seq " + std::to_string(seq_len) +
+                            ", decode steps " + std::to_string(n_decode) + ") exceeds the contexts (batch " + std::to_string(max_b) + ", seq " +
+                            std::to_string(BertParams.max_seq_len) + ", cache " + std::to_string(BertParams.max_cache_len) + ")");
+        return ok;
+    }
+    bool decode_fits(int batch_size, int past, int n_steps, const char* who) {
+        const int max_b = _pool_total ? _ctx_batch : BertParams.max_batch_size;
+        const bool ok = batch_size > 0 && past >= 0 && n_steps > 0 && batch_size <= max_b && BertParams.max_cache_len > 0 &&
+                        past + n_steps <= BertParams.max_cache_len;
+        if (!ok && error_code() == 0)
+            set_error_state(LG_ERR_INVALID, std::string(who) + ": decode request (batch " + std::to_string(batch_size) + ", past " + std::to_string(past) +
+                            ", steps " + std::to_string(n_steps) + ") exceeds the contexts (batch " + std::to_string(max_b) + ", cache " +
+                            std::to_string(BertParams.max_cache_len) + ")");
+        return ok;
     }
     // contexts in creation order (tests compare a request's output buffer with a plain sequential run)
     const ReqCtx* context(int i) const { return (i >= 0 && i < (int)_all_ctx.size()) ? _all_ctx[i] : nullptr; }
+    // Blocks while every context is in flight -- but only if a scheduler loop is running that can return one; with no loop
+    // running (requests queued up front, more of them than contexts) it fails with nullptr instead of waiting forever.
     ReqCtx* acquire_ctx() {
         std::unique_lock<std::mutex> lk(_pool_mutex);
-        _pool_cv.wait(lk, [this] { return !_pool.empty(); });
+        _pool_cv.wait(lk, [this] { return !_pool.empty() || !_running.load(); });
+        if (_pool.empty()) return nullptr;
         ReqCtx* c = _pool.front();
         _pool.erase(_pool.begin());
         return c;
@@ -251,6 +309,10 @@ class Scheduler {
     }
     // Profiles one decode step at `past` cached positions; keys are {1000 + k, bs, past}.
     void profile_decode(int bs, int past, int itr = 20) {
+        if (bs > BertParams.max_batch_size || BertParams.max_cache_len <= 0 || past < 0 || past >= BertParams.max_cache_len) {
+            if (error_code() == 0) set_error_state(LG_ERR_INVALID, "profile_decode: batch or cached positions exceed the model's KV cache");
+            return;
+        }
         std::vector<FuncWrap> vec = _model->forward_decode(input, output, bs, past, 0);
         const int count = _model->kernels_per_layer(true);
         for (int k = 0; k < count; k++) vec[k].callback(DParams0);
@@ -272,6 +334,8 @@ class Scheduler {
     ContentionSample profile_contention(int bs, int seq, int dec_bs, int past, int trials = 3) {
         ContentionSample r = {0.f, 0.f, 0.f, -1.f, 0};
         if (_all_ctx.empty() || BertParams.max_cache_len <= 0) return r;
+        if (bs <= 0 || seq <= 0 || bs > BertParams.max_batch_size || seq > BertParams.max_seq_len || dec_bs <= 0 || dec_bs > _ctx_batch ||
+            past < 0 || past >= BertParams.max_cache_len) return r;
         ReqCtx* c = _all_ctx[0];
         std::vector<FuncWrap> pre = _model->forward(input, output, bs, seq);
         std::vector<FuncWrap> A;
@@ -319,11 +383,90 @@ class Scheduler {
         return r;
     }
 
+    struct PartitionSample { float main_ms, sub_ms, main_part_ms, sub_part_ms, factor, gain; int sub_repeats; };
+    // Measures a partitioned co-run: the MFMA-bound kernels of one prefill layer (bs x seq) on the MFMA side's compute units
+    // next to `reps` decode steps (dec_bs sequences, `past` cached positions) on the HBM side's, against both run one after the
+    // other on the whole chip.  factor = stand-alone ms of decode work completed per stand-alone ms of prefill work while both
+    // run; gain = whole-chip back-to-back time / partitioned co-run time of the same work.  Fills partition_table (both
+    // directions) when gain exceeds min_gain, clears it otherwise.  Needs enable_partition, a pool context and a KV cache.
+    PartitionSample profile_partition(int bs, int seq, int dec_bs, int past, int trials = 3, float min_gain = 1.02f) {
+        PartitionSample r = {0.f, 0.f, 0.f, 0.f, -1.f, 0.f, 0};
+        if (partition_hbm_cus <= 0 || _all_ctx.empty() || BertParams.max_cache_len <= 0) return r;
+        if (bs <= 0 || seq <= 0 || bs > BertParams.max_batch_size || seq > BertParams.max_seq_len || dec_bs <= 0 || dec_bs > _ctx_batch ||
+            past < 0 || past >= BertParams.max_cache_len) return r;
+        ReqCtx* c = _all_ctx[0];
+        std::vector<FuncWrap> pre = _model->forward(input, output, bs, seq);
+        std::vector<FuncWrap> A;
+        for (int k = 0; k < BertParams.kernel_num; k++)
+            if (pre[k].rclass == MFMA_BOUND) A.push_back(pre[k]);
+        const int kd = _model->kernels_per_layer(true);
+        std::vector<FuncWrap> dec = _model->forward_decode(c->dec_a, c->dec_b, dec_bs, past, c->slot, c->ws);
+        std::vector<FuncWrap> B(dec.begin(), dec.begin() + kd);
+        if (A.empty() || B.empty()) return r;
+        void *e0 = nullptr, *eA = nullptr, *eB = nullptr;
+        note_status(lg_event_create(&e0), "lg_event_create");
+        note_status(lg_event_create(&eA), "lg_event_create");
+        note_status(lg_event_create(&eB), "lg_event_create");
+        for (int k = 0; k < BertParams.kernel_num; k++) pre[k].callback(DParams0);
+        auto run = [&](const DynamicInitParam& DA, const DynamicInitParam& DB, int nA, int nB, float& tA, float& tB) {
+            note_status(lg_device_synchronize(), "lg_device_synchronize");
+            note_status(lg_event_record(e0, DA.stream), "lg_event_record");
+            note_status(lg_stream_wait_event(DB.stream, e0), "lg_stream_wait_event");
+            for (int i = 0; i < nA; ++i) for (auto& f : A) f.callback(DA);
+            for (int i = 0; i < nB; ++i) for (auto& f : B) f.callback(DB);
+            note_status(lg_event_record(eA, DA.stream), "lg_event_record");
+            note_status(lg_event_record(eB, DB.stream), "lg_event_record");
+            note_status(lg_event_synchronize(eA), "lg_event_synchronize");
+            note_status(lg_event_synchronize(eB), "lg_event_synchronize");
+            note_status(lg_event_elapsed_ms(&tA, e0, eA), "lg_event_elapsed_ms");
+            note_status(lg_event_elapsed_ms(&tB, e0, eB), "lg_event_elapsed_ms");
+        };
+        const DynamicInitParam& PM = *_part[0][MFMA_BOUND];
+        const DynamicInitParam& SH = *_part[1][HBM_BOUND];
+        float a, b, main_full = 1e30f, sub_full = 1e30f;
+        run(DParams0, DParams1, 1, 1, a, b);  // warm-up on the whole chip and on the shares
+        run(PM, SH, 1, 1, a, b);
+        for (int t = 0; t < trials; ++t) { run(DParams0, DParams1, 1, 0, a, b); main_full = std::min(main_full, a); }
+        for (int t = 0; t < trials; ++t) { run(DParams0, DParams1, 0, 1, a, b); sub_full = std::min(sub_full, b); }
+        // as many decode steps as finish together with the prefill kernels: start from the whole-chip ratio, correct once
+        int reps = std::max(1, (int)(main_full / std::max(sub_full, 1e-6f) + 0.5f));
+        float best_a = 0.f, best_b = 0.f;
+        for (int pass = 0; pass < 2; ++pass) {
+            float best = 1e30f;
+            for (int t = 0; t < trials; ++t) {
+                run(PM, SH, 1, reps, a, b);
+                if (std::max(a, b) < best) { best = std::max(a, b); best_a = a; best_b = b; }
+            }
+            if (pass == 0) {
+                const int adj = std::max(1, (int)((float)reps * best_a / std::max(best_b, 1e-6f) + 0.5f));
+                if (adj == reps) break;
+                reps = adj;
+            }
+        }
+        lg_event_destroy(e0); lg_event_destroy(eA); lg_event_destroy(eB);
+        r.main_ms = main_full; r.sub_ms = sub_full; r.main_part_ms = best_a; r.sub_part_ms = best_b; r.sub_repeats = reps;
+        // decode work per millisecond of co-run, times how long the prefill kernels take there, per millisecond of their own
+        r.factor = ((float)reps * sub_full / std::max(best_b, 1e-6f)) * best_a / std::max(main_full, 1e-6f);
+        r.gain = (main_full + (float)reps * sub_full) / std::max(std::max(best_a, best_b), 1e-6f);
+        if (r.gain >= min_gain && r.factor > 0.f) {
+            partition_table[MFMA_BOUND][HBM_BOUND] = r.factor;
+            partition_table[HBM_BOUND][MFMA_BOUND] = 1.0f / r.factor;
+        } else {
+            partition_table[MFMA_BOUND][HBM_BOUND] = partition_table[HBM_BOUND][MFMA_BOUND] = -1.f;
+        }
+        return r;
+    }
+
     // ---- serve  (schedule.h:159-172) ------------------------------------------------------------------------
     // Builds the launch vector of one request (prefill of batch_size x seq_len, then n_decode decode steps), stamps
     // kernel indices and profiled durations, and queues it.
-    void serve(int batch_size, int seq_len, int n_decode = 0) {
+    bool serve(int batch_size, int seq_len, int n_decode = 0) {
+        if (!request_fits(batch_size, seq_len, n_decode, "serve")) return false;
         ReqCtx* ctx = _pool_total ? acquire_ctx() : nullptr;  // without a pool all requests share the default buffers
+        if (_pool_total && !ctx) {
+            if (error_code() == 0) set_error_state(LG_ERR_INVALID, "serve: every request context is in flight and no scheduler loop is running to return one");
+            return false;
+        }
         T* in = ctx ? ctx->input : input;
         T* out = ctx ? ctx->output : output;
         T* ws = ctx ? ctx->ws : nullptr;
@@ -369,17 +512,24 @@ class Scheduler {
         Sample* sample = new Sample(vec, profiling_decompse_res_dict, batch_size, seq_len, BertParams.factor, policy, axis);
         sample->user = ctx;
         sample->merge_minor = merge_minor;
+        sample->key_seq = seq_bucket > 1 ? (seq_len + seq_bucket - 1) / seq_bucket * seq_bucket : seq_len;
         {
             std::lock_guard<std::mutex> lk(_q_mutex);
             sample->id = _next_id++;
             _main_q.push_back(sample);
         }
+        return true;
     }
 
     // Queues a request that consists of decode steps only: `n_steps` single-token steps for `batch_size` sequences that
     // already have `past` cached positions (cache contents are whatever the slot holds).  No reference counterpart.
-    void serve_decode(int batch_size, int past, int n_steps) {
+    bool serve_decode(int batch_size, int past, int n_steps) {
+        if (!decode_fits(batch_size, past, n_steps, "serve_decode")) return false;
         ReqCtx* ctx = _pool_total ? acquire_ctx() : nullptr;
+        if (_pool_total && !ctx) {
+            if (error_code() == 0) set_error_state(LG_ERR_INVALID, "serve_decode: every request context is in flight and no scheduler loop is running to return one");
+            return false;
+        }
         T* din = ctx ? ctx->dec_a : input;
         T* dout = ctx ? ctx->dec_b : output;
         T* ws = ctx ? ctx->ws : nullptr;
@@ -405,6 +555,7 @@ class Scheduler {
             sample->id = _next_id++;
             _main_q.push_back(sample);
         }
+        return true;
     }
 
     size_t queued() {
@@ -417,6 +568,7 @@ class Scheduler {
         if (!exe_vec.empty() && exe_vec[0]->empty()) {
             Sample* tmp = exe_vec[0];
             recs.push_back(tmp->get_recording());
+            sub_profile_misses += tmp->sub_profile_misses;
             exe_vec.erase(exe_vec.begin());
             _retired.push_back(tmp);
         }
@@ -434,6 +586,7 @@ class Scheduler {
 
     // ---- baseline: one request at a time on stream 0  (schedule.h:204-219) -----------------------------------------
     void run_sequential() {
+        RunningGuard running(this);
         float time_planned = 0;
         note_status(lg_event_record(Wait_EVENT, DParams0.stream), "lg_event_record");
         while (!(_stop.load() && drained())) {
@@ -450,6 +603,13 @@ class Scheduler {
 
     // ---- Liger: interleave the waiting requests into the primary's windows  (schedule.h:221-278) ----------------------
     void run_stream_sync() {
+        RunningGuard running(this);
+        // two requests on two streams must not share buffers: without per-request contexts only one request may be in flight
+        if (_pool_total == 0 && schedule_deep > 1) {
+            if (error_code() == 0) set_error_state(LG_ERR_INVALID, "run_stream_sync: interleaving needs per-request contexts (make_pool) or schedule_deep 1");
+            _drop_queued();
+            return;
+        }
         float time_planned = 0.0f;
         int main_class = 0;
         note_status(lg_event_record(Wait_EVENT, DParams0.stream), "lg_event_record");
@@ -457,20 +617,44 @@ class Scheduler {
         while (!(_stop.load() && drained())) {
             update_vec();
             if (exe_vec.empty()) continue;
-            // hybrid synchronisation: the host waits for everything before the last kernel of the previous round,
-            // stream 1 waits (on the device) for the end of the previous round
-            note_status(lg_event_synchronize(Wait_EVENT), "lg_event_synchronize");
-            note_status(lg_stream_wait_event(DParams1.stream, Main_EVENT), "lg_stream_wait_event");
             Sample* head = exe_vec.at(0);
+            // Partitioned round?  Only while a waiting request has work of the other class at its head, and only for as much
+            // primary time as that work needs; the primary then runs on its class's share of the compute units, the
+            // secondaries on the other share.  Otherwise (and always without enable_partition) the round is the reference's:
+            // primary on stream 0, secondaries on stream 1, both on the whole chip.
+            const DynamicInitParam* Dp = &DParams0;
+            const DynamicInitParam* Ds = &DParams1;
+            float part_factor = -1.f, cap = 0.f;
+            if (partition_hbm_cus > 0 && policy == RESOURCE && !head->empty()) {
+                const int mc = head->next_class();
+                const int sc = mc == MFMA_BOUND ? HBM_BOUND : (mc == HBM_BOUND ? MFMA_BOUND : -1);
+                if (sc >= 0 && partition_table[mc][sc] > 0.f) {
+                    float need = 0.f;
+                    for (size_t s = 1; s < exe_vec.size(); s++)
+                        if (!exe_vec[s]->empty()) need += exe_vec[s]->run_ahead_duration(mc);
+                    if (need >= partition_min_ms) {
+                        part_factor = partition_table[mc][sc];
+                        cap = need / part_factor;
+                        Dp = _part[0][mc].get();
+                        Ds = _part[1][sc].get();
+                        partition_rounds++;
+                    }
+                }
+            }
+            // hybrid synchronisation: the host waits for everything before the last kernel of the previous round,
+            // the secondary stream waits (on the device) for the end of the previous round
+            note_status(lg_event_synchronize(Wait_EVENT), "lg_event_synchronize");
+            note_status(lg_stream_wait_event(Ds->stream, Main_EVENT), "lg_stream_wait_event");
             while (!head->empty()) {
                 main_class = head->next_class();
-                if (head->is_switch()) {
-                    note_status(lg_event_record(Wait_EVENT, DParams0.stream), "lg_event_record");
-                    time_planned += head->dequeue(DParams0, 1, time_planned);
-                    note_status(lg_event_record(Main_EVENT, DParams0.stream), "lg_event_record");
+                const bool capped = part_factor > 0.f && time_planned + head->duration(1, time_planned) >= cap;
+                if (head->is_switch() || capped) {
+                    note_status(lg_event_record(Wait_EVENT, Dp->stream), "lg_event_record");
+                    time_planned += head->dequeue(*Dp, 1, time_planned);
+                    note_status(lg_event_record(Main_EVENT, Dp->stream), "lg_event_record");
                     break;
                 }
-                time_planned += head->dequeue(DParams0, 1, time_planned);
+                time_planned += head->dequeue(*Dp, 1, time_planned);
             }
             rounds++;
             // time_planned stays in units of the primary's time; a secondary kernel of stand-alone duration d uses up
@@ -479,7 +663,7 @@ class Scheduler {
                 Sample* sub = exe_vec.at(s);
                 while (time_planned > 0 && !sub->empty()) {
                     if (sub->is_same_class(main_class)) break;
-                    const float f = contention(main_class, sub->next_class());
+                    const float f = part_factor > 0.f ? part_factor : contention(main_class, sub->next_class());
                     float avail = time_planned * f;
                     if (sub->duration(0, avail) > avail) {
                         if (sub->type() == GEMM && sub->possible_duration(avail)) {
@@ -488,7 +672,7 @@ class Scheduler {
                         }
                         time_planned = 0.0f;
                     } else {
-                        time_planned -= sub->dequeue(DParams1, 0, avail) / f;
+                        time_planned -= sub->dequeue(*Ds, 0, avail) / f;
                         secondary_launches++;
                     }
                 }
@@ -509,13 +693,14 @@ class Scheduler {
         _epoch_host = std::chrono::steady_clock::now();
         for (auto& r : recs) { lg_event_destroy(r.start); lg_event_destroy(r.stop); }
         recs.clear();
-        rounds = secondary_launches = splits = 0;
+        rounds = secondary_launches = splits = partition_rounds = 0;
     }
 
     // ---- request simulator  (schedule.h:285-321) ---------------------------------------------------------------------
     // Replays `trace` in real time on a second host thread, then requests stop.
     void serving(const std::vector<TraceRequest>& trace) {
         if (_thread.joinable()) _thread.join();
+        _running.store(true);  // a loop is about to run: serve() may wait for a context instead of failing
         _thread = std::thread([this, trace]() {
             const auto t0 = std::chrono::steady_clock::now();
             for (const auto& r : trace) {
@@ -588,6 +773,19 @@ class Scheduler {
     }
 
   private:
+    std::atomic<bool> _running{false};
+    int _ctx_batch = 0;
+    struct RunningGuard {
+        Scheduler* s;
+        explicit RunningGuard(Scheduler* s_) : s(s_) { s->_running.store(true); }
+        ~RunningGuard() { s->_running.store(false); s->_pool_cv.notify_all(); }
+    };
+    void _drop_queued() {
+        std::lock_guard<std::mutex> lk(_q_mutex);
+        for (Sample* smp : _main_q) delete smp;
+        _main_q.clear();
+    }
+    std::unique_ptr<DynamicInitParam> _part[2][2];  // CU-masked streams of partitioned rounds: [role][class]
     void* _epoch_event = nullptr;
     std::chrono::steady_clock::time_point _epoch_host;
     std::vector<Sample*> _retired;
@@ -609,6 +807,9 @@ class Scheduler {
     void _finish() {
         note_status(lg_stream_synchronize(DParams0.stream), "lg_stream_synchronize");
         note_status(lg_stream_synchronize(DParams1.stream), "lg_stream_synchronize");
+        for (int role = 0; role < 2; ++role)
+            for (int cls = 0; cls < 2; ++cls)
+                if (_part[role][cls]) note_status(lg_stream_synchronize(_part[role][cls]->stream), "lg_stream_synchronize");
         _reclaim();
         if (_thread.joinable()) _thread.join();
     }

@@ -101,39 +101,61 @@ def kernel_only(args, capi, host, model, x, y, B, S, H, stream):
     print(json.dumps({"kernel": name, "iters": args.iters, "avg_ms_hip_events": round(ms, 5)}))
 
 
-def bench_cfg4(capi, host, weight_layout):
-    """BASELINE config 4: a prefill request (batch 4 x seq 512) is decomposed by factor 1, 2, 4, 8 (token rows) and
-    interleaved on two streams with a decode batch (32 sequences, 1024 cached positions, 8 steps); makespan against
-    sequential launch of the same two requests.  The decode batch is the primary request (its HBM-bound kernels open the
-    windows), the prefill's MFMA-bound GEMMs are the ones split to fit them."""
+def bench_cfg4(capi, host, weight_layout, factors=(1, 2, 4, 8), shares=(0, 64, 96, 128), repeats=3):
+    """BASELINE config 4: a prefill request (batch 4 x seq 512) is decomposed by `factors` (token rows) and interleaved on two
+    streams with a decode batch (32 sequences, 1024 cached positions, 8 steps); makespan against sequential launch of the same
+    two requests.  The decode batch is the primary request (its HBM-bound kernels open the windows), the prefill's MFMA-bound
+    GEMMs are the ones split to fit them.  `shares` = compute units given to the HBM-bound side in co-running rounds (0: both
+    streams on the whole chip, as the reference runs them).  Each request has its own context (buffers, workspace, cache slots)."""
     c = CFG2
     out = []
-    model = host.Model(capi.F16, 36, 512, c["heads_global"], c["d"], layer_num=1, world_size=c["world_size"], ffn_inner=c["ffn_global"],
+    model = host.Model(capi.F16, 64, 512, c["heads_global"], c["d"], layer_num=1, world_size=c["world_size"], ffn_inner=c["ffn_global"],
                        causal=True, fused=True, max_cache_len=1024 + 64, weight_layout=weight_layout, seed=0)
-    for factor in (1, 2, 4, 8):
+    partition = {}
+    for factor in factors:
         sched = host.Scheduler(model, schedule_deep=6, contention_factor=0.8, policy=host.POLICY_RESOURCE,
-                               axis=host.SPLIT_TOKEN_ROWS, seq_bucket=64, ignore_num=0, pool_count=0)
+                               axis=host.SPLIT_TOKEN_ROWS, seq_bucket=64, ignore_num=0, pool_count=2, ctx_batch=32)
         sched.set_factor(factor)
         sched.profile(4, 512, 512, 1, 10)
         sched.profile_decode(32, 1024, 10)
-        res = {"factor": factor}
-        res["streams_verified_concurrent"] = sched.streams_concurrent
-        for mode, name, merge in ((host.MODE_SEQUENTIAL, "sequential", False), (host.MODE_LIGER, "interleaved", False),
-                                  (host.MODE_LIGER, "interleaved_minor_merged", True)):
-            sched.set_merge_minor(merge)
+        res = {"factor": factor, "streams_verified_concurrent": sched.streams_concurrent}
+
+        def best_of(mode):
             best = None
-            for _ in range(3):
+            for _ in range(repeats):
                 sched.serve_decode(32, 1000, 8)
                 sched.serve(4, 512, 0)
                 r = sched.run_queued(mode)
                 if best is None or r["total_duration_ms"] < best["total_duration_ms"]:
                     best = r
-            res[name] = {"makespan_ms": round(best["total_duration_ms"], 4), "secondary_launches": best["secondary_launches"],
-                         "splits": best["splits"], "rounds": best["rounds"]}
+            return {"makespan_ms": round(best["total_duration_ms"], 4), "secondary_launches": best["secondary_launches"],
+                    "splits": best["splits"], "rounds": best["rounds"], "partition_rounds": best["partition_rounds"]}
+
+        sched.set_merge_minor(False)
+        res["sequential"] = best_of(host.MODE_SEQUENTIAL)
+        res["interleaved"] = best_of(host.MODE_LIGER)
+        sched.set_merge_minor(True)
+        res["interleaved_minor_merged"] = best_of(host.MODE_LIGER)
+        for share in shares:
+            if share == 0:
+                continue
+            sched.enable_partition(share)
+            meas = sched.profile_partition(4, 512, 32, 1024)
+            partition[share] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in meas.items()}
+            key = "partitioned_%d_hbm_cus" % share
+            if sched.partition_factor(1, 0) <= 0:
+                res[key] = {"skipped": "a partitioned co-run does not beat back-to-back execution (gain %.3f)" % meas["gain"]}
+                continue
+            res[key] = best_of(host.MODE_LIGER)
+            res[key]["speedup"] = round(res["sequential"]["makespan_ms"] / res[key]["makespan_ms"], 4)
+        sched.enable_partition(0)
         res["speedup"] = round(res["sequential"]["makespan_ms"] / res["interleaved"]["makespan_ms"], 4)
         res["speedup_minor_merged"] = round(res["sequential"]["makespan_ms"] / res["interleaved_minor_merged"]["makespan_ms"], 4)
         out.append(res)
-    return {"workload": "cfg4: prefill B4 S512 (split by token rows) || decode B32 L1024 x 8 steps, one layer shard", "results": out}
+    return {"workload": "cfg4: prefill B4 S512 (split by token rows) || decode B32 L1024 x 8 steps, one layer shard",
+            "partition_measurement": {"what": "MFMA-bound kernels of the prefill layer on 256 - n compute units || decode steps on n, "
+                                              "against both back to back on the whole chip", "by_hbm_cus": partition},
+            "results": out}
 
 
 def bench_cfg5(capi, host, weight_layout, n_requests):

@@ -5,8 +5,12 @@
  * src/layer/func_wrapper.h bind into a FuncWrap.  Conventions, identical to the reference's:
  *   - asynchronous: work is enqueued on `stream` (a hipStream_t passed as void*; NULL = default
  *     stream) and the call returns without waiting;
- *   - device pointers are owned by the caller; nothing here allocates or frees (lg_malloc & co.
- *     below are thin runtime wrappers for host code that does not include HIP headers);
+ *   - device pointers are owned by the caller; no kernel entry point allocates, frees or blocks (lg_malloc & co. below
+ *     are thin runtime wrappers for host code that does not include HIP headers).  The one piece of device memory the
+ *     library owns is a 64 MiB split-K workspace per stream, allocated by lg_stream_create* / lg_stream_attach and freed
+ *     by lg_stream_destroy / lg_stream_detach -- the counterpart of the workspace a cuBLAS handle owns (context.h:20-29
+ *     binds one handle per stream).  A GEMM on a stream the library was never told about still runs, on kernels that
+ *     need no workspace (slower for fewer than 257 token rows);
  *   - several kernels work in place, exactly where the reference's do.
  * Differences: every function returns an int status instead of asserting --
  *   LG_OK, LG_ERR_INVALID (bad / unsupported shape or pointer), LG_ERR_LAUNCH (HIP error; text via
@@ -48,8 +52,16 @@ int lg_memcpy_d2d_async(void* dst, const void* src, size_t bytes, void* stream);
 int lg_memset_async(void* dst, int value, size_t bytes, void* stream);
 int lg_device_synchronize(void);
 int lg_stream_create(void** stream);          /* non-blocking stream, default priority */
+/* Tells the library about a stream it did not create (the null stream, another runtime's stream): allocates its split-K
+ * workspace and records how many compute units its kernels run on (cu_count 0 = all of the device), which is what the
+ * launchers size their grids for.  On a stream that is already known only a non-zero cu_count changes anything.  lg_stream_detach frees the workspace (after
+ * synchronising the stream); lg_stream_cu_count returns the recorded count (the device's for an unknown stream). */
+int lg_stream_attach(void* stream, int cu_count);
+int lg_stream_detach(void* stream);
+int lg_stream_cu_count(void* stream);
 /* Non-blocking stream whose kernels run only on the compute units whose bit is set in cu_mask (mask_words 32-bit
- * words, bit i of word w = CU 32*w + i; at least one bit must be set).  Takes the place of the two stream priorities
+ * words, bit i of word w = mask bit 32*w + i; on this GPU bit i selects a unit of accelerator die i mod 8, and every die must
+ * keep at least one unit).  The launchers size their grids for the number of selected units.  Takes the place of the two stream priorities
  * the reference gives its streams (context.h:28-29, schedule.h:54-55): on this platform the two streams of the scheduler
  * are separated in space, not by priority. */
 int lg_stream_create_cu_mask(void** stream, const unsigned* cu_mask, int mask_words);

@@ -6,6 +6,7 @@
 // policy (src/schedule.h:221-278, src/init.h:121-259 of the reference) can be asserted launch by launch on a machine
 // without a GPU.  Memory "on the device" is ordinary host memory that is never dereferenced by the fake kernels.
 #include <algorithm>
+#include <cmath>
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
@@ -16,7 +17,17 @@
 
 namespace {
 
-struct Stream { double ready = 0; int id = 0; };
+struct Stream {
+    double ready = 0;
+    int id = 0;
+    int cus = 256;                  // compute units of the stream (a CU-masked stream has fewer)
+    unsigned mask[8] = {~0u, ~0u, ~0u, ~0u, ~0u, ~0u, ~0u, ~0u};
+};
+bool share_cus(const Stream* a, const Stream* b) {
+    for (int w = 0; w < 8; ++w)
+        if (a->mask[w] & b->mask[w]) return true;
+    return false;
+}
 struct Event { double time = 0; bool recorded = false; };
 struct Launch {
     int stream; char name[48]; long long a, b, c;  // problem size (m, n, k) or (rows, cols, 0)
@@ -29,6 +40,9 @@ double g_launch_cost = 0.002;   // host time per launch call
 double g_mfma_rate = 1.0e9;     // flop per virtual ms
 double g_hbm_rate = 1.0e6;      // bytes per virtual ms
 double g_corun_speed = 1.0;     // a kernel launched while another stream is busy runs at this fraction of its speed
+double g_share_exp[2] = {1.0, 1.0};  // a kernel on a stream with `cus` of 256 compute units costs (256 / cus)^exp times more:
+                                     // [0] matrix kernels, [1] memory kernels (1 = proportional, < 1 = the share hurts less)
+thread_local int g_cost_kind = 1;    // kind of the cost computed last on this thread (0 matrix, 1 memory)
 std::vector<Stream*> g_streams;
 std::vector<Launch> g_trace;
 Stream g_default;
@@ -45,15 +59,18 @@ int launch(void* stream, const char* name, long long a, long long b, long long c
     l.name[sizeof(l.name) - 1] = 0;
     l.a = a; l.b = b; l.c = c; l.p0 = p0; l.p1 = p1; l.p2 = p2;
     l.start = std::max(s->ready, g_host_now);
-    bool other_busy = (s != &g_default && g_default.ready > l.start);
-    for (auto* o : g_streams) other_busy = other_busy || (o != s && o->ready > l.start);
+    // a kernel on a CU-masked stream runs on its share of the chip: cost x 256 / cus; a kernel launched while another stream
+    // that shares compute units with this one is busy runs at g_corun_speed of its speed
+    bool other_busy = (s != &g_default && g_default.ready > l.start && share_cus(s, &g_default));
+    for (auto* o : g_streams) other_busy = other_busy || (o != s && o->ready > l.start && share_cus(s, o));
+    cost *= std::pow(256.0 / (double)s->cus, g_share_exp[g_cost_kind]);
     l.end = l.start + (other_busy ? cost / g_corun_speed : cost);
     s->ready = l.end;
     g_trace.push_back(l);
     return LG_OK;
 }
-double gemm_cost(long long m, long long n, long long k) { return 0.003 + 2.0 * m * n * k / g_mfma_rate; }
-double mem_cost(double bytes) { return 0.003 + bytes / g_hbm_rate; }
+double gemm_cost(long long m, long long n, long long k) { g_cost_kind = 0; return 0.003 + 2.0 * m * n * k / g_mfma_rate; }
+double mem_cost(double bytes) { g_cost_kind = 1; return 0.003 + bytes / g_hbm_rate; }
 
 }  // namespace
 
@@ -64,6 +81,7 @@ void fake_reset(void) {
     std::lock_guard<std::mutex> lk(g_mu);
     g_trace.clear();
     g_corun_speed = 1.0;
+    g_share_exp[0] = g_share_exp[1] = 1.0;
     g_host_now = 0;
     g_default.ready = 0;
     for (auto* s : g_streams) s->ready = 0;
@@ -72,6 +90,7 @@ void fake_set_rates(double mfma_flop_per_ms, double hbm_bytes_per_ms, double lau
     g_mfma_rate = mfma_flop_per_ms; g_hbm_rate = hbm_bytes_per_ms; g_launch_cost = launch_cost_ms;
 }
 void fake_set_corun_speed(double speed) { g_corun_speed = speed > 0 ? speed : 1.0; }
+void fake_set_share_model(double matrix_exp, double memory_exp) { g_share_exp[0] = matrix_exp; g_share_exp[1] = memory_exp; }
 int fake_trace_count(void) { std::lock_guard<std::mutex> lk(g_mu); return (int)g_trace.size(); }
 int fake_trace_get(int i, int* stream, char* name, int name_len, long long* abc, unsigned long long* ptrs, double* start_end) {
     std::lock_guard<std::mutex> lk(g_mu);
@@ -130,12 +149,19 @@ int lg_stream_create_concurrent(void** stream, void* other, int* verified) {
 }
 int lg_stream_create_cu_mask(void** stream, const unsigned* cu_mask, int mask_words) {
     if (!stream || !cu_mask || mask_words <= 0) return LG_ERR_INVALID;
-    bool any = false;
-    for (int w = 0; w < mask_words; ++w) any = any || cu_mask[w] != 0u;
-    if (!any) return LG_ERR_INVALID;
-    return lg_stream_create(stream);  // the virtual-time backend has no notion of compute units
+    int cus = 0;
+    for (int b = 0; b < mask_words * 32 && b < 256; ++b) cus += (cu_mask[b >> 5] >> (b & 31)) & 1u;
+    if (cus == 0) return LG_ERR_INVALID;
+    const int rc = lg_stream_create(stream);
+    Stream* s = (Stream*)*stream;
+    s->cus = cus;
+    for (int w = 0; w < 8; ++w) s->mask[w] = w < mask_words ? cu_mask[w] : 0u;
+    return rc;
 }
 int lg_stream_destroy(void*) { return LG_OK; }
+int lg_stream_attach(void*, int cu_count) { return cu_count < 0 ? LG_ERR_INVALID : LG_OK; }
+int lg_stream_detach(void*) { return LG_OK; }
+int lg_stream_cu_count(void* stream) { return stream ? S(stream)->cus : 256; }
 int lg_stream_synchronize(void* stream) { std::lock_guard<std::mutex> lk(g_mu); g_host_now = std::max(g_host_now, S(stream)->ready); return LG_OK; }
 int lg_stream_wait_event(void* stream, void* event) {
     std::lock_guard<std::mutex> lk(g_mu);

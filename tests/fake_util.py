@@ -18,6 +18,7 @@ class Fake:
         self.lib.fake_set_rates.argtypes = [C.c_double, C.c_double, C.c_double]
         self.lib.fake_host_now.restype = C.c_double
         self.lib.fake_set_corun_speed.argtypes = [C.c_double]
+        self.lib.fake_set_share_model.argtypes = [C.c_double, C.c_double]
 
     def close(self):
         self.host.lib = self._prev
@@ -31,6 +32,10 @@ class Fake:
     def set_corun_speed(self, speed):
         """A kernel launched while another stream is busy runs at `speed` (0..1] of its stand-alone speed."""
         self.lib.fake_set_corun_speed(speed)
+
+    def set_share_model(self, matrix_exp, memory_exp):
+        """A kernel on a stream with `cus` of 256 compute units costs (256 / cus) ** exp times its whole-chip cost."""
+        self.lib.fake_set_share_model(matrix_exp, memory_exp)
 
     def trace(self):
         out = []

@@ -12,6 +12,9 @@ class Dev:
         self.lib = liger.capi.lib
         self.device = torch.device("cuda:0")
         torch.cuda.set_device(0)
+        # the device library is told about the stream the tests launch on (it allocates that stream's split-K workspace)
+        rc = self.lib.lg_stream_attach(C.c_void_p(self.stream), 0)
+        assert rc == 0, self.capi.last_error()
 
     @property
     def stream(self):

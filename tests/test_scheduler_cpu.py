@@ -397,3 +397,176 @@ def test_merged_minor_kernels_keep_a_prefill_in_one_run(fake):
     assert merged["secondary_launches"] > 5
     b_rows = [e for e in t1 if (e["name"] in ("gemm", "gemm_fused") and e["n"] == 64) or (e["name"] == "layer_norm" and e["m"] == 64)]
     assert all(y["start"] >= x["end"] - 1e-12 for x, y in zip(b_rows, b_rows[1:]))   # B's own order is kept
+
+
+def test_requests_that_exceed_the_contexts_are_refused_on_the_host(fake):
+    """Shapes decide how far a launch vector writes into a request's buffers and KV-cache slots, so every entry point that
+    builds one checks them first and launches nothing (no kernel may write outside its buffers)."""
+    host = fake.host
+    m = small_model(host, max_batch=4, cache=80)      # max_seq 64, cache 80 rows, 4 slots
+    s = host.Scheduler(m, policy=host.POLICY_RESOURCE, pool_count=2, ctx_batch=2)
+    s.profile(1, 64, 64, 1, 2)
+    fake.reset()
+    for bad in ((3, 64, 0),      # batch beyond the contexts' batch
+                (1, 65, 0),      # sequence beyond max_seq_len
+                (1, 64, 17),     # 64 + 17 decode steps do not fit 80 cache rows
+                ):
+        with pytest.raises(host.capi.LigerError):
+            s.serve(*bad)
+    with pytest.raises(host.capi.LigerError):
+        s.serve_decode(1, 70, 11)                      # past + steps beyond the cache
+    with pytest.raises(host.capi.LigerError):
+        s.serve_decode(3, 10, 1)                       # batch beyond the contexts' batch
+    with pytest.raises(host.capi.LigerError):
+        s.profile_decode(1, 80)                        # position 80 is outside an 80-row cache
+    with pytest.raises(host.capi.LigerError):
+        s.profile_contention(1, 64, 3, 10)             # decode batch beyond the context
+    with pytest.raises(host.capi.LigerError):
+        m.run(0x1000, 0x2000, 2, 64, cache_slot=3)     # slots 3, 4 of 4
+    with pytest.raises(host.capi.LigerError):
+        m.run_decode(0x1000, 0x2000, 1, 80, cache_slot=0)
+    with pytest.raises(host.capi.LigerError):
+        m.time_kernels(0x1000, 0x2000, 5, 64)          # batch beyond max_batch
+    with pytest.raises(host.capi.LigerError):
+        m.time_kernels(0x1000, 0x2000, 1, 1, decode_past=80, cache_slot=0)
+    nocache = small_model(host, cache=0, fused=False)
+    s2 = host.Scheduler(nocache, pool_count=1, ctx_batch=1)
+    with pytest.raises(host.capi.LigerError):
+        s2.serve(1, 32, 1)                             # decode steps without a KV cache
+    with pytest.raises(host.capi.LigerError):
+        s2.serve_decode(1, 0, 1)
+    assert fake.trace() == []                          # nothing was launched by any of the refused calls
+    # what fits is still accepted afterwards
+    s.serve(2, 64, 16)
+    assert s.run_queued(host.MODE_SEQUENTIAL)["records"] == 1
+
+
+def test_more_queued_requests_than_contexts_fail_instead_of_deadlocking(fake):
+    host = fake.host
+    m = small_model(host)
+    s = host.Scheduler(m, pool_count=2, ctx_batch=1)
+    s.serve(1, 32)
+    s.serve(1, 32)
+    with pytest.raises(host.capi.LigerError, match="no scheduler loop"):
+        s.serve(1, 32)                                 # no loop is running that could return a context
+    assert s.run_queued(host.MODE_LIGER)["records"] == 2
+    s.serve(1, 32)                                     # contexts are back
+    assert s.run_queued(host.MODE_LIGER)["records"] == 1
+
+
+def test_interleaving_without_request_contexts_is_refused(fake):
+    """Two requests on two streams that share the model's default buffers would race: run_stream_sync needs a pool."""
+    host = fake.host
+    m = small_model(host)
+    s = host.Scheduler(m, schedule_deep=6, pool_count=0)
+    s.serve(1, 32)
+    s.serve(1, 32)
+    with pytest.raises(host.capi.LigerError, match="per-request contexts"):
+        s.run_queued(host.MODE_LIGER)
+    s1 = host.Scheduler(m, schedule_deep=1, pool_count=0)   # one request in flight at a time: allowed
+    s1.serve(1, 32)
+    assert s1.run_queued(host.MODE_LIGER)["records"] == 1
+
+
+def test_request_off_the_profile_grid_is_still_split(fake):
+    """Durations are looked up at seq rounded up to the profile grid; the decomposition table must be looked up with the
+    same key, or requests whose length is not itself a profiled key would never be split."""
+    host = fake.host
+    m = small_model(host, factor=4)
+    s = host.Scheduler(m, contention_factor=0.8, policy=host.POLICY_RESOURCE, seq_bucket=16, pool_count=3, ctx_batch=1)
+    s.profile(1, 48, 64, 16, 2)
+    fake.reset()
+    s.serve(1, 64)
+    s.serve(1, 52)            # looked up at 64
+    r = s.run_queued(host.MODE_LIGER)
+    assert r["records"] == 2 and r["profile_misses"] == 0 and r["sub_profile_misses"] == 0
+    assert r["splits"] >= 1   # the worked example's split of B's out_proj happens for the off-grid request too
+    pieces = [e for e in fake.trace() if e["name"] == "gemm" and e["n"] == 52 and e["m"] < 256]
+    assert sum(e["m"] for e in pieces) == 256
+
+
+def test_cu_mask_streams_need_every_die_and_report_their_share(fake):
+    import ctypes as C
+    lib = fake.lib
+    st = C.c_void_p()
+    mask = (C.c_uint * 8)(0xffffffff, 0xffffffff, 0, 0, 0, 0, 0, 0)       # 64 units
+    assert lib.lg_stream_create_cu_mask(C.byref(st), mask, 8) == 0
+    lib.lg_stream_cu_count.argtypes = [C.c_void_p]
+    assert lib.lg_stream_cu_count(st) == 64 and lib.lg_stream_cu_count(None) == 256
+    empty = (C.c_uint * 8)()
+    assert lib.lg_stream_create_cu_mask(C.byref(st), empty, 8) != 0
+
+
+def _partition_setup(fake, factor_hbm_main=None):
+    host = fake.host
+    m = small_model(host, factor=4, layers=2, max_batch=4, cache=128)
+    s = host.Scheduler(m, contention_factor=0.8, policy=host.POLICY_RESOURCE, seq_bucket=16, pool_count=3, ctx_batch=1)
+    s.profile(1, 48, 64, 16, 2)
+    for past in (48, 64, 80):
+        s.profile_decode(1, past, 2)
+    s.set_merge_minor(True)
+    s.enable_partition(128)
+    if factor_hbm_main is not None:
+        s.set_partition_factor(HBM, MFMA, factor_hbm_main)
+        s.set_partition_factor(MFMA, HBM, 1.0 / factor_hbm_main)
+    return host, m, s
+
+
+def test_partitioned_rounds_run_only_while_the_other_class_has_work(fake):
+    """Decode request A (HBM-bound, primary) and prefill request B (MFMA-bound, waiting).  With a partition, A's kernels run
+    on the HBM side's compute units and B's on the MFMA side's for exactly as long as B has work; afterwards A is back on
+    the whole chip (stream 0).  Every entry is launched once, each request in its own order."""
+    host, m, s = _partition_setup(fake, factor_hbm_main=1.0)
+    fake.reset()
+    s.serve_decode(1, 48, 24)     # A: 24 decode steps x 2 layers x 7 kernels, one long HBM-bound run
+    s.serve(1, 64, 0)             # B: two prefill layers, one MFMA-bound run (minor kernels merged)
+    r = s.run_queued(host.MODE_LIGER)
+    t = fake.trace()
+    assert r["records"] == 2 and r["partition_rounds"] >= 1 and r["secondary_launches"] >= 18
+    ids = sorted({e["stream"] for e in t})
+    b_rows = [e for e in t if (e["name"] in ("gemm", "gemm_fused") and e["n"] == 64) or (e["name"] == "layer_norm" and e["m"] == 64) or e["name"] == "attn_prefill"]
+    a_rows = [e for e in t if e not in b_rows]
+    assert len(b_rows) == 18 + r["splits"] and len(a_rows) == 24 * 2 * 7
+    # B ran on one masked stream only; A on another masked stream while B had work, on stream 0 (the lowest id) afterwards
+    b_streams = {e["stream"] for e in b_rows}
+    a_streams = [e["stream"] for e in a_rows]
+    assert len(b_streams) == 1 and b_streams.isdisjoint(a_streams) and ids[0] not in b_streams
+    assert a_streams[0] != ids[0] and a_streams[-1] == ids[0]
+    switch = a_streams.index(ids[0])
+    assert all(x == a_streams[0] for x in a_streams[:switch]) and all(x == ids[0] for x in a_streams[switch:])
+    # the partitioned part of A is about as long as B's work divided by the factor (1.0): B's stand-alone time on the whole chip
+    b_work = sum((e["end"] - e["start"]) / 2.0 for e in b_rows)          # measured on 128 of 256 units: twice the whole-chip cost
+    a_part = sum((e["end"] - e["start"]) / 2.0 for e in a_rows[:switch])
+    assert a_part == pytest.approx(b_work, rel=0.25)
+    for rows in (a_rows, b_rows):
+        assert all(y["start"] >= x["end"] - 1e-12 for x, y in zip(rows, rows[1:]))
+    # no partition factor for the pair -> the same requests never leave the whole-chip streams
+    s.set_partition_factor(HBM, MFMA, -1.0)
+    fake.reset()
+    s.serve_decode(1, 48, 24)
+    s.serve(1, 64, 0)
+    r2 = s.run_queued(host.MODE_LIGER)
+    assert r2["partition_rounds"] == 0 and len({e["stream"] for e in fake.trace()}) <= 2
+
+
+@pytest.mark.parametrize("matrix_exp,memory_exp,pays", [(1.0, 1.0, False), (0.5, 0.2, True)])
+def test_measured_partition_follows_the_backend_model(fake, matrix_exp, memory_exp, pays):
+    """profile_partition runs the prefill's MFMA-bound kernels on 128 of 256 compute units next to decode steps on the other
+    128.  When a share costs in proportion (exponent 1) both sides take twice as long and nothing is gained: the table stays
+    empty and rounds are never partitioned.  When a share hurts less than in proportion the co-run wins, and factor and gain
+    follow from the model: matrix kernels 2^a times slower, memory kernels 2^b."""
+    host, m, s = _partition_setup(fake)
+    fake.reset()
+    fake.set_share_model(matrix_exp, memory_exp)
+    r = s.profile_partition(1, 64, 1, 64)
+    slow_a, slow_b = 2.0 ** matrix_exp, 2.0 ** memory_exp
+    assert r["main_part_ms"] == pytest.approx(r["main_ms"] * slow_a, rel=0.1)
+    # a decode step mixes memory kernels with (tiny) matrix kernels: its slow-down lies between the two
+    slow_sub = r["sub_part_ms"] / (r["sub_repeats"] * r["sub_ms"])
+    assert min(slow_a, slow_b) * 0.9 <= slow_sub <= max(slow_a, slow_b) * 1.1
+    assert r["factor"] == pytest.approx(slow_a / slow_sub, rel=0.1)
+    if pays:
+        assert r["gain"] > 1.2
+        assert s.partition_factor(MFMA, HBM) == pytest.approx(r["factor"]) and s.partition_factor(HBM, MFMA) == pytest.approx(1 / r["factor"])
+    else:
+        assert r["gain"] < 1.02 and s.partition_factor(MFMA, HBM) < 0 and s.partition_factor(HBM, MFMA) < 0
