@@ -10,8 +10,8 @@
 namespace lg {
 
 int launch_gemm_fast_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t stream, bool* handled);
-int launch_gemm_skinny_f16(const GemmArgs& g, const GemmGroup& grp, int wlayout, int batch, hipStream_t stream, bool* handled);
-int launch_gemv_f16(const GemmArgs& g, const GemmGroup& grp, int wlayout, int batch, hipStream_t stream, bool* handled);
+int launch_gemm_skinny_f16(const GemmArgs& g, const GemmGroup& grp, const RowMap* rows, int wlayout, int batch, hipStream_t stream, bool* handled);
+int launch_gemv_f16(const GemmArgs& g, const GemmGroup& grp, const RowMap* rows, int wlayout, int batch, hipStream_t stream, bool* handled);
 
 // ---------------------------------------------------------------------------------------------------
 // fp16 generic kernel
@@ -150,9 +150,9 @@ static int gemm_f16_dispatch(GemmArgs g, int wlayout, int batch, hipStream_t str
     int rc = launch_gemm_fast_f16(g, wlayout, batch, stream, &handled);
     if (handled) return rc;
     const GemmGroup one = single_group(g);
-    rc = launch_gemv_f16(g, one, wlayout, batch, stream, &handled);
+    rc = launch_gemv_f16(g, one, nullptr, wlayout, batch, stream, &handled);
     if (handled) return rc;
-    rc = launch_gemm_skinny_f16(g, one, wlayout, batch, stream, &handled);
+    rc = launch_gemm_skinny_f16(g, one, nullptr, wlayout, batch, stream, &handled);
     if (handled) return rc;
     const bool aligned = aligned16(g.X) && aligned16(g.W) && aligned16(g.Y) && (g.ldx % 8 == 0) && (g.ldw % 8 == 0) &&
                          (g.strideX % 8 == 0) && (g.strideW % 8 == 0) && (g.strideY % 4 == 0) &&
@@ -273,7 +273,7 @@ int lg_gemm_strided_batched_f16(int transa, int transb, int m, int n, int k, con
     g.X = (const half_t*)B; g.ldx = ldb; g.strideX = strideB;
     g.W = (const half_t*)A; g.ldw = lda; g.strideW = strideA;
     g.Y = (half_t*)C; g.ldy = ldc; g.strideY = strideC;
-    g.epi = Epilogue{LG_EPI_NONE, nullptr, 0, 0, 0};
+    g.epi = Epilogue{LG_EPI_NONE, nullptr, 0, 0, 0, 0};
     return gemm_f16_dispatch(g, transa ? W_NK : W_KN, batch, (hipStream_t)stream);
 }
 
@@ -304,7 +304,7 @@ int lg_gemm_fused_f16(int transa, int m, int n, int k, const void* A, int lda, c
     g.X = (const half_t*)B; g.ldx = ldb; g.strideX = 0;
     g.W = (const half_t*)A; g.ldw = lda; g.strideW = 0;
     g.Y = (half_t*)C; g.ldy = ldc; g.strideY = 0;
-    g.epi = Epilogue{epilogue, (const half_t*)bias, epi_arg0, epi_arg1, epi_arg2};
+    g.epi = Epilogue{epilogue, (const half_t*)bias, epi_arg0, epi_arg1, epi_arg2, 0};
     return gemm_f16_dispatch(g, transa ? W_NK : W_KN, 1, (hipStream_t)stream);
 }
 
@@ -348,11 +348,11 @@ int lg_gemm_fused_grouped_f16(int transa, int m, int n, int k, int count, const 
             g.X = (const half_t*)B; g.ldx = ldb; g.strideX = 0;
             g.W = grp.W[0]; g.ldw = lda; g.strideW = 0;
             g.Y = grp.Y[0]; g.ldy = grp.ldy[0]; g.strideY = 0;
-            g.epi = Epilogue{epilogue, grp.bias[0], epi_arg0, epi_arg1, heads_total};
+            g.epi = Epilogue{epilogue, grp.bias[0], epi_arg0, epi_arg1, heads_total, 0};
             bool handled = false;
-            int rc = launch_gemv_f16(g, grp, W_NK, 1, (hipStream_t)stream, &handled);
+            int rc = launch_gemv_f16(g, grp, nullptr, W_NK, 1, (hipStream_t)stream, &handled);
             if (handled) return rc;
-            rc = launch_gemm_skinny_f16(g, grp, W_NK, 1, (hipStream_t)stream, &handled);
+            rc = launch_gemm_skinny_f16(g, grp, nullptr, W_NK, 1, (hipStream_t)stream, &handled);
             if (handled) return rc;
         }
     }
@@ -360,6 +360,75 @@ int lg_gemm_fused_grouped_f16(int transa, int m, int n, int k, int count, const 
         int rc = lg_gemm_fused_f16(transa, m, n, k, A[i], lda, B, ldb, C[i], ldc[i], epilogue, epilogue != LG_EPI_NONE ? bias[i] : nullptr,
                                    epi_arg0, epi_arg1, epi_arg2, stream);
         if (rc) return rc;
+    }
+    return LG_OK;
+}
+
+int lg_gemm_fused_grouped_rows_f16(int transa, int m, int n, int k, int count, const void* const* A, int lda, const void* B, int ldb,
+                                   void* const* C, const int* ldc, const void* const* bias, int size_per_head, int heads_total,
+                                   const int* use_rows, const int* slot, const int* pos, void* stream) {
+    const int d = size_per_head;
+    if (count < 1 || count > LG_MAX_GROUP || !A || !C || !ldc || !bias || !use_rows) {
+        set_error("gemm_fused_grouped_rows_f16: count must be 1..%d and the pointer arrays non-null", LG_MAX_GROUP);
+        return LG_ERR_INVALID;
+    }
+    if (m < 0 || n < 0 || k < 0 || n > LG_ROWMAP_MAX) { set_error("gemm_fused_grouped_rows_f16: at most %d token rows (n = %d)", LG_ROWMAP_MAX, n); return LG_ERR_INVALID; }
+    if (m == 0 || n == 0) return LG_OK;
+    if (d <= 0 || m % d != 0 || d % 4 != 0 || heads_total < m / d) {
+        set_error("gemm_fused_grouped_rows_f16: size_per_head must divide the features and be a multiple of 4, heads_total >= features / size_per_head");
+        return LG_ERR_INVALID;
+    }
+    bool any_rows = false;
+    for (int i = 0; i < count; ++i) any_rows = any_rows || use_rows[i] != 0;
+    if (any_rows && (!slot || !pos)) { set_error("gemm_fused_grouped_rows_f16: null slot / pos array"); return LG_ERR_INVALID; }
+    RowMap rm{};
+    for (int r = 0; r < n && any_rows; ++r) {
+        if (slot[r] < 0 || pos[r] < 0) { set_error("gemm_fused_grouped_rows_f16: token row %d: slot %d, pos %d", r, slot[r], pos[r]); return LG_ERR_INVALID; }
+        rm.slot[r] = slot[r];
+        rm.pos[r] = pos[r];
+    }
+    GemmGroup grp{};
+    grp.count = count;
+    for (int i = 0; i < count; ++i) {
+        int rc = check_blas_args("gemm_fused_grouped_rows_f16", transa, 0, m, n, k, A[i], lda, B, ldb, C[i], m > 1 ? m : 1, 1);
+        if (rc) return rc;
+        if (!bias[i]) { set_error("gemm_fused_grouped_rows_f16: null bias"); return LG_ERR_INVALID; }
+        if (ldc[i] < 1) { set_error("gemm_fused_grouped_rows_f16: ldc (rows per head slot) must be >= 1"); return LG_ERR_INVALID; }
+        for (int r = 0; r < n && use_rows[i]; ++r)
+            if (pos[r] >= ldc[i]) { set_error("gemm_fused_grouped_rows_f16: token row %d: pos %d outside the %d rows of a head slot", r, pos[r], ldc[i]); return LG_ERR_INVALID; }
+        grp.W[i] = (const half_t*)A[i];
+        grp.Y[i] = (half_t*)C[i];
+        grp.bias[i] = (const half_t*)bias[i];
+        grp.ldy[i] = ldc[i];
+        grp.rows[i] = use_rows[i] ? 1 : 0;
+    }
+    if (transa == 1) {
+        GemmArgs g;
+        g.M = n; g.N = m; g.K = k;
+        g.X = (const half_t*)B; g.ldx = ldb; g.strideX = 0;
+        g.W = grp.W[0]; g.ldw = lda; g.strideW = 0;
+        g.Y = grp.Y[0]; g.ldy = grp.ldy[0]; g.strideY = 0;
+        g.epi = Epilogue{LG_EPI_BIAS_HEADS_ROWS, grp.bias[0], 1, d, heads_total, grp.rows[0]};
+        bool handled = false;
+        int rc = launch_gemv_f16(g, grp, &rm, W_NK, 1, (hipStream_t)stream, &handled);
+        if (handled) return rc;
+        rc = launch_gemm_skinny_f16(g, grp, &rm, W_NK, 1, (hipStream_t)stream, &handled);
+        if (handled) return rc;
+    }
+    // anything the weight-streaming kernels do not take: plain calls, one per member -- and one per token row for a member
+    // whose rows go to their own places
+    for (int i = 0; i < count; ++i) {
+        if (!use_rows[i]) {
+            int rc = lg_gemm_fused_f16(transa, m, n, k, A[i], lda, B, ldb, C[i], ldc[i], LG_EPI_BIAS_HEADS, bias[i], 1, d, heads_total, stream);
+            if (rc) return rc;
+            continue;
+        }
+        for (int r = 0; r < n; ++r) {
+            half_t* dst = (half_t*)C[i] + ((int64_t)slot[r] * heads_total * ldc[i] + pos[r]) * d;
+            int rc = lg_gemm_fused_f16(transa, m, 1, k, A[i], lda, (const half_t*)B + (int64_t)r * ldb, ldb, dst, ldc[i], LG_EPI_BIAS_HEADS,
+                                       bias[i], 1, d, heads_total, stream);
+            if (rc) return rc;
+        }
     }
     return LG_OK;
 }

@@ -16,6 +16,16 @@ struct Epilogue {
     int seq;              // LG_EPI_BIAS_HEADS: tokens per sequence
     int d;                // LG_EPI_BIAS_HEADS: size_per_head
     int heads_total;      // LG_EPI_BIAS_HEADS: heads per batch entry in the destination (>= N / d)
+    int rows;             // LG_EPI_BIAS_HEADS_ROWS: 1 = token row m goes to (slot[m], pos[m]) of the RowMap, 0 = to (m, 0)
+};
+
+// kernel-internal epilogue: LG_EPI_BIAS_HEADS for one token per sequence, where every token row has its own destination
+// (batch entry, position) -- the K and V rows of decode steps of different requests batched into one launch
+constexpr int LG_EPI_BIAS_HEADS_ROWS = 4;
+constexpr int LG_ROWMAP_MAX = LG_ATTN_DECODE_MAX_SEQS;
+struct RowMap {  // passed by value with the launch
+    int slot[LG_ROWMAP_MAX];
+    int pos[LG_ROWMAP_MAX];
 };
 
 struct GemmArgs {
@@ -35,6 +45,7 @@ struct GemmGroup {
     half_t* Y[LG_MAX_GROUP];
     const half_t* bias[LG_MAX_GROUP];
     int64_t ldy[LG_MAX_GROUP];
+    int rows[LG_MAX_GROUP];  // LG_EPI_BIAS_HEADS_ROWS: whether the member's token rows follow the RowMap
 };
 __device__ __forceinline__ void select_group(GemmArgs& g, const GemmGroup& grp) {
     if (grp.count > 1) {
@@ -43,6 +54,7 @@ __device__ __forceinline__ void select_group(GemmArgs& g, const GemmGroup& grp) 
         g.Y = grp.Y[gi];
         g.epi.bias = grp.bias[gi];
         g.ldy = grp.ldy[gi];
+        g.epi.rows = grp.rows[gi];
     }
 }
 
@@ -50,14 +62,14 @@ __device__ __forceinline__ void select_group(GemmArgs& g, const GemmGroup& grp) 
 inline GemmGroup single_group(const GemmArgs& g) {
     GemmGroup grp{};
     grp.count = 1;
-    grp.W[0] = g.W; grp.Y[0] = g.Y; grp.bias[0] = g.epi.bias; grp.ldy[0] = g.ldy;
+    grp.W[0] = g.W; grp.Y[0] = g.Y; grp.bias[0] = g.epi.bias; grp.ldy[0] = g.ldy; grp.rows[0] = g.epi.rows;
     return grp;
 }
 // what the vectorised loads and stores of the weight-streaming kernels need of every member of the group
 inline bool group_aligned(const GemmArgs& g, const GemmGroup& grp) {
     for (int i = 0; i < grp.count; ++i) {
         if (!aligned16(grp.W[i]) || !aligned16(grp.Y[i])) return false;
-        if (g.epi.kind == LG_EPI_BIAS_HEADS ? (g.epi.d % 4 != 0) : (grp.ldy[i] % 4 != 0)) return false;
+        if ((g.epi.kind == LG_EPI_BIAS_HEADS || g.epi.kind == LG_EPI_BIAS_HEADS_ROWS) ? (g.epi.d % 4 != 0) : (grp.ldy[i] % 4 != 0)) return false;
     }
     return true;
 }
@@ -79,7 +91,8 @@ __device__ __forceinline__ half4_t lds_read_tr4(const half_t* p) {
 
 // Applies the epilogue to 4 consecutive output columns n..n+3 of token row m and stores them.
 template <int EPI>
-__device__ __forceinline__ void epilogue_store4(const GemmArgs& g, half_t* Yb, int m, int n, float4_t acc, bool vec_ok) {
+__device__ __forceinline__ void epilogue_store4(const GemmArgs& g, half_t* Yb, int m, int n, float4_t acc, bool vec_ok,
+                                                const RowMap* rm = nullptr) {
     if (m >= g.M || n >= g.N) return;
     float v[4] = {acc[0], acc[1], acc[2], acc[3]};
     if (EPI != LG_EPI_NONE) {
@@ -92,7 +105,12 @@ __device__ __forceinline__ void epilogue_store4(const GemmArgs& g, half_t* Yb, i
         for (int r = 0; r < 4; ++r) v[r] = gelu_tanh(v[r]);
     }
     int64_t base;
-    if (EPI == LG_EPI_BIAS_HEADS) {
+    if (EPI == LG_EPI_BIAS_HEADS_ROWS) {
+        // one token per sequence: row m -> [slot, head, pos, e] with ldy rows reserved per (slot, head)
+        const int b = g.epi.rows ? rm->slot[m] : m, s = g.epi.rows ? rm->pos[m] : 0;
+        const int head = n / g.epi.d, e = n % g.epi.d;
+        base = (((int64_t)b * g.epi.heads_total + head) * g.ldy + s) * (int64_t)g.epi.d + e;
+    } else if (EPI == LG_EPI_BIAS_HEADS) {
         // [M = b*seq + s, N = head*d + e]  ->  [b, head, s, e] with ldy rows reserved per (b, head)
         const int b = m / g.epi.seq, s = m % g.epi.seq;
         const int head = n / g.epi.d, e = n % g.epi.d;

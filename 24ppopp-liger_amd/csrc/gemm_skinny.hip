@@ -128,7 +128,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_nk_kernel(GemmArgs g, int ksl
 // MFMA tile (8 loads per chunk), so its rolling pipeline is DEPTH chunks deep: two chunks (16 loads per lane, as in the sliced
 // kernel) for blocks of 4, 6 or 8 waves, four chunks for the 2-wave block, which then keeps the 64 KiB of a 4-wave block in flight.
 template <int MT, int EPI, int NWV, int DEPTH>
-__global__ __launch_bounds__(64 * NWV) void gemm_skinny_direct_kernel(GemmArgs g, GemmGroup grp) {
+__global__ __launch_bounds__(64 * NWV) void gemm_skinny_direct_kernel(GemmArgs g, GemmGroup grp, RowMap rm) {
     constexpr int THREADS = 64 * NWV;
     select_group(g, grp);
     __shared__ __attribute__((aligned(16))) half_t xs[2][16 * MT * SK_XS];
@@ -216,26 +216,27 @@ __global__ __launch_bounds__(64 * NWV) void gemm_skinny_direct_kernel(GemmArgs g
         for (int d = 0; d < DEPTH; ++d) do_chunk(ch + d, d & 1, bf[d]);
     }
 #pragma unroll
-    for (int i = 0; i < MT; ++i) epilogue_store4<EPI>(g, g.Y, i * 16 + l16, n0 + 4 * lk, acc[i], true);
+    for (int i = 0; i < MT; ++i) epilogue_store4<EPI>(g, g.Y, i * 16 + l16, n0 + 4 * lk, acc[i], true, &rm);
 }
 
 template <int MT, int NWV, int DEPTH>
-static void launch_direct(const GemmArgs& g, const GemmGroup& grp, hipStream_t stream) {
+static void launch_direct(const GemmArgs& g, const GemmGroup& grp, const RowMap& rm, hipStream_t stream) {
     const dim3 grid((g.N + 16 * NWV - 1) / (16 * NWV), grp.count), block(64 * NWV);
     switch (g.epi.kind) {
-        case LG_EPI_NONE: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_NONE, NWV, DEPTH>), grid, block, 0, stream, g, grp); break;
-        case LG_EPI_BIAS: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_BIAS, NWV, DEPTH>), grid, block, 0, stream, g, grp); break;
-        case LG_EPI_BIAS_GELU: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_BIAS_GELU, NWV, DEPTH>), grid, block, 0, stream, g, grp); break;
-        default: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_BIAS_HEADS, NWV, DEPTH>), grid, block, 0, stream, g, grp); break;
+        case LG_EPI_NONE: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_NONE, NWV, DEPTH>), grid, block, 0, stream, g, grp, rm); break;
+        case LG_EPI_BIAS: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_BIAS, NWV, DEPTH>), grid, block, 0, stream, g, grp, rm); break;
+        case LG_EPI_BIAS_GELU: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_BIAS_GELU, NWV, DEPTH>), grid, block, 0, stream, g, grp, rm); break;
+        case LG_EPI_BIAS_HEADS_ROWS: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_BIAS_HEADS_ROWS, NWV, DEPTH>), grid, block, 0, stream, g, grp, rm); break;
+        default: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_BIAS_HEADS, NWV, DEPTH>), grid, block, 0, stream, g, grp, rm); break;
     }
 }
 template <int NWV, int DEPTH>
-static void launch_direct_mt(const GemmArgs& g, const GemmGroup& grp, hipStream_t stream) {
+static void launch_direct_mt(const GemmArgs& g, const GemmGroup& grp, const RowMap& rm, hipStream_t stream) {
     switch ((g.M + 15) / 16) {
-        case 1: launch_direct<1, NWV, DEPTH>(g, grp, stream); break;
-        case 2: launch_direct<2, NWV, DEPTH>(g, grp, stream); break;
-        case 3: launch_direct<3, NWV, DEPTH>(g, grp, stream); break;
-        default: launch_direct<4, NWV, DEPTH>(g, grp, stream); break;
+        case 1: launch_direct<1, NWV, DEPTH>(g, grp, rm, stream); break;
+        case 2: launch_direct<2, NWV, DEPTH>(g, grp, rm, stream); break;
+        case 3: launch_direct<3, NWV, DEPTH>(g, grp, rm, stream); break;
+        default: launch_direct<4, NWV, DEPTH>(g, grp, rm, stream); break;
     }
 }
 
@@ -273,11 +274,13 @@ void launch_splitk_reduce(const GemmArgs& g, const float* partial, int nsplit, h
 }
 
 // grp.count > 1: handled only if the unsliced kernels apply (the caller then falls back to one launch per member)
-int launch_gemm_skinny_f16(const GemmArgs& g, const GemmGroup& grp, int wlayout, int batch, hipStream_t stream, bool* handled) {
+int launch_gemm_skinny_f16(const GemmArgs& g, const GemmGroup& grp, const RowMap* rows, int wlayout, int batch, hipStream_t stream, bool* handled) {
     *handled = false;
     if (batch != 1 || wlayout != W_NK) return LG_OK;
     if (g.M <= 0 || g.M > 64 || g.N < 512 || g.K < 1024 || (g.K % SK_KC) || (g.N % 4)) return LG_OK;
     if (!aligned16(g.X) || (g.ldx % 8) || (g.ldw % 8) || !group_aligned(g, grp)) return LG_OK;
+    if (g.epi.kind == LG_EPI_BIAS_HEADS_ROWS && !rows) return LG_OK;
+    const RowMap rm = rows ? *rows : RowMap{};
     const int mt = (g.M + 15) / 16;
     const StreamInfo si = stream_info(stream);
     const int cus = si.cus;  // compute units this stream's kernels run on: "one round of blocks" means this many
@@ -295,15 +298,15 @@ int launch_gemm_skinny_f16(const GemmArgs& g, const GemmGroup& grp, int wlayout,
             if (blocks < cus * 3 / 4 || (blocks > cus && blocks < 4 * cus)) continue;
             *handled = true;
             switch (w) {
-                case 128: launch_direct_mt<8, 2>(g, grp, stream); break;
-                case 96: launch_direct_mt<6, 2>(g, grp, stream); break;
-                case 64: launch_direct_mt<4, 2>(g, grp, stream); break;
-                default: launch_direct<1, 2, 4>(g, grp, stream); break;
+                case 128: launch_direct_mt<8, 2>(g, grp, rm, stream); break;
+                case 96: launch_direct_mt<6, 2>(g, grp, rm, stream); break;
+                case 64: launch_direct_mt<4, 2>(g, grp, rm, stream); break;
+                default: launch_direct<1, 2, 4>(g, grp, rm, stream); break;
             }
             return check_launch("gemm_f16_skinny");
         }
     }
-    if (grp.count > 1) return LG_OK;
+    if (grp.count > 1 || g.epi.kind == LG_EPI_BIAS_HEADS_ROWS) return LG_OK;  // the sliced kernels take plain single problems only
     const int nblk = (g.N + SK_BN - 1) / SK_BN;
     // K-slices: as few as fill the chip.  One block of 4 waves keeps 64 KiB of weight loads in flight, which is enough for one
     // CU; more slices only add fp32 partials and reduce work (six GEMMs of a decode step at 32 token rows on 256 CUs: 344 us

@@ -31,7 +31,7 @@ __device__ __forceinline__ float dot8(half8_t w, half8_t x, float acc) {
 
 // MR = staged token rows (1, 2 or 4; rows >= M are zero)
 template <int MR, int EPI>
-__global__ __launch_bounds__(256) void gemv_nk_kernel(GemmArgs g, GemmGroup members) {
+__global__ __launch_bounds__(256) void gemv_nk_kernel(GemmArgs g, GemmGroup members, RowMap rm) {
     extern __shared__ __attribute__((aligned(16))) half_t xs[];  // [MR][K]
     select_group(g, members);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -95,12 +95,12 @@ __global__ __launch_bounds__(256) void gemv_nk_kernel(GemmArgs g, GemmGroup memb
             float4_t out;
 #pragma unroll
             for (int r = 0; r < 4; ++r) out[r] = wave_sum(acc[q * 4 + r][m]);
-            if (lane == 0 && m < g.M) epilogue_store4<EPI>(g, g.Y, m, n0 + q * 4, out, true);
+            if (lane == 0 && m < g.M) epilogue_store4<EPI>(g, g.Y, m, n0 + q * 4, out, true, &rm);
         }
     }
 }
 
-int launch_gemv_f16(const GemmArgs& g, const GemmGroup& grp, int wlayout, int batch, hipStream_t stream, bool* handled) {
+int launch_gemv_f16(const GemmArgs& g, const GemmGroup& grp, const RowMap* rows, int wlayout, int batch, hipStream_t stream, bool* handled) {
     *handled = false;
     if (batch != 1 || wlayout != W_NK) return LG_OK;
     if (g.M <= 0 || g.M > 4 || g.N < 256 || (g.N % 4) || g.K < GV_KSTEP * GV_U || (g.K % (GV_KSTEP * GV_U))) return LG_OK;
@@ -108,14 +108,16 @@ int launch_gemv_f16(const GemmArgs& g, const GemmGroup& grp, int wlayout, int ba
     const size_t smem = (size_t)mr * g.K * sizeof(half_t);
     if (smem > (size_t)GV_MAX_LDS) return LG_OK;
     if (!aligned16(g.X) || (g.ldx % 8) || (g.ldw % 8) || !group_aligned(g, grp)) return LG_OK;
+    if (g.epi.kind == LG_EPI_BIAS_HEADS_ROWS && (!rows || g.M > LG_ROWMAP_MAX)) return LG_OK;
     *handled = true;
+    const RowMap rm = rows ? *rows : RowMap{};
     const dim3 grid((g.N + 4 * GV_ROWS - 1) / (4 * GV_ROWS), grp.count), block(256);
 #define LG_GV(MR_, E_)                                                                                              \
     do {                                                                                                            \
         /* set once per instantiation; the initialisation of a function-local static is thread-safe */              \
         static const hipError_t attr_rc = hipFuncSetAttribute((const void*)gemv_nk_kernel<MR_, E_>, hipFuncAttributeMaxDynamicSharedMemorySize, GV_MAX_LDS); \
         (void)attr_rc;                                                                                              \
-        hipLaunchKernelGGL((gemv_nk_kernel<MR_, E_>), grid, block, smem, stream, g, grp);                              \
+        hipLaunchKernelGGL((gemv_nk_kernel<MR_, E_>), grid, block, smem, stream, g, grp, rm);                              \
     } while (0)
 #define LG_GV_MR(E_)                                 \
     switch (mr) {                                    \
@@ -127,6 +129,7 @@ int launch_gemv_f16(const GemmArgs& g, const GemmGroup& grp, int wlayout, int ba
         case LG_EPI_NONE: LG_GV_MR(LG_EPI_NONE); break;
         case LG_EPI_BIAS: LG_GV_MR(LG_EPI_BIAS); break;
         case LG_EPI_BIAS_GELU: LG_GV_MR(LG_EPI_BIAS_GELU); break;
+        case LG_EPI_BIAS_HEADS_ROWS: LG_GV_MR(LG_EPI_BIAS_HEADS_ROWS); break;
         default: LG_GV_MR(LG_EPI_BIAS_HEADS); break;
     }
 #undef LG_GV_MR

@@ -44,6 +44,7 @@ SIGNATURES = {
     "lgh_model_describe": (_i, [_p, _i, _i, _i, C.c_char_p, _i]),
     "lgh_model_run": (_i, [_p, _p, _p, _i, _i, _p, _p, _i]),
     "lgh_model_run_decode": (_i, [_p, _p, _p, _i, _i, _i, _p, _p]),
+    "lgh_model_run_decode_seqs": (_i, [_p, _p, _p, _i, C.POINTER(_i), C.POINTER(_i), _p, _p]),
     "lgh_model_time_kernels": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, C.POINTER(_f), _i]),
     "lgh_model_time_one": (_f, [_p, _p, _p, _i, _i, _i, _i, _i, _i]),
     "lgh_sched_create": (_p, [_p, _i, _f, _i, _i, _i, _i, _i, _i]),
@@ -197,6 +198,12 @@ class Model:
     def run_decode(self, input_ptr, output_ptr, batch, past, cache_slot=0, workspace_ptr=None, stream=None):
         check(lib.lgh_model_run_decode(self.h, input_ptr, output_ptr, batch, past, cache_slot, workspace_ptr, stream),
               "lgh_model_run_decode")
+
+    def run_decode_seqs(self, input_ptr, output_ptr, slots, pasts, workspace_ptr=None, stream=None):
+        """One decode step for sequences in cache slots `slots` that hold `pasts` positions each."""
+        n = len(slots)
+        check(lib.lgh_model_run_decode_seqs(self.h, input_ptr, output_ptr, n, (C.c_int * n)(*slots), (C.c_int * n)(*pasts),
+                                            workspace_ptr, stream), "lgh_model_run_decode_seqs")
 
     def time_kernels(self, input_ptr, output_ptr, batch, seq, decode_past=-1, cache_slot=-1, iters=20, trials=3):
         out = (C.c_float * 4096)()

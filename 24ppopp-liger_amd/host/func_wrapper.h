@@ -32,6 +32,19 @@ inline void GemmExGrouped3(const DynamicInitParam& DParams, const GemmDesc& q, c
                                           q.epi_d, q.epi_heads_total, DParams.stream), "lg_gemm_fused_grouped_f16");
 }
 
+// The same for sequences in arbitrary cache slots at different positions: q goes to row r of its buffer, the K and V rows of
+// token r to position pos[r] of cache slot slot[r].  `n` sequences; slot / pos are copied into the launch.
+inline void GemmExGrouped3Rows(const DynamicInitParam& DParams, const GemmDesc& q, const GemmDesc& k, const GemmDesc& v, const int* slot,
+                               const int* pos) {
+    const void* A[3] = {q.A, k.A, v.A};
+    void* C[3] = {q.C, k.C, v.C};
+    const int ldc[3] = {q.ldc, k.ldc, v.ldc};
+    const void* bias[3] = {q.bias, k.bias, v.bias};
+    const int use_rows[3] = {0, 1, 1};
+    note_status(lg_gemm_fused_grouped_rows_f16(q.transa, q.m, q.n, q.k, 3, A, q.lda, q.B, q.ldb, C, ldc, bias, q.epi_d, q.epi_heads_total,
+                                               use_rows, slot, pos, DParams.stream), "lg_gemm_fused_grouped_rows_f16");
+}
+
 inline void GemmStridedBatchedEx(const DynamicInitParam& DParams, int dtype, int transa, int transb, int m, int n, int k,
                                  const void* A, int lda, long long strideA, const void* B, int ldb, long long strideB,
                                  void* C, int ldc, long long strideC, int batchCount) {

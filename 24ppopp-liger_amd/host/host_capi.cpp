@@ -48,6 +48,7 @@ struct ModelBase {
     virtual ~ModelBase() {}
     virtual std::vector<FuncWrap> build(void* in, void* out, int batch, int seq, void* ws, int slot) = 0;
     virtual std::vector<FuncWrap> build_decode(void* in, void* out, int batch, int past, int slot, void* ws) = 0;
+    virtual std::vector<FuncWrap> build_decode_seqs(void* in, void* out, const std::vector<int>& slots, const std::vector<int>& pasts, void* ws) = 0;
     virtual int64_t workspace_elems(int batch, int seq) = 0;
     virtual int kernels_per_layer(bool decode) = 0;
     virtual std::vector<ParamRef> params() = 0;
@@ -181,6 +182,9 @@ struct ModelT : ModelBase {
     }
     std::vector<FuncWrap> build_decode(void* in, void* out, int batch, int past, int slot, void* ws) override {
         return m->forward_decode((T*)in, (T*)out, batch, past, slot, (T*)(ws ? ws : default_ws));
+    }
+    std::vector<FuncWrap> build_decode_seqs(void* in, void* out, const std::vector<int>& slots, const std::vector<int>& pasts, void* ws) override {
+        return m->forward_decode_seqs((T*)in, (T*)out, slots, pasts, (T*)(ws ? ws : default_ws));
     }
     int64_t workspace_elems(int batch, int seq) override { return m->workspace_elems(batch, seq); }
     int kernels_per_layer(bool decode) override { return m->kernels_per_layer(decode); }
@@ -335,6 +339,23 @@ int lgh_model_run_decode(void* model, void* input, void* output, int batch, int 
         return fail("lgh_model_run_decode: bad arguments");
     DynamicInitParam D(stream ? stream : mb->stream0->stream, 0);
     for (auto& f : mb->build_decode(input, output, batch, past, cache_slot, workspace)) f.callback(D);
+    return first_error();
+}
+
+// One decode step for `batch` sequences that sit in cache slots slot[i] with past[i] cached positions each (decode steps of
+// different requests as one launch vector); input / output are [batch, hidden].
+int lgh_model_run_decode_seqs(void* model, void* input, void* output, int batch, const int* slot, const int* past, void* workspace,
+                              void* stream) {
+    ModelBase* mb = (ModelBase*)model;
+    if (!mb || batch <= 0 || batch > mb->P.max_batch_size || batch > LG_ATTN_DECODE_MAX_SEQS || !slot || !past || !input || !output ||
+        mb->P.max_cache_len <= 0)
+        return fail("lgh_model_run_decode_seqs: bad arguments");
+    std::vector<int> slots(slot, slot + batch), pasts(past, past + batch);
+    for (int i = 0; i < batch; ++i)
+        if (slots[i] < 0 || slots[i] >= mb->P.max_batch_size || pasts[i] < 0 || pasts[i] >= mb->P.max_cache_len)
+            return fail("lgh_model_run_decode_seqs: a position or cache slot lies outside the KV cache");
+    DynamicInitParam D(stream ? stream : mb->stream0->stream, 0);
+    for (auto& f : mb->build_decode_seqs(input, output, slots, pasts, workspace)) f.callback(D);
     return first_error();
 }
 

@@ -513,6 +513,66 @@ class Bert_MHA {
         FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
         return FuncWrapVec;
     }
+
+    // One decode step for sequences that sit in arbitrary cache slots at different positions (decode steps of different
+    // requests as one launch vector): sequence i reads and extends cache slot slots[i], which holds pasts[i] positions.
+    // Same entries as forward_decode, with the per-sequence variants of the kernels that touch the cache.
+    std::vector<FuncWrap> forward_decode_seqs(T* input, T* output, const std::vector<int>& slots, const std::vector<int>& pasts,
+                                              T* ws = nullptr) {
+        FuncWrapVec.clear();
+        if (!ws) ws = workspace;
+        const int batch = (int)slots.size();
+        const MhaBuffers<T> b = slice(ws, batch, 1);
+        const int h = heads(), d = BertParams.size_per_head, Lmax = BertParams.max_cache_len;
+        bool ok = k_cache && batch > 0 && batch <= LG_ATTN_DECODE_MAX_SEQS && pasts.size() == slots.size();
+        for (int i = 0; i < batch && ok; ++i) ok = slots[i] >= 0 && slots[i] < BertParams.max_batch_size && pasts[i] >= 0 && pasts[i] < Lmax;
+        if (!ok) {
+            set_error_state(LG_ERR_INVALID, "Bert_MHA::forward_decode_seqs: a position or cache slot lies outside the KV cache");
+            return FuncWrapVec;
+        }
+        const float sc = scalar;
+        T *kc = k_cache, *vc = v_cache;
+        void* dws = b.decode_ws;
+        std::vector<int> lens(pasts);
+        for (int& l : lens) l += 1;
+        std::vector<FuncWrap> v;
+        if (BertParams.fused) {
+            Linear_Col<T>* lin[3] = {linear_q_col, linear_k_col, linear_v_col};
+            T* dst[3] = {b.q_buf, kc, vc};
+            const T* bias[3] = {q_bias, k_bias, v_bias};
+            GemmDesc g[3];
+            for (int t = 0; t < 3; ++t) {
+                g[t] = lin[t]->desc(input, dst[t], batch);
+                g[t].bias = bias[t];
+                g[t].epi_seq = 1; g[t].epi_d = d; g[t].epi_heads_total = h;
+                g[t].ldc = (t == 0) ? 1 : Lmax;
+            }
+            const GemmDesc gq = g[0], gk = g[1], gv = g[2];
+            FuncWrapVec.push_back(FuncWrap(1.0f, COMPUTATION, [gq, gk, gv, slots, pasts](const DynamicInitParam& D) {
+                GemmExGrouped3Rows(D, gq, gk, gv, slots.data(), pasts.data());
+            }, "qkv_gemm(decode)", HBM_BOUND));
+        } else {
+            v = linear_q_col->forward(input, b.q, batch); v[0].label = "q_gemm(decode)"; v[0].rclass = HBM_BOUND;
+            FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
+            v = linear_k_col->forward(input, b.k, batch); v[0].label = "k_gemm(decode)"; v[0].rclass = HBM_BOUND;
+            FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
+            v = linear_v_col->forward(input, b.v, batch); v[0].label = "v_gemm(decode)"; v[0].rclass = HBM_BOUND;
+            FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
+            T *qbias = q_bias, *kbias = k_bias, *vbias = v_bias;
+            FuncWrapVec.push_back(FuncWrap(0.05f, COMPUTATION, [=](const DynamicInitParam& D) {
+                note_status(lg_kv_append_varlen_f16(b.q_buf, kc, vc, b.q, qbias, b.k, kbias, b.v, vbias, batch, h, d, slots.data(), pasts.data(),
+                                                    Lmax, D.stream), "lg_kv_append_varlen_f16");
+            }, "kv_append"));
+            FuncWrapVec.back().minor = true;
+        }
+        FuncWrapVec.push_back(FuncWrap(0.15f, COMPUTATION, [=](const DynamicInitParam& D) {
+            note_status(lg_attn_decode_varlen_f16(b.q_buf, kc, vc, b.attn_out, dws, batch, h, d, slots.data(), lens.data(), Lmax, sc, D.stream),
+                        "lg_attn_decode_varlen_f16");
+        }, "attn_decode"));
+        v = linear_w_row->forward(b.attn_out, output, batch); v[0].label = "out_proj(decode)"; v[0].rclass = HBM_BOUND;
+        FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
+        return FuncWrapVec;
+    }
 };
 
 // ---------------------------------------------------------------------------------------------------
@@ -562,11 +622,12 @@ class Bert_Encoder {
 
     // bert.h:59-79: MHA -> LN -> MLP -> LN (POST_NORESID).  PRE_LN_RESID chains layer_norm -> MHA ->
     // add_bias_input_layernorm_2 -> MLP -> add_bias_input.
+    // slots / pasts (both or neither): a decode step over sequences in arbitrary cache slots at different positions
     std::vector<FuncWrap> forward(T* input, T* output, int batch_size, int seq_len, T* ws = nullptr, int cache_slot = -1,
-                                  int decode_past = -1) {
+                                  int decode_past = -1, const std::vector<int>* slots = nullptr, const std::vector<int>* pasts = nullptr) {
         FuncWrapVec.clear();
         if (!ws) ws = workspace;
-        const bool decode = decode_past >= 0;
+        const bool decode = decode_past >= 0 || slots;
         const int seq = decode ? 1 : seq_len;
         const int M = batch_size * seq;
         T* attn_ws = ws;
@@ -577,6 +638,7 @@ class Bert_Encoder {
         T* pre_ln_out = mlp_out + align_up((int64_t)M * n);
         auto append = [&](std::vector<FuncWrap> v) { FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end()); };
         auto mha = [&](T* in, T* out) {
+            if (slots) return MHA->forward_decode_seqs(in, out, *slots, *pasts, attn_ws);
             return decode ? MHA->forward_decode(in, out, batch_size, decode_past, cache_slot, attn_ws)
                           : MHA->forward(in, out, batch_size, seq_len, attn_ws, cache_slot);
         };
@@ -648,6 +710,17 @@ class Bert_Model {
         if (!ws) ws = workspace;
         for (int i = 0; i < BertParams.layer_num; i++) {
             std::vector<FuncWrap> v = encoders[i]->forward(i == 0 ? input : output, output, batch_size, seq_len, ws, cache_slot);
+            FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
+        }
+        return FuncWrapVec;
+    }
+    // one decode step through all layers for sequences in arbitrary cache slots at different positions
+    std::vector<FuncWrap> forward_decode_seqs(T* input, T* output, const std::vector<int>& slots, const std::vector<int>& pasts, T* ws = nullptr) {
+        FuncWrapVec.clear();
+        if (!ws) ws = workspace;
+        if (slots.empty() || slots.size() != pasts.size()) return FuncWrapVec;
+        for (int i = 0; i < BertParams.layer_num; i++) {
+            std::vector<FuncWrap> v = encoders[i]->forward(i == 0 ? input : output, output, (int)slots.size(), 1, ws, -1, -1, &slots, &pasts);
             FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
         }
         return FuncWrapVec;

@@ -182,19 +182,30 @@ class Scheduler {
     bool enable_partition(int hbm_cus, int total_cus = 256) {
         if (hbm_cus <= 0 || hbm_cus % 8 != 0 || hbm_cus >= total_cus || total_cus > 256 || total_cus % 8 != 0) return false;
         if (partition_hbm_cus == hbm_cus) return true;
-        unsigned hbm_mask[8] = {0}, mfma_mask[8] = {0};
-        for (int b = 0; b < total_cus; ++b) (b < hbm_cus ? hbm_mask : mfma_mask)[b >> 5] |= 1u << (b & 31);
-        for (int role = 0; role < 2; ++role) {
-            _part[role][MFMA_BOUND].reset(new DynamicInitParam(mfma_mask, 8, 2 + 2 * role + MFMA_BOUND));
-            _part[role][HBM_BOUND].reset(new DynamicInitParam(hbm_mask, 8, 2 + 2 * role + HBM_BOUND));
+        // the streams of a share are created once and kept (every CU-masked stream is a hardware queue of its own)
+        auto it = _part_streams.find(hbm_cus);
+        if (it == _part_streams.end()) {
+            unsigned hbm_mask[8] = {0}, mfma_mask[8] = {0};
+            for (int b = 0; b < total_cus; ++b) (b < hbm_cus ? hbm_mask : mfma_mask)[b >> 5] |= 1u << (b & 31);
+            PartStreams ps;
+            for (int role = 0; role < 2; ++role) {
+                ps.d[role][MFMA_BOUND].reset(new DynamicInitParam(mfma_mask, 8, 2 + 2 * role + MFMA_BOUND));
+                ps.d[role][HBM_BOUND].reset(new DynamicInitParam(hbm_mask, 8, 2 + 2 * role + HBM_BOUND));
+            }
+            if (first_error()) { partition_hbm_cus = 0; return false; }
+            it = _part_streams.emplace(hbm_cus, std::move(ps)).first;
         }
-        if (first_error()) { partition_hbm_cus = 0; return false; }
+        for (int role = 0; role < 2; ++role)
+            for (int cls = 0; cls < 2; ++cls) _part[role][cls] = it->second.d[role][cls].get();
         partition_hbm_cus = hbm_cus;
+        // factors measured for another share do not carry over
+        for (int a = 0; a < 3; ++a)
+            for (int b = 0; b < 3; ++b) partition_table[a][b] = -1.f;
         return true;
     }
     void disable_partition() { partition_hbm_cus = 0; }
     const DynamicInitParam* partition_stream(int role, int cls) const {
-        return (partition_hbm_cus > 0 && (cls == MFMA_BOUND || cls == HBM_BOUND)) ? _part[role][cls].get() : nullptr;
+        return (partition_hbm_cus > 0 && (cls == MFMA_BOUND || cls == HBM_BOUND)) ? _part[role][cls] : nullptr;
     }
 
     // ---- per-request contexts ------------------------------------------------------------------------------
@@ -635,8 +646,8 @@ class Scheduler {
                     if (need >= partition_min_ms) {
                         part_factor = partition_table[mc][sc];
                         cap = need / part_factor;
-                        Dp = _part[0][mc].get();
-                        Ds = _part[1][sc].get();
+                        Dp = _part[0][mc];
+                        Ds = _part[1][sc];
                         partition_rounds++;
                     }
                 }
@@ -785,7 +796,9 @@ class Scheduler {
         for (Sample* smp : _main_q) delete smp;
         _main_q.clear();
     }
-    std::unique_ptr<DynamicInitParam> _part[2][2];  // CU-masked streams of partitioned rounds: [role][class]
+    struct PartStreams { std::unique_ptr<DynamicInitParam> d[2][2]; };
+    std::map<int, PartStreams> _part_streams;                              // by HBM-side share, created once
+    DynamicInitParam* _part[2][2] = {{nullptr, nullptr}, {nullptr, nullptr}};  // CU-masked streams of partitioned rounds: [role][class]
     void* _epoch_event = nullptr;
     std::chrono::steady_clock::time_point _epoch_host;
     std::vector<Sample*> _retired;

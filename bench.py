@@ -158,9 +158,10 @@ def bench_cfg4(capi, host, weight_layout, factors=(1, 2, 4, 8), shares=(0, 64, 9
             "results": out}
 
 
-def bench_cfg5(capi, host, weight_layout, n_requests):
+def bench_cfg5(capi, host, weight_layout, n_requests, rates=(4.0, 8.0, 16.0), shares=(64, 128), runs=1):
     """BASELINE config 5: Poisson arrivals at 4, 8, 16 req/s through 4 stacked layer shards; prompts U[128, 1024]
-    (rounded to 64), 32 decode tokens each; mean and p99 request latency with interleaving on and off."""
+    (rounded to 64), 32 decode tokens each; mean and p99 request latency with interleaving on and off.  `runs` > 1 repeats
+    every (rate, mode) and reports the mean and the spread of the mean latency over the runs."""
     c = CFG2
     pool = 16
     model = host.Model(capi.F16, pool, 1024, c["heads_global"], c["d"], layer_num=4, world_size=c["world_size"], ffn_inner=c["ffn_global"],
@@ -175,29 +176,51 @@ def bench_cfg5(capi, host, weight_layout, n_requests):
     # measured contention: the MFMA-bound kernels of a 512-token prefill next to batch-1 decode steps at 512 cached positions
     meas = sched.profile_contention(1, 512, 1, 512)
     table = {"mfma_main_hbm_sub": sched.contention(0, 1), "hbm_main_mfma_sub": sched.contention(1, 0)}
+    part_meas = {}
+    part_factor = {}
+    for share in shares:
+        sched.enable_partition(share)
+        pm = sched.profile_partition(1, 512, 1, 512)
+        part_meas[share] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in pm.items()}
+        part_factor[share] = (sched.partition_factor(0, 1), sched.partition_factor(1, 0))
+    sched.enable_partition(0)
+    modes = [(host.MODE_SEQUENTIAL, "scheduling_off", False, False, 0), (host.MODE_LIGER, "scheduling_on", False, False, 0),
+             (host.MODE_LIGER, "scheduling_on_measured_contention", True, False, 0),
+             (host.MODE_LIGER, "scheduling_on_minor_kernels_merged", False, True, 0)]
+    for share in shares:
+        if part_factor[share][0] > 0:
+            modes.append((host.MODE_LIGER, "scheduling_on_partitioned_%d_hbm_cus" % share, False, True, share))
     out = []
-    for lam in (4.0, 8.0, 16.0):
+    for lam in rates:
         trace = host.make_poisson_trace(lam, n_requests, 1, 128, 1024, 64, 32, 0)
         row = {"lambda_req_s": lam, "requests": n_requests}
-        for mode, name, measured, merge_minor in ((host.MODE_SEQUENTIAL, "scheduling_off", False, False), (host.MODE_LIGER, "scheduling_on", False, False),
-                                                 (host.MODE_LIGER, "scheduling_on_measured_contention", True, False),
-                                                 (host.MODE_LIGER, "scheduling_on_minor_kernels_merged", False, True)):
+        for mode, name, measured, merge_minor, share in modes:
             sched.set_contention(0, 1, table["mfma_main_hbm_sub"] if measured else -1.0)
             sched.set_contention(1, 0, table["hbm_main_mfma_sub"] if measured else -1.0)
             sched.set_merge_minor(merge_minor)
-            r = sched.run_trace(trace, mode)
+            sched.enable_partition(share)
+            if share:
+                sched.set_partition_factor(0, 1, part_factor[share][0])
+                sched.set_partition_factor(1, 0, part_factor[share][1])
+            reps = [sched.run_trace(trace, mode) for _ in range(runs)]
+            r = reps[0]
             # latency = arrival -> completion on one clock; the reference's sum (first launch - arrival) + (start event -> stop
             # event) is kept beside it: it under-counts when a start event is held up on the device
-            row[name] = {"mean_latency_ms": round(r["avg_e2e_ms"], 3), "p99_latency_ms": round(r["p99_e2e_ms"], 3),
+            means = [x["avg_e2e_ms"] for x in reps]
+            row[name] = {"mean_latency_ms": round(sum(means) / len(means), 3), "p99_latency_ms": round(sum(x["p99_e2e_ms"] for x in reps) / len(reps), 3),
+                         "mean_latency_runs_ms": [round(v, 3) for v in means],
                          "mean_cpu_plus_gpu_ms": round(r["avg_latency_ms"], 3),
                          "mean_gpu_ms": round(r["avg_gpu_ms"], 3), "mean_queue_ms": round(r["avg_queue_ms"], 3),
                          "throughput_req_s": round(r["throughput"], 3), "records": r["records"],
-                         "secondary_launches": r["secondary_launches"], "splits": r["splits"], "profile_misses": r["profile_misses"]}
+                         "secondary_launches": r["secondary_launches"], "splits": r["splits"], "profile_misses": r["profile_misses"],
+                         "partition_rounds": r["partition_rounds"]}
         out.append(row)
+    sched.enable_partition(0)
     return {"workload": "cfg5: 4 layer shards, Poisson arrivals, prompts U[128,1024] rounded to 64, 32 decode tokens", "profile_seconds": round(prof_s, 1),
             "streams_verified_concurrent": sched.streams_concurrent,
             "contention_measurement": {k: (round(v, 4) if isinstance(v, float) else v) for k, v in meas.items()},
-            "contention_table": {k: round(v, 4) for k, v in table.items()}, "results": out}
+            "contention_table": {k: round(v, 4) for k, v in table.items()},
+            "partition_measurement": part_meas, "results": out}
 
 
 def main():

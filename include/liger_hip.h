@@ -35,6 +35,9 @@ extern "C" {
 #define LG_F32 0
 #define LG_F16 1
 
+/* most sequences one launch of the per-sequence (varlen / rows) decode entry points can carry */
+#define LG_ATTN_DECODE_MAX_SEQS 64
+
 /* ---- library / device ------------------------------------------------------------------------ */
 const char* lg_last_error(void);
 const char* lg_version(void);
@@ -193,6 +196,15 @@ int lg_gemm_fused_grouped_f16(int transa, int m, int n, int k, int count, const 
                               int ldb, void* const* C, const int* ldc, int epilogue, const void* const* bias,
                               int epi_arg0, int epi_arg1, int epi_arg2, void* stream);
 
+/* The Q, K and V projections of a decode step over sequences that sit in arbitrary cache slots at different positions (decode
+ * steps of different requests batched into one launch): lg_gemm_fused_grouped_f16 with the heads epilogue and one token per
+ * sequence, except that a member i with use_rows[i] != 0 writes token row r to position pos[r] of batch entry slot[r] of its
+ * destination C[i] = [slots, heads_total, ldc[i], size_per_head] (a KV cache) instead of to position 0 of entry r.  slot and
+ * pos are HOST arrays of n ints, copied into the launch (n <= LG_ATTN_DECODE_MAX_SEQS).  No reference counterpart. */
+int lg_gemm_fused_grouped_rows_f16(int transa, int m, int n, int k, int count, const void* const* A, int lda, const void* B,
+                                   int ldb, void* const* C, const int* ldc, const void* const* bias, int size_per_head,
+                                   int heads_total, const int* use_rows, const int* slot, const int* pos, void* stream);
+
 /* ---- attention kernels with no reference counterpart --------------------------------------------- */
 /* Fused prefill attention: out = softmax(q k^T * scalar + maskterm) v with the reference's softmax
  * semantics (-10000 additive mask, +1e-6 in the denominator); replaces launch-vector entries 4,5,6 (and 7
@@ -214,7 +226,6 @@ int lg_attn_decode_f16(const void* q, const void* k_cache, const void* v_cache, 
 /* The same over sequences that differ in length and sit in arbitrary cache slots (decode steps of different requests
  * batched into one launch): sequence b reads slot[b] of the caches [slots,h,max_len,d] and attends to its first len[b]
  * positions.  slot and len are HOST arrays of `batch` ints, copied into the launch (batch <= LG_ATTN_DECODE_MAX_SEQS). */
-#define LG_ATTN_DECODE_MAX_SEQS 64
 int lg_attn_decode_varlen_f16(const void* q, const void* k_cache, const void* v_cache, void* out, void* workspace,
                               int batch, int head_num, int size_per_head, const int* slot, const int* len, int max_len,
                               float scalar, void* stream);

@@ -227,6 +227,10 @@ int lg_gemm_strided_batched_f32(int, int, int m, int n, int k, const float* A, i
 int lg_gemm_strided_batched_f16(int, int, int m, int n, int k, const void* A, int, int64_t, const void* B, int, int64_t, void* C, int, int64_t, int batch, void* stream) { return launch(stream, "gemm_batched", m, n, k, A, B, C, gemm_cost((long long)m * batch, n, k)); }
 int lg_gemm_fused_f16(int, int m, int n, int k, const void* A, int, const void* B, int, void* C, int, int, const void*, int, int, int, void* stream) { return launch(stream, "gemm_fused", m, n, k, A, B, C, gemm_cost(m, n, k)); }
 int lg_gemm_fused_grouped_f16(int, int m, int n, int k, int count, const void* const* A, int, const void* B, int, void* const* C, const int*, int, const void* const*, int, int, int, void* stream) { return launch(stream, "gemm_fused_grouped", (long long)m * count, n, k, A[0], B, C[0], gemm_cost((long long)m * count, n, k)); }
+int lg_gemm_fused_grouped_rows_f16(int, int m, int n, int k, int count, const void* const* A, int, const void* B, int, void* const* C, const int*, const void* const*, int, int, const int*, const int* slot, const int*, void* stream) {
+    (void)slot;
+    return launch(stream, "gemm_fused_grouped_rows", (long long)m * count, n, k, A[0], B, C[0], gemm_cost((long long)m * count, n, k));
+}
 int lg_attn_prefill_f16(const void* q, const void* k, const void*, const void*, void* out, int b, int s, int h, int d, int, float, int, int, void* stream) { return launch(stream, "attn_prefill", (long long)b * h, s, d, q, k, out, gemm_cost((long long)b * h * s, s, 2 * d)); }
 size_t lg_attn_decode_workspace_bytes(int, int, int, int) { return 1024; }
 int lg_attn_decode_f16(const void* q, const void* kc, const void*, void* out, void*, int b, int h, int d, int len, int, float, void* stream) { return launch(stream, "attn_decode", (long long)b * h, len, d, q, kc, out, mem_cost(4.0 * b * h * len * d)); }

@@ -302,3 +302,47 @@ def test_grouped_gemm_other_epilogues_and_counts(dev, po, M, count, epi):
         y = po.gemm(X, Ws[t], 1)
         ref = y if epi == "none" else (po.round_f16(y + bs[t]) if epi == "bias" else po.add_bias_gelu(y.copy(), bs[t], 1))
         assert max_rel_err(got[:, :N], ref) < 4e-3
+
+
+@pytest.mark.parametrize("M,N,K,transa", [(3, 1024, 2048, 1), (12, 6144, 2048, 1), (40, 6144, 4096, 1), (5, 512, 512, 1), (6, 1024, 2048, 0)])
+def test_grouped_gemm_with_a_destination_per_token_row(dev, po, M, N, K, transa):
+    """Q, K and V of a decode step whose sequences sit in arbitrary cache slots at different positions: q goes to row r, the
+    K and V rows of token r to (slot[r], head, pos[r]) of a cache [slots, heads, rows, d].  Shapes for the matrix-vector
+    kernel (M <= 4), the weight-streaming kernel, and the plain-call fallback (small N, or weights stored [in, out]).  Checked
+    against the oracle's GEMM + bias scattered by numpy, bit-for-bit untouched elsewhere."""
+    import ctypes as C
+    d = 128
+    h = N // d
+    slots, rows = 7, 24
+    X = rnd(po, M * K, 80, 1).reshape(M, K)
+    Ws = [rnd(po, K * N, 81 + t, 1, 0.05).reshape(K, N) for t in range(3)]
+    bs = [rnd(po, N, 84 + t, 1, 0.3) for t in range(3)]
+    dA = [dev.up(np.ascontiguousarray(W.T) if transa else W, 1) for W in Ws]
+    dB = [dev.up(b, 1) for b in bs]
+    dX = dev.up(X, 1)
+    cells = [(11 * r + 5) % (slots * rows) for r in range(M)]      # distinct (slot, position) cells, scattered
+    slot, pos = [c % slots for c in cells], [c // slots for c in cells]
+    q = dev.empty((M, h, d), 1); q.zero_()
+    kc0 = rnd(po, slots * h * rows * d, 90, 1).reshape(slots, h, rows, d)
+    vc0 = rnd(po, slots * h * rows * d, 91, 1).reshape(slots, h, rows, d)
+    dkc, dvc = dev.up(kc0, 1), dev.up(vc0, 1)
+    arr = lambda ptrs: (C.c_void_p * 3)(*ptrs)
+    lda = K if transa else N
+    dev.call("lg_gemm_fused_grouped_rows_f16", transa, N, M, K, 3, arr([a.data_ptr() for a in dA]), lda, dX, K,
+             arr([q.data_ptr(), dkc.data_ptr(), dvc.data_ptr()]), (C.c_int * 3)(1, rows, rows), arr([b.data_ptr() for b in dB]),
+             d, h, (C.c_int * 3)(0, 1, 1), (C.c_int * M)(*slot), (C.c_int * M)(*pos))
+    ref = [po.round_f16(po.gemm(X, Ws[t], 1) + bs[t]).reshape(M, h, d) for t in range(3)]
+    assert max_rel_err(dev.down(q), ref[0]) < 4e-3
+    for got, base, want in ((dev.down(dkc), kc0, ref[1]), (dev.down(dvc), vc0, ref[2])):
+        exp = base.copy()
+        touched = np.zeros(base.shape[:3], dtype=bool)
+        for r in range(M):
+            exp[slot[r], :, pos[r], :] = want[r]
+            touched[slot[r], :, pos[r]] = True
+        assert np.array_equal(got[~touched], base[~touched]), "rows other than the addressed ones were written"
+        assert max_rel_err(got[touched], exp[touched]) < 4e-3
+    # rows outside the destination are refused on the host
+    bad = (C.c_int * M)(*([rows] + pos[1:]))
+    assert dev.call_rc("lg_gemm_fused_grouped_rows_f16", transa, N, M, K, 3, arr([a.data_ptr() for a in dA]), lda, dX, K,
+                       arr([q.data_ptr(), dkc.data_ptr(), dvc.data_ptr()]), (C.c_int * 3)(1, rows, rows), arr([b.data_ptr() for b in dB]),
+                       d, h, (C.c_int * 3)(0, 1, 1), (C.c_int * M)(*slot), bad) == dev.capi.ERR_INVALID

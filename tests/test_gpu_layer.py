@@ -118,6 +118,48 @@ def test_decode_step_matches_oracle(dev, po, host):
         tok = po.round_f16(ref)
 
 
+@pytest.mark.parametrize("heads,d,lens", [(4, 64, [40, 17, 33]), (8, 128, [64, 5, 23, 48, 9, 31])])
+def test_decode_step_over_sequences_of_different_lengths(dev, po, host, heads, d, lens):
+    """Decode steps of different requests as one launch vector: sequences of different lengths, prefilled one by one into
+    scattered cache slots, take one batched step (per-sequence K/V destinations in the Q/K/V epilogue, per-sequence lengths
+    in the attention).  Every sequence must equal the oracle's decoder step over its own cache, and its cache rows the
+    oracle's; a second step checks that the first one appended K and V where the next one reads them."""
+    F, Lmax, slots_total = 512, 72, 8
+    H = heads * d
+    n = len(lens)
+    slots = [(3 * i + 1) % slots_total for i in range(n)]         # scattered, not in sequence order
+    m = host.Model(1, slots_total, max(lens), heads, d, layer_num=1, ffn_inner=F, causal=True, fused=True, max_cache_len=Lmax, seed=5)
+    w = oracle_weights(m.download_params())
+    kcs, vcs = [], []
+    for i, S in enumerate(lens):
+        x = po.fill_normal(S * H, 5, 200 + i, 0.0, 1.0, 1).reshape(S, H)
+        dx, dy = dev.up(x, 1), dev.empty((S, H), 1)
+        m.run(dx.data_ptr(), dy.data_ptr(), 1, S, None, dev.stream, cache_slot=slots[i])
+        q = po.gemm(x, w["wq"], 1); k = po.gemm(x, w["wk"], 1); v = po.gemm(x, w["wv"], 1)
+        _, kb, vb = po.add_qkv_bias_transpose(q, w["bq"], k, w["bk"], v, w["bv"], 1, S, heads, d, 1)
+        kc = np.zeros((1, heads, Lmax, d), dtype=np.float32); vc = np.zeros_like(kc)
+        kc[:, :, :S] = kb; vc[:, :, :S] = vb
+        kcs.append(kc); vcs.append(vc)
+    dev.sync()
+    tok = po.fill_normal(n * H, 5, 300, 0.0, 1.0, 1).reshape(n, H)
+    pasts = list(lens)
+    for step in range(2):
+        dt_in, dt_out = dev.up(tok, 1), dev.empty((n, H), 1)
+        m.run_decode_seqs(dt_in.data_ptr(), dt_out.data_ptr(), slots, pasts, None, dev.stream)
+        got = dev.down(dt_out)
+        nxt = np.empty_like(tok)
+        for i in range(n):
+            shape = dict(batch=1, seq=lens[i], hidden=H, head_num=heads, size_per_head=d, ffn_inner=F, causal=1, norm_mode=0, dtype=1)
+            ref = po.decoder_step(shape, w, tok[i:i + 1], kcs[i], vcs[i], pasts[i])   # appends to the oracle-side cache
+            assert max_rel_err(got[i:i + 1], ref) < 1e-2, "step %d, sequence %d (slot %d, %d cached)" % (step, i, slots[i], pasts[i])
+            nxt[i] = po.round_f16(ref)[0]
+        tok = nxt
+        pasts = [p + 1 for p in pasts]
+    # a request outside the cache is refused before anything is launched
+    with pytest.raises(dev.capi.LigerError):
+        m.run_decode_seqs(dt_in.data_ptr(), dt_out.data_ptr(), slots, [Lmax] * n, None, dev.stream)
+
+
 @pytest.mark.parametrize("dtype,fused", [(0, False), (1, False), (1, True)])
 @pytest.mark.parametrize("norm_mode", [0, 1])
 def test_geglu_layer(dev, po, host, dtype, fused, norm_mode):
