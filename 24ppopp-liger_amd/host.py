@@ -25,7 +25,7 @@ class Report(C.Structure):
     _fields_ = [("records", _i), ("avg_latency_ms", _d), ("p99_latency_ms", _d), ("avg_gpu_ms", _d),
                 ("avg_queue_ms", _d), ("total_duration_ms", _d), ("throughput", _d), ("rounds", _i),
                 ("secondary_launches", _i), ("splits", _i), ("profile_misses", _i), ("avg_e2e_ms", _d), ("p99_e2e_ms", _d),
-                ("partition_rounds", _i), ("sub_profile_misses", _i)]
+                ("partition_rounds", _i), ("sub_profile_misses", _i), ("batched_steps", _i), ("batched_rows", _i)]
 
     def as_dict(self):
         return {n: getattr(self, n) for n, _ in self._fields_}
@@ -53,6 +53,8 @@ SIGNATURES = {
     "lgh_sched_profile_contention": (_i, [_p, _i, _i, _i, _i, C.POINTER(_f)]),
     "lgh_sched_set_contention": (_i, [_p, _i, _i, _f]),
     "lgh_sched_enable_partition": (_i, [_p, _i]),
+    "lgh_sched_enable_batch_decode": (_i, [_p, _i, _i]),
+    "lgh_sched_ctx_decode_ptrs": (_i, [_p, _i, C.POINTER(_p), C.POINTER(_p)]),
     "lgh_sched_profile_partition": (_i, [_p, _i, _i, _i, _i, C.POINTER(_f)]),
     "lgh_sched_set_partition_factor": (_i, [_p, _i, _i, _f]),
     "lgh_sched_get_partition_factor": (_f, [_p, _i, _i]),
@@ -235,6 +237,15 @@ class Scheduler:
         out = (_f * 5)()
         check(lib.lgh_sched_profile_contention(self.h, bs, seq, dec_bs, past, out), "lgh_sched_profile_contention")
         return {"main_ms": out[0], "sub_ms": out[1], "both_ms": out[2], "hidden": out[3], "sub_repeats": int(out[4])}
+
+    def enable_batch_decode(self, on=True, steps_ahead=0):
+        """Requests that are in their decode steps at the same time share one launch vector per step."""
+        check(lib.lgh_sched_enable_batch_decode(self.h, int(bool(on)), steps_ahead), "lgh_sched_enable_batch_decode")
+
+    def ctx_decode_ptrs(self, i):
+        a, b = _p(), _p()
+        check(lib.lgh_sched_ctx_decode_ptrs(self.h, i, C.byref(a), C.byref(b)), "lgh_sched_ctx_decode_ptrs")
+        return a.value, b.value
 
     def enable_partition(self, hbm_cus):
         """Co-running rounds give the HBM-bound side `hbm_cus` compute units and the MFMA-bound side the rest (0 = off)."""

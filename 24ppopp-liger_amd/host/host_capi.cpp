@@ -33,6 +33,9 @@ struct SchedBase {
     virtual bool set_partition_factor(int main_class, int sub_class, float v) = 0;
     virtual float get_partition_factor(int main_class, int sub_class) = 0;
     virtual void extra_counters(int* out2) = 0;
+    virtual bool enable_batch_decode(bool on, int steps_ahead) = 0;
+    virtual void batch_counters(int* out2) = 0;
+    virtual bool ctx_decode_ptrs(int i, void** a, void** b) = 0;
     virtual void set_factor(int factor) = 0;
     virtual bool ctx_ptrs(int i, void** in, void** out) = 0;
     virtual Report run_queued(int mode, int* counters) = 0;
@@ -130,6 +133,17 @@ struct SchedT : SchedBase {
         return (main_class < 0 || main_class > 2 || sub_class < 0 || sub_class > 2) ? -1.f : s->partition_table[main_class][sub_class];
     }
     void extra_counters(int* out2) override { out2[0] = s->partition_rounds; out2[1] = s->sub_profile_misses; }
+    bool enable_batch_decode(bool on, int steps_ahead) override {
+        if (steps_ahead > 0) s->decode_steps_ahead = steps_ahead;
+        return s->enable_batch_decode(on);
+    }
+    void batch_counters(int* out2) override { out2[0] = s->batched_steps; out2[1] = s->batched_rows; }
+    bool ctx_decode_ptrs(int i, void** a, void** b) override {
+        auto* c = s->context(i);
+        if (!c) return false;
+        *a = c->dec_a; *b = c->dec_b;
+        return true;
+    }
     void set_factor(int factor) override { s->BertParams.factor = factor; }
     bool ctx_ptrs(int i, void** in, void** out) override {
         auto* c = s->context(i);
@@ -391,6 +405,7 @@ struct LghReport {
     int rounds, secondary_launches, splits, profile_misses;
     double avg_e2e_ms, p99_e2e_ms;  // arrival -> completion on one clock
     int partition_rounds, sub_profile_misses;
+    int batched_steps, batched_rows;
 };
 
 // policy: 0 = classic (communication vs rest), 1 = resource classes (MFMA-bound vs HBM-bound)
@@ -447,6 +462,20 @@ int lgh_sched_set_partition_factor(void* sched, int main_class, int sub_class, f
 float lgh_sched_get_partition_factor(void* sched, int main_class, int sub_class) {
     return sched ? ((SchedBase*)sched)->get_partition_factor(main_class, sub_class) : -1.f;
 }
+// Requests that are in their decode steps at the same time share one launch vector per step (Scheduler::enable_batch_decode);
+// needs a pool, a KV cache and one cache slot more than the pool uses.  steps_ahead > 0 sets how many steps one vector holds
+// while nothing waits to join.
+int lgh_sched_enable_batch_decode(void* sched, int on, int steps_ahead) {
+    if (!sched || !((SchedBase*)sched)->enable_batch_decode(on != 0, steps_ahead))
+        return fail("lgh_sched_enable_batch_decode: needs per-request contexts, a KV cache and max_batch >= pool_count * ctx_batch + 1");
+    return LG_OK;
+}
+// the decode ping-pong buffers [ctx_batch, hidden] of the i-th context: after n decode steps a request's last hidden state is in
+// the second one when n is odd, in the first when n is even
+int lgh_sched_ctx_decode_ptrs(void* sched, int i, void** dec_a, void** dec_b) {
+    if (!sched || !dec_a || !dec_b || !((SchedBase*)sched)->ctx_decode_ptrs(i, dec_a, dec_b)) return fail("lgh_sched_ctx_decode_ptrs: no such context");
+    return LG_OK;
+}
 // main_class / sub_class: 0 = MFMA-bound, 1 = HBM-bound, 2 = link-bound; a negative value restores the constant factor
 int lgh_sched_set_contention(void* sched, int main_class, int sub_class, float value) {
     if (!sched || !((SchedBase*)sched)->set_contention(main_class, sub_class, value)) return fail("lgh_sched_set_contention: bad arguments");
@@ -487,6 +516,7 @@ int lgh_sched_run_trace(void* sched, int mode, const double* arrival_s, const in
     out->throughput = r.throughput; out->rounds = c[0]; out->secondary_launches = c[1]; out->splits = c[2]; out->profile_misses = c[3];
     out->avg_e2e_ms = r.avg_e2e_ms; out->p99_e2e_ms = r.p99_e2e_ms;
     { int x[2] = {0, 0}; ((SchedBase*)sched)->extra_counters(x); out->partition_rounds = x[0]; out->sub_profile_misses = x[1]; }
+    { int x[2] = {0, 0}; ((SchedBase*)sched)->batch_counters(x); out->batched_steps = x[0]; out->batched_rows = x[1]; }
     return first_error();
 }
 // Deterministic variant for tests: requests are queued up front with lgh_sched_serve (no request thread, no real-time
@@ -526,6 +556,7 @@ int lgh_sched_run_queued(void* sched, int mode, LghReport* out) {
     out->throughput = r.throughput; out->rounds = c[0]; out->secondary_launches = c[1]; out->splits = c[2]; out->profile_misses = c[3];
     out->avg_e2e_ms = r.avg_e2e_ms; out->p99_e2e_ms = r.p99_e2e_ms;
     { int x[2] = {0, 0}; ((SchedBase*)sched)->extra_counters(x); out->partition_rounds = x[0]; out->sub_profile_misses = x[1]; }
+    { int x[2] = {0, 0}; ((SchedBase*)sched)->batch_counters(x); out->batched_steps = x[0]; out->batched_rows = x[1]; }
     return first_error();
 }
 // the report arithmetic alone (known-answer tests against the reference's published logs)
@@ -535,7 +566,7 @@ int lgh_summarize(const double* cpu_ms, const double* gpu_ms, int n, double tota
     out->records = r.records; out->avg_latency_ms = r.avg_latency_ms; out->p99_latency_ms = r.p99_latency_ms;
     out->avg_gpu_ms = r.avg_gpu_ms; out->avg_queue_ms = r.avg_queue_ms; out->total_duration_ms = r.total_duration_ms;
     out->throughput = r.throughput; out->rounds = out->secondary_launches = out->splits = out->profile_misses = 0;
-    out->avg_e2e_ms = out->p99_e2e_ms = 0; out->partition_rounds = out->sub_profile_misses = 0;
+    out->avg_e2e_ms = out->p99_e2e_ms = 0; out->partition_rounds = out->sub_profile_misses = 0; out->batched_steps = out->batched_rows = 0;
     return LG_OK;
 }
 int lgh_make_poisson_trace(double lambda, int n, int batch, int seq_lo, int seq_hi, int seq_round, int n_decode, uint64_t seed,

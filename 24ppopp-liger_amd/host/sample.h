@@ -89,6 +89,7 @@ class Sample {
     int key_seq = 0;            // seq_len on the profile grid (set by the scheduler; seq_len when there is no grid)
     int sub_profile_misses = 0; // GEMMs that could not be split because the decomposition table has no entry for them
     int id = 0;
+    int n_decode_pending = 0;   // decode steps the owner still has to run for this request once the prefill vector is done
     bool merge_minor = false;  // see _neutral(); false = every entry keeps its own class (the reference's behaviour)
     void* user = nullptr;  // owner's per-request context (buffers), opaque here
 

@@ -149,6 +149,17 @@ class Scheduler {
     // that work lasts; all other rounds run on the whole chip.  partition_table[main][sub] = stand-alone milliseconds of
     // class-`sub` work that complete per stand-alone millisecond of the class-`main` primary in a partitioned round
     // (measured by profile_partition; <= 0: partitioning that pair does not pay and is not done).
+    // ---- decode steps of different requests as one launch vector (enable_batch_decode) ------------------------------------
+    // A request's decode steps stream the whole weight shard for one token row; requests that are in their decode steps at the
+    // same time therefore share one launch vector per step (per-sequence cache slots and lengths in the kernels that touch the
+    // cache), which reads the weights once for all of them.  The batched step is scheduled like one more request that is always
+    // last in line: the prefill of a newly arrived request goes ahead of it as the primary, the batch's HBM-bound kernels are
+    // interleaved into that prefill's MFMA-bound windows, and the request joins the batch at the first step boundary after its
+    // prefill.  No reference counterpart (the reference has no
+    // decode phase); without it every request runs its own decode steps, as in run_sequential.
+    bool batch_decode = false;
+    int decode_steps_ahead = 4;       // steps per batched launch vector while nothing waits to join (1 otherwise)
+    int batched_steps = 0, batched_rows = 0;   // steps launched, and token rows they carried (holes included)
     int partition_hbm_cus = 0;
     float partition_table[3][3] = {{-1.f, -1.f, -1.f}, {-1.f, -1.f, -1.f}, {-1.f, -1.f, -1.f}};
     float partition_min_ms = 0.05f;   // less waiting work than this is not worth a partitioned round
@@ -230,6 +241,22 @@ class Scheduler {
         _ctx_batch = ctx_batch;
         note_status(lg_device_synchronize(), "lg_device_synchronize");
     }
+    // Batched decode needs one more cache slot than the contexts use (rows of the batch that belong to no request in its
+    // decode steps are pointed at it) and the batch's own token-row buffer and workspace.
+    bool enable_batch_decode(bool on = true) {
+        if (!on) { batch_decode = false; return true; }
+        const int rows = _pool_total * _ctx_batch;
+        if (rows <= 0 || BertParams.max_cache_len <= 0 || rows + 1 > BertParams.max_batch_size || rows > LG_ATTN_DECODE_MAX_SEQS) return false;
+        if (!_dec_x) {
+            const int H = BertParams.head_num * BertParams.size_per_head;
+            _dec_x = dev_alloc<T>((int64_t)rows * H);
+            _dec_ws = dev_alloc<T>(_model->workspace_elems(rows, 1));
+            note_status(lg_memset_async(_dec_x, 0, (size_t)rows * H * sizeof(T), nullptr), "lg_memset_async");
+            note_status(lg_device_synchronize(), "lg_device_synchronize");
+        }
+        batch_decode = true;
+        return first_error() == 0;
+    }
     // Shapes a request may have: they decide how far the launch vector writes into the request's buffers, its workspace and
     // its KV-cache slots, so they are checked once here, on the host, before anything is built or launched.
     bool request_fits(int batch_size, int seq_len, int n_decode, const char* who) {
@@ -260,8 +287,12 @@ class Scheduler {
         std::unique_lock<std::mutex> lk(_pool_mutex);
         _pool_cv.wait(lk, [this] { return !_pool.empty() || !_running.load(); });
         if (_pool.empty()) return nullptr;
-        ReqCtx* c = _pool.front();
-        _pool.erase(_pool.begin());
+        // the free context with the lowest cache slot: the rows of a batched decode step then stay dense
+        size_t pick = 0;
+        for (size_t i = 1; i < _pool.size(); ++i)
+            if (_pool[i]->slot < _pool[pick]->slot) pick = i;
+        ReqCtx* c = _pool[pick];
+        _pool.erase(_pool.begin() + pick);
         return c;
     }
     void release_ctx(ReqCtx* c) {
@@ -279,6 +310,19 @@ class Scheduler {
         }
         profile_misses++;
         return 0.f;  // the reference's operator[] yields 0 for a missing key as well
+    }
+
+    // duration of decode-step entry `name` for `bs` token rows at `past` cached positions: the profiled batch at or below bs
+    // that exists (a step is weight-streaming bound: its time moves little with the number of rows)
+    float lookup_decode(int name, int bs, int past) {
+        const int key_past = seq_bucket > 1 ? (past + seq_bucket - 1) / seq_bucket * seq_bucket : past;
+        for (int b = bs; b >= 1; --b) {
+            auto it = profiling_res_dict.find({name, b, key_past});
+            if (it == profiling_res_dict.end()) it = profiling_res_dict.find({name, b, past});
+            if (it != profiling_res_dict.end()) return it->second;
+        }
+        profile_misses++;
+        return 0.f;
     }
 
     void profile_vector(std::vector<FuncWrap>& vec, int count, int name_base, int bs, int key_seq, int itr) {
@@ -482,6 +526,7 @@ class Scheduler {
         T* out = ctx ? ctx->output : output;
         T* ws = ctx ? ctx->ws : nullptr;
         const int slot = (ctx && BertParams.max_cache_len > 0) ? ctx->slot : -1;
+        std::unique_lock<std::mutex> build_lock(_build_mutex);  // the layer classes keep per-call state: one builder at a time
         std::vector<FuncWrap> vec = _model->forward(in, out, batch_size, seq_len, ws, slot);
         for (int i = 0; i < BertParams.layer_num; i++)
             for (int j = 0; j < BertParams.kernel_num; j++) {
@@ -489,7 +534,8 @@ class Scheduler {
                 f.name = j;
                 f.duration = lookup(j, batch_size, seq_len);
             }
-        if (n_decode > 0 && ctx && slot >= 0) {
+        const bool defer_decode = batch_decode && n_decode > 0 && ctx && slot >= 0;  // the decode steps join the batched launch vector
+        if (n_decode > 0 && ctx && slot >= 0 && !defer_decode) {
             const int H = BertParams.head_num * BertParams.size_per_head;
             const int kd = _model->kernels_per_layer(true);
             T* din = ctx->dec_a;
@@ -520,10 +566,12 @@ class Scheduler {
                 std::swap(din, dout);
             }
         }
+        build_lock.unlock();
         Sample* sample = new Sample(vec, profiling_decompse_res_dict, batch_size, seq_len, BertParams.factor, policy, axis);
         sample->user = ctx;
         sample->merge_minor = merge_minor;
         sample->key_seq = seq_bucket > 1 ? (seq_len + seq_bucket - 1) / seq_bucket * seq_bucket : seq_len;
+        sample->n_decode_pending = defer_decode ? n_decode : 0;
         {
             std::lock_guard<std::mutex> lk(_q_mutex);
             sample->id = _next_id++;
@@ -546,6 +594,7 @@ class Scheduler {
         T* ws = ctx ? ctx->ws : nullptr;
         const int slot = ctx ? ctx->slot : 0;
         const int kd = _model->kernels_per_layer(true);
+        std::unique_lock<std::mutex> build_lock(_build_mutex);
         std::vector<FuncWrap> vec;
         for (int t = 0; t < n_steps; ++t) {
             const int p = past + t;
@@ -558,6 +607,7 @@ class Scheduler {
             vec.insert(vec.end(), dv.begin(), dv.end());
             std::swap(din, dout);
         }
+        build_lock.unlock();
         Sample* sample = new Sample(vec, profiling_decompse_res_dict, batch_size, past, BertParams.factor, policy, axis);
         sample->user = ctx;
         sample->merge_minor = merge_minor;
@@ -576,7 +626,8 @@ class Scheduler {
 
     // ---- admission / retirement  (schedule.h:175-202) ------------------------------------------------------------
     void update_vec() {
-        if (!exe_vec.empty() && exe_vec[0]->empty()) {
+        if (batch_decode) _update_decode_batch();
+        if (!exe_vec.empty() && exe_vec[0] != _dec_sample && exe_vec[0]->empty()) {
             Sample* tmp = exe_vec[0];
             recs.push_back(tmp->get_recording());
             sub_profile_misses += tmp->sub_profile_misses;
@@ -584,16 +635,18 @@ class Scheduler {
             _retired.push_back(tmp);
         }
         _reclaim();
-        for (size_t i = exe_vec.size(); i < (size_t)schedule_deep; i++) {
+        const size_t deep = (size_t)schedule_deep + (_dec_sample ? 1 : 0);  // the batched step does not use up a request's place
+        for (size_t i = exe_vec.size(); i < deep; i++) {
             std::lock_guard<std::mutex> lk(_q_mutex);
             if (_main_q.empty()) break;
-            exe_vec.push_back(_main_q.front());
+            // the batched decode step stays last: a request's prefill goes ahead of it (the request then joins the batch)
+            exe_vec.insert(_dec_sample ? exe_vec.end() - 1 : exe_vec.end(), _main_q.front());
             _main_q.pop_front();
         }
         if (exe_vec.empty()) std::this_thread::sleep_for(std::chrono::microseconds(100));
     }
 
-    bool drained() { return exe_vec.empty() && queued() == 0; }
+    bool drained() { return exe_vec.empty() && queued() == 0 && _dec_seqs.empty(); }
 
     // ---- baseline: one request at a time on stream 0  (schedule.h:204-219) -----------------------------------------
     void run_sequential() {
@@ -704,6 +757,9 @@ class Scheduler {
         _epoch_host = std::chrono::steady_clock::now();
         for (auto& r : recs) { lg_event_destroy(r.start); lg_event_destroy(r.stop); }
         recs.clear();
+        for (void* e : _dec_prefill_events) lg_event_destroy(e);
+        _dec_prefill_events.clear();
+        batched_steps = batched_rows = 0;
         rounds = secondary_launches = splits = partition_rounds = 0;
     }
 
@@ -784,6 +840,156 @@ class Scheduler {
     }
 
   private:
+    // ---- batched decode steps ---------------------------------------------------------------------------------------------
+    struct DecodeSeq {
+        ReqCtx* ctx;
+        int batch, seq_len, past, remaining, n_decode;
+        bool joined;
+        void *start, *prefill_done, *done;   // events: first prefill kernel, last prefill kernel, last decode kernel
+        double cpu_time;
+        std::chrono::steady_clock::time_point arrive;
+    };
+    std::vector<DecodeSeq> _dec_seqs;        // requests in (or about to join) their decode steps
+    Sample* _dec_sample = nullptr;           // launch vector of the batched step(s) being launched; last in exe_vec while it exists
+    T *_dec_x = nullptr, *_dec_ws = nullptr; // token rows [contexts x ctx_batch, hidden] (a step runs in place) and its workspace
+    std::vector<std::pair<void*, ReqCtx*>> _dec_done;   // (completion event, context to hand back)
+    std::mutex _build_mutex;
+
+    // requests whose prefill vector has been launched completely move on to the decode batch
+    void _collect_prefilled() {
+        for (size_t i = 0; i < exe_vec.size();) {
+            Sample* smp = exe_vec[i];
+            if (smp == _dec_sample || !smp->empty() || smp->n_decode_pending <= 0) { ++i; continue; }
+            DecodeSeq q;
+            q.ctx = (ReqCtx*)smp->user;
+            q.batch = smp->batch_size; q.seq_len = smp->seq_len; q.past = smp->seq_len;
+            q.remaining = q.n_decode = smp->n_decode_pending;
+            q.joined = false;
+            q.start = smp->start; q.prefill_done = smp->stop; q.done = nullptr;
+            note_status(lg_event_create(&q.done), "lg_event_create");
+            q.cpu_time = smp->time_cpu_elapsed();
+            q.arrive = smp->sample_arrive;
+            sub_profile_misses += smp->sub_profile_misses;
+            _dec_seqs.push_back(q);
+            exe_vec.erase(exe_vec.begin() + i);
+            delete smp;
+        }
+    }
+
+    // Builds the launch vector of the next batched step(s): [join] step [retire] step [retire] ...
+    //   join:   every request that has finished its prefill since the last vector waits (on the device) for its last prefill
+    //           kernel and copies the hidden state of its last token into its row of the batch;
+    //   step:   one decode step over rows 0 .. highest row in use (rows of no request point at the spare cache slot);
+    //   retire: requests that have run their last step copy their row out and record their completion event.
+    void _build_decode_vector() {
+        const int H = BertParams.head_num * BertParams.size_per_head;
+        const size_t row_bytes = (size_t)H * sizeof(T);
+        const int kd = _model->kernels_per_layer(true);
+        const int spare_slot = _pool_total * _ctx_batch;
+        bool waiting = queued() > 0;
+        for (Sample* smp : exe_vec) waiting = waiting || smp != _dec_sample;
+        int steps = 1;
+        if (!waiting) {
+            steps = 0;
+            for (const DecodeSeq& q : _dec_seqs) steps = std::max(steps, q.remaining);
+            steps = std::max(1, std::min(steps, decode_steps_ahead));
+        }
+        std::vector<FuncWrap> vec;
+        // join
+        {
+            std::vector<DecodeSeq*> joiners;
+            for (DecodeSeq& q : _dec_seqs)
+                if (!q.joined) { joiners.push_back(&q); q.joined = true; }
+            if (!joiners.empty()) {
+                struct Join { void* done; const char* src; char* dst; int batch, seq_len; };
+                std::vector<Join> js;
+                for (DecodeSeq* q : joiners)
+                    js.push_back({q->prefill_done, (const char*)q->ctx->output, (char*)_dec_x + (size_t)q->ctx->slot * row_bytes, q->batch, q->seq_len});
+                FuncWrap f(0.005f, COMPUTATION, [js, row_bytes](const DynamicInitParam& D) {
+                    for (const Join& j : js) {
+                        note_status(lg_stream_wait_event(D.stream, j.done), "lg_stream_wait_event");
+                        for (int b = 0; b < j.batch; ++b)
+                            note_status(lg_memcpy_d2d_async(j.dst + (size_t)b * row_bytes, j.src + ((size_t)(b + 1) * j.seq_len - 1) * row_bytes,
+                                                            row_bytes, D.stream), "lg_memcpy_d2d_async");
+                    }
+                }, "join_decode_batch");
+                f.minor = true; f.name = 900; f.duration = 0.005f;
+                vec.push_back(f);
+            }
+        }
+        std::unique_lock<std::mutex> build_lock(_build_mutex);
+        for (int st = 0; st < steps; ++st) {
+            int rows = 0, longest = 0;
+            for (const DecodeSeq& q : _dec_seqs)
+                if (q.remaining > 0) { rows = std::max(rows, q.ctx->slot + q.batch); longest = std::max(longest, q.past); }
+            if (rows == 0) break;
+            std::vector<int> slots(rows, spare_slot), pasts(rows, 0);
+            for (const DecodeSeq& q : _dec_seqs)
+                if (q.remaining > 0)
+                    for (int b = 0; b < q.batch; ++b) { slots[q.ctx->slot + b] = q.ctx->slot + b; pasts[q.ctx->slot + b] = q.past; }
+            std::vector<FuncWrap> dv = _model->forward_decode_seqs(_dec_x, _dec_x, slots, pasts, _dec_ws);
+            for (size_t j = 0; j < dv.size(); ++j) {
+                dv[j].name = 1000 + (int)(j % kd);
+                dv[j].duration = lookup_decode(dv[j].name, rows, longest);
+            }
+            vec.insert(vec.end(), dv.begin(), dv.end());
+            batched_steps++;
+            batched_rows += rows;
+            // retire
+            struct Retire { void* done; const char* src; char* dst; int batch; };
+            std::vector<Retire> rs;
+            for (DecodeSeq& q : _dec_seqs) {
+                if (q.remaining <= 0) continue;
+                q.past++;
+                if (--q.remaining > 0) continue;
+                char* out = (char*)((q.n_decode & 1) ? q.ctx->dec_b : q.ctx->dec_a);   // where the request's own decode steps would leave it
+                rs.push_back({q.done, (const char*)_dec_x + (size_t)q.ctx->slot * row_bytes, out, q.batch});
+                recs.push_back(recorder{q.cpu_time, q.start, q.done, q.batch, q.seq_len, q.arrive});
+                _dec_done.push_back({q.done, q.ctx});
+                _dec_prefill_events.push_back(q.prefill_done);
+            }
+            if (!rs.empty()) {
+                FuncWrap f(0.005f, COMPUTATION, [rs, row_bytes](const DynamicInitParam& D) {
+                    for (const Retire& r : rs) {
+                        note_status(lg_memcpy_d2d_async(r.dst, r.src, (size_t)r.batch * row_bytes, D.stream), "lg_memcpy_d2d_async");
+                        note_status(lg_event_record(r.done, D.stream), "lg_event_record");
+                    }
+                }, "retire_from_decode_batch");
+                f.minor = true; f.name = 901; f.duration = 0.005f;
+                vec.push_back(f);
+            }
+            _dec_seqs.erase(std::remove_if(_dec_seqs.begin(), _dec_seqs.end(), [](const DecodeSeq& q) { return q.remaining <= 0; }), _dec_seqs.end());
+        }
+        build_lock.unlock();
+        if (vec.empty()) return;
+        _dec_sample = new Sample(vec, profiling_decompse_res_dict, 1, 1, 1, policy, axis);
+        _dec_sample->merge_minor = true;   // join / retire entries never end a run
+        _dec_sample->id = -1;
+        exe_vec.push_back(_dec_sample);
+    }
+
+    void _update_decode_batch() {
+        _collect_prefilled();
+        if (_dec_sample && _dec_sample->empty()) {
+            exe_vec.erase(std::find(exe_vec.begin(), exe_vec.end(), _dec_sample));
+            lg_event_destroy(_dec_sample->start);
+            lg_event_destroy(_dec_sample->stop);
+            delete _dec_sample;
+            _dec_sample = nullptr;
+        }
+        if (!_dec_sample && !_dec_seqs.empty()) _build_decode_vector();
+        // contexts of requests whose last decode kernel has finished go back to the pool
+        for (size_t i = 0; i < _dec_done.size();) {
+            if (lg_event_query(_dec_done[i].first) == LG_OK) {
+                release_ctx(_dec_done[i].second);
+                _dec_done.erase(_dec_done.begin() + i);
+            } else {
+                ++i;
+            }
+        }
+    }
+    std::vector<void*> _dec_prefill_events;  // destroyed with the run's records
+
     std::atomic<bool> _running{false};
     int _ctx_batch = 0;
     struct RunningGuard {
@@ -824,6 +1030,8 @@ class Scheduler {
             for (int cls = 0; cls < 2; ++cls)
                 if (_part[role][cls]) note_status(lg_stream_synchronize(_part[role][cls]->stream), "lg_stream_synchronize");
         _reclaim();
+        for (auto& d : _dec_done) release_ctx(d.second);   // every stream has been synchronised: their kernels are done
+        _dec_done.clear();
         if (_thread.joinable()) _thread.join();
     }
 };

@@ -158,13 +158,13 @@ def bench_cfg4(capi, host, weight_layout, factors=(1, 2, 4, 8), shares=(0, 64, 9
             "results": out}
 
 
-def bench_cfg5(capi, host, weight_layout, n_requests, rates=(4.0, 8.0, 16.0), shares=(64, 128), runs=1):
+def bench_cfg5(capi, host, weight_layout, n_requests, rates=(4.0, 8.0, 16.0), shares=(64, 128), runs=1, decode_steps_ahead=2):
     """BASELINE config 5: Poisson arrivals at 4, 8, 16 req/s through 4 stacked layer shards; prompts U[128, 1024]
     (rounded to 64), 32 decode tokens each; mean and p99 request latency with interleaving on and off.  `runs` > 1 repeats
     every (rate, mode) and reports the mean and the spread of the mean latency over the runs."""
     c = CFG2
     pool = 16
-    model = host.Model(capi.F16, pool, 1024, c["heads_global"], c["d"], layer_num=4, world_size=c["world_size"], ffn_inner=c["ffn_global"],
+    model = host.Model(capi.F16, pool + 1, 1024, c["heads_global"], c["d"], layer_num=4, world_size=c["world_size"], ffn_inner=c["ffn_global"],
                        causal=True, fused=True, max_cache_len=1024 + 64, weight_layout=weight_layout, factor=8, seed=0)
     sched = host.Scheduler(model, schedule_deep=6, contention_factor=0.8, policy=host.POLICY_RESOURCE, axis=host.SPLIT_TOKEN_ROWS,
                            seq_bucket=64, ignore_num=5, pool_count=pool, ctx_batch=1)
@@ -172,6 +172,10 @@ def bench_cfg5(capi, host, weight_layout, n_requests, rates=(4.0, 8.0, 16.0), sh
     sched.profile(1, 128, 1024, 64, 5)
     for past in range(128, 1024 + 64 + 1, 64):
         sched.profile_decode(1, min(past, 1024 + 63), 5)
+    # batched decode steps: a few batch sizes on a coarser grid of cached positions (looked up at or below the batch)
+    for bs in (2, 3, 4, 6, 8, 12, 16):
+        for past in range(128, 1024 + 64 + 1, 64):
+            sched.profile_decode(bs, min(past, 1024 + 63), 3)
     prof_s = time.perf_counter() - t0
     # measured contention: the MFMA-bound kernels of a 512-token prefill next to batch-1 decode steps at 512 cached positions
     meas = sched.profile_contention(1, 512, 1, 512)
@@ -184,20 +188,27 @@ def bench_cfg5(capi, host, weight_layout, n_requests, rates=(4.0, 8.0, 16.0), sh
         part_meas[share] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in pm.items()}
         part_factor[share] = (sched.partition_factor(0, 1), sched.partition_factor(1, 0))
     sched.enable_partition(0)
-    modes = [(host.MODE_SEQUENTIAL, "scheduling_off", False, False, 0), (host.MODE_LIGER, "scheduling_on", False, False, 0),
-             (host.MODE_LIGER, "scheduling_on_measured_contention", True, False, 0),
-             (host.MODE_LIGER, "scheduling_on_minor_kernels_merged", False, True, 0)]
+    # (mode, name, measured contention, minor kernels merged, HBM-side compute units of partitioned rounds, batched decode)
+    modes = [(host.MODE_SEQUENTIAL, "scheduling_off", False, False, 0, False), (host.MODE_LIGER, "scheduling_on", False, False, 0, False),
+             (host.MODE_LIGER, "scheduling_on_measured_contention", True, False, 0, False),
+             (host.MODE_LIGER, "scheduling_on_minor_kernels_merged", False, True, 0, False)]
     for share in shares:
         if part_factor[share][0] > 0:
-            modes.append((host.MODE_LIGER, "scheduling_on_partitioned_%d_hbm_cus" % share, False, True, share))
+            modes.append((host.MODE_LIGER, "scheduling_on_partitioned_%d_hbm_cus" % share, False, True, share, False))
+    modes.append((host.MODE_SEQUENTIAL, "batched_decode_without_interleaving", False, True, 0, True))
+    modes.append((host.MODE_LIGER, "scheduling_on_batched_decode", False, True, 0, True))
+    for share in shares:
+        if part_factor[share][0] > 0:
+            modes.append((host.MODE_LIGER, "scheduling_on_batched_decode_partitioned_%d_hbm_cus" % share, False, True, share, True))
     out = []
     for lam in rates:
         trace = host.make_poisson_trace(lam, n_requests, 1, 128, 1024, 64, 32, 0)
         row = {"lambda_req_s": lam, "requests": n_requests}
-        for mode, name, measured, merge_minor, share in modes:
+        for mode, name, measured, merge_minor, share, batched in modes:
             sched.set_contention(0, 1, table["mfma_main_hbm_sub"] if measured else -1.0)
             sched.set_contention(1, 0, table["hbm_main_mfma_sub"] if measured else -1.0)
             sched.set_merge_minor(merge_minor)
+            sched.enable_batch_decode(batched, decode_steps_ahead)
             sched.enable_partition(share)
             if share:
                 sched.set_partition_factor(0, 1, part_factor[share][0])
@@ -213,9 +224,11 @@ def bench_cfg5(capi, host, weight_layout, n_requests, rates=(4.0, 8.0, 16.0), sh
                          "mean_gpu_ms": round(r["avg_gpu_ms"], 3), "mean_queue_ms": round(r["avg_queue_ms"], 3),
                          "throughput_req_s": round(r["throughput"], 3), "records": r["records"],
                          "secondary_launches": r["secondary_launches"], "splits": r["splits"], "profile_misses": r["profile_misses"],
-                         "partition_rounds": r["partition_rounds"]}
+                         "partition_rounds": r["partition_rounds"], "batched_steps": r["batched_steps"],
+                         "rows_per_batched_step": round(r["batched_rows"] / r["batched_steps"], 2) if r["batched_steps"] else None}
         out.append(row)
     sched.enable_partition(0)
+    sched.enable_batch_decode(False)
     return {"workload": "cfg5: 4 layer shards, Poisson arrivals, prompts U[128,1024] rounded to 64, 32 decode tokens", "profile_seconds": round(prof_s, 1),
             "streams_verified_concurrent": sched.streams_concurrent,
             "contention_measurement": {k: (round(v, 4) if isinstance(v, float) else v) for k, v in meas.items()},

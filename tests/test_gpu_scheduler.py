@@ -73,6 +73,61 @@ def test_prefill_plus_decode_trace_on_gpu(dev, host):
         assert r["avg_latency_ms"] > 0 and r["p99_latency_ms"] >= r["avg_latency_ms"] * 0.5
 
 
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("partition", [0, 128])
+def test_batched_decode_equals_every_request_on_its_own(dev, host, mode, partition):
+    """Requests of different prompt lengths and decode lengths, all in flight at once: with batched decode steps (and the
+    prefills interleaved into them, optionally on a CU partition) every request must end with the hidden state it gets when it
+    runs alone, step by step, on the same model.  A step over several rows may take another weight-streaming kernel than a step
+    over one row, so values may differ by the rounding of the fp32 summation order, never by more."""
+    if mode == 0 and partition:
+        pytest.skip("partitioned rounds belong to the interleaving scheduler")
+    heads, d, F, layers, pool = 8, 128, 2048, 2, 6
+    H = heads * d
+    m = host.Model(1, pool + 1, 128, heads, d, layer_num=layers, ffn_inner=F, causal=True, fused=True, max_cache_len=192, factor=4,
+                   weight_layout=1, seed=5)
+    s = host.Scheduler(m, policy=host.POLICY_RESOURCE, axis=host.SPLIT_TOKEN_ROWS, seq_bucket=32, ignore_num=0, pool_count=pool, ctx_batch=1)
+    s.profile(1, 32, 128, 32, 3)
+    for bs in (1, 2, 4, 6):
+        for past in (32, 64, 96, 128, 160):
+            s.profile_decode(bs, past, 3)
+    s.set_merge_minor(True)
+    s.enable_batch_decode(True, 2)
+    if partition:
+        s.enable_partition(partition)
+        s.set_partition_factor(0, 1, 1.0)     # every co-running round is partitioned, whatever a measurement would say
+        s.set_partition_factor(1, 0, 1.0)
+    reqs = [(1, 96, 7), (1, 33, 12), (1, 128, 3), (1, 64, 9), (1, 50, 1), (1, 120, 10)]
+    for r in reqs:
+        s.serve(*r)
+    rep = s.run_queued(host.MODE_LIGER if mode else host.MODE_SEQUENTIAL)
+    torch.cuda.synchronize()
+    assert rep["records"] == len(reqs) and rep["profile_misses"] == 0
+    assert rep["batched_steps"] < sum(n for _, _, n in reqs)
+    if partition and mode:
+        assert rep["partition_rounds"] > 0
+    for i, (_, S, n) in enumerate(reqs):
+        pin, pout = s.ctx_ptrs(i)
+        da, db = s.ctx_decode_ptrs(i)
+        got = torch.empty(H, device="cuda", dtype=torch.float16)
+        dev.capi.call("lg_memcpy_d2d_async", got.data_ptr(), db if n % 2 else da, H * 2, None)
+        # the request alone: prefill into its context's cache slot, then n single steps
+        y = torch.empty(S, H, device="cuda", dtype=torch.float16)
+        torch.cuda.synchronize()
+        m.run(pin, y.data_ptr(), 1, S, None, None, cache_slot=i)     # on the model's own stream
+        torch.cuda.synchronize()
+        a = y[S - 1:S].clone()
+        b = torch.empty_like(a)
+        torch.cuda.synchronize()
+        for t in range(n):
+            m.run_decode(a.data_ptr(), b.data_ptr(), 1, S + t, i, None, None)
+            a, b = b, a
+        torch.cuda.synchronize()
+        ref = a[0].float()
+        err = float((got.float() - ref).abs().max() / ref.abs().max())
+        assert err < 1e-2, "request %d (prompt %d, %d steps): max rel err %g" % (i, S, n, err)
+
+
 def test_measured_contention_on_gpu(dev, host):
     """The contention measurement runs on the device, yields a fraction in [0.05, 1] consistent with its three times, and
     a trace scheduled with the measured table completes like one scheduled with the constant."""

@@ -570,3 +570,57 @@ def test_measured_partition_follows_the_backend_model(fake, matrix_exp, memory_e
         assert s.partition_factor(MFMA, HBM) == pytest.approx(r["factor"]) and s.partition_factor(HBM, MFMA) == pytest.approx(1 / r["factor"])
     else:
         assert r["gain"] < 1.02 and s.partition_factor(MFMA, HBM) < 0 and s.partition_factor(HBM, MFMA) < 0
+
+
+@pytest.mark.parametrize("mode_name", ["liger", "sequential"])
+def test_batched_decode_steps_share_one_launch_vector(fake, mode_name):
+    """Requests that are in their decode steps at the same time run one step together (per-sequence cache slots and lengths),
+    a request joins at the first step boundary after its prefill and leaves after its last step.  Invariants: every request
+    runs exactly its number of decode steps; fewer batched steps are launched than the requests have steps in total; a
+    request's row is copied in after its last prefill kernel and copied out after its last step; rows that belong to no
+    request point at the spare cache slot."""
+    host = fake.host
+    pool = 3
+    m = host.Model(1, pool + 1, 64, 4, 64, layer_num=2, ffn_inner=512, causal=True, fused=True, max_cache_len=128, factor=4, seed=0)
+    s = host.Scheduler(m, contention_factor=0.8, policy=host.POLICY_RESOURCE, seq_bucket=16, pool_count=pool, ctx_batch=1)
+    s.profile(1, 32, 64, 16, 2)
+    for bs in (1, 2, 3):
+        for past in (32, 48, 64, 80):
+            s.profile_decode(bs, past, 2)
+    s.set_merge_minor(True)
+    s.enable_batch_decode(True, 2)
+    reqs = [(1, 48, 5), (1, 64, 3), (1, 32, 6)]
+    fake.reset()
+    for r in reqs:
+        s.serve(*r)
+    rep = s.run_queued(host.MODE_LIGER if mode_name == "liger" else host.MODE_SEQUENTIAL)
+    t = fake.trace()
+    assert rep["records"] == 3 and rep["profile_misses"] == 0
+    steps = [e for e in t if e["name"] == "attn_decode_varlen"]
+    layers = 2
+    assert len(steps) == rep["batched_steps"] * layers
+    total_steps = sum(n for _, _, n in reqs)
+    assert max(n for _, _, n in reqs) <= rep["batched_steps"] < total_steps          # some steps were shared
+    # keys attended per step = sum over the live sequences of (cached + 1); a row of no request attends to 1 key of the spare slot.
+    # Summed over all steps of one layer: every request contributes sum_{t < n} (seq + t + 1); the rest are holes (1 key each)
+    keys = sum(e["n"] for e in steps[::layers])
+    rows = sum(e["m"] // 4 for e in steps[::layers])          # 4 heads
+    own = sum(sum(seq + t + 1 for t in range(n)) for _, seq, n in reqs)
+    holes = rows - total_steps
+    assert rows == rep["batched_rows"] and holes >= 0 and keys == own + holes
+    copies = [e for e in t if e["name"] == "memcpy_d2d"]
+    assert len(copies) == 2 * len(reqs)                        # one row in, one row out per request
+    # a request's row is copied into the batch only after its last prefill kernel: the three prefills end with a LayerNorm over
+    # 48, 64 and 32 token rows; the copy-in of the context with the matching output buffer starts after it
+    for i, (_, seq, _) in enumerate(reqs):
+        pin, pout = s.ctx_ptrs(i)
+        last_ln = [e for e in t if e["name"] == "layer_norm" and e["m"] == seq][-1]
+        assert last_ln["C"] == pout
+        row_bytes = 256 * 2
+        join = [e for e in copies if e["A"] == pout + (seq - 1) * row_bytes]
+        assert len(join) == 1 and join[0]["start"] >= last_ln["end"] - 1e-12
+    # no batched decode without the spare cache slot
+    m2 = host.Model(1, pool, 64, 4, 64, layer_num=1, ffn_inner=512, causal=True, fused=True, max_cache_len=128, seed=0)
+    s2 = host.Scheduler(m2, pool_count=pool, ctx_batch=1)
+    with pytest.raises(host.capi.LigerError):
+        s2.enable_batch_decode(True)
