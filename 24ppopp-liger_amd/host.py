@@ -41,6 +41,7 @@ SIGNATURES = {
     "lgh_model_stream": (_p, [_p]),
     "lgh_model_param_count": (_i, [_p]),
     "lgh_model_param_info": (_i, [_p, _i, C.c_char_p, _i, C.POINTER(_p), C.POINTER(_i64), C.POINTER(_i), C.POINTER(_i), C.POINTER(_i)]),
+    "lgh_model_kv_cache": (_i, [_p, _i, C.POINTER(_p), C.POINTER(_p)]),
     "lgh_model_describe": (_i, [_p, _i, _i, _i, C.c_char_p, _i]),
     "lgh_model_run": (_i, [_p, _p, _p, _i, _i, _p, _p, _i]),
     "lgh_model_run_decode": (_i, [_p, _p, _p, _i, _i, _i, _p, _p]),
@@ -54,6 +55,7 @@ SIGNATURES = {
     "lgh_sched_set_contention": (_i, [_p, _i, _i, _f]),
     "lgh_sched_enable_partition": (_i, [_p, _i]),
     "lgh_sched_enable_batch_decode": (_i, [_p, _i, _i]),
+    "lgh_sched_set_recycle_contexts": (_i, [_p, _i]),
     "lgh_sched_ctx_decode_ptrs": (_i, [_p, _i, C.POINTER(_p), C.POINTER(_p)]),
     "lgh_sched_profile_partition": (_i, [_p, _i, _i, _i, _i, C.POINTER(_f)]),
     "lgh_sched_set_partition_factor": (_i, [_p, _i, _i, _f]),
@@ -186,6 +188,31 @@ class Model:
             res[name] = a
         return res
 
+    def upload_params(self, values):
+        """Overwrites parameters with host values: name -> array in the logical orientation download_params returns
+        (weight matrices [in, out] whatever their storage layout, vectors flat)."""
+        info = self.param_info()
+        dt = np.float16 if self.dtype == capi.F16 else np.float32
+        for name, a in values.items():
+            if name not in info:
+                raise KeyError("no parameter named %r" % name)
+            i = info[name]
+            a = np.asarray(a, dtype=np.float32)
+            if i["rows"] > 1:
+                if a.shape != (i["rows"], i["cols"]):
+                    raise ValueError("%s: expected shape %s, got %s" % (name, (i["rows"], i["cols"]), a.shape))
+                a = a.T if i["transposed"] else a
+            raw = np.ascontiguousarray(a, dtype=dt).ravel()
+            if raw.size != i["elems"]:
+                raise ValueError("%s: expected %d elements, got %d" % (name, i["elems"], raw.size))
+            capi.check(capi.lib.lg_memcpy_h2d(_p(i["ptr"]), raw.ctypes.data_as(_p), raw.size * self.es), "lg_memcpy_h2d")
+
+    def kv_cache(self, layer=0):
+        """(k_cache, v_cache) device pointers of one layer: [max_batch, local heads, max_cache_len, size_per_head]."""
+        k, v = _p(), _p()
+        check(lib.lgh_model_kv_cache(self.h, layer, C.byref(k), C.byref(v)), "lgh_model_kv_cache")
+        return k.value, v.value
+
     def describe(self, batch, seq, decode_past=-1):
         buf = C.create_string_buffer(1 << 16)
         n = lib.lgh_model_describe(self.h, batch, seq, decode_past, buf, 1 << 16)
@@ -241,6 +268,10 @@ class Scheduler:
     def enable_batch_decode(self, on=True, steps_ahead=0):
         """Requests that are in their decode steps at the same time share one launch vector per step."""
         check(lib.lgh_sched_enable_batch_decode(self.h, int(bool(on)), steps_ahead), "lgh_sched_enable_batch_decode")
+
+    def set_recycle_contexts(self, on):
+        """False: finished requests keep their context (and results) until the next run starts."""
+        check(lib.lgh_sched_set_recycle_contexts(self.h, int(bool(on))), "lgh_sched_set_recycle_contexts")
 
     def ctx_decode_ptrs(self, i):
         a, b = _p(), _p()

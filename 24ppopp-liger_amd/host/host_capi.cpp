@@ -35,6 +35,7 @@ struct SchedBase {
     virtual void extra_counters(int* out2) = 0;
     virtual bool enable_batch_decode(bool on, int steps_ahead) = 0;
     virtual void batch_counters(int* out2) = 0;
+    virtual void set_recycle(bool on) = 0;
     virtual bool ctx_decode_ptrs(int i, void** a, void** b) = 0;
     virtual void set_factor(int factor) = 0;
     virtual bool ctx_ptrs(int i, void** in, void** out) = 0;
@@ -56,6 +57,7 @@ struct ModelBase {
     virtual int kernels_per_layer(bool decode) = 0;
     virtual std::vector<ParamRef> params() = 0;
     virtual size_t elem_size() = 0;
+    virtual bool kv_cache(int layer, void** k, void** v) = 0;
     BertInitParam P;
     StaticInitParam S;
     void* default_ws = nullptr;
@@ -138,6 +140,7 @@ struct SchedT : SchedBase {
         return s->enable_batch_decode(on);
     }
     void batch_counters(int* out2) override { out2[0] = s->batched_steps; out2[1] = s->batched_rows; }
+    void set_recycle(bool on) override { s->recycle_contexts = on; }
     bool ctx_decode_ptrs(int i, void** a, void** b) override {
         auto* c = s->context(i);
         if (!c) return false;
@@ -204,6 +207,12 @@ struct ModelT : ModelBase {
     int kernels_per_layer(bool decode) override { return m->kernels_per_layer(decode); }
     std::vector<ParamRef> params() override { return m->params(); }
     size_t elem_size() override { return sizeof(T); }
+    bool kv_cache(int layer, void** k, void** v) override {
+        if (layer < 0 || layer >= (int)m->encoders.size() || !m->encoders[layer]->MHA->k_cache) return false;
+        *k = m->encoders[layer]->MHA->k_cache;
+        *v = m->encoders[layer]->MHA->v_cache;
+        return true;
+    }
 };
 
 int fail(const char* msg) {
@@ -316,6 +325,13 @@ int lgh_model_param_info(void* model, int idx, char* name, int name_len, void** 
     if (rows) *rows = ps[idx].rows;
     if (cols) *cols = ps[idx].cols;
     if (transposed) *transposed = ps[idx].transposed;
+    return LG_OK;
+}
+
+// Device pointers of layer `layer`'s KV cache [max_batch, local heads, max_cache_len, size_per_head] (K and V), for callers that
+// manage cache contents themselves (loading a saved cache, tests).
+int lgh_model_kv_cache(void* model, int layer, void** k_cache, void** v_cache) {
+    if (!model || !k_cache || !v_cache || !((ModelBase*)model)->kv_cache(layer, k_cache, v_cache)) return fail("lgh_model_kv_cache: no such layer or no KV cache");
     return LG_OK;
 }
 
@@ -468,6 +484,13 @@ float lgh_sched_get_partition_factor(void* sched, int main_class, int sub_class)
 int lgh_sched_enable_batch_decode(void* sched, int on, int steps_ahead) {
     if (!sched || !((SchedBase*)sched)->enable_batch_decode(on != 0, steps_ahead))
         return fail("lgh_sched_enable_batch_decode: needs per-request contexts, a KV cache and max_batch >= pool_count * ctx_batch + 1");
+    return LG_OK;
+}
+// on = 0: a finished request's context stays out of the pool until the next run, so that a run of no more requests than
+// contexts leaves every request's results in a context of its own (requests take the free context with the lowest index)
+int lgh_sched_set_recycle_contexts(void* sched, int on) {
+    if (!sched) return fail("lgh_sched_set_recycle_contexts: null");
+    ((SchedBase*)sched)->set_recycle(on != 0);
     return LG_OK;
 }
 // the decode ping-pong buffers [ctx_batch, hidden] of the i-th context: after n decode steps a request's last hidden state is in

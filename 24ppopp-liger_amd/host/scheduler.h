@@ -232,6 +232,8 @@ class Scheduler {
             c->ws = dev_alloc<T>(we);
             c->dec_a = dev_alloc<T>((int64_t)ctx_batch * H);
             c->dec_b = dev_alloc<T>((int64_t)ctx_batch * H);
+            dev_fill_normal(c->dec_a, (int64_t)ctx_batch * H, 1234, 60000 + _pool_total, 0.f, 1.f);  // input of a decode-only request
+            dev_fill_const(c->dec_b, (int64_t)ctx_batch * H, 0.f);
             c->slot = _pool_total * ctx_batch;
             dev_fill_normal(c->input, io, 1234, 50000 + _pool_total, 0.f, 1.f);
             _pool.push_back(c);
@@ -295,7 +297,11 @@ class Scheduler {
         _pool.erase(_pool.begin() + pick);
         return c;
     }
+    // recycle_contexts = false keeps a finished request's context (and with it its results) out of the pool until the next
+    // run starts: a run of no more requests than contexts then leaves every request's output in a context of its own
+    bool recycle_contexts = true;
     void release_ctx(ReqCtx* c) {
+        if (!recycle_contexts) { _held.push_back(c); return; }
         { std::lock_guard<std::mutex> lk(_pool_mutex); _pool.push_back(c); }
         _pool_cv.notify_one();
     }
@@ -749,6 +755,11 @@ class Scheduler {
     void run_stop() { _stop.store(true); }
     void reset_run() {
         _stop.store(false);
+        if (!_held.empty()) {
+            { std::lock_guard<std::mutex> lk(_pool_mutex); for (ReqCtx* c : _held) _pool.push_back(c); }
+            _held.clear();
+            _pool_cv.notify_all();
+        }
         // epoch of the run: an event whose host time is known (the stream is idle, so it completes as it is recorded)
         if (!_epoch_event) note_status(lg_event_create(&_epoch_event), "lg_event_create");
         note_status(lg_stream_synchronize(DParams0.stream), "lg_stream_synchronize");
@@ -991,6 +1002,7 @@ class Scheduler {
     std::vector<void*> _dec_prefill_events;  // destroyed with the run's records
 
     std::atomic<bool> _running{false};
+    std::vector<ReqCtx*> _held;   // contexts of finished requests kept back while recycle_contexts is off
     int _ctx_batch = 0;
     struct RunningGuard {
         Scheduler* s;

@@ -24,7 +24,9 @@ class Dev:
         """numpy float32 array -> device tensor of dtype ('f32' | 'f16')."""
         t = torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32))
         t = t.to(self.device)
-        return t.half() if dtype in ("f16", 1) else t
+        t = t.half() if dtype in ("f16", 1) else t
+        torch.cuda.synchronize()   # callers may launch on another stream than torch's
+        return t
 
     def empty(self, shape, dtype):
         return torch.empty(shape, device=self.device, dtype=torch.float16 if dtype in ("f16", 1) else torch.float32)

@@ -139,3 +139,37 @@ def test_full_size_decode_step_against_oracle(dev, po, host, batch):
         ref = po.decoder_step(shape, w, tok, kc, vc, S + step)   # also appends this step's K/V rows to kc / vc
         assert max_rel_err(dev.down(dt_out), ref) < 1e-2
         tok = po.round_f16(ref)
+
+
+def test_cfg3_full_decode_step_against_oracle(dev, po, host):
+    """BASELINE config 3 as a whole: batch 32, one new token per sequence, 1024 cached positions with K/V ~ N(0, 1), on the
+    full layer shard.  The cache contents are written into the model's KV cache from the host, so the oracle's decoder step
+    sees the same numbers; the 32-row Q/K/V, output and FFN GEMMs take the weight-streaming kernel at K = 12288 / 6144 /
+    16384, the grouped Q/K/V launch appends row 1024, the attention reads 1025 positions."""
+    Bd, h, L, Lmax = 32, 48, 1024, 1032
+    m = host.Model(1, Bd, 8, 96, D, layer_num=1, world_size=2, ffn_inner=2 * F, norm_mode=0, causal=True, fused=True,
+                   max_cache_len=Lmax, weight_layout=1, seed=2)
+    w = {k[len("layer0."):]: v for k, v in m.download_params().items() if k.startswith("layer0.")}
+    kc = np.zeros((Bd, h, Lmax, D), dtype=np.float32)
+    vc = np.zeros_like(kc)
+    kc[:, :, :L] = po.fill_normal(Bd * h * L * D, 2, 51, 0.0, 1.0, 1).reshape(Bd, h, L, D)
+    vc[:, :, :L] = po.fill_normal(Bd * h * L * D, 2, 52, 0.0, 1.0, 1).reshape(Bd, h, L, D)
+    pk, pv = m.kv_cache(0)
+    for ptr, a in ((pk, kc), (pv, vc)):
+        t = dev.up(a, 1)
+        dev.capi.call("lg_memcpy_d2d_async", ptr, t.data_ptr(), t.numel() * 2, None)
+        torch.cuda.synchronize()
+        del t
+    tok = po.fill_normal(Bd * H, 2, 100, 0.0, 1.0, 1).reshape(Bd, H)
+    dt_in, dt_out = dev.up(tok, 1), dev.empty((Bd, H), 1)
+    m.run_decode(dt_in.data_ptr(), dt_out.data_ptr(), Bd, L, 0, None, dev.stream)
+    got = dev.down(dt_out)
+    shape = dict(batch=Bd, seq=L, hidden=H, head_num=h, size_per_head=D, ffn_inner=F, causal=1, norm_mode=0, dtype=1)
+    ref = po.decoder_step(shape, w, tok, kc, vc, L)
+    assert max_rel_err(got, ref) < 1e-2
+    # the step appended its K and V rows at position 1024 of every sequence (the oracle did the same to its arrays)
+    back = torch.empty(Bd, h, Lmax, D, device="cuda", dtype=torch.float16)
+    dev.capi.call("lg_memcpy_d2d_async", back.data_ptr(), pk, back.numel() * 2, None)
+    torch.cuda.synchronize()
+    assert max_rel_err(back[:, :, L].float().cpu().numpy(), kc[:, :, L]) < 4e-3
+    assert torch.equal(back[:, :, :L].cpu(), torch.from_numpy(kc[:, :, :L]).half())

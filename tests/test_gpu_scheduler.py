@@ -128,6 +128,113 @@ def test_batched_decode_equals_every_request_on_its_own(dev, host, mode, partiti
         assert err < 1e-2, "request %d (prompt %d, %d steps): max rel err %g" % (i, S, n, err)
 
 
+CFG = dict(hidden=12288, heads_global=96, d=128, ffn_global=32768, world_size=2)   # GLM-130B, one TP=2 shard
+
+
+def _read(dev, ptr, elems):
+    t = torch.empty(elems, device="cuda", dtype=torch.float16)
+    dev.capi.call("lg_memcpy_d2d_async", t.data_ptr(), ptr, elems * 2, None)
+    torch.cuda.synchronize()
+    return t.float()
+
+
+def test_cfg4_decomposition_sweep_at_its_real_shapes(dev, host):
+    """BASELINE config 4: a prefill request of batch 4 x seq 512 on the TP=2 layer shard, decomposed by 1, 2, 4 and 8 along
+    its token rows and interleaved on two streams with a decode batch of 32 sequences at 1024 cached positions (3 steps, so
+    that the prefill does not fit the decode window whole and something has to be split).  Durations come from profiling on
+    the device.  For every factor both requests must end with the result of their sequential run: the pieces of a split
+    GEMM tile its output exactly, and the two streams are ordered.  A piece of at most 256 token rows may sum K in slices
+    where the whole GEMM does not, so values may differ by the rounding of one fp32 summation order."""
+    c = CFG
+    H = c["hidden"]
+    m = host.Model(1, 64, 512, c["heads_global"], c["d"], layer_num=1, world_size=c["world_size"], ffn_inner=c["ffn_global"], causal=True,
+                   fused=True, max_cache_len=1024 + 64, weight_layout=1, seed=0)
+    s = host.Scheduler(m, schedule_deep=6, contention_factor=0.8, policy=host.POLICY_RESOURCE, axis=host.SPLIT_TOKEN_ROWS, seq_bucket=64,
+                       ignore_num=0, pool_count=2, ctx_batch=32)
+    s.set_merge_minor(True)
+    s.profile_decode(32, 1024, 5)
+
+    tokens = _read(dev, s.ctx_decode_ptrs(0)[0], 32 * H).half()   # the decode request's input rows (its steps overwrite them)
+
+    def run(mode):
+        dev.capi.call("lg_memcpy_d2d_async", s.ctx_decode_ptrs(0)[0], tokens.data_ptr(), 32 * H * 2, None)
+        torch.cuda.synchronize()
+        s.serve_decode(32, 1000, 3)       # context 0
+        s.serve(4, 512, 0)                # context 1
+        r = s.run_queued(mode)
+        torch.cuda.synchronize()
+        assert r["records"] == 2 and r["profile_misses"] == 0
+        return r, _read(dev, s.ctx_decode_ptrs(0)[1], 32 * H), _read(dev, s.ctx_ptrs(1)[1], 4 * 512 * H)
+
+    s.profile(4, 512, 512, 1, 5)
+    _, dec_ref, pre_ref = run(host.MODE_SEQUENTIAL)
+    assert bool(torch.isfinite(dec_ref).all()) and bool(torch.isfinite(pre_ref).all())
+    for factor in (1, 2, 4, 8):
+        s.set_factor(factor)
+        s.profile(4, 512, 512, 1, 5)      # durations of the whole GEMMs and of their 1/f .. (f-1)/f pieces
+        # The decode request's three steps open one window.  Its budget is set so that the prefill's attention block fits and
+        # 0.62 of FFN-1 is left: FFN-1 does not fit whole, half of it does -- whatever this GPU's timings are today.
+        step_ms = sum(s.lookup(1000 + j, 32, 1024) for j in range(m.kernels_per_layer(decode=True)))
+        d = [s.lookup(j, 4, 512) for j in range(m.kernels_per_layer())]
+        assert [e["label"] for e in m.describe(4, 512)][6] == "ffn1+bias+gelu" and step_ms > 0 and min(d) > 0
+        s.set_contention(1, 0, (sum(d[:6]) + 0.62 * d[6]) / (3 * step_ms))
+        r, dec, pre = run(host.MODE_LIGER)
+        assert r["secondary_launches"] > 0
+        assert (r["splits"] > 0) == (factor > 1), "factor %d: %d splits" % (factor, r["splits"])
+        assert r["sub_profile_misses"] == 0
+        for name, got, ref in (("decode", dec, dec_ref), ("prefill", pre, pre_ref)):
+            err = float((got - ref).abs().max() / ref.abs().max())
+            assert err < 4e-3, "factor %d: the %s request differs from its sequential run (%g)" % (factor, name, err)
+    # the same on a CU partition (128 units for the HBM-bound side): results unchanged
+    s.enable_partition(128)
+    s.set_partition_factor(0, 1, 1.0)
+    s.set_partition_factor(1, 0, 1.0)
+    r, dec, pre = run(host.MODE_LIGER)
+    assert r["partition_rounds"] > 0
+    assert float((dec - dec_ref).abs().max() / dec_ref.abs().max()) < 4e-3 and float((pre - pre_ref).abs().max() / pre_ref.abs().max()) < 4e-3
+
+
+def test_cfg5_mixed_trace_at_its_real_shapes(dev, host):
+    """BASELINE config 5, shortened: 12 Poisson arrivals at 16 requests/s through 4 stacked TP=2 layer shards, prompts uniform
+    in [128, 1024] (rounded to 64), 32 decode tokens each, durations profiled on the device.  Every request must end with the
+    hidden state of its sequential run -- with interleaving, and with interleaving plus batched decode steps (where a step over
+    several rows may take another weight-streaming kernel than a step over one row: rounding of the fp32 summation order)."""
+    c = CFG
+    H, n = c["hidden"], 12
+    m = host.Model(1, n + 1, 1024, c["heads_global"], c["d"], layer_num=4, world_size=c["world_size"], ffn_inner=c["ffn_global"], causal=True,
+                   fused=True, max_cache_len=1024 + 64, weight_layout=1, factor=8, seed=0)
+    s = host.Scheduler(m, schedule_deep=6, contention_factor=0.8, policy=host.POLICY_RESOURCE, axis=host.SPLIT_TOKEN_ROWS, seq_bucket=64,
+                       ignore_num=0, pool_count=n, ctx_batch=1)
+    s.profile(1, 128, 1024, 64, 3)
+    for bs in (1, 2, 3, 4, 6, 8, 12):
+        for past in range(128, 1024 + 64 + 1, 64):
+            s.profile_decode(bs, min(past, 1024 + 63), 3)
+    s.set_merge_minor(True)
+    s.set_recycle_contexts(False)         # request i keeps context i: its result stays readable after the run
+    trace = host.make_poisson_trace(16.0, n, 1, 128, 1024, 64, 32, 0)
+    gaps = np.diff([0.0] + [t["arrival_s"] for t in trace])
+    assert all(128 <= t["seq"] <= 1024 and t["seq"] % 64 == 0 for t in trace) and 0.02 < gaps.mean() < 0.2
+
+    def run(mode, batched):
+        s.enable_batch_decode(batched, 2)
+        r = s.run_trace(trace, mode)
+        torch.cuda.synchronize()
+        assert r["records"] == n and r["profile_misses"] == 0
+        return r, [_read(dev, s.ctx_decode_ptrs(i)[0], H) for i in range(n)]   # 32 steps: the last state is in the first buffer
+
+    _, ref = run(host.MODE_SEQUENTIAL, False)
+    assert all(bool(torch.isfinite(x).all()) for x in ref)
+    r_on, on = run(host.MODE_LIGER, False)
+    r_b, batched = run(host.MODE_LIGER, True)
+    assert r_b["batched_steps"] > 0
+    for i in range(n):
+        e1 = float((on[i] - ref[i]).abs().max() / ref[i].abs().max())
+        e2 = float((batched[i] - ref[i]).abs().max() / ref[i].abs().max())
+        assert e1 < 4e-3, "request %d (prompt %d) differs from its sequential run with interleaving: %g" % (i, trace[i]["seq"], e1)
+        assert e2 < 1e-2, "request %d (prompt %d) differs from its sequential run with batched decode steps: %g" % (i, trace[i]["seq"], e2)
+    assert r_b["avg_e2e_ms"] > 0 and r_on["avg_e2e_ms"] > 0
+
+
 def test_measured_contention_on_gpu(dev, host):
     """The contention measurement runs on the device, yields a fraction in [0.05, 1] consistent with its three times, and
     a trace scheduled with the measured table completes like one scheduled with the constant."""

@@ -624,3 +624,49 @@ def test_batched_decode_steps_share_one_launch_vector(fake, mode_name):
     s2 = host.Scheduler(m2, pool_count=pool, ctx_batch=1)
     with pytest.raises(host.capi.LigerError):
         s2.enable_batch_decode(True)
+
+
+@pytest.mark.parametrize("factor", [2, 4, 8])
+@pytest.mark.parametrize("axis", [0, 1])
+def test_cfg4_shapes_pieces_cover_the_prefill_exactly(fake, factor, axis):
+    """BASELINE config 4 at its real shapes on the virtual-time backend, where every launch is visible: prefill batch 4 x seq
+    512 on the TP=2 GLM-130B layer shard, decomposed by `factor`, next to a decode batch of 32 sequences at 1024 cached
+    positions.  Whatever is split, the pieces of every weight GEMM of the prefill must cover its 2048 token rows (or its
+    output features) exactly once, in order, with the operand pointers offset accordingly."""
+    host = fake.host
+    m = host.Model(1, 64, 512, 96, 128, layer_num=1, world_size=2, ffn_inner=32768, causal=True, fused=True, max_cache_len=1088, factor=factor, seed=0)
+    s = host.Scheduler(m, contention_factor=0.8, policy=host.POLICY_RESOURCE, axis=axis, seq_bucket=64, pool_count=2, ctx_batch=32)
+    s.set_factor(factor)
+    s.profile(4, 512, 512, 1, 2)
+    s.profile_decode(32, 1024, 2)
+    s.set_merge_minor(True)
+    fake.reset()
+    s.serve_decode(32, 1000, 3)   # three steps: a window that holds the attention block of the prefill and part of FFN-1
+    s.serve(4, 512, 0)
+    r = s.run_queued(host.MODE_LIGER)
+    t = fake.trace()
+    assert r["records"] == 2 and r["splits"] > 0 and r["profile_misses"] == 0 and r["sub_profile_misses"] == 0
+    H, Hl, F, M = 12288, 6144, 16384, 2048
+    pin, pout = s.ctx_ptrs(1)
+    gemms = [e for e in t if e["name"] in ("gemm", "gemm_fused") and e["n"] != 32]      # the prefill's (the decode batch has 32 rows)
+    by_weight = {}
+    for e in gemms:
+        by_weight.setdefault(e["A"] if axis == 1 else None, []).append(e)
+    if axis == 1:   # token-row pieces share the weight pointer: group by it
+        assert len(by_weight) == 6
+        widths = sorted(v[0]["m"] for v in by_weight.values())
+        assert widths == sorted([Hl, Hl, Hl, H, F, H])
+        n_split = 0
+        for v in by_weight.values():
+            v.sort(key=lambda e: e["B"])
+            assert sum(e["n"] for e in v) == M
+            k = v[0]["k"]
+            for a, b in zip(v, v[1:]):
+                assert b["B"] - a["B"] == a["n"] * k * 2        # the next piece's activations start where this one's end
+            n_split += len(v) > 1
+        # the three head-transposing projections are always split by output features (token rows would move the batch decode)
+        assert n_split >= 1
+    else:           # output-feature pieces: every piece shares the activations; weights / outputs advance by whole features
+        total = sum(e["m"] * e["n"] for e in gemms)
+        assert total == M * (3 * Hl + H + F + H) and all(e["n"] == M for e in gemms)
+        assert len(gemms) > 6
