@@ -101,10 +101,10 @@ def kernel_only(args, capi, host, model, x, y, B, S, H, stream):
     print(json.dumps({"kernel": name, "iters": args.iters, "avg_ms_hip_events": round(ms, 5)}))
 
 
-def bench_cfg4(capi, host, weight_layout, factors=(1, 2, 4, 8), shares=(0, 64, 96, 128), repeats=3):
+def bench_cfg4(capi, host, weight_layout, factors=(1, 2, 4, 8), shares=(0, 64, 96, 128), repeats=3, decode_steps=8):
     """BASELINE config 4: a prefill request (batch 4 x seq 512) is decomposed by `factors` (token rows) and interleaved on two
-    streams with a decode batch (32 sequences, 1024 cached positions, 8 steps); makespan against sequential launch of the same
-    two requests.  The decode batch is the primary request (its HBM-bound kernels open the windows), the prefill's MFMA-bound
+    streams with a decode batch (32 sequences, 1024 cached positions, `decode_steps` steps: 8 steps hold the whole prefill in
+    their window, 4 do not, so that a GEMM has to be split); makespan against sequential launch of the same two requests.  The decode batch is the primary request (its HBM-bound kernels open the windows), the prefill's MFMA-bound
     GEMMs are the ones split to fit them.  `shares` = compute units given to the HBM-bound side in co-running rounds (0: both
     streams on the whole chip, as the reference runs them).  Each request has its own context (buffers, workspace, cache slots)."""
     c = CFG2
@@ -123,7 +123,7 @@ def bench_cfg4(capi, host, weight_layout, factors=(1, 2, 4, 8), shares=(0, 64, 9
         def best_of(mode):
             best = None
             for _ in range(repeats):
-                sched.serve_decode(32, 1000, 8)
+                sched.serve_decode(32, 1000, decode_steps)
                 sched.serve(4, 512, 0)
                 r = sched.run_queued(mode)
                 if best is None or r["total_duration_ms"] < best["total_duration_ms"]:
@@ -152,13 +152,13 @@ def bench_cfg4(capi, host, weight_layout, factors=(1, 2, 4, 8), shares=(0, 64, 9
         res["speedup"] = round(res["sequential"]["makespan_ms"] / res["interleaved"]["makespan_ms"], 4)
         res["speedup_minor_merged"] = round(res["sequential"]["makespan_ms"] / res["interleaved_minor_merged"]["makespan_ms"], 4)
         out.append(res)
-    return {"workload": "cfg4: prefill B4 S512 (split by token rows) || decode B32 L1024 x 8 steps, one layer shard",
+    return {"workload": "cfg4: prefill B4 S512 (split by token rows) || decode B32 L1024 x %d steps, one layer shard" % decode_steps,
             "partition_measurement": {"what": "MFMA-bound kernels of the prefill layer on 256 - n compute units || decode steps on n, "
                                               "against both back to back on the whole chip", "by_hbm_cus": partition},
             "results": out}
 
 
-def bench_cfg5(capi, host, weight_layout, n_requests, rates=(4.0, 8.0, 16.0), shares=(64, 128), runs=1, decode_steps_ahead=2):
+def bench_cfg5(capi, host, weight_layout, n_requests, rates=(4.0, 8.0, 16.0), shares=(64, 128), runs=1, decode_steps_ahead=2, short=False):
     """BASELINE config 5: Poisson arrivals at 4, 8, 16 req/s through 4 stacked layer shards; prompts U[128, 1024]
     (rounded to 64), 32 decode tokens each; mean and p99 request latency with interleaving on and off.  `runs` > 1 repeats
     every (rate, mode) and reports the mean and the spread of the mean latency over the runs."""
@@ -195,6 +195,8 @@ def bench_cfg5(capi, host, weight_layout, n_requests, rates=(4.0, 8.0, 16.0), sh
     for share in shares:
         if part_factor[share][0] > 0:
             modes.append((host.MODE_LIGER, "scheduling_on_partitioned_%d_hbm_cus" % share, False, True, share, False))
+    if short:   # off / on / on with batched decode steps (the default bench run)
+        modes = [modes[0], modes[3]]
     modes.append((host.MODE_SEQUENTIAL, "batched_decode_without_interleaving", False, True, 0, True))
     modes.append((host.MODE_LIGER, "scheduling_on_batched_decode", False, True, 0, True))
     for share in shares:
@@ -219,7 +221,7 @@ def bench_cfg5(capi, host, weight_layout, n_requests, rates=(4.0, 8.0, 16.0), sh
             # event) is kept beside it: it under-counts when a start event is held up on the device
             means = [x["avg_e2e_ms"] for x in reps]
             row[name] = {"mean_latency_ms": round(sum(means) / len(means), 3), "p99_latency_ms": round(sum(x["p99_e2e_ms"] for x in reps) / len(reps), 3),
-                         "mean_latency_runs_ms": [round(v, 3) for v in means],
+                         "mean_latency_runs_ms": [round(v, 3) for v in means], "mean_latency_spread_ms": round(max(means) - min(means), 3),
                          "mean_cpu_plus_gpu_ms": round(r["avg_latency_ms"], 3),
                          "mean_gpu_ms": round(r["avg_gpu_ms"], 3), "mean_queue_ms": round(r["avg_queue_ms"], 3),
                          "throughput_req_s": round(r["throughput"], 3), "records": r["records"],
@@ -236,6 +238,58 @@ def bench_cfg5(capi, host, weight_layout, n_requests, rates=(4.0, 8.0, 16.0), sh
             "partition_measurement": part_meas, "results": out}
 
 
+def derived_peaks(info):
+    """Roofline denominators re-derived from the device properties: matrix peak = CUs x 4096 fp16 flop per clock and CU x
+    engine clock; memory peak = bus width x memory clock x 2 transfers per clock (as the runtime reports them)."""
+    flops = info["cu_count"] * 4096 * info["clock_khz"] * 1e3 / 1e12
+    gbs = info["bus_width_bits"] / 8 * info["mem_clock_khz"] * 1e3 * 2 / 1e9
+    return {"fp16_mfma_TFLOPs": round(flops, 1), "hbm_GBps": round(gbs, 1),
+            "formula": "%d CUs x 4096 flop/clk x %.3f GHz; %d bit x %.3f GHz x 2" % (info["cu_count"], info["clock_khz"] / 1e6,
+                                                                                     info["bus_width_bits"], info["mem_clock_khz"] / 1e6)}
+
+
+def time_layer(capi, host, weight_layout, fused, steps, warmup):
+    """Times the cfg2 prefill layer shard and the cfg3 decode step in one weight layout; returns (model, x, y, results)."""
+    import torch
+    c = CFG2
+    B, S, H = c["batch"], c["seq"], c["hidden"]
+    M = B * S
+    model = host.Model(capi.F16, 32, S, c["heads_global"], c["d"], layer_num=1, world_size=c["world_size"], ffn_inner=c["ffn_global"],
+                       norm_mode=host.POST_NORESID, causal=True, fused=fused, max_cache_len=CFG3["cache_len"] + 32 if fused else 0,
+                       weight_layout=weight_layout, seed=0)
+    x = torch.empty(M, H, device="cuda", dtype=torch.float16)
+    capi.call("lg_fill_normal_f16", x.data_ptr(), x.numel(), 0, 99, 0.0, 1.0, None)
+    y = torch.empty_like(x)
+    torch.cuda.synchronize()
+    stream = model.stream
+    for _ in range(warmup):
+        model.run(x.data_ptr(), y.data_ptr(), B, S, None, stream)
+    capi.call("lg_stream_synchronize", stream)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        model.run(x.data_ptr(), y.data_ptr(), B, S, None, stream)
+    capi.call("lg_stream_synchronize", stream)
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
+    # per-kernel durations: HIP events on the launch stream, 2 warm-ups + 20 launches, min of 3 (the reference's profiler protocol)
+    desc = model.describe(B, S)
+    times = model.time_kernels(x.data_ptr(), y.data_ptr(), B, S)
+    kernels = [{"idx": e["idx"], "kernel": e["label"], "class": e["class"], "ms": round(t, 4)} for e, t in zip(desc, times)]
+    decode = None
+    if fused:
+        Bd, L = CFG3["batch"], CFG3["cache_len"]
+        xd = torch.empty(Bd, H, device="cuda", dtype=torch.float16)
+        capi.call("lg_fill_normal_f16", xd.data_ptr(), xd.numel(), 0, 98, 0.0, 1.0, None)
+        yd = torch.empty_like(xd)
+        torch.cuda.synchronize()
+        ddesc = model.describe(Bd, 1, decode_past=L - 1)
+        dtimes = model.time_kernels(xd.data_ptr(), yd.data_ptr(), Bd, 1, decode_past=L - 1, cache_slot=0)
+        decode = {"kernels": [{"idx": e["idx"], "kernel": e["label"], "ms": round(t, 4)} for e, t in zip(ddesc, dtimes)],
+                  "ms_per_layer_shard": round(sum(dtimes), 4)}
+    return model, x, y, {"ms_per_step": ms_per_step, "kernels": kernels, "sum_kernel_ms": sum(times), "decode": decode}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -243,9 +297,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--unfused", action="store_true", help="time the reference-shaped 14-entry assembly instead")
-    ap.add_argument("--cfg4", action="store_true", help="also run the decomposition sweep (BASELINE config 4)")
-    ap.add_argument("--cfg5", action="store_true", help="also run the mixed request trace (BASELINE config 5); takes minutes")
+    ap.add_argument("--no-scheduler", action="store_true", help="skip the short config-4 / config-5 scheduler records")
+    ap.add_argument("--cfg4", action="store_true", help="run the full decomposition sweep (BASELINE config 4) instead of the short record")
+    ap.add_argument("--cfg5", action="store_true", help="run the full mixed request trace (BASELINE config 5; minutes) instead of the short record")
     ap.add_argument("--cfg5-requests", type=int, default=60)
+    ap.add_argument("--cfg5-runs", type=int, default=3)
     ap.add_argument("--kernel-only", default=None,
                     help="launch only the named launch-vector entry (e.g. 'ffn1+bias+gelu', 'attn_decode', 'layer_norm') or "
                          "'copy' (a plain 128 MiB read + 128 MiB write kernel) --iters times; for rocprofv3 runs")
@@ -268,36 +324,20 @@ def main():
     B, S, H = c["batch"], c["seq"], c["hidden"]
     M = B * S
     fused = not args.unfused
-    model = host.Model(capi.F16, 32, S, c["heads_global"], c["d"], layer_num=1, world_size=c["world_size"], ffn_inner=c["ffn_global"],
-                       norm_mode=host.POST_NORESID, causal=True, fused=fused, max_cache_len=CFG3["cache_len"] + 32 if fused else 0,
-                       weight_layout=args.weight_layout, seed=0)
-    x = torch.empty(M, H, device="cuda", dtype=torch.float16)
-    capi.call("lg_fill_normal_f16", x.data_ptr(), x.numel(), 0, 99, 0.0, 1.0, None)
-    y = torch.empty_like(x)
-    stream = model.stream
 
     if args.kernel_only:
-        kernel_only(args, capi, host, model, x, y, B, S, H, stream)
+        model = host.Model(capi.F16, 32, S, c["heads_global"], c["d"], layer_num=1, world_size=c["world_size"], ffn_inner=c["ffn_global"],
+                           norm_mode=host.POST_NORESID, causal=True, fused=fused, max_cache_len=CFG3["cache_len"] + 32 if fused else 0,
+                           weight_layout=args.weight_layout, seed=0)
+        x = torch.empty(M, H, device="cuda", dtype=torch.float16)
+        capi.call("lg_fill_normal_f16", x.data_ptr(), x.numel(), 0, 99, 0.0, 1.0, None)
+        y = torch.empty_like(x)
+        torch.cuda.synchronize()
+        kernel_only(args, capi, host, model, x, y, B, S, H, model.stream)
         return
 
-    def step():
-        model.run(x.data_ptr(), y.data_ptr(), B, S, None, stream)
-
-    for _ in range(args.warmup):
-        step()
-    capi.call("lg_stream_synchronize", stream)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    capi.call("lg_stream_synchronize", stream)
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
-
-    # per-kernel durations: HIP events on the launch stream, 2 warm-ups + 20 launches, min of 3 (the reference's profiler protocol)
-    desc = model.describe(B, S)
-    times = model.time_kernels(x.data_ptr(), y.data_ptr(), B, S)
-    kernels = [{"idx": e["idx"], "kernel": e["label"], "class": e["class"], "ms": round(t, 4)} for e, t in zip(desc, times)]
+    model, x, y, res = time_layer(capi, host, args.weight_layout, fused, args.steps, args.warmup)
+    ms_per_step, kernels = res["ms_per_step"], res["kernels"]
     fl = gemm_flops_cfg2()
     label_flops = {"q_gemm": fl["q"], "k_gemm": fl["k"], "v_gemm": fl["v"], "out_proj": fl["out"], "ffn1": fl["ffn1"], "ffn2": fl["ffn2"],
                    "q_gemm+bias+heads": fl["q"], "k_gemm+bias+heads": fl["k"], "v_gemm+bias+heads": fl["v"], "ffn1+bias+gelu": fl["ffn1"]}
@@ -306,38 +346,39 @@ def main():
     for k in kernels:
         if k["kernel"] in label_flops:
             k["tflops"] = round(label_flops[k["kernel"]] / (k["ms"] * 1e-3) / 1e12, 1)
+            k["traffic"] = measured_traffic(k["kernel"])
             gemm_ms += k["ms"]
             gemm_fl += label_flops[k["kernel"]]
-    # dominant kernel = the FFN GEMM with the largest share of the step
-    dom = max((k for k in kernels if k["kernel"] in label_flops), key=lambda k: k["ms"])
+    # dominant kernel = FFN-1 (with FFN-2 the largest share of the step's flops; always the same one, so that the counter
+    # traffic on file belongs to it)
+    dom = [k for k in kernels if k["kernel"] in ("ffn1+bias+gelu", "ffn1")][0]
     dom_fl = label_flops[dom["kernel"]]
     achieved = dom_fl / (dom["ms"] * 1e-3) / 1e12
     roofline = {"bound": "mfma", "kernel": dom["kernel"], "achieved": round(achieved, 1), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / PEAK_FP16_TFLOPS, 4), "traffic": measured_traffic(dom["kernel"]),
-                "all_gemms_tflops": round(gemm_fl / (gemm_ms * 1e-3) / 1e12, 1)}
+                "all_gemms_tflops": round(gemm_fl / (gemm_ms * 1e-3) / 1e12, 1),
+                "all_gemms_frac": round(gemm_fl / (gemm_ms * 1e-3) / 1e12 / PEAK_FP16_TFLOPS, 4)}
     ln = [k for k in kernels if k["kernel"] == "layer_norm"]
     ln_gbs = (2 * M * H * 2) / (min(k["ms"] for k in ln) * 1e-3) / 1e9 if ln else None
 
     # decode step of the same shard (BASELINE config 3): batch 32, one token, 1024 cached positions
     decode = None
-    if fused:
+    if res["decode"]:
         Bd, L = CFG3["batch"], CFG3["cache_len"]
-        xd = torch.empty(Bd, H, device="cuda", dtype=torch.float16)
-        capi.call("lg_fill_normal_f16", xd.data_ptr(), xd.numel(), 0, 98, 0.0, 1.0, None)
-        yd = torch.empty_like(xd)
-        ddesc = model.describe(Bd, 1, decode_past=L - 1)
-        dtimes = model.time_kernels(xd.data_ptr(), yd.data_ptr(), Bd, 1, decode_past=L - 1, cache_slot=0)
-        dk = [{"idx": e["idx"], "kernel": e["label"], "ms": round(t, 4)} for e, t in zip(ddesc, dtimes)]
+        dk = res["decode"]["kernels"]
+        step_ms = res["decode"]["ms_per_layer_shard"]
         attn = [k for k in dk if k["kernel"] == "attn_decode"][0]
         kv_bytes = 2 * Bd * 48 * L * 128 * 2
         w_bytes = (3 * H * 6144 + 6144 * H + 2 * H * 16384) * 2
         gemm_dec_ms = sum(k["ms"] for k in dk if "gemm" in k["kernel"] or "proj" in k["kernel"] or "ffn" in k["kernel"])
-        decode = {"workload": "cfg3: batch 32, 1 new token, 1024 cached positions", "ms_per_layer_shard": round(sum(dtimes), 4),
-                  "tokens_per_s": round(Bd / (sum(dtimes) * 1e-3), 1), "kernels": dk,
+        decode = {"workload": "cfg3: batch 32, 1 new token, 1024 cached positions", "ms_per_layer_shard": step_ms,
+                  "tokens_per_s": round(Bd / (step_ms * 1e-3), 1), "kernels": dk,
+                  "hbm_floor_ms": round((w_bytes + kv_bytes) / (PEAK_HBM_GBS * 1e9) * 1e3, 4),
                   "roofline_attn_decode": {"bound": "hbm", "achieved": round(kv_bytes / (attn["ms"] * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
                                            "unit": "GB/s", "frac": round(kv_bytes / (attn["ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
                                            "traffic": measured_traffic("attn_decode")},
-                  "skinny_gemms": {"ms": round(gemm_dec_ms, 4), "weight_GBps": round(w_bytes / (gemm_dec_ms * 1e-3) / 1e9, 1)}}
+                  "skinny_gemms": {"ms": round(gemm_dec_ms, 4), "weight_GBps": round(w_bytes / (gemm_dec_ms * 1e-3) / 1e9, 1),
+                                   "frac": round(w_bytes / (gemm_dec_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}}
 
     out = {
         "metric": "ms/layer-shard prefill (GLM-130B TP=2 shard, B8 S512, causal, fp16)",
@@ -351,19 +392,41 @@ def main():
         "roofline": roofline,
         "layer_norm_GBps": round(ln_gbs, 1) if ln_gbs else None,
         "kernels": kernels,
-        "sum_kernel_ms": round(sum(times), 4),
+        "sum_kernel_ms": round(res["sum_kernel_ms"], 4),
         "decode": decode,
         "device": info,
-        "peaks": {"fp16_mfma_TFLOPs": PEAK_FP16_TFLOPS, "hbm_GBps": PEAK_HBM_GBS},
+        "peaks": {"fp16_mfma_TFLOPs": PEAK_FP16_TFLOPS, "hbm_GBps": PEAK_HBM_GBS, "source": "published MI355X figures (the roofline denominators)",
+                  "derived_from_device_properties": derived_peaks(info)},
     }
+    del model, x, y
+    torch.cuda.empty_cache()
+    # the same layer with the weights stored the other way round (0 = [in, out], the layout the reference's (N,N) cuBLAS call implies)
+    other = 1 - args.weight_layout
+    m2, x2, y2, r2 = time_layer(capi, host, other, fused, max(5, args.steps // 2), 2)
+    out["reference_layout" if other == 0 else "out_in_layout"] = {
+        "weights": "[in, out]" if other == 0 else "[out, in]", "ms_per_layer_shard_prefill": round(r2["ms_per_step"], 4),
+        "ms_per_layer_shard_decode": r2["decode"]["ms_per_layer_shard"] if r2["decode"] else None,
+        "prefill_gemm_tflops": {k["kernel"]: round(label_flops[k["kernel"]] / (k["ms"] * 1e-3) / 1e12, 1) for k in r2["kernels"] if k["kernel"] in label_flops},
+        "decode_kernels_ms": {k["kernel"]: k["ms"] for k in r2["decode"]["kernels"]} if r2["decode"] else None}
+    del m2, x2, y2
+    torch.cuda.empty_cache()
     if not args.no_cpu_baseline:
         from oracle import pyoracle as po
         out["cpu_baseline"] = cpu_baseline(po)
-    del model
-    if args.cfg4:
-        out["cfg4"] = bench_cfg4(capi, host, args.weight_layout)
-    if args.cfg5:
-        out["cfg5"] = bench_cfg5(capi, host, args.weight_layout, args.cfg5_requests)
+    if fused and not args.no_scheduler:
+        # scheduler records: the decomposition sweep against a decode batch (config 4) and the mixed trace (config 5); short
+        # versions by default so that the whole run stays within minutes, the full sweeps with --cfg4 / --cfg5
+        if args.cfg4:
+            out["cfg4"] = bench_cfg4(capi, host, args.weight_layout)
+            out["cfg4_split_forced"] = bench_cfg4(capi, host, args.weight_layout, decode_steps=4)
+        else:
+            out["cfg4"] = bench_cfg4(capi, host, args.weight_layout, factors=(1, 8), shares=(0, 128), repeats=3)
+            out["cfg4_split_forced"] = bench_cfg4(capi, host, args.weight_layout, factors=(8,), shares=(0, 128), repeats=3, decode_steps=4)
+        torch.cuda.empty_cache()
+        if args.cfg5:
+            out["cfg5"] = bench_cfg5(capi, host, args.weight_layout, args.cfg5_requests, runs=args.cfg5_runs)
+        else:
+            out["cfg5"] = bench_cfg5(capi, host, args.weight_layout, 40, rates=(16.0,), shares=(128,), runs=3, short=True)
     print(json.dumps(out))
 
 
