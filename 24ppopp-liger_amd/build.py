@@ -24,7 +24,7 @@ HIP_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument", "-Wno-option-ignored",
 ]
-HIP_SOURCES = ["runtime.hip", "elementwise.hip", "attention_aux.hip", "gemm.hip", "gemm_fast.hip", "gemm_skinny.hip", "gemv.hip", "attention.hip",
+HIP_SOURCES = ["runtime.hip", "elementwise.hip", "attention_aux.hip", "gemm.hip", "gemm_fast.hip", "gemm_skinny.hip", "gemm_skinny_kn.hip", "gemv.hip", "attention.hip",
                "attention_prefill.hip"]
 
 

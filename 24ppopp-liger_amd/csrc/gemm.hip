@@ -12,6 +12,7 @@ namespace lg {
 int launch_gemm_fast_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t stream, bool* handled);
 int launch_gemm_skinny_f16(const GemmArgs& g, const GemmGroup& grp, const RowMap* rows, int wlayout, int batch, hipStream_t stream, bool* handled);
 int launch_gemv_f16(const GemmArgs& g, const GemmGroup& grp, const RowMap* rows, int wlayout, int batch, hipStream_t stream, bool* handled);
+int launch_gemm_skinny_kn_f16(const GemmArgs& g, const RowMap* rows, int wlayout, int batch, hipStream_t stream, bool* handled);
 
 // ---------------------------------------------------------------------------------------------------
 // fp16 generic kernel
@@ -153,6 +154,8 @@ static int gemm_f16_dispatch(GemmArgs g, int wlayout, int batch, hipStream_t str
     rc = launch_gemv_f16(g, one, nullptr, wlayout, batch, stream, &handled);
     if (handled) return rc;
     rc = launch_gemm_skinny_f16(g, one, nullptr, wlayout, batch, stream, &handled);
+    if (handled) return rc;
+    rc = launch_gemm_skinny_kn_f16(g, nullptr, wlayout, batch, stream, &handled);
     if (handled) return rc;
     const bool aligned = aligned16(g.X) && aligned16(g.W) && aligned16(g.Y) && (g.ldx % 8 == 0) && (g.ldw % 8 == 0) &&
                          (g.strideX % 8 == 0) && (g.strideW % 8 == 0) && (g.strideY % 4 == 0) &&
@@ -414,6 +417,24 @@ int lg_gemm_fused_grouped_rows_f16(int transa, int m, int n, int k, int count, c
         if (handled) return rc;
         rc = launch_gemm_skinny_f16(g, grp, &rm, W_NK, 1, (hipStream_t)stream, &handled);
         if (handled) return rc;
+    }
+    if (transa == 0) {
+        // weights stored [in, out]: one launch of the LDS-transposing weight-streaming kernel per member
+        bool all = true;
+        for (int i = 0; i < count && all; ++i) {
+            GemmArgs g;
+            g.M = n; g.N = m; g.K = k;
+            g.X = (const half_t*)B; g.ldx = ldb; g.strideX = 0;
+            g.W = grp.W[i]; g.ldw = lda; g.strideW = 0;
+            g.Y = grp.Y[i]; g.ldy = grp.ldy[i]; g.strideY = 0;
+            g.epi = Epilogue{LG_EPI_BIAS_HEADS_ROWS, grp.bias[i], 1, d, heads_total, grp.rows[i]};
+            bool handled = false;
+            int rc = launch_gemm_skinny_kn_f16(g, &rm, W_KN, 1, (hipStream_t)stream, &handled);
+            if (rc) return rc;
+            all = handled;
+            if (!handled && i > 0) { set_error("gemm_fused_grouped_rows_f16: members of one group must take the same kernel"); return LG_ERR_INVALID; }
+        }
+        if (all) return LG_OK;
     }
     // anything the weight-streaming kernels do not take: plain calls, one per member -- and one per token row for a member
     // whose rows go to their own places

@@ -89,6 +89,21 @@ __device__ __forceinline__ half4_t lds_read_tr4(const half_t* p) {
     return __builtin_bit_cast(half4_t, r);
 }
 
+// ---- direct-to-LDS loads and the bank-conflict swizzles of the LDS-tiled kernels -------------------------------------------
+typedef __attribute__((address_space(3))) void lds_void_t;
+typedef __attribute__((address_space(1))) const void gbl_void_t;
+
+__device__ __forceinline__ void load_lds16(const half_t* gptr, half_t* lds_wave_base) {
+    // every lane supplies its own global address; the 64 x 16 bytes land contiguously at lds_wave_base
+    __builtin_amdgcn_global_load_lds((gbl_void_t*)gptr, (lds_void_t*)lds_wave_base, 16, 0, 0);
+}
+
+// swizzles: position (in 16-byte chunks) of logical chunk c in row r of the [rows][64] tiles; block (32 bytes) of
+// logical block b in row k of a [64][128 or 256] weight tile
+__device__ __forceinline__ int swz_a(int row, int c) { return c ^ ((row >> 1) & 7); }
+// the 32 lanes served together by one transposed read touch rows k0..k0+3 and k0+8..k0+11: eight distinct XOR values
+__device__ __forceinline__ int swz_b(int k, int blk) { return blk ^ ((k & 3) | ((k >> 1) & 4)); }
+
 // Applies the epilogue to 4 consecutive output columns n..n+3 of token row m and stores them.
 template <int EPI>
 __device__ __forceinline__ void epilogue_store4(const GemmArgs& g, half_t* Yb, int m, int n, float4_t acc, bool vec_ok,
@@ -133,6 +148,6 @@ constexpr int LG_EPI_PARTIAL = 100;  // kernel-internal: store the fp32 accumula
 // The fp32 partials live in the stream's workspace (StreamInfo::ws, allocated when the stream was created or attached); a
 // launcher never allocates: with no workspace, or one that is too small, it slices K less or not at all.
 // Y = epilogue(sum over the nsplit K-slices in slice order) of the fp32 partials [nsplit][M][N]
-void launch_splitk_reduce(const GemmArgs& g, const float* partial, int nsplit, hipStream_t stream);
+void launch_splitk_reduce(const GemmArgs& g, const float* partial, int nsplit, hipStream_t stream, const RowMap* rows = nullptr);
 
 }  // namespace lg

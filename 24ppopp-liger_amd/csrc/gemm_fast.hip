@@ -33,20 +33,6 @@ constexpr int F_THREADS = 512;
 constexpr int X_STAGES = 3, W_STAGES = 2;
 constexpr int lds_halves(int NJ) { return X_STAGES * FB_M * FB_K + W_STAGES * FB_K * 64 * NJ; }
 
-typedef __attribute__((address_space(3))) void lds_void_t;
-typedef __attribute__((address_space(1))) const void gbl_void_t;
-
-__device__ __forceinline__ void load_lds16(const half_t* gptr, half_t* lds_wave_base) {
-    // every lane supplies its own global address; the 64 x 16 bytes land contiguously at lds_wave_base
-    __builtin_amdgcn_global_load_lds((gbl_void_t*)gptr, (lds_void_t*)lds_wave_base, 16, 0, 0);
-}
-
-// swizzles: position (in 16-byte chunks) of logical chunk c in row r of the [rows][64] tiles; block (32 bytes) of
-// logical block b in row k of the [64][256] tile
-__device__ __forceinline__ int swz_a(int row, int c) { return c ^ ((row >> 1) & 7); }
-// the 32 lanes served together by one transposed read touch rows k0..k0+3 and k0+8..k0+11: eight distinct XOR values
-__device__ __forceinline__ int swz_b(int k, int blk) { return blk ^ ((k & 3) | ((k >> 1) & 4)); }
-
 template <int WL, int EPI, int NJ>
 __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles_m, int tiles_n, float* partial, int kt_per_split, int cus) {
     constexpr int FB_N = 64 * NJ;

@@ -242,7 +242,7 @@ static void launch_direct_mt(const GemmArgs& g, const GemmGroup& grp, const RowM
 
 // sums the K-slices and applies the epilogue; one thread per 4 consecutive output columns
 template <int EPI>
-__global__ __launch_bounds__(256) void gemm_skinny_reduce_kernel(GemmArgs g, const float* partial, int nsplit) {
+__global__ __launch_bounds__(256) void gemm_skinny_reduce_kernel(GemmArgs g, const float* partial, int nsplit, RowMap rm) {
     const int64_t quads = (int64_t)g.M * ((g.N + 3) / 4);
     for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < quads; q += (int64_t)gridDim.x * blockDim.x) {
         const int nq = (g.N + 3) / 4;
@@ -256,20 +256,22 @@ __global__ __launch_bounds__(256) void gemm_skinny_reduce_kernel(GemmArgs g, con
                 for (int r = 0; r < 4 && n + r < g.N; ++r) s[r] += p[r];
             }
         }
-        epilogue_store4<EPI>(g, g.Y, m, n, s, true);
+        epilogue_store4<EPI>(g, g.Y, m, n, s, true, &rm);
     }
 }
 
-void launch_splitk_reduce(const GemmArgs& g, const float* partial, int nsplit, hipStream_t stream) {
+void launch_splitk_reduce(const GemmArgs& g, const float* partial, int nsplit, hipStream_t stream, const RowMap* rows) {
     const dim3 block(256);
     const int64_t quads = (int64_t)g.M * ((g.N + 3) / 4);
     int rgrid = (int)((quads + 255) / 256);
     if (rgrid > 4096) rgrid = 4096;
+    const RowMap rm = rows ? *rows : RowMap{};
     switch (g.epi.kind) {
-        case LG_EPI_NONE: hipLaunchKernelGGL((gemm_skinny_reduce_kernel<LG_EPI_NONE>), dim3(rgrid), block, 0, stream, g, partial, nsplit); break;
-        case LG_EPI_BIAS: hipLaunchKernelGGL((gemm_skinny_reduce_kernel<LG_EPI_BIAS>), dim3(rgrid), block, 0, stream, g, partial, nsplit); break;
-        case LG_EPI_BIAS_GELU: hipLaunchKernelGGL((gemm_skinny_reduce_kernel<LG_EPI_BIAS_GELU>), dim3(rgrid), block, 0, stream, g, partial, nsplit); break;
-        default: hipLaunchKernelGGL((gemm_skinny_reduce_kernel<LG_EPI_BIAS_HEADS>), dim3(rgrid), block, 0, stream, g, partial, nsplit); break;
+        case LG_EPI_NONE: hipLaunchKernelGGL((gemm_skinny_reduce_kernel<LG_EPI_NONE>), dim3(rgrid), block, 0, stream, g, partial, nsplit, rm); break;
+        case LG_EPI_BIAS: hipLaunchKernelGGL((gemm_skinny_reduce_kernel<LG_EPI_BIAS>), dim3(rgrid), block, 0, stream, g, partial, nsplit, rm); break;
+        case LG_EPI_BIAS_GELU: hipLaunchKernelGGL((gemm_skinny_reduce_kernel<LG_EPI_BIAS_GELU>), dim3(rgrid), block, 0, stream, g, partial, nsplit, rm); break;
+        case LG_EPI_BIAS_HEADS_ROWS: hipLaunchKernelGGL((gemm_skinny_reduce_kernel<LG_EPI_BIAS_HEADS_ROWS>), dim3(rgrid), block, 0, stream, g, partial, nsplit, rm); break;
+        default: hipLaunchKernelGGL((gemm_skinny_reduce_kernel<LG_EPI_BIAS_HEADS>), dim3(rgrid), block, 0, stream, g, partial, nsplit, rm); break;
     }
 }
 
