@@ -33,12 +33,24 @@ constexpr int F_THREADS = 512;
 constexpr int X_STAGES = 3, W_STAGES = 2;
 constexpr int lds_halves(int NJ) { return X_STAGES * FB_M * FB_K + W_STAGES * FB_K * 64 * NJ; }
 
+// [64 k][64 NJ n] weight tile: which logical 32-byte block sits at block position `pos` of row k (swz_kn), and at which position
+// logical block `blk` sits (unswz_kn).  Power-of-two widths XOR (an involution); the 192-wide tile has 12 blocks to a row and
+// rotates instead: its rows are 96 dwords apart, so rows k and k + 2 (and k + 8, k + 10: the other half of the 32 lanes that one
+// transposed read serves together) would share banks, and a rotation by ((k >> 1) & 1) + 2 ((k >> 3) & 1) blocks separates them.
+template <int NJ> __device__ __forceinline__ int swz_kn(int k, int pos) {
+    if (NJ == 3) { const int b = pos + ((k >> 1) & 1) + 2 * ((k >> 3) & 1); return b >= 12 ? b - 12 : b; }
+    return swz_b(k, pos);
+}
+template <int NJ> __device__ __forceinline__ int unswz_kn(int k, int blk) {
+    if (NJ == 3) { const int p = blk - ((k >> 1) & 1) - 2 * ((k >> 3) & 1); return p < 0 ? p + 12 : p; }
+    return swz_b(k, blk);
+}
+
 template <int WL, int EPI, int NJ>
 __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles_m, int tiles_n, float* partial, int kt_per_split, int cus) {
     constexpr int FB_N = 64 * NJ;
     constexpr int X_TILE = FB_M * FB_K, W_TILE = FB_K * FB_N;  // halves per ring slot
     constexpr int WCH = (FB_K * FB_N) / 512 / 8;  // 1 KiB chunks of the W tile per wave (= NJ)
-    static_assert(WL == W_NK || NJ == 4 || NJ == 2, "the [in, out] weight tile needs a power-of-two number of lanes per k-row");
     extern __shared__ __attribute__((aligned(16))) half_t smem[];  // X ring (3 tiles), then W ring (2 tiles)
     half_t* const xring = smem;
     half_t* const wring = smem + X_STAGES * X_TILE;
@@ -107,9 +119,11 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles
             woff[i] = (unsigned)(row * (int)g.ldw + c * 8) * 2u;
         } else {
             // W tile [64 k][FB_N n]: a k-row is FB_N / 8 lanes wide, chunk q = 64 / (FB_N / 8) consecutive k-rows
+            // (the 192-wide tile has 24 lanes to a k-row, so a chunk's lanes straddle rows: every lane finds its own row and place)
             constexpr int LPR = FB_N / 8;
-            const int k = q * (64 / LPR) + lane / LPR, p = lane % LPR;
-            const int blk = swz_b(k, p >> 1);
+            const int f = q * 64 + lane;
+            const int k = f / LPR, p = f % LPR;
+            const int blk = swz_kn<NJ>(k, p >> 1);
             woff[i] = (unsigned)(k * (int)g.ldw + (blk * 2 + (p & 1)) * 8) * 2u;
         }
     }
@@ -143,8 +157,8 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles
         } else {
             const int blk = wn * NJ + u;                     // 32-byte block = 16 output columns
             const int k = ks * 32 + lk * 8 + (l16 >> 2);     // this lane's source row of the first 4x16 read
-            const half4_t lo = lds_read_tr4(&ws[k * FB_N + swz_b(k, blk) * 16 + (l16 & 3) * 4]);
-            const half4_t hi = lds_read_tr4(&ws[(k + 4) * FB_N + swz_b(k + 4, blk) * 16 + (l16 & 3) * 4]);
+            const half4_t lo = lds_read_tr4(&ws[k * FB_N + unswz_kn<NJ>(k, blk) * 16 + (l16 & 3) * 4]);
+            const half4_t hi = lds_read_tr4(&ws[(k + 4) * FB_N + unswz_kn<NJ>(k + 4, blk) * 16 + (l16 & 3) * 4]);
             b[u] = half8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         }
     };
@@ -338,7 +352,6 @@ int launch_gemm_fast_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t 
     long best_cost = 0;
     for (int nj = 4; nj >= 2; --nj) {
         if (g.N % (64 * nj)) continue;
-        if (nj == 3 && wlayout != W_NK) continue;
         const long tiles = (long)tiles_m * (g.N / (64 * nj));
         // narrower tiles move more operand bytes per flop: about 3 % / 35 % more time per unit of width (measured)
         const long cost = ((tiles + si.cus - 1) / si.cus) * nj * (nj == 4 ? 100 : nj == 3 ? 103 : 135);
@@ -354,6 +367,7 @@ int launch_gemm_fast_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t 
         else rc = launch_fast_epi<W_NK, 2>(g, tiles_m, tiles_n, si, stream);
     } else {
         if (best_nj == 4) rc = launch_fast_epi<W_KN, 4>(g, tiles_m, tiles_n, si, stream);
+        else if (best_nj == 3) rc = launch_fast_epi<W_KN, 3>(g, tiles_m, tiles_n, si, stream);
         else rc = launch_fast_epi<W_KN, 2>(g, tiles_m, tiles_n, si, stream);
     }
     return rc != LG_OK ? rc : check_launch("gemm_f16_fast");
