@@ -4,8 +4,14 @@
 // keeps its softmax semantics: t = q.k * scalar + (1 - mask) * (-10000), p = exp(t - max t), out = sum p v / (sum p +
 // 1e-6).  The S x S score matrix never touches HBM.
 //
-// Work split: one block = 128 queries of one (batch, head); 4 waves x 32 queries.  K and V tiles of 64 keys are staged
-// in LDS.  Everything is computed transposed so that no cross-lane data movement is needed between the two GEMMs:
+// Work split: one block = 32 NW queries of one (batch, head), NW waves x 32 queries (NW = 4; blocks of 8 waves halve the tile
+// loads per query and measure the same).  K and V tiles of 64 keys go from global
+// memory straight into LDS (direct-to-LDS loads, no VGPR staging) into a ring of two tiles each: the loads of tile t+1 are
+// issued right after the barrier that publishes tile t and run under tile t's MFMAs, one barrier per tile.  The LDS position of a
+// lane's 16 bytes is fixed by the load instruction, so the tiles are made bank-conflict-free by rotating, through the global
+// address each lane loads from, the 16-byte chunks (K) or 32-byte blocks (V) of row r by r places: the 16 rows that one
+// fragment read touches then fall into 16 different bank groups.  Rows beyond the sequence are read from its last row and
+// masked out of the softmax.  Everything is computed transposed so that no cross-lane data movement is needed between the two GEMMs:
 //   S^T[key, q] = K[key, :] . Q[q, :]      A = K tile (16-byte LDS reads), B = Q (registers, loaded once)
 //   O^T[d, q]  += V^T[d, key] * P^T[key, q] A = V tile through the gfx950 transposed LDS read, B = P^T, which is
 //                                           exactly the accumulator layout S^T came out in (4 consecutive keys per
@@ -16,21 +22,27 @@
 
 namespace lg {
 
-constexpr int PF_BQ = 128;  // queries per block
 constexpr int PF_BC = 64;   // keys per LDS tile
 
-template <int D, bool CAUSAL, bool HAS_MASK>
-__global__ __launch_bounds__(256) void attn_prefill_kernel(const half_t* __restrict__ q_buf, const half_t* __restrict__ k_buf,
+template <int D, int NW, bool CAUSAL, bool HAS_MASK>
+// two waves per SIMD (at most 256 registers): the softmax arithmetic of one wave runs under the MFMAs of the other
+__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(const half_t* __restrict__ q_buf, const half_t* __restrict__ k_buf,
                                                            const half_t* __restrict__ v_buf, const half_t* __restrict__ mask,
                                                            half_t* out, int seq, int head_num, int kv_rows, float scalar,
                                                            int out_layout) {
-    constexpr int KS = D + 8;       // LDS row stride in halves
     constexpr int DC = D / 32;      // 32-wide d chunks (k steps of the S^T GEMM)
     constexpr int DT = D / 16;      // 16-wide d tiles (rows of O^T)
-    __shared__ __attribute__((aligned(16))) half_t Ks[PF_BC * KS];
-    __shared__ __attribute__((aligned(16))) half_t Vs[PF_BC * KS];
+    constexpr int CPR = D / 8;      // 16-byte chunks per row
+    constexpr int BPR = D / 16;     // 32-byte blocks per row
+    constexpr int TILE = PF_BC * D; // halves per tile
+    constexpr int PF_BQ = 32 * NW;  // queries per block
+    constexpr int LPT = TILE / 8 / (64 * NW);  // direct-to-LDS loads per thread and tile (K and V each)
+    static_assert(TILE % (8 * 64 * NW) == 0, "a tile must be a whole number of 1 KiB wave loads per wave");
+    __shared__ __attribute__((aligned(16))) half_t Ks[2][TILE];
+    __shared__ __attribute__((aligned(16))) half_t Vs[2][TILE];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l16 = lane & 15, g = lane >> 4;
     const int bh = blockIdx.y;                 // b * head_num + head
     const int b = bh / head_num, head = bh % head_num;
@@ -40,6 +52,49 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const half_t* __restr
     const half_t* Q = q_buf + (int64_t)bh * seq * D;
     const half_t* K = k_buf + (int64_t)bh * kv_rows * D;
     const half_t* V = v_buf + (int64_t)bh * kv_rows * D;
+
+    // position of logical chunk c (K) / block blk (V) in row r of a tile
+    constexpr bool P2 = (CPR & (CPR - 1)) == 0;   // power-of-two row: 16 rows further on the rotation is the same again
+    auto kpos = [](int r, int c) { return P2 ? ((c + r) & (CPR - 1)) : (c + r) % CPR; };
+    auto vpos = [](int r, int blk) { return P2 ? ((blk + r) & (BPR - 1)) : (blk + r) % BPR; };
+    // LDS offsets (in halves) of this lane's fragment reads.  With a power-of-two row the rotation of rows r and r + 16 is the
+    // same, so one offset per d-chunk serves every 16-row group (the group's distance folds into the instruction's offset field).
+    constexpr int KG = P2 ? 1 : 4, VG = P2 ? 1 : 4;
+    int kfrag[KG][DC], vfrag[VG][DT];
+#pragma unroll
+    for (int kt = 0; kt < KG; ++kt)
+#pragma unroll
+        for (int dc = 0; dc < DC; ++dc) kfrag[kt][dc] = (kt * 16 + l16) * D + kpos(kt * 16 + l16, dc * 4 + g) * 8;
+#pragma unroll
+    for (int vg = 0; vg < VG; ++vg)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            const int row = vg * 16 + 4 * g + (l16 >> 2);
+            vfrag[vg][dt] = row * D + vpos(row, dt) * 16 + 4 * (l16 & 3);
+        }
+
+    // this thread's loads of one tile: LDS chunk f = (i * 4 + wave) * 64 + lane sits in row f / CPR at position f % CPR and must
+    // receive the logical chunk that belongs there
+    int lrow[LPT];
+    unsigned koff[LPT], voff[LPT];
+#pragma unroll
+    for (int i = 0; i < LPT; ++i) {
+        const int f = (i * NW + wave) * 64 + lane;
+        const int r = f / CPR, p = f % CPR;
+        lrow[i] = r;
+        const int kc = (p - r % CPR + CPR) % CPR;                       // kpos(r, kc) == p
+        const int vb = ((p >> 1) - r % BPR + BPR) % BPR;                // vpos(r, vb) == p >> 1
+        koff[i] = (unsigned)(kc * 8);
+        voff[i] = (unsigned)((vb * 2 + (p & 1)) * 8);
+    }
+    auto issue = [&](int k0, int buf) {
+#pragma unroll
+        for (int i = 0; i < LPT; ++i) {
+            const int64_t row = min(k0 + lrow[i], seq - 1);             // rows beyond the sequence: its last row, masked later
+            load_lds16(K + row * D + koff[i], &Ks[buf][(i * NW + wave) * 512]);
+            load_lds16(V + row * D + voff[i], &Vs[buf][(i * NW + wave) * 512]);
+        }
+    };
 
     // Q fragments: qf[qt][dc] = Q[qw + qt*16 + l16][dc*32 + 8g .. +8]
     half8_t qf[2][DC];
@@ -61,28 +116,20 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const half_t* __restr
     float m_run[2] = {-1e30f, -1e30f};
     float l_run[2] = {0.f, 0.f};  // per-lane partial sums (this lane's keys only)
 
+    const float sl2 = scalar * 1.4426950408889634f;            // scores in log2 units
+    constexpr float MASK_L2 = -10000.0f * 1.4426950408889634f;  // the reference's additive mask term, in the same units
     const int kv_end = CAUSAL ? min(seq, q0 + PF_BQ) : seq;
-    for (int k0 = 0; k0 < kv_end; k0 += PF_BC) {
-        __syncthreads();  // previous tile fully consumed
-        // stage K and V tiles: 64 rows x D halves each; rows beyond seq are zero-filled
-        constexpr int VPR = D / 8;               // 16-byte vectors per row
-        constexpr int NVEC = PF_BC * VPR;        // per tile
-#pragma unroll
-        for (int i = 0; i < NVEC / 256; ++i) {
-            const int v = tid + 256 * i;
-            const int row = v / VPR, c = v % VPR;
-            half8_t kk = half8_t{0, 0, 0, 0, 0, 0, 0, 0}, vv = kk;
-            if (k0 + row < seq) {
-                kk = *reinterpret_cast<const half8_t*>(K + (int64_t)(k0 + row) * D + c * 8);
-                vv = *reinterpret_cast<const half8_t*>(V + (int64_t)(k0 + row) * D + c * 8);
-            }
-            *reinterpret_cast<half8_t*>(&Ks[row * KS + c * 8]) = kk;
-            *reinterpret_cast<half8_t*>(&Vs[row * KS + c * 8]) = vv;
-        }
-        __syncthreads();
-        // a wave whose queries all lie before this key tile has nothing to do here (causal), but must keep hitting the
-        // barriers above, so only the math is skipped
+    issue(0, 0);
+    for (int k0 = 0, t = 0; k0 < kv_end; k0 += PF_BC, ++t) {
+        const int buf = t & 1;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's part of tile t has landed
+        __syncthreads();  // tile t is visible to every wave, and every wave is done with tile t-1: its buffer is refilled now
+        if (k0 + PF_BC < kv_end) issue(k0 + PF_BC, buf ^ 1);
+        // a wave whose queries all lie before this key tile has nothing to do here (causal), but keeps loading and hitting
+        // the barrier, so only the math is skipped
         if (CAUSAL && k0 > qw + 31) continue;
+        const half_t* ks = Ks[buf];
+        const half_t* vs = Vs[buf];
 
         // ---- S^T = K Q^T ------------------------------------------------------------------------------------
         float4_t s[4][2];
@@ -92,48 +139,65 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const half_t* __restr
             s[kt][1] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int dc = 0; dc < DC; ++dc) {
-                const half8_t a = *reinterpret_cast<const half8_t*>(&Ks[(kt * 16 + l16) * KS + dc * 32 + g * 8]);
+                const half8_t a = *reinterpret_cast<const half8_t*>(&ks[P2 ? kfrag[0][dc] + kt * 16 * D : kfrag[kt % KG][dc]]);
                 s[kt][0] = mfma16(a, qf[0][dc], s[kt][0]);
                 s[kt][1] = mfma16(a, qf[1][dc], s[kt][1]);
             }
         }
         // ---- scale, mask, online softmax (per query column) -----------------------------------------------------
+        // Scores are kept in log2 units (scale folded with log2 e: exp(t - m) = exp2(t' - m')), so that a score costs one
+        // multiply, one max, one subtract, one exp2 and one add.  The causal comparison is only made on tiles that reach above
+        // the diagonal of the wave's first query, the end-of-sequence test only on the last tile (both wave-uniform).
+        const bool diag = CAUSAL && (k0 + PF_BC - 1 > qw);
+        const bool tail = k0 + PF_BC > seq;
 #pragma unroll
         for (int qt = 0; qt < 2; ++qt) {
             const int q = qw + qt * 16 + l16;
-            float mx = -1e30f;
 #pragma unroll
-            for (int kt = 0; kt < 4; ++kt) {
-                float mterm[4] = {0.f, 0.f, 0.f, 0.f};
-                if (HAS_MASK) {
+            for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) s[kt][qt][r] *= sl2;
+            if (HAS_MASK) {
+#pragma unroll
+                for (int kt = 0; kt < 4; ++kt) {
                     const int key = k0 + kt * 16 + 4 * g;
                     if (q < seq) {
 #pragma unroll
                         for (int r = 0; r < 4; ++r)
-                            if (key + r < seq) mterm[r] = (1.0f - (float)mask[((int64_t)b * seq + q) * seq + key + r]) * -10000.0f;
+                            if (key + r < seq) s[kt][qt][r] += (1.0f - (float)mask[((int64_t)b * seq + q) * seq + key + r]) * MASK_L2;
                     }
                 }
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int key = k0 + kt * 16 + 4 * g + r;
-                    float t = s[kt][qt][r] * scalar + mterm[r];
-                    if (CAUSAL && key > q) t += -10000.0f;
-                    if (key >= seq) t = -1e30f;  // beyond the sequence: not part of the row at all
-                    s[kt][qt][r] = t;
-                    mx = fmaxf(mx, t);
-                }
             }
+            if (diag) {
+#pragma unroll
+                for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (k0 + kt * 16 + 4 * g + r > q) s[kt][qt][r] += MASK_L2;
+            }
+            if (tail) {
+#pragma unroll
+                for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (k0 + kt * 16 + 4 * g + r >= seq) s[kt][qt][r] = -1e30f;  // beyond the sequence: not part of the row at all
+            }
+            float mx = -1e30f;
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[kt][qt][r]);
             mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
             const float m_new = fmaxf(m_run[qt], mx);
-            const float corr = __expf(m_run[qt] - m_new);
+            const float corr = __builtin_amdgcn_exp2f(m_run[qt] - m_new);
             m_run[qt] = m_new;
             float ls = 0.f;
 #pragma unroll
             for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const float p = __expf(s[kt][qt][r] - m_new);
+                    const float p = __builtin_amdgcn_exp2f(s[kt][qt][r] - m_new);
                     s[kt][qt][r] = p;
                     ls += p;
                 }
@@ -153,16 +217,16 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const half_t* __restr
             }
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
-                const int col = dt * 16 + 4 * (l16 & 3);
-                const int row = (2 * j) * 16 + 4 * g + (l16 >> 2);
-                const half4_t lo = lds_read_tr4(&Vs[row * KS + col]);
-                const half4_t hi = lds_read_tr4(&Vs[(row + 16) * KS + col]);
+                // logical 32-byte block dt of rows 32 j + 4 g + l16 / 4 and 16 rows further on, this lane's 8 bytes inside it
+                const half4_t lo = lds_read_tr4(&vs[P2 ? vfrag[0][dt] + (2 * j) * 16 * D : vfrag[(2 * j) % VG][dt]]);
+                const half4_t hi = lds_read_tr4(&vs[P2 ? vfrag[0][dt] + (2 * j + 1) * 16 * D : vfrag[(2 * j + 1) % VG][dt]]);
                 const half8_t a = half8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                 o[dt][0] = mfma16(a, pf[0], o[dt][0]);
                 o[dt][1] = mfma16(a, pf[1], o[dt][1]);
             }
         }
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
     // ---- normalise and store ----------------------------------------------------------------------------------------
 #pragma unroll
@@ -184,16 +248,17 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const half_t* __restr
     }
 }
 
-template <int D>
+template <int D, int NW>
 static void launch_prefill(const half_t* q, const half_t* k, const half_t* v, const half_t* mask, half_t* out, int batch,
                            int seq, int head_num, int kv_rows, float scalar, int causal, int out_layout, hipStream_t st) {
-    dim3 grid((seq + PF_BQ - 1) / PF_BQ, batch * head_num);
+    constexpr int BQ = 32 * NW;
+    dim3 grid((seq + BQ - 1) / BQ, batch * head_num), block(64 * NW);
     if (causal)
-        hipLaunchKernelGGL((attn_prefill_kernel<D, true, false>), grid, dim3(256), 0, st, q, k, v, mask, out, seq, head_num, kv_rows, scalar, out_layout);
+        hipLaunchKernelGGL((attn_prefill_kernel<D, NW, true, false>), grid, block, 0, st, q, k, v, mask, out, seq, head_num, kv_rows, scalar, out_layout);
     else if (mask)
-        hipLaunchKernelGGL((attn_prefill_kernel<D, false, true>), grid, dim3(256), 0, st, q, k, v, mask, out, seq, head_num, kv_rows, scalar, out_layout);
+        hipLaunchKernelGGL((attn_prefill_kernel<D, NW, false, true>), grid, block, 0, st, q, k, v, mask, out, seq, head_num, kv_rows, scalar, out_layout);
     else
-        hipLaunchKernelGGL((attn_prefill_kernel<D, false, false>), grid, dim3(256), 0, st, q, k, v, mask, out, seq, head_num, kv_rows, scalar, out_layout);
+        hipLaunchKernelGGL((attn_prefill_kernel<D, NW, false, false>), grid, block, 0, st, q, k, v, mask, out, seq, head_num, kv_rows, scalar, out_layout);
 }
 
 }  // namespace lg
@@ -217,13 +282,13 @@ extern "C" int lg_attn_prefill_f16(const void* q_buf, const void* k_buf, const v
     if ((int64_t)batch * head_num > 65535) { set_error("attn_prefill: batch * head_num > 65535"); return LG_ERR_INVALID; }
     scalar = (float)(half_t)scalar;
     if (size_per_head == 128)
-        launch_prefill<128>((const half_t*)q_buf, (const half_t*)k_buf, (const half_t*)v_buf, (const half_t*)attr_mask,
+        launch_prefill<128, 4>((const half_t*)q_buf, (const half_t*)k_buf, (const half_t*)v_buf, (const half_t*)attr_mask,
                             (half_t*)out, batch, seq, head_num, kv_rows, scalar, causal, out_layout, (hipStream_t)stream);
     else if (size_per_head == 96)
-        launch_prefill<96>((const half_t*)q_buf, (const half_t*)k_buf, (const half_t*)v_buf, (const half_t*)attr_mask,
+        launch_prefill<96, 4>((const half_t*)q_buf, (const half_t*)k_buf, (const half_t*)v_buf, (const half_t*)attr_mask,
                            (half_t*)out, batch, seq, head_num, kv_rows, scalar, causal, out_layout, (hipStream_t)stream);
     else
-        launch_prefill<64>((const half_t*)q_buf, (const half_t*)k_buf, (const half_t*)v_buf, (const half_t*)attr_mask,
+        launch_prefill<64, 4>((const half_t*)q_buf, (const half_t*)k_buf, (const half_t*)v_buf, (const half_t*)attr_mask,
                            (half_t*)out, batch, seq, head_num, kv_rows, scalar, causal, out_layout, (hipStream_t)stream);
     return check_launch("attn_prefill");
 }
