@@ -14,6 +14,8 @@ enum LnMode { LN_PLAIN = 0, LN_ADD_INPLACE = 1, LN_ADD_STORE = 2 };
 //   LN_PLAIN        x = src                                   dst = LN(x)
 //   LN_ADD_INPLACE  x = src + add + bias        (fp32)        dst = LN(x)          (dst may alias src)
 //   LN_ADD_STORE    x = T(add + src + bias); sum_out = x      dst = LN(x)          (sum_out may alias src)
+//                   with the mean taken over the unrounded fp32 sums and the variance and output over the stored x,
+//                   as the reference kernel does (cuda_kernels.cu:377-408)
 template <typename T, int MODE, int NV>
 __global__ __launch_bounds__(256) void ln_vec_kernel(const T* __restrict__ src, const T* __restrict__ add,
                                                      const T* __restrict__ bias, const T* __restrict__ gamma,
@@ -37,19 +39,21 @@ __global__ __launch_bounds__(256) void ln_vec_kernel(const T* __restrict__ src, 
 #pragma unroll
                 for (int j = 0; j < VN; ++j) {
                     float t = r.get(j) + a.get(j) + b.get(j);
+                    local += t;  // the mean sums the unrounded value in every mode
                     if (MODE == LN_ADD_STORE) {
                         s.set(j, t);
-                        t = s.get(j);  // statistics use the stored (rounded) value
+                        t = s.get(j);  // variance and output use the stored (rounded) value
                     }
                     x[i][j] = t;
                 }
                 if (MODE == LN_ADD_STORE) *reinterpret_cast<V*>(sum_out + row + (int64_t)v * VN) = s;
             } else {
 #pragma unroll
-                for (int j = 0; j < VN; ++j) x[i][j] = a.get(j);
+                for (int j = 0; j < VN; ++j) {
+                    x[i][j] = a.get(j);
+                    local += x[i][j];
+                }
             }
-#pragma unroll
-            for (int j = 0; j < VN; ++j) local += x[i][j];
         } else {
 #pragma unroll
             for (int j = 0; j < VN; ++j) x[i][j] = 0.f;
@@ -95,10 +99,7 @@ __global__ __launch_bounds__(256) void ln_scalar_kernel(const T* src, const T* a
     for (int i = threadIdx.x; i < n; i += blockDim.x) {
         float t = ldf(src + row + i);
         if (MODE != LN_PLAIN) t = ldf(add + row + i) + t + ldf(bias + i);
-        if (MODE == LN_ADD_STORE) {
-            stf(sum_out + row + i, t);
-            t = ldf(sum_out + row + i);
-        }
+        if (MODE == LN_ADD_STORE) stf(sum_out + row + i, t);  // the mean still sums the unrounded t
         local += t;
     }
     const float mean = block_sum(local, scratch) / (float)n;

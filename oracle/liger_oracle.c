@@ -272,10 +272,12 @@ void lo_add_bias_geglu(float* out, const float* in, const float* bias, int m, in
 /* LayerNorm family                                                                            */
 /* ------------------------------------------------------------------------------------------ */
 /* two-pass statistics exactly as layer_norm_kernel_generalize does them (cuda_kernels.cu:463-508):
- * mean = sum/n; var = sum((x-mean)^2)/n; scale = rsqrt(var + 1e-6) */
-static void ln_row(const float* x, const float* gamma, const float* beta, float* y, int n, int dtype) {
+ * mean = sum/n; var = sum((x-mean)^2)/n; scale = rsqrt(var + 1e-6).
+ * `msrc` holds the values the mean is summed over (x itself for every kernel but add_bias_input_layernorm_2). */
+static void ln_row2(const float* x, const float* msrc, const float* gamma, const float* beta, float* y, int n,
+                    int dtype) {
     double s = 0.0; /* the GPU tree-reduces in fp32; double here is the mathematically cleaner stand-in */
-    for (int j = 0; j < n; ++j) s += x[j];
+    for (int j = 0; j < n; ++j) s += msrc[j];
     float mean = (float)(s / n);
     double v = 0.0;
     for (int j = 0; j < n; ++j) {
@@ -284,6 +286,10 @@ static void ln_row(const float* x, const float* gamma, const float* beta, float*
     }
     float rstd = 1.0f / sqrtf((float)(v / n) + 1e-6f);
     for (int j = 0; j < n; ++j) y[j] = st(((x[j] - mean) * rstd) * gamma[j] + beta[j], dtype);
+}
+
+static void ln_row(const float* x, const float* gamma, const float* beta, float* y, int n, int dtype) {
+    ln_row2(x, x, gamma, beta, y, n, dtype);
 }
 
 void lo_layer_norm(const float* in, const float* gamma, const float* beta, float* out, int m, int n,
@@ -307,8 +313,9 @@ void lo_add_bias_input_layernorm(float* out, const float* input, const float* bi
     }
 }
 
-/* cuda_kernels.cu:360-409: output += input + bias (stored, rounded to T), then
- * norm_output = LN(output) computed from the STORED values. */
+/* cuda_kernels.cu:360-409: output = T(input + output + bias) is stored; the mean is summed over the UNROUNDED fp32
+ * sums (:377-384), the variance and the normalised output re-read the stored, rounded values (:392-408).  In half
+ * precision the two differ by the mean rounding error of the row, which a row of near-ties makes visible. */
 void lo_add_bias_input_layernorm_2(const float* input, const float* gamma, const float* beta,
                                    const float* bias, float* output, float* norm_output, int m, int n,
                                    int dtype) {
@@ -316,16 +323,16 @@ void lo_add_bias_input_layernorm_2(const float* input, const float* gamma, const
     for (int i = 0; i < m; ++i) {
         float* o = output + (int64_t)i * n;
         const float* in = input + (int64_t)i * n;
+        float* raw = (float*)malloc(sizeof(float) * (size_t)n);
         for (int j = 0; j < n; ++j) {
             float t = in[j];
             t += o[j];
             t += bias[j];
+            raw[j] = t;
             o[j] = st(t, dtype);
         }
-        /* the reference sums the unrounded fp32 values for the mean (:377-384) but re-reads the stored
-         * values for the variance and the output (:392-408); the stored values are used for all three
-         * here, the difference is below fp16 resolution of the result */
-        ln_row(o, gamma, beta, norm_output + (int64_t)i * n, n, dtype);
+        ln_row2(o, raw, gamma, beta, norm_output + (int64_t)i * n, n, dtype);
+        free(raw);
     }
 }
 
@@ -382,24 +389,29 @@ void lo_add_fused_qkv_bias_transpose(float* q_buf, float* k_buf, float* v_buf, c
                     }
 }
 
-/* attention_kernels.cu:480-519 (fp32 math) and :525-576 (half2 specialisation):
- *   t = qk*scalar + (1-mask)*(-10000);  p = exp(t - max t);  out = p * (1/(sum p + 1e-6)).
- * The half specialisation forms t in half (scale product rounded, mask term rounded, sum rounded),
- * subtracts the max in half and exponentiates in half (h2exp); max and sum are fp32. */
+/* attn_softmax_kernelLauncher (attention_kernels.cu:621-680) picks one of three arithmetic variants by seq and T:
+ *   t = qk*scalar + (1-mask)*(-10000);  e = exp(t - max t);  s = sum e + 1e-6
+ *   odd seq (softmax_kernel / _v2, :397-478)            fp32 math, out = T(e / s)
+ *   even seq <= 32, or float (_v3_LE32 / _v3, :482-617) fp32 math, out = T(e * (1/s))
+ *   even seq > 32 and half (half2 _v3, :525-576)        t formed in half (scale product, 1-mask, its product with
+ *       -10000 and the sum each rounded), max subtracted and exponentiated in half (h2exp), the two columns a thread
+ *       holds (2i, 2i+1) added IN HALF before the fp32 block sum, 1/s rounded to half, product in half. */
 void lo_attn_softmax(float* buffer, const float* attr_mask, int batch, int seq, int head_num,
                      float scalar, int dtype) {
     const float sc = st(scalar, dtype); /* bert_layer.h:94 stores the scalar as T */
+    const int half2_path = dtype != LO_F32 && seq % 2 == 0 && seq > 32;
+    const int divide = seq % 2 != 0;
 #pragma omp parallel for collapse(2) schedule(static)
     for (int b = 0; b < batch; ++b)
         for (int h = 0; h < head_num; ++h) {
-            float* t = (float*)malloc(sizeof(float) * (size_t)seq);
+            float* t = (float*)malloc(sizeof(float) * (size_t)(seq > 0 ? seq : 1));
             for (int sq = 0; sq < seq; ++sq) {
                 float* row = buffer + (((int64_t)b * head_num + h) * seq + sq) * seq;
                 const float* mrow = attr_mask + ((int64_t)b * seq + sq) * seq;
                 float mx = -1e20f;
                 for (int j = 0; j < seq; ++j) {
                     float v;
-                    if (dtype == LO_F32) {
+                    if (!half2_path) {
                         v = row[j] * sc + (1.0f - mrow[j]) * -10000.0f;
                     } else {
                         float mterm = lo_round_f16(lo_round_f16(1.0f - mrow[j]) * -10000.0f);
@@ -409,18 +421,28 @@ void lo_attn_softmax(float* buffer, const float* attr_mask, int batch, int seq, 
                     mx = v > mx ? v : mx;
                 }
                 float sum = 0.f;
-                for (int j = 0; j < seq; ++j) {
-                    float e;
-                    if (dtype == LO_F32) {
-                        e = expf(t[j] - mx);
-                    } else {
-                        e = lo_round_f16(expf(lo_round_f16(t[j] - lo_round_f16(mx))));
+                if (!half2_path) {
+                    for (int j = 0; j < seq; ++j) {
+                        t[j] = expf(t[j] - mx);
+                        sum += t[j];
                     }
-                    t[j] = e;
-                    sum += e;
+                } else {
+                    for (int j = 0; j < seq; j += 2) {
+                        t[j] = lo_round_f16(expf(lo_round_f16(t[j] - mx)));
+                        t[j + 1] = lo_round_f16(expf(lo_round_f16(t[j + 1] - mx)));
+                        sum += lo_round_f16(t[j] + t[j + 1]);
+                    }
                 }
-                float inv = 1.0f / (sum + 1e-6f);
-                for (int j = 0; j < seq; ++j) row[j] = st(t[j] * st(inv, dtype), dtype);
+                if (divide) {
+                    const float s = sum + 1e-6f;
+                    for (int j = 0; j < seq; ++j) row[j] = st(t[j] / s, dtype);
+                } else if (!half2_path) {
+                    const float inv = 1.0f / (sum + 1e-6f);
+                    for (int j = 0; j < seq; ++j) row[j] = st(t[j] * inv, dtype);
+                } else {
+                    const float inv = lo_round_f16(1.0f / (sum + 1e-6f));
+                    for (int j = 0; j < seq; ++j) row[j] = lo_round_f16(t[j] * inv);
+                }
             }
             free(t);
         }

@@ -88,6 +88,26 @@ def test_add_bias_input_layernorm_family(dev, po, dt, m, n):
     assert max_rel_err(dev.down(d_out), ref) < tol(dt)
 
 
+@pytest.mark.parametrize("n", [64, 12288, 100, 33])
+def test_layernorm_2_f16_row_of_near_ties(dev, po, n):
+    """add_bias_input_layernorm_2 in half on a row whose every sum 1 + 2^-11 ties down to 1.0: the stored sums are all 1.0,
+    the mean comes from the unrounded sums (cuda_kernels.cu:377-384), variance and output from the stored ones (:392-408),
+    so every output is -u / sqrt(u^2 + 1e-6) = -0.43877 with u = 2^-11 (0 if the mean came from the stored values, -0.48828
+    if the variance came from the unrounded ones).  n = 64 and 12288 take the register-cached kernel, 100 and 33 the scalar
+    one."""
+    u = 2.0 ** -11
+    m = 5
+    inp = np.ones((m, n), dtype=np.float32)
+    out0 = np.full((m, n), u, dtype=np.float32)
+    g, b, z = np.ones(n, dtype=np.float32), np.zeros(n, dtype=np.float32), np.zeros(n, dtype=np.float32)
+    ref_sum, ref_norm = po.add_bias_input_layernorm_2(inp, g, b, z, out0.copy(), 1)
+    d_out, d_norm = dev.up(out0, 1), dev.empty((m, n), 1)
+    dev.call("lg_add_bias_input_layernorm_2_f16", dev.up(inp, 1), dev.up(g, 1), dev.up(b, 1), dev.up(z, 1), d_out, d_norm, m, n)
+    assert np.array_equal(dev.down(d_out), ref_sum) and np.all(ref_sum == 1.0)
+    got = dev.down(d_norm)
+    assert np.abs(got - ref_norm).max() <= 2.0 ** -11 and np.abs(got + 0.43877).max() < 5e-4
+
+
 @pytest.mark.parametrize("dt", [0, 1])
 @pytest.mark.parametrize("B,S,h,d", [(2, 32, 4, 64), (2, 8, 12, 128), (1, 5, 3, 20), (3, 7, 2, 9)])
 def test_qkv_bias_transpose_and_back(dev, po, dt, B, S, h, d):

@@ -282,3 +282,146 @@ def test_decoder_step_equals_prefill_of_extended_sequence(po):
     shape = dict(shape1, seq=S)
     out = po.decoder_step(shape, w, np.ascontiguousarray(x[:, S]), kc, vc, S)
     assert np.abs(out - full[:, S]).max() < 1e-4
+
+
+# ---- fp16 rounding points ---------------------------------------------------------------------------------------------
+# Each case below is built so that the half instantiation's result differs visibly from what fp32 arithmetic (or a
+# different placement of the roundings) would give; the expected values follow from the IEEE binary16 grid by hand:
+# spacing 2^-10 in [1, 2), 2^-11 in [0.5, 1), 8 in [8192, 16384); ties go to the even significand.
+U = 2.0 ** -11          # half an ulp of 1.0: 1 + U ties to 1.0, 1 + 3U ties to 1 + 4U
+
+
+def _h(x):
+    return np.asarray(x, dtype=np.float32).astype(np.float16).astype(np.float32)
+
+
+def test_f16_add_bias_input_rounds_twice_left_to_right(po):
+    """cuda_kernels.cu:438-452, half: output + input is rounded before bias is added.  (1 + U) ties to 1, then (1 + U)
+    ties to 1 again; one rounding of the exact sum, or adding input + bias first, gives 1 + 2U."""
+    out = np.array([[1.0, 1.0, 1.0, 2.0 * U]], dtype=np.float32)
+    inp = np.array([[U, U, 3 * U, 1.0]], dtype=np.float32)
+    bias = np.array([U, 0.0, U, U], dtype=np.float32)
+    got = po.add_bias_input(out.copy(), bias, inp, 1)
+    #   (1+U)->1, +U -> 1 | (1+U)->1 | (1+3U)->1+4U, +U -> 1+5U ties to 1+4U | (2U+1) exact, +U -> 1+3U ties to 1+4U
+    assert got.tolist() == [[1.0, 1.0, 1.0 + 4 * U, 1.0 + 4 * U]]
+    assert float(_h(1.0 + U + U)) == 1.0 + 2 * U                      # what a single rounding would have given
+    assert po.add_bias_input(out.copy(), bias, inp, 0).tolist() == [[1.0 + 2 * U, 1.0 + U, 1.0 + 4 * U, 1.0 + 3 * U]]
+
+
+def test_f16_layernorm_2_mean_from_unrounded_sums_rest_from_stored(po):
+    """cuda_kernels.cu:377-408, half: the stored sum is rounded, the mean is taken over the unrounded fp32 sums, variance
+    and output over the stored values.  A constant row 1 + U stores 1.0 everywhere, so mean = 1 + U, every deviation is
+    -U, var = U^2 and y = -U / sqrt(U^2 + 1e-6) = -0.43877; taking the mean from the stored values would give 0, taking
+    the variance from the unrounded values would give -U / sqrt(1e-6) = -0.48828."""
+    n = 64
+    inp = np.ones((2, n), dtype=np.float32)
+    out = np.full((2, n), U, dtype=np.float32)
+    g = np.ones(n, dtype=np.float32)
+    b = np.zeros(n, dtype=np.float32)
+    stored, normed = po.add_bias_input_layernorm_2(inp, g, b, np.zeros(n, dtype=np.float32), out.copy(), 1)
+    assert np.all(stored == 1.0)
+    want = -U / np.sqrt(np.float64(U) ** 2 + 1e-6)
+    assert abs(want + 0.43877) < 1e-5
+    assert np.all(normed == _h(want))
+    # the in-place sibling (cuda_kernels.cu:115-185) never stores the sum: every statistic sees 1 + U and the row is flat
+    flat = po.add_bias_input_layernorm(out.copy(), inp, np.zeros(n, dtype=np.float32), g, b, 1)
+    assert np.all(flat == 0.0)
+    # fp32 instantiation: nothing is rounded, the row is flat as well
+    _, n32 = po.add_bias_input_layernorm_2(inp, g, b, np.zeros(n, dtype=np.float32), out.copy(), 0)
+    assert np.all(np.abs(n32) < 1e-6)
+
+
+def test_f16_softmax_half2_variant_rounding_points(po):
+    """attention_kernels.cu:525-576 (half, even seq > 32)."""
+    S = 64
+    ones = np.ones((1, S, S), dtype=np.float32)
+    e8 = float(_h(np.exp(np.float32(-8.0))))
+    # (1) mask term on the spacing-8 grid: a fully masked row with scores 5 and 3 has t = -9995 -> -9992 and
+    #     t = -9997 -> -10000, eight apart instead of two
+    qk = np.full((1, 1, S, S), 3.0, dtype=np.float32)
+    qk[0, 0, :, 0] = 5.0
+    p = po.attn_softmax(qk.copy(), np.zeros((1, S, S), dtype=np.float32), 1.0, 1)
+    #     pair (0, 1) sums to 1 + e8 -> 1.0 in half, the other 31 pairs to 2 e8 exactly
+    inv = float(_h(1.0 / (np.float32(1.0) + np.float32(62.0 * e8) + np.float32(1e-6))))
+    assert np.all(p[0, 0, :, 0] == float(_h(inv))) and np.all(p[0, 0, :, 1:] == float(_h(e8 * inv)))
+    assert abs(p[0, 0, 0, 1] / p[0, 0, 0, 0] - np.exp(-8.0)) < 2e-6 and np.exp(-2.0) > 0.1
+    # (2) the two columns a thread holds are added in half: 1 + exp(-8) -> 1.0, so 1/s rounds to 1.0; with the small term
+    #     in another pair the fp32 sum keeps it and 1/s = 0.999665 rounds down to 1 - U
+    m = np.zeros((1, S, S), dtype=np.float32)
+    m[0, :, 0] = m[0, :, 1] = m[0, :, 2] = 1.0
+    a = np.zeros((1, 1, S, S), dtype=np.float32)
+    a[0, 0, :, 1] = -8.0
+    a[0, 0, :, 2] = -30.0                                    # exp(-30) is 0 in half
+    pa = po.attn_softmax(a.copy(), m, 1.0, 1)
+    assert np.all(pa[0, 0, :, 0] == 1.0) and np.all(pa[0, 0, :, 1] == e8) and np.all(pa[0, 0, :, 2:] == 0.0)
+    a[0, 0, :, 1], a[0, 0, :, 2] = -30.0, -8.0
+    pb = po.attn_softmax(a.copy(), m, 1.0, 1)
+    assert np.all(pb[0, 0, :, 0] == 1.0 - U) and np.all(pb[0, 0, :, 2] == float(_h(e8 * (1.0 - U))))
+    # (3) constant row, all-ones mask: every e is 1, the sum 48 is exact, out = half(1 / (48 + 1e-6))
+    S3 = 48
+    c = po.attn_softmax(np.full((1, 2, S3, S3), 2.5, dtype=np.float32), np.ones((1, S3, S3), dtype=np.float32), 0.125, 1)
+    assert np.all(c == float(_h(np.float32(1.0) / (np.float32(48.0) + np.float32(1e-6)))))
+    # (4) the scalar is a half and the scale product is rounded: half(0.011) = 0.0110015869140625 takes 1028 to
+    #     11.30963 -> 11.3125 and 1024 to 11.265625 (exact), 0.046875 apart; an fp32 scalar 0.011 would give
+    #     11.308 -> 11.3046875 and the same 11.265625, 0.0390625 apart
+    z = np.full((1, 1, S, S), 1024.0, dtype=np.float32)
+    z[0, 0, :, 0] = 1028.0
+    pz = po.attn_softmax(z.copy(), ones, 0.011, 1)
+    e1 = float(_h(np.exp(np.float32(-0.046875))))
+    sz = np.float32(float(_h(1.0 + e1))) + np.float32(62.0 * e1) + np.float32(1e-6)
+    iz = float(_h(np.float32(1.0) / sz))
+    assert np.all(pz[0, 0, :, 0] == iz) and np.all(pz[0, 0, :, 1:] == float(_h(e1 * iz)))
+    assert abs(pz[0, 0, 0, 1] / pz[0, 0, 0, 0] - np.exp(-0.046875)) < 1.5e-3 < abs(np.exp(-0.0390625) - np.exp(-0.046875)) / 4
+
+
+def test_f16_softmax_small_and_odd_rows_use_fp32_math(po):
+    """attention_kernels.cu:621-680: half rows with even seq <= 32 (softmax_kernel_v3_LE32) and odd seq (softmax_kernel /
+    _v2) are computed in fp32 and rounded once, so a fully masked row keeps the true score differences (two apart, not
+    eight as in the half2 variant)."""
+    for S in (16, 32, 33, 7):
+        qk = np.full((1, 1, S, S), 3.0, dtype=np.float32)
+        qk[0, 0, :, 0] = 5.0
+        p = po.attn_softmax(qk.copy(), np.zeros((1, S, S), dtype=np.float32), 1.0, 1)
+        e2 = np.exp(np.float32(-2.0))
+        s = np.float32(1.0) + np.float32(S - 1) * e2 + np.float32(1e-6)
+        assert np.abs(p[0, 0, :, 0] - _h(1.0 / s)).max() <= 2.0 ** -12, S     # within one half ulp of the closed form
+        assert np.abs(p[0, 0, :, 1] / p[0, 0, :, 0] - e2).max() < 2e-3, S
+    # the half2 variant at S = 34 has the ratio exp(-8)
+    S = 34
+    qk = np.full((1, 1, S, S), 3.0, dtype=np.float32)
+    qk[0, 0, :, 0] = 5.0
+    p = po.attn_softmax(qk.copy(), np.zeros((1, S, S), dtype=np.float32), 1.0, 1)
+    assert np.abs(p[0, 0, :, 1] / p[0, 0, :, 0] - np.exp(-8.0)).max() < 1e-5
+
+
+def test_f16_gelu_rounding_points_exhaustive(po):
+    """cuda_kernels.cu:17-29,72-84 (half2): x = half(v + b); x3 = half(x * half(x * x)); cdf in fp32 from x and x3, rounded
+    to half; out = half(x * cdf).  Checked over every finite half value against numpy's binary16 arithmetic, plus one value
+    derived by hand."""
+    # by hand: v = 1, b = U -> x = 1.0 (tie to even); cdf(1) = 0.84119199 -> 1723 * 2^-11 = 0.84130859375
+    one = po.add_bias_gelu(np.array([[1.0, 1.0]], dtype=np.float32), np.array([U, 0.0], dtype=np.float32), 1)
+    assert one.tolist() == [[0.84130859375, 0.84130859375]]
+    assert float(_h(np.float32(1.0 + U) * 0.5 * (1 + np.tanh(0.7978845608 * ((1 + U) + 0.044715 * (1 + U) ** 3))))) == 0.841796875
+    bits = np.arange(0, 1 << 16, dtype=np.uint16)
+    x = bits.view(np.float16)
+    x = x[np.isfinite(x)]
+    n = x.size - x.size % 2
+    x = x[:n]
+    with np.errstate(over="ignore", invalid="ignore"):
+        x3 = x * (x * x)                                     # float16 arithmetic: each product rounded
+        arg = np.float32(0.7978845608028654) * (x.astype(np.float32) + np.float32(0.044715) * x3.astype(np.float32))
+        cdf = (np.float32(0.5) * (np.float32(1.0) + np.tanh(arg.astype(np.float64)).astype(np.float32))).astype(np.float16)
+        want = (x * cdf).astype(np.float32)
+    got = po.add_bias_gelu(x.astype(np.float32).reshape(1, n), np.zeros(n, dtype=np.float32), 1)[0]
+    both_nan = np.isnan(want) & np.isnan(got)
+    diff = ~both_nan & (want != got)
+    # tanhf is not correctly rounded everywhere: allow a last-place difference of the cdf at a handful of points
+    assert diff.sum() <= 8, diff.sum()
+    assert np.all(np.abs(want[diff] - got[diff]) <= np.abs(want[diff]) * 2.0 ** -9)
+    # the check discriminates: cubing in fp32 (one rounding instead of two) disagrees at thousands of points
+    with np.errstate(over="ignore", invalid="ignore"):
+        xf = x.astype(np.float32)
+        arg1 = np.float32(0.7978845608028654) * (xf + np.float32(0.044715) * (xf * xf * xf).astype(np.float16).astype(np.float32))
+        cdf1 = (np.float32(0.5) * (np.float32(1.0) + np.tanh(arg1.astype(np.float64)).astype(np.float32))).astype(np.float16)
+        alt = (x * cdf1).astype(np.float32)
+    assert ((alt != got) & ~(np.isnan(alt) & np.isnan(got))).sum() > 100
