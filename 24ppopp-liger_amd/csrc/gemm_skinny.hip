@@ -123,18 +123,38 @@ __global__ __launch_bounds__(256) void gemm_skinny_nk_kernel(GemmArgs g, int ksl
 }
 
 // ---- whole K in one block ------------------------------------------------------------------------------------------------
-// When N alone gives enough blocks K is not sliced at all: a block = NWV waves x 16 output features walks the whole of K, the
-// epilogue is applied to the accumulators, and there are no fp32 partials and no second kernel.  A wave owns one 16-feature
-// MFMA tile (8 loads per chunk), so its rolling pipeline is DEPTH chunks deep: two chunks (16 loads per lane, as in the sliced
-// kernel) for blocks of 4, 6 or 8 waves, four chunks for the 2-wave block, which then keeps the 64 KiB of a 4-wave block in flight.
+// When N alone gives enough work K is not sliced at all: a wave owns one 16-feature MFMA tile and walks the whole of K for it,
+// the epilogue is applied to the accumulators, and there are no fp32 partials and no second kernel.  The 16-feature tiles of the
+// problem (of all members of a group, which share X) are dealt out in runs of consecutive tiles to a grid of exactly one block per
+// compute unit, NWV = ceil(tiles / CUs) waves a block, with the last wave having a tile only in the first blocks.  Every wave streams the same number of bytes, and one block per compute unit measured
+// fastest (32 token rows, 256 CUs: 12288 features as 256 blocks of 3 waves 75.7 us at K = 16384 and 25.8 us at K = 6144, as 192
+// blocks of 4 waves 86.1 and 29.7 us).
+// A wave's rolling pipeline is DEPTH chunks deep (8 loads per chunk): two chunks for blocks of 3 to 8 waves, four chunks for the
+// 2-wave block, which then keeps the 64 KiB of a 4-wave block in flight.
 template <int MT, int EPI, int NWV, int DEPTH>
-__global__ __launch_bounds__(64 * NWV) void gemm_skinny_direct_kernel(GemmArgs g, GemmGroup grp, RowMap rm) {
+__global__ __launch_bounds__(64 * NWV) void gemm_skinny_direct_kernel(GemmArgs g, GemmGroup grp, RowMap rm, int tiles_per_member) {
     constexpr int THREADS = 64 * NWV;
-    select_group(g, grp);
     __shared__ __attribute__((aligned(16))) half_t xs[2][16 * MT * SK_XS];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l16 = lane & 15, lk = lane >> 4;
-    const int n0 = blockIdx.x * (16 * NWV) + wave * 16;
+    // the tiles of all members, laid end to end, are dealt out in runs of consecutive tiles: the first `full` blocks take NWV
+    // tiles each, the others NWV - 1; a wave without a tile keeps the block's loads, barriers and arithmetic but reads one and
+    // the same weight chunk over and over (cache hits) and stores nothing
+    const int tiles = tiles_per_member * grp.count;
+    const int full = tiles - (NWV - 1) * (int)gridDim.x;  // 1 .. gridDim.x (the launcher's choice of grid and NWV)
+    const int b = blockIdx.x;
+    const int tile = b * (NWV - 1) + min(b, full) + wave;
+    const bool active = wave < NWV - 1 || b < full;
+    const int member = min(tile / tiles_per_member, grp.count - 1);
+    const int n0 = active ? (tile - member * tiles_per_member) * 16 : 0;
+    const int wstep = active ? SK_KC : 0;
+    if (grp.count > 1) {
+        g.W = grp.W[member];
+        g.Y = grp.Y[member];
+        g.epi.bias = grp.bias[member];
+        g.ldy = grp.ldy[member];
+        g.epi.rows = grp.rows[member];
+    }
     const int nchunks = g.K / SK_KC;  // a multiple of DEPTH (the launcher checks)
     const int rot = blockIdx.x % nchunks;  // rotated chunk order, see gemm_skinny_nk_kernel
     auto chunk_at = [&](int i) { int c = rot + i; while (c >= nchunks) c -= nchunks; return c; };
@@ -180,7 +200,7 @@ __global__ __launch_bounds__(64 * NWV) void gemm_skinny_direct_kernel(GemmArgs g
         if (d == DEPTH - 2) load_x(chunk_at(0), xq[0]);
         if (d == DEPTH - 1) load_x(chunk_at(1), xq[1]);
 #pragma unroll
-        for (int s = 0; s < 8; ++s) bf[d][s] = *reinterpret_cast<const half8_t*>(w0 + chunk_at(d) * SK_KC + s * 32);
+        for (int s = 0; s < 8; ++s) bf[d][s] = *reinterpret_cast<const half8_t*>(w0 + chunk_at(d) * wstep + s * 32);
         asm volatile("" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
     }
@@ -192,7 +212,7 @@ __global__ __launch_bounds__(64 * NWV) void gemm_skinny_direct_kernel(GemmArgs g
     // end wrap around to valid addresses and are never multiplied.
     auto do_chunk = [&](int ch, int buf, half8_t (&b)[8]) {
         load_x(chunk_at(ch + 2), xq[buf]);
-        const half_t* wn = w0 + chunk_at(ch + DEPTH) * SK_KC;
+        const half_t* wn = w0 + chunk_at(ch + DEPTH) * wstep;
         // compiler-only fences keep every load where it is written (left alone, the compiler moves the X loads to the end
         // of the chunk, right in front of the LDS stores that wait for them)
         asm volatile("" ::: "memory");
@@ -216,27 +236,29 @@ __global__ __launch_bounds__(64 * NWV) void gemm_skinny_direct_kernel(GemmArgs g
         for (int d = 0; d < DEPTH; ++d) do_chunk(ch + d, d & 1, bf[d]);
     }
 #pragma unroll
-    for (int i = 0; i < MT; ++i) epilogue_store4<EPI>(g, g.Y, i * 16 + l16, n0 + 4 * lk, acc[i], true, &rm);
+    for (int i = 0; i < MT; ++i)
+        if (active) epilogue_store4<EPI>(g, g.Y, i * 16 + l16, n0 + 4 * lk, acc[i], true, &rm);
 }
 
 template <int MT, int NWV, int DEPTH>
-static void launch_direct(const GemmArgs& g, const GemmGroup& grp, const RowMap& rm, hipStream_t stream) {
-    const dim3 grid((g.N + 16 * NWV - 1) / (16 * NWV), grp.count), block(64 * NWV);
+static void launch_direct(const GemmArgs& g, const GemmGroup& grp, const RowMap& rm, int nblocks, hipStream_t stream) {
+    const dim3 grid(nblocks), block(64 * NWV);
+    const int tpm = (g.N + 15) / 16;
     switch (g.epi.kind) {
-        case LG_EPI_NONE: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_NONE, NWV, DEPTH>), grid, block, 0, stream, g, grp, rm); break;
-        case LG_EPI_BIAS: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_BIAS, NWV, DEPTH>), grid, block, 0, stream, g, grp, rm); break;
-        case LG_EPI_BIAS_GELU: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_BIAS_GELU, NWV, DEPTH>), grid, block, 0, stream, g, grp, rm); break;
-        case LG_EPI_BIAS_HEADS_ROWS: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_BIAS_HEADS_ROWS, NWV, DEPTH>), grid, block, 0, stream, g, grp, rm); break;
-        default: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_BIAS_HEADS, NWV, DEPTH>), grid, block, 0, stream, g, grp, rm); break;
+        case LG_EPI_NONE: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_NONE, NWV, DEPTH>), grid, block, 0, stream, g, grp, rm, tpm); break;
+        case LG_EPI_BIAS: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_BIAS, NWV, DEPTH>), grid, block, 0, stream, g, grp, rm, tpm); break;
+        case LG_EPI_BIAS_GELU: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_BIAS_GELU, NWV, DEPTH>), grid, block, 0, stream, g, grp, rm, tpm); break;
+        case LG_EPI_BIAS_HEADS_ROWS: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_BIAS_HEADS_ROWS, NWV, DEPTH>), grid, block, 0, stream, g, grp, rm, tpm); break;
+        default: hipLaunchKernelGGL((gemm_skinny_direct_kernel<MT, LG_EPI_BIAS_HEADS, NWV, DEPTH>), grid, block, 0, stream, g, grp, rm, tpm); break;
     }
 }
 template <int NWV, int DEPTH>
-static void launch_direct_mt(const GemmArgs& g, const GemmGroup& grp, const RowMap& rm, hipStream_t stream) {
+static void launch_direct_mt(const GemmArgs& g, const GemmGroup& grp, const RowMap& rm, int nblocks, hipStream_t stream) {
     switch ((g.M + 15) / 16) {
-        case 1: launch_direct<1, NWV, DEPTH>(g, grp, rm, stream); break;
-        case 2: launch_direct<2, NWV, DEPTH>(g, grp, rm, stream); break;
-        case 3: launch_direct<3, NWV, DEPTH>(g, grp, rm, stream); break;
-        default: launch_direct<4, NWV, DEPTH>(g, grp, rm, stream); break;
+        case 1: launch_direct<1, NWV, DEPTH>(g, grp, rm, nblocks, stream); break;
+        case 2: launch_direct<2, NWV, DEPTH>(g, grp, rm, nblocks, stream); break;
+        case 3: launch_direct<3, NWV, DEPTH>(g, grp, rm, nblocks, stream); break;
+        default: launch_direct<4, NWV, DEPTH>(g, grp, rm, nblocks, stream); break;
     }
 }
 
@@ -286,24 +308,26 @@ int launch_gemm_skinny_f16(const GemmArgs& g, const GemmGroup& grp, const RowMap
     const int mt = (g.M + 15) / 16;
     const StreamInfo si = stream_info(stream);
     const int cus = si.cus;  // compute units this stream's kernels run on: "one round of blocks" means this many
-    // Unsliced blocks need a block width (128, 96, 64 or, up to 16 token rows, 32 features) that gives one round of blocks on
-    // the stream's CUs, 3/4 of them to all of them (fewer leave CUs idle; a few more than a round double the time of the CUs
-    // that get two), or so many blocks that the last, partial round does not matter.  The widest such block re-reads the token
-    // rows least.
+    // Unsliced: the 16-feature tiles are dealt to one block per compute unit of the stream, 2 to 8 waves a block (the partly
+    // filled last wave sits in the first blocks only).  That needs enough tiles to give most compute units two waves, whole
+    // pipeline depths of chunks, and for the 2-wave block (four chunks deep) registers for one row tile only.  Problems with more
+    // tiles than 8 waves a block take many rounds of 4-wave blocks, where the partial last round no longer matters.
     {
-        const int widths[4] = {128, 96, 64, 32};
-        for (int wi = 0; wi < 4; ++wi) {
-            const int w = widths[wi];
-            // whole pipeline depths of chunks; the 2-wave block's registers hold its four-chunk pipeline for one row tile only
-            if (w == 32 ? (mt != 1 || g.K % (4 * SK_KC) != 0) : (g.K % (2 * SK_KC) != 0)) continue;
-            const int blocks = (g.N + w - 1) / w * grp.count;
-            if (blocks < cus * 3 / 4 || (blocks > cus && blocks < 4 * cus)) continue;
+        const int tiles = (g.N + 15) / 16 * grp.count;
+        int nwv = (tiles + cus - 1) / cus, nblocks = cus;
+        if (nwv > 8 && tiles >= 16 * cus) { nwv = 4; nblocks = (tiles + 3) / 4; }
+        if (nwv == 7) { nwv = 8; nblocks = (tiles + 7) / 8; }
+        const bool deep = nwv == 2;
+        if (nwv >= 2 && nwv <= 8 && tiles >= cus * 3 / 2 && g.K % ((deep ? 4 : 2) * SK_KC) == 0 && (!deep || mt == 1) &&
+            (int64_t)(nwv - 1) * nblocks < tiles && tiles <= (int64_t)nwv * nblocks) {  // what the kernel's dealing assumes
             *handled = true;
-            switch (w) {
-                case 128: launch_direct_mt<8, 2>(g, grp, rm, stream); break;
-                case 96: launch_direct_mt<6, 2>(g, grp, rm, stream); break;
-                case 64: launch_direct_mt<4, 2>(g, grp, rm, stream); break;
-                default: launch_direct<1, 2, 4>(g, grp, rm, stream); break;
+            switch (nwv) {
+                case 2: launch_direct<1, 2, 4>(g, grp, rm, nblocks, stream); break;
+                case 3: launch_direct_mt<3, 2>(g, grp, rm, nblocks, stream); break;
+                case 4: launch_direct_mt<4, 2>(g, grp, rm, nblocks, stream); break;
+                case 5: launch_direct_mt<5, 2>(g, grp, rm, nblocks, stream); break;
+                case 6: launch_direct_mt<6, 2>(g, grp, rm, nblocks, stream); break;
+                default: launch_direct_mt<8, 2>(g, grp, rm, nblocks, stream); break;
             }
             return check_launch("gemm_f16_skinny");
         }
