@@ -119,6 +119,15 @@ __global__ __launch_bounds__(256) void gemm_f16_generic(GemmArgs g) {
     }
 
     const bool vec_ok = ALIGNED && (EPI == LG_EPI_BIAS_HEADS ? (g.epi.d % 4 == 0) : (g.ldy % 4 == 0));
+    if (EPI == LG_EPI_BIAS_GEGLU) {
+        // a wave's four 16-feature tiles are two (gate, up) pairs (N % 32 == 0, tiles start at multiples of 64)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; j += 2)
+                epilogue_geglu4(g, Y, m0 + wm * 64 + i * 16 + l16, n0 + wn * 64 + j * 16 + 4 * lk, acc[i][j], acc[i][j + 1], vec_ok);
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -140,6 +149,7 @@ static void launch_generic_epi(const GemmArgs& g, dim3 grid, hipStream_t stream)
         case LG_EPI_NONE: hipLaunchKernelGGL((gemm_f16_generic<WL, LG_EPI_NONE, ALIGNED>), grid, dim3(256), 0, stream, g); break;
         case LG_EPI_BIAS: hipLaunchKernelGGL((gemm_f16_generic<WL, LG_EPI_BIAS, ALIGNED>), grid, dim3(256), 0, stream, g); break;
         case LG_EPI_BIAS_GELU: hipLaunchKernelGGL((gemm_f16_generic<WL, LG_EPI_BIAS_GELU, ALIGNED>), grid, dim3(256), 0, stream, g); break;
+        case LG_EPI_BIAS_GEGLU: hipLaunchKernelGGL((gemm_f16_generic<WL, LG_EPI_BIAS_GEGLU, ALIGNED>), grid, dim3(256), 0, stream, g); break;
         default: hipLaunchKernelGGL((gemm_f16_generic<WL, LG_EPI_BIAS_HEADS, ALIGNED>), grid, dim3(256), 0, stream, g); break;
     }
 }
@@ -288,10 +298,11 @@ int lg_gemm_f16(int transa, int transb, int m, int n, int k, const void* A, int 
 int lg_gemm_fused_f16(int transa, int m, int n, int k, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
                       int epilogue, const void* bias, int epi_arg0, int epi_arg1, int epi_arg2, void* stream) {
     int rc = check_blas_args("gemm_fused_f16", transa, 0, m, n, k, A, lda, B, ldb, C,
-                             epilogue == LG_EPI_BIAS_HEADS ? (m > 1 ? m : 1) : ldc, 1);
+                             epilogue == LG_EPI_BIAS_HEADS ? (m > 1 ? m : 1) : (epilogue == LG_EPI_BIAS_GEGLU ? (ldc < m / 2 ? 0 : m) : ldc), 1);
     if (rc) return rc;
-    if (epilogue < LG_EPI_NONE || epilogue > LG_EPI_BIAS_HEADS) { set_error("gemm_fused_f16: unknown epilogue %d", epilogue); return LG_ERR_INVALID; }
+    if (epilogue != LG_EPI_BIAS_GEGLU && (epilogue < LG_EPI_NONE || epilogue > LG_EPI_BIAS_HEADS)) { set_error("gemm_fused_f16: unknown epilogue %d", epilogue); return LG_ERR_INVALID; }
     if (epilogue != LG_EPI_NONE && !bias) { set_error("gemm_fused_f16: epilogue needs a bias"); return LG_ERR_INVALID; }
+    if (epilogue == LG_EPI_BIAS_GEGLU && m % 32 != 0) { set_error("gemm_fused_f16: the GeGLU epilogue needs features %% 32 == 0 (gate and up interleaved in groups of 16)"); return LG_ERR_INVALID; }
     if (epilogue == LG_EPI_BIAS_HEADS) {
         const int seq = epi_arg0, d = epi_arg1;
         if (seq <= 0 || d <= 0 || m % d != 0 || n % seq != 0 || d % 4 != 0 || ldc < seq ||

@@ -143,6 +143,24 @@ __device__ __forceinline__ void epilogue_store4(const GemmArgs& g, half_t* Yb, i
     }
 }
 
+// LG_EPI_BIAS_GEGLU: `gate` holds features n..n+3 of token row m (n % 32 < 16: a gate group), `up` features n+16..n+19 (the up
+// columns of the same indices); the product goes to columns (n / 32) * 16 + n % 16 .. + 3 of the [M, N / 2] output.
+__device__ __forceinline__ void epilogue_geglu4(const GemmArgs& g, half_t* Yb, int m, int n, float4_t gate, float4_t up, bool vec_ok) {
+    if (m >= g.M || n >= g.N) return;
+    float v[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+        v[r] = gelu_tanh(gate[r] + (float)g.epi.bias[n + r]) * (up[r] + (float)g.epi.bias[n + 16 + r]);
+    const int64_t base = (int64_t)m * g.ldy + (n >> 5) * 16 + (n & 15);
+    if (vec_ok) {
+        half4_t o = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+        *reinterpret_cast<half4_t*>(Yb + base) = o;
+    } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) Yb[base + r] = (half_t)v[r];
+    }
+}
+
 // ---- split-K support shared by the weight-streaming and the pipelined kernel (gemm_skinny.hip) --------------------------
 constexpr int LG_EPI_PARTIAL = 100;  // kernel-internal: store the fp32 accumulators of K-slice `split` to partial[split][M][N]
 // The fp32 partials live in the stream's workspace (StreamInfo::ws, allocated when the stream was created or attached); a

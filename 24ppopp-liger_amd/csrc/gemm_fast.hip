@@ -245,6 +245,35 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles
         }
         return;
     }
+    if (EPI == LG_EPI_BIAS_GEGLU) {
+        // the wave's 16-feature tiles are (gate, up) pairs (NJ even): out[m][(n / 32) * 16 + n % 16 ..] = gelu(gate + b) * (up + b)
+        float bg[NJ / 2 + 1][4], bu[NJ / 2 + 1][4];
+        int col[NJ / 2 + 1];
+#pragma unroll
+        for (int jp = 0; jp < NJ / 2; ++jp) {
+            const int n = n0 + wn * (16 * NJ) + jp * 32 + 4 * lk;
+            const half4_t g4 = *reinterpret_cast<const half4_t*>(g.epi.bias + n);
+            const half4_t u4 = *reinterpret_cast<const half4_t*>(g.epi.bias + n + 16);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) { bg[jp][r] = (float)g4[r]; bu[jp][r] = (float)u4[r]; }
+            col[jp] = (n >> 5) * 16 + (n & 15);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int m = m0 + wm * 128 + i * 16 + l16;
+            if (m >= g.M) continue;
+            half_t* yrow = g.Y + (int64_t)m * g.ldy;
+#pragma unroll
+            for (int jp = 0; jp < NJ / 2; ++jp) {
+                float v[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) v[r] = gelu_tanh(acc[i][2 * jp][r] + bg[jp][r]) * (acc[i][(2 * jp + 1) % NJ][r] + bu[jp][r]);
+                const half4_t o = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+                *reinterpret_cast<half4_t*>(yrow + col[jp]) = o;
+            }
+        }
+        return;
+    }
     float bias_v[NJ][4];
     int64_t col_off[NJ];
 #pragma unroll
@@ -326,6 +355,9 @@ static int launch_fast_epi(const GemmArgs& g, int tiles_m, int tiles_n, const St
             case LG_EPI_NONE: LG_FAST(LG_EPI_NONE); break;
             case LG_EPI_BIAS: LG_FAST(LG_EPI_BIAS); break;
             case LG_EPI_BIAS_GELU: LG_FAST(LG_EPI_BIAS_GELU); break;
+            case LG_EPI_BIAS_GEGLU:
+                if constexpr (NJ % 2 == 0) LG_FAST(LG_EPI_BIAS_GEGLU);  // the launcher picks an even tile width for it
+                break;
             default: LG_FAST(LG_EPI_BIAS_HEADS); break;
         }
     }
@@ -352,6 +384,7 @@ int launch_gemm_fast_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t 
     long best_cost = 0;
     for (int nj = 4; nj >= 2; --nj) {
         if (g.N % (64 * nj)) continue;
+        if (nj == 3 && g.epi.kind == LG_EPI_BIAS_GEGLU) continue;  // a wave must hold whole (gate, up) pairs of 16-feature tiles
         const long tiles = (long)tiles_m * (g.N / (64 * nj));
         // narrower tiles move more operand bytes per flop: about 3 % / 35 % more time per unit of width (measured)
         const long cost = ((tiles + si.cus - 1) / si.cus) * nj * (nj == 4 ? 100 : nj == 3 ? 103 : 135);

@@ -282,8 +282,32 @@ __global__ __launch_bounds__(256) void gemm_skinny_reduce_kernel(GemmArgs g, con
     }
 }
 
+// GeGLU: one thread per 4 consecutive OUTPUT columns; it sums the slices of the gate quad and of the up quad 16 features on
+__global__ __launch_bounds__(256) void gemm_skinny_reduce_geglu_kernel(GemmArgs g, const float* partial, int nsplit) {
+    const int nq = g.N / 8;  // output quads per token row (N % 32 == 0)
+    const int64_t quads = (int64_t)g.M * nq;
+    for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < quads; q += (int64_t)gridDim.x * blockDim.x) {
+        const int m = (int)(q / nq), c = (int)(q % nq) * 4;
+        const int n = (c >> 4) * 32 + (c & 15);
+        float4_t sg = float4_t{0.f, 0.f, 0.f, 0.f}, su = float4_t{0.f, 0.f, 0.f, 0.f};
+        for (int sp = 0; sp < nsplit; ++sp) {
+            const float* p = partial + ((int64_t)sp * g.M + m) * g.N + n;
+            sg += *reinterpret_cast<const float4_t*>(p);
+            su += *reinterpret_cast<const float4_t*>(p + 16);
+        }
+        epilogue_geglu4(g, g.Y, m, n, sg, su, (g.ldy % 4 == 0) && aligned_dev16(g.Y));
+    }
+}
+
 void launch_splitk_reduce(const GemmArgs& g, const float* partial, int nsplit, hipStream_t stream, const RowMap* rows) {
     const dim3 block(256);
+    if (g.epi.kind == LG_EPI_BIAS_GEGLU) {
+        const int64_t gq = (int64_t)g.M * (g.N / 8);
+        int gg = (int)((gq + 255) / 256);
+        if (gg > 4096) gg = 4096;
+        hipLaunchKernelGGL(gemm_skinny_reduce_geglu_kernel, dim3(gg), block, 0, stream, g, partial, nsplit);
+        return;
+    }
     const int64_t quads = (int64_t)g.M * ((g.N + 3) / 4);
     int rgrid = (int)((quads + 255) / 256);
     if (rgrid > 4096) rgrid = 4096;
@@ -306,6 +330,9 @@ int launch_gemm_skinny_f16(const GemmArgs& g, const GemmGroup& grp, const RowMap
     if (g.epi.kind == LG_EPI_BIAS_HEADS_ROWS && !rows) return LG_OK;
     const RowMap rm = rows ? *rows : RowMap{};
     const int mt = (g.M + 15) / 16;
+    // GeGLU pairs features 16 apart, which sit in different waves of the unsliced kernel: such problems take the sliced kernel
+    // below (one slice when N alone fills the chip), whose reduce step forms the product
+    const bool geglu = g.epi.kind == LG_EPI_BIAS_GEGLU;
     const StreamInfo si = stream_info(stream);
     const int cus = si.cus;  // compute units this stream's kernels run on: "one round of blocks" means this many
     // Unsliced: the 16-feature tiles are dealt to one block per compute unit of the stream, 2 to 8 waves a block (the partly
@@ -318,7 +345,7 @@ int launch_gemm_skinny_f16(const GemmArgs& g, const GemmGroup& grp, const RowMap
         if (nwv > 8 && tiles >= 16 * cus) { nwv = 4; nblocks = (tiles + 3) / 4; }
         if (nwv == 7) { nwv = 8; nblocks = (tiles + 7) / 8; }
         const bool deep = nwv == 2;
-        if (nwv >= 2 && nwv <= 8 && tiles >= cus * 3 / 2 && g.K % ((deep ? 4 : 2) * SK_KC) == 0 && (!deep || mt == 1) &&
+        if (!geglu && nwv >= 2 && nwv <= 8 && tiles >= cus * 3 / 2 && g.K % ((deep ? 4 : 2) * SK_KC) == 0 && (!deep || mt == 1) &&
             (int64_t)(nwv - 1) * nblocks < tiles && tiles <= (int64_t)nwv * nblocks) {  // what the kernel's dealing assumes
             *handled = true;
             switch (nwv) {

@@ -109,6 +109,7 @@ int launch_gemv_f16(const GemmArgs& g, const GemmGroup& grp, const RowMap* rows,
     if (smem > (size_t)GV_MAX_LDS) return LG_OK;
     if (!aligned16(g.X) || (g.ldx % 8) || (g.ldw % 8) || !group_aligned(g, grp)) return LG_OK;
     if (g.epi.kind == LG_EPI_BIAS_HEADS_ROWS && (!rows || g.M > LG_ROWMAP_MAX)) return LG_OK;
+    if (g.epi.kind == LG_EPI_BIAS_GEGLU) return LG_OK;  // pairs features 16 apart: left to the sliced kernel and its reduce step
     *handled = true;
     const RowMap rm = rows ? *rows : RowMap{};
     const dim3 grid((g.N + 4 * GV_ROWS - 1) / (4 * GV_ROWS), grp.count), block(256);

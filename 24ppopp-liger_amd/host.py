@@ -130,6 +130,19 @@ def make_poisson_trace(lam, n, batch, seq_lo, seq_hi, seq_round, n_decode, seed)
     return [{"arrival_s": arr[i], "batch": batch, "seq": seq[i], "n_decode": n_decode} for i in range(n)]
 
 
+def _interleave16(n, inverse=False):
+    """Index vector of the stored order of n = 2 f features [first half | second half] interleaved in groups of 16:
+    stored[p] = logical[idx[p]] (inverse: logical[c] = stored[idx[c]])."""
+    f = n // 2
+    p = np.arange(n)
+    idx = (p // 32) * 16 + p % 16 + np.where(p % 32 >= 16, f, 0)
+    if not inverse:
+        return idx
+    inv = np.empty(n, dtype=np.int64)
+    inv[idx] = p
+    return inv
+
+
 class Model:
     """One tensor-parallel shard of a stack of encoder layers, assembled as launch vectors by the C++ runtime."""
 
@@ -158,7 +171,8 @@ class Model:
         return lib.lgh_model_stream(self.h)
 
     def param_info(self):
-        """name -> dict(ptr, elems, rows, cols, transposed); rows x cols is the logical [in, out] shape"""
+        """name -> dict(ptr, elems, rows, cols, transposed, interleave16); rows x cols is the logical [in, out] shape;
+        interleave16: the out dimension (or the vector) is stored with its two halves interleaved in groups of 16"""
         out = {}
         for i in range(lib.lgh_model_param_count(self.h)):
             name = C.create_string_buffer(128)
@@ -166,7 +180,8 @@ class Model:
             r, c, t = _i(), _i(), _i()
             check(lib.lgh_model_param_info(self.h, i, name, 128, C.byref(ptr), C.byref(n), C.byref(r), C.byref(c), C.byref(t)),
                   "lgh_model_param_info")
-            out[name.value.decode()] = dict(ptr=ptr.value, elems=n.value, rows=r.value, cols=c.value, transposed=t.value)
+            out[name.value.decode()] = dict(ptr=ptr.value, elems=n.value, rows=r.value, cols=c.value, transposed=t.value & 1,
+                                            interleave16=(t.value >> 1) & 1)
         return out
 
     def params(self):
@@ -184,8 +199,9 @@ class Model:
             a = raw.astype(np.float32)
             if info["rows"] > 1:
                 a = a.reshape(info["cols"], info["rows"]).T if info["transposed"] else a.reshape(info["rows"], info["cols"])
-                a = np.ascontiguousarray(a)
-            res[name] = a
+            if info["interleave16"]:
+                a = a[..., _interleave16(a.shape[-1], inverse=True)]
+            res[name] = np.ascontiguousarray(a)
         return res
 
     def upload_params(self, values):
@@ -201,6 +217,9 @@ class Model:
             if i["rows"] > 1:
                 if a.shape != (i["rows"], i["cols"]):
                     raise ValueError("%s: expected shape %s, got %s" % (name, (i["rows"], i["cols"]), a.shape))
+            if i["interleave16"]:
+                a = a[..., _interleave16(a.shape[-1])]
+            if i["rows"] > 1:
                 a = a.T if i["transposed"] else a
             raw = np.ascontiguousarray(a, dtype=dt).ravel()
             if raw.size != i["elems"]:

@@ -47,7 +47,9 @@ struct ParamRef {
     void* ptr;
     int64_t elems;
     int rows = 1, cols = 0;   // logical shape [in, out] of a weight matrix (vectors: rows = 1)
-    int transposed = 0;       // 1: stored as [out, in]
+    int transposed = 0;       // bit 0: stored as [out, in]; bit 1: the out dimension (or the vector) is stored with its two
+                              // halves interleaved in groups of 16 (stored group 2g = logical [16g, 16g+16) of the first
+                              // half, stored group 2g+1 = the same range of the second half)
 };
 
 // ---------------------------------------------------------------------------------------------------
@@ -63,12 +65,13 @@ class Linear_Col {  // linear.h:68-109: output features split across ranks
     std::vector<FuncWrap> FuncWrapVec;
 
     int weight_layout = 0;  // 0: [k, n_local] row-major; 1: [n_local, k] row-major (multiplied with transa = T)
+    int interleave16 = 0;   // 1: output features stored as (gate, up) groups of 16 (the GeGLU epilogue's order)
 
     Linear_Col(const StaticInitParam& SParams_, const int& k_, const int& n_, int weight_layout_ = 0)
         : k(k_), n(n_), SParams(SParams_), weight_layout(weight_layout_) {
         weights = dev_alloc<T>((size_t)k * n / SParams.world_size);
     }
-    ParamRef param(const std::string& name) { return ParamRef{name, weights, (int64_t)k * n_local(), k, n_local(), weight_layout}; }
+    ParamRef param(const std::string& name) { return ParamRef{name, weights, (int64_t)k * n_local(), k, n_local(), weight_layout | (interleave16 << 1)}; }
     int n_local() const { return n / SParams.world_size; }
     void init_weights(uint64_t seed, uint64_t tensor_id, float stddev = 0.02f) {
         dev_fill_normal(weights, (int64_t)k * n_local(), seed, tensor_id, 0.f, stddev);
@@ -178,6 +181,7 @@ class Bert_MLP {
         // GeGLU: FFN-1 produces [gate | up], 2 F local columns
         linear_col = new Linear_Col<T>(SParam, k, intermediate_size * gate_mult(), BertParams.weight_layout);
         linear_row = new Linear_Row<T>(SParam, intermediate_size, k, BertParams.weight_layout);
+        linear_col->interleave16 = geglu_fused() ? 1 : 0;
         bias = dev_alloc<T>(f_local() * gate_mult());
         bias2 = dev_alloc<T>(k);
         dev_fill_const(bias, f_local() * gate_mult(), 0.f);
@@ -185,10 +189,17 @@ class Bert_MLP {
     }
     int f_local() const { return intermediate_size / SParam.world_size; }
     int gate_mult() const { return BertParams.ffn_act == FFN_GEGLU ? 2 : 1; }
-    // elements of the FFN-1 output buffer per token (GeGLU keeps [gate | up] and the product)
+    // GeGLU in the fused fp16 assembly: FFN-1's weight and bias are stored with gate and up interleaved in groups of 16 features,
+    // and the product is formed in the GEMM's epilogue (no [gate | up] buffer, no separate pass over it)
+    static bool geglu_fused(const BertInitParam& P, const StaticInitParam& S, int hidden) {
+        const int64_t F = (P.ffn_inner > 0 ? P.ffn_inner : 4 * hidden) / S.world_size;
+        return P.ffn_act == FFN_GEGLU && P.fused && dtype_of<T>::value == LG_F16 && F % 16 == 0;
+    }
+    bool geglu_fused() const { return geglu_fused(BertParams, SParam, n); }
+    // elements of the FFN-1 output buffer per token (unfused GeGLU keeps [gate | up] and the product)
     static int64_t inner_per_token(const BertInitParam& P, const StaticInitParam& S, int hidden) {
         const int64_t F = (P.ffn_inner > 0 ? P.ffn_inner : 4 * hidden) / S.world_size;
-        return P.ffn_act == FFN_GEGLU ? 3 * F : F;
+        return (P.ffn_act == FFN_GEGLU && !geglu_fused(P, S, hidden)) ? 3 * F : F;
     }
     void init_weights(uint64_t seed, uint64_t base) {
         linear_col->init_weights(seed, base + 0);
@@ -198,7 +209,7 @@ class Bert_MLP {
     }
     void params(const std::string& prefix, std::vector<ParamRef>& out) {
         out.push_back(linear_col->param(prefix + "w1"));
-        out.push_back({prefix + "b1", bias, f_local() * gate_mult(), 1, f_local() * gate_mult(), 0});
+        out.push_back({prefix + "b1", bias, f_local() * gate_mult(), 1, f_local() * gate_mult(), geglu_fused() ? 2 : 0});
         out.push_back(linear_row->param(prefix + "w2"));
         out.push_back({prefix + "b2", bias2, k, 1, k, 0});
     }
@@ -207,7 +218,13 @@ class Bert_MLP {
         FuncWrapVec.clear();
         if (!inner) inner = linear_row_output;
         const int F = f_local();
-        if (BertParams.ffn_act == FFN_GEGLU) {
+        if (geglu_fused()) {
+            GemmDesc g = linear_col->desc(input, inner, m);
+            g.epilogue = LG_EPI_BIAS_GEGLU;
+            g.bias = bias;
+            g.ldc = F;
+            FuncWrapVec.push_back(FuncWrap(1.0f, GEMM, [g](const DynamicInitParam& D) { GemmEx(D, g); }, g, "ffn1+bias+geglu"));
+        } else if (BertParams.ffn_act == FFN_GEGLU) {
             // inner holds [m, F] (the product) followed by [m, 2F] (gate | up)
             T* gu = inner + (int64_t)m * F;
             std::vector<FuncWrap> v = linear_col->forward(input, gu, m);

@@ -174,7 +174,7 @@ inline SubDict SubFileToDict(const std::string& filename) {
 // The reference scales cuBLAS's m by n/factor without moving any pointer, so all of its pieces recompute the leading
 // columns; here the weight / bias / output (or activation / output) pointers are offset so that the pieces of one
 // GEMM tile its output exactly.  Unit boundaries are rounded to the epilogue's granularity (whole heads for the
-// head-transposing epilogue, 8 elements otherwise) so that every piece keeps the vectorised paths.
+// head-transposing epilogue, whole gate/up groups for the GeGLU epilogue, 8 elements otherwise) so that every piece keeps the vectorised paths.
 inline int split_point(int extent, int unit, int factor, int gran) {
     if (unit <= 0) return 0;
     if (unit >= factor) return extent;
@@ -188,11 +188,13 @@ inline FuncWrap decompose_callback(const FuncWrap& old_func, int factor, int n, 
     const size_t es = (g.dtype == LG_F16) ? 2 : 4;
     if (g.epilogue == LG_EPI_BIAS_HEADS) axis = SPLIT_OUT_COLS;  // token rows would move the (batch, seq) decode of rows
     if (axis == SPLIT_OUT_COLS) {
-        const int gran = (g.epilogue == LG_EPI_BIAS_HEADS) ? g.epi_d : 8;
+        // GeGLU: whole (gate, up) groups of 32 features, which produce 16 output columns
+        const int gran = (g.epilogue == LG_EPI_BIAS_HEADS) ? g.epi_d : (g.epilogue == LG_EPI_BIAS_GEGLU ? 32 : 8);
         const int c0 = split_point(g.m, start, factor, gran), c1 = split_point(g.m, start + n, factor, gran);
         g.A = (const char*)g.A + (g.transa ? (size_t)c0 * g.lda : (size_t)c0) * es;
         if (g.bias) g.bias = (const char*)g.bias + (size_t)c0 * es;
         if (g.epilogue == LG_EPI_BIAS_HEADS) g.C = (char*)g.C + (size_t)(c0 / g.epi_d) * g.ldc * g.epi_d * es;
+        else if (g.epilogue == LG_EPI_BIAS_GEGLU) g.C = (char*)g.C + (size_t)(c0 / 2) * es;
         else g.C = (char*)g.C + (size_t)c0 * es;
         g.m = c1 - c0;
     } else {

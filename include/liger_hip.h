@@ -180,6 +180,11 @@ int lg_gemm_strided_batched_f16(int transa, int transb, int m, int n, int k, con
                                size_per_head, epi_arg2 = heads per batch entry in C (0 -> m / size_per_head;
                                larger when C is a slice of a wider buffer), and ldc = rows reserved per
                                (batch, head) in C (>= seq; > seq when C is a KV cache)                     */
+#define LG_EPI_BIAS_GEGLU 5 /* the m output features are the gate and up halves of a GeGLU FFN-1, interleaved in groups
+                               of 16: features [32g, 32g+16) are gate columns [16g, 16g+16), features [32g+16, 32g+32)
+                               the up columns of the same indices (A and bias are stored in that order); C is
+                               [n tokens, m/2] (ldc >= m/2) with C[t, c] = gelu_tanh(gate_c + bias) * (up_c + bias)
+                               == lg_gemm + lg_add_bias_geglu on the de-interleaved operands.  m % 32 == 0.   */
 /* lg_gemm_f16 with a fused epilogue (the bias / GELU / head-transpose kernels that follow the GEMMs in
  * the launch vector, bert_layer.h:54-56,139-142, folded into the GEMM's store).  No reference
  * counterpart; results equal the two-kernel sequence up to one fp16 rounding. */

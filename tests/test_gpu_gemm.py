@@ -56,6 +56,55 @@ def test_gemm(dev, po, dt, transa, M, N, K):
     assert max_rel_err(C2, ref) < 1e-5
 
 
+def _interleave16(n):
+    """stored order of n = 2 f features [gate | up] interleaved in groups of 16: stored[p] = logical[idx[p]]"""
+    p = np.arange(n)
+    return (p // 32) * 16 + p % 16 + np.where(p % 32 >= 16, n // 2, 0)
+
+
+# (tokens, f, k): the pipelined kernel with 256- and 128-wide tiles, the generic kernel (ragged k / tokens / f % 64 != 0),
+# the weight-streaming kernels (few tokens; one slice and several), a single token row
+GEGLU_SHAPES = [(512, 512, 256), (256, 192, 128), (300, 1024, 192), (70, 48, 72), (130, 16, 40), (32, 2048, 1024),
+                (32, 256, 2048), (8, 8192, 512), (1, 512, 2048), (64, 1024, 1536), (4096, 256, 64)]
+
+
+@pytest.mark.parametrize("transa", [0, 1])
+@pytest.mark.parametrize("M,F,K", GEGLU_SHAPES)
+def test_gemm_geglu_epilogue(dev, po, transa, M, F, K):
+    """FFN-1 of a GeGLU MLP with the product formed in the GEMM's epilogue: the weight [K, 2F] = [gate | up] and its bias are
+    handed over with gate and up interleaved in groups of 16 features, the result [M, F] must equal the oracle's
+    GEMM -> bias + GeGLU on the plain operands."""
+    X = rnd(po, M * K, 40, 1).reshape(M, K)
+    W = rnd(po, K * 2 * F, 41, 1, 0.05).reshape(K, 2 * F)
+    bias = rnd(po, 2 * F, 42, 1, 0.3)
+    ref = po.add_bias_geglu(po.gemm(X, W, 1), bias, 1)
+    idx = _interleave16(2 * F)
+    Ws, bs = np.ascontiguousarray(W[:, idx]), np.ascontiguousarray(bias[idx])
+    A, lda = (np.ascontiguousarray(Ws.T), K) if transa else (Ws, 2 * F)
+    dY = dev.empty((M, F), 1)
+    dev.call("lg_gemm_fused_f16", transa, 2 * F, M, K, dev.up(A, 1), lda, dev.up(X, 1), K, dY, F, 5, dev.up(bs, 1), 0, 0, 0)
+    assert max_rel_err(dev.down(dY), ref) < 4e-3
+    # a wider destination (ldc > f) leaves the columns beyond f alone
+    wide = dev.up(np.full((M, F + 8), 7.0, dtype=np.float32), 1)
+    dev.call("lg_gemm_fused_f16", transa, 2 * F, M, K, dev.up(A, 1), lda, dev.up(X, 1), K, wide, F + 8, 5, dev.up(bs, 1), 0, 0, 0)
+    got = dev.down(wide)
+    assert np.all(got[:, F:] == 7.0) and max_rel_err(got[:, :F], ref) < 4e-3
+
+
+def test_gemm_geglu_epilogue_rejects_bad_shapes(dev):
+    x = dev.empty((4, 64), 1)
+    w = dev.empty((48, 64), 1)
+    y = dev.empty((4, 24), 1)
+    b = dev.empty((48,), 1)
+    with pytest.raises(dev.capi.LigerError):   # features not a multiple of 32
+        dev.call("lg_gemm_fused_f16", 1, 48, 4, 64, w, 64, x, 64, y, 24, 5, b, 0, 0, 0)
+    w2, b2 = dev.empty((64, 64), 1), dev.empty((64,), 1)
+    with pytest.raises(dev.capi.LigerError):   # ldc below features / 2
+        dev.call("lg_gemm_fused_f16", 1, 64, 4, 64, w2, 64, x, 64, y, 24, 5, b2, 0, 0, 0)
+    with pytest.raises(dev.capi.LigerError):   # no bias
+        dev.call("lg_gemm_fused_f16", 1, 64, 4, 64, w2, 64, x, 64, y, 32, 5, None, 0, 0, 0)
+
+
 @pytest.mark.parametrize("dt", [0, 1])
 def test_gemm_subrange_concatenation_is_exact(dev, po, dt):
     """Decomposition invariant: computing column slices / row slices of Y separately (pointer offsets, same
