@@ -9,7 +9,7 @@
 
 namespace lg {
 
-int launch_gemm_fast_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t stream, bool* handled);
+int launch_gemm_fast_f16(const GemmArgs& g, const GemmGroup& grp, int wlayout, int batch, hipStream_t stream, bool* handled);
 int launch_gemm_skinny_f16(const GemmArgs& g, const GemmGroup& grp, const RowMap* rows, int wlayout, int batch, hipStream_t stream, bool* handled);
 int launch_gemv_f16(const GemmArgs& g, const GemmGroup& grp, const RowMap* rows, int wlayout, int batch, hipStream_t stream, bool* handled);
 int launch_gemm_skinny_kn_f16(const GemmArgs& g, const RowMap* rows, int wlayout, int batch, hipStream_t stream, bool* handled);
@@ -158,9 +158,9 @@ static int gemm_f16_dispatch(GemmArgs g, int wlayout, int batch, hipStream_t str
     if (g.M == 0 || g.N == 0 || batch == 0) return LG_OK;
     if (g.K == 0) { set_error("gemm: k == 0 is not supported"); return LG_ERR_INVALID; }
     bool handled = false;
-    int rc = launch_gemm_fast_f16(g, wlayout, batch, stream, &handled);
-    if (handled) return rc;
     const GemmGroup one = single_group(g);
+    int rc = launch_gemm_fast_f16(g, one, wlayout, batch, stream, &handled);
+    if (handled) return rc;
     rc = launch_gemv_f16(g, one, nullptr, wlayout, batch, stream, &handled);
     if (handled) return rc;
     rc = launch_gemm_skinny_f16(g, one, nullptr, wlayout, batch, stream, &handled);
@@ -329,10 +329,11 @@ int lg_gemm_fused_grouped_f16(int transa, int m, int n, int k, int count, const 
         set_error("gemm_fused_grouped_f16: count must be 1..%d and the pointer arrays non-null", LG_MAX_GROUP);
         return LG_ERR_INVALID;
     }
-    // the weight-streaming kernels run the whole group as one launch; every other case is `count` plain calls
+    // the pipelined kernel (many token rows, either weight layout) and the weight-streaming kernels (few token rows, weights
+    // [out, in]) run the whole group as one launch; every other case is `count` plain calls
     GemmGroup grp{};
     grp.count = count;
-    bool one_launch = transa == 1 && m > 0 && n > 0 && k > 0 && count > 1 && B != nullptr;
+    bool one_launch = m > 0 && n > 0 && k > 0 && count > 1 && B != nullptr;
     for (int i = 0; i < count; ++i) {
         grp.W[i] = (const half_t*)A[i];
         grp.Y[i] = (half_t*)C[i];
@@ -364,10 +365,14 @@ int lg_gemm_fused_grouped_f16(int transa, int m, int n, int k, int count, const 
             g.Y = grp.Y[0]; g.ldy = grp.ldy[0]; g.strideY = 0;
             g.epi = Epilogue{epilogue, grp.bias[0], epi_arg0, epi_arg1, heads_total, 0};
             bool handled = false;
-            int rc = launch_gemv_f16(g, grp, nullptr, W_NK, 1, (hipStream_t)stream, &handled);
+            int rc = launch_gemm_fast_f16(g, grp, transa ? W_NK : W_KN, 1, (hipStream_t)stream, &handled);
             if (handled) return rc;
-            rc = launch_gemm_skinny_f16(g, grp, nullptr, W_NK, 1, (hipStream_t)stream, &handled);
-            if (handled) return rc;
+            if (transa == 1) {
+                rc = launch_gemv_f16(g, grp, nullptr, W_NK, 1, (hipStream_t)stream, &handled);
+                if (handled) return rc;
+                rc = launch_gemm_skinny_f16(g, grp, nullptr, W_NK, 1, (hipStream_t)stream, &handled);
+                if (handled) return rc;
+            }
         }
     }
     for (int i = 0; i < count; ++i) {

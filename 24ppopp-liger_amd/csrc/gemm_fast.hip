@@ -47,7 +47,7 @@ template <int NJ> __device__ __forceinline__ int unswz_kn(int k, int blk) {
 }
 
 template <int WL, int EPI, int NJ>
-__global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles_m, int tiles_n, float* partial, int kt_per_split, int cus) {
+__global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, GemmGroup grp, int tiles_m, int tiles_n, float* partial, int kt_per_split, int cus) {
     constexpr int FB_N = 64 * NJ;
     constexpr int X_TILE = FB_M * FB_K, W_TILE = FB_K * FB_N;  // halves per ring slot
     constexpr int WCH = (FB_K * FB_N) / 512 / 8;  // 1 KiB chunks of the W tile per wave (= NJ)
@@ -94,6 +94,17 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles
             tm = bid % tiles_m;
             tn = bid / tiles_m;
         }
+    }
+    // a group (problems that share X and the shape: the Q, K and V projections) lays its members' tile columns side by side;
+    // from here on g is the member's problem and n0 a feature index inside it
+    if (grp.count > 1) {
+        const int per = tiles_n / grp.count;
+        const int member = tn / per;
+        tn -= member * per;
+        g.W = grp.W[member];
+        g.Y = grp.Y[member];
+        g.epi.bias = grp.bias[member];
+        g.ldy = grp.ldy[member];
     }
     const int m0 = tm * FB_M, n0 = tn * FB_N;
     // K-slice of this workgroup (blockIdx.y; the whole K when the launch is not split): k-tiles [kt0, kt0 + ktiles)
@@ -318,7 +329,7 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, int tiles
 }
 
 template <int WL, int NJ>
-static int launch_fast_epi(const GemmArgs& g, int tiles_m, int tiles_n, const StreamInfo& si, hipStream_t stream) {
+static int launch_fast_epi(const GemmArgs& g, const GemmGroup& grp, int tiles_m, int tiles_n, const StreamInfo& si, hipStream_t stream) {
     const int tiles = tiles_m * tiles_n, ktiles = g.K / FB_K;
     const int cus = si.cus;
     // At most 256 token rows (one row of tiles, the continuation of the weight-streaming kernel's regime): the time is set by
@@ -327,7 +338,7 @@ static int launch_fast_epi(const GemmArgs& g, int tiles_m, int tiles_n, const St
     // holds, none on a stream without one).  Larger M never splits K, so that a token row's result does not depend on how many
     // other rows are in the batch (each output is one sequential sum over k).
     int nsplit = 1;
-    if (tiles_m == 1 && tiles <= cus / 2 && si.ws) {
+    if (tiles_m == 1 && tiles <= cus / 2 && si.ws && grp.count == 1) {
         nsplit = cus / tiles;
         if (nsplit > ktiles / 8) nsplit = ktiles / 8;
         if (nsplit > 16) nsplit = 16;
@@ -345,7 +356,7 @@ static int launch_fast_epi(const GemmArgs& g, int tiles_m, int tiles_n, const St
         /* set once per instantiation; the initialisation of a function-local static is thread-safe */              \
         static const hipError_t attr_rc = hipFuncSetAttribute((const void*)gemm_f16_fast<WL, E, NJ>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
         (void)attr_rc;                                                                                              \
-        hipLaunchKernelGGL((gemm_f16_fast<WL, E, NJ>), grid, block, smem, stream, g, tiles_m, tiles_n, partial, kt_per_split, cus); \
+        hipLaunchKernelGGL((gemm_f16_fast<WL, E, NJ>), grid, block, smem, stream, g, grp, tiles_m, tiles_n, partial, kt_per_split, cus); \
     } while (0)
     if (nsplit > 1) {
         LG_FAST(LG_EPI_PARTIAL);
@@ -365,7 +376,7 @@ static int launch_fast_epi(const GemmArgs& g, int tiles_m, int tiles_n, const St
     return LG_OK;
 }
 
-int launch_gemm_fast_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t stream, bool* handled) {
+int launch_gemm_fast_f16(const GemmArgs& g, const GemmGroup& grp, int wlayout, int batch, hipStream_t stream, bool* handled) {
     *handled = false;
     if (batch != 1) return LG_OK;
     if (g.K % FB_K || g.M <= 0 || g.N <= 0 || g.K <= 0) return LG_OK;
@@ -373,10 +384,14 @@ int launch_gemm_fast_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t 
     // for every token count the weight-streaming kernel does not take (M = 128: 182 us vs 331 us in the generic kernel for a
     // 16384 x 12288 weight), because with few token rows the time is set by how fast the weights stream in.
     if (g.M <= 64) return LG_OK;
-    if (!aligned16(g.X) || !aligned16(g.W) || !aligned16(g.Y) || (g.ldx % 8) || (g.ldw % 8)) return LG_OK;
+    if (!aligned16(g.X) || (g.ldx % 8) || (g.ldw % 8)) return LG_OK;
     if (g.ldx >= (1 << 22) || g.ldw >= (1 << 22)) return LG_OK;  // 256 rows x ld must fit the 31-bit tile offsets
-    if (g.epi.kind == LG_EPI_BIAS_HEADS ? (g.epi.d % 4 != 0) : (g.ldy % 4 != 0)) return LG_OK;
-    if (g.epi.kind != LG_EPI_NONE && (reinterpret_cast<uintptr_t>(g.epi.bias) & 7u)) return LG_OK;  // 8-byte bias loads
+    for (int i = 0; i < grp.count; ++i) {
+        if (!aligned16(grp.W[i]) || !aligned16(grp.Y[i])) return LG_OK;
+        if (g.epi.kind == LG_EPI_BIAS_HEADS ? (g.epi.d % 4 != 0) : (grp.ldy[i] % 4 != 0)) return LG_OK;
+        if (g.epi.kind != LG_EPI_NONE && (reinterpret_cast<uintptr_t>(grp.bias[i]) & 7u)) return LG_OK;  // 8-byte bias loads
+    }
+    if (grp.count > 1 && g.M <= FB_M) return LG_OK;  // one row of tiles may want K-slices, which take single problems only
     // tile width: the one that needs the least work-rounds on the stream's CUs (rounds x tile width); ties go to the wider tile
     const StreamInfo si = stream_info(stream);
     const int tiles_m = (g.M + FB_M - 1) / FB_M;
@@ -385,23 +400,23 @@ int launch_gemm_fast_f16(const GemmArgs& g, int wlayout, int batch, hipStream_t 
     for (int nj = 4; nj >= 2; --nj) {
         if (g.N % (64 * nj)) continue;
         if (nj == 3 && g.epi.kind == LG_EPI_BIAS_GEGLU) continue;  // a wave must hold whole (gate, up) pairs of 16-feature tiles
-        const long tiles = (long)tiles_m * (g.N / (64 * nj));
+        const long tiles = (long)tiles_m * (g.N / (64 * nj)) * grp.count;
         // narrower tiles move more operand bytes per flop: about 3 % / 35 % more time per unit of width (measured)
         const long cost = ((tiles + si.cus - 1) / si.cus) * nj * (nj == 4 ? 100 : nj == 3 ? 103 : 135);
         if (!best_nj || cost < best_cost) { best_nj = nj; best_cost = cost; }
     }
     if (!best_nj) return LG_OK;
     *handled = true;
-    const int tiles_n = g.N / (64 * best_nj);
+    const int tiles_n = g.N / (64 * best_nj) * grp.count;
     int rc;
     if (wlayout == W_NK) {
-        if (best_nj == 4) rc = launch_fast_epi<W_NK, 4>(g, tiles_m, tiles_n, si, stream);
-        else if (best_nj == 3) rc = launch_fast_epi<W_NK, 3>(g, tiles_m, tiles_n, si, stream);
-        else rc = launch_fast_epi<W_NK, 2>(g, tiles_m, tiles_n, si, stream);
+        if (best_nj == 4) rc = launch_fast_epi<W_NK, 4>(g, grp, tiles_m, tiles_n, si, stream);
+        else if (best_nj == 3) rc = launch_fast_epi<W_NK, 3>(g, grp, tiles_m, tiles_n, si, stream);
+        else rc = launch_fast_epi<W_NK, 2>(g, grp, tiles_m, tiles_n, si, stream);
     } else {
-        if (best_nj == 4) rc = launch_fast_epi<W_KN, 4>(g, tiles_m, tiles_n, si, stream);
-        else if (best_nj == 3) rc = launch_fast_epi<W_KN, 3>(g, tiles_m, tiles_n, si, stream);
-        else rc = launch_fast_epi<W_KN, 2>(g, tiles_m, tiles_n, si, stream);
+        if (best_nj == 4) rc = launch_fast_epi<W_KN, 4>(g, grp, tiles_m, tiles_n, si, stream);
+        else if (best_nj == 3) rc = launch_fast_epi<W_KN, 3>(g, grp, tiles_m, tiles_n, si, stream);
+        else rc = launch_fast_epi<W_KN, 2>(g, grp, tiles_m, tiles_n, si, stream);
     }
     return rc != LG_OK ? rc : check_launch("gemm_f16_fast");
 }

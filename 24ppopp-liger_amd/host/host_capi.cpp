@@ -257,8 +257,9 @@ void* lgh_model_create(int dtype, int max_batch, int max_seq, int head_num, int 
     return lgh_model_create_ex(dtype, max_batch, max_seq, head_num, size_per_head, layer_num, world_size, ffn_inner, norm_mode, causal,
                                fused, max_cache_len, factor, weight_layout, 0, 0, seed);
 }
-// ffn_act: 0 GELU, 1 GeGLU (FFN-1 is [H, 2F] = [gate | up]); packed_qkv: 1 = one [H, 3 Hl] projection + the fused
-// bias/transpose kernel (reference-shaped assembly without KV cache only)
+// ffn_act: 0 GELU, 1 GeGLU (FFN-1 is [H, 2F] = [gate | up]); packed_qkv: 1 = one [H, 3 Hl] projection, columns [q | k | v] (the
+// reference-shaped assembly follows it with the fused bias/transpose kernel, the fused assembly routes the columns in the GEMM's
+// epilogue; decode steps read the same packed parameters)
 void* lgh_model_create_ex(int dtype, int max_batch, int max_seq, int head_num, int size_per_head, int layer_num, int world_size,
                           int ffn_inner, int norm_mode, int causal, int fused, int max_cache_len, int factor, int weight_layout,
                           int ffn_act, int packed_qkv, uint64_t seed) {
@@ -269,7 +270,6 @@ void* lgh_model_create_ex(int dtype, int max_batch, int max_seq, int head_num, i
     }
     if (fused && dtype != 1) { fail("lgh_model_create: the fused assembly is fp16 only"); return nullptr; }
     if (max_cache_len > 0 && !fused) { fail("lgh_model_create: the KV cache needs the fused assembly"); return nullptr; }
-    if (packed_qkv && (fused || max_cache_len > 0)) { fail("lgh_model_create: the packed QKV projection belongs to the reference-shaped assembly (fused = 0, no KV cache)"); return nullptr; }
     if ((ffn_act != 0 && ffn_act != 1) || (packed_qkv != 0 && packed_qkv != 1)) { fail("lgh_model_create: bad ffn_act / packed_qkv"); return nullptr; }
     BertInitParam P(max_batch, max_seq, head_num, size_per_head, layer_num, 0, factor, 0);
     P.ffn_act = ffn_act; P.packed_qkv = packed_qkv;

@@ -67,20 +67,25 @@ class Linear_Col {  // linear.h:68-109: output features split across ranks
     int weight_layout = 0;  // 0: [k, n_local] row-major; 1: [n_local, k] row-major (multiplied with transa = T)
     int interleave16 = 0;   // 1: output features stored as (gate, up) groups of 16 (the GeGLU epilogue's order)
 
+    int lda_view = 0;       // > 0: `weights` points into a wider matrix with this leading dimension (one of q / k / v inside the
+                            // packed [H, 3 Hl] projection); the object then owns and initialises nothing
+
     Linear_Col(const StaticInitParam& SParams_, const int& k_, const int& n_, int weight_layout_ = 0)
         : k(k_), n(n_), SParams(SParams_), weight_layout(weight_layout_) {
         weights = dev_alloc<T>((size_t)k * n / SParams.world_size);
     }
+    Linear_Col(const StaticInitParam& SParams_, const int& k_, const int& n_, int weight_layout_, T* view, int lda)
+        : k(k_), n(n_), weights(view), SParams(SParams_), weight_layout(weight_layout_), lda_view(lda) {}
     ParamRef param(const std::string& name) { return ParamRef{name, weights, (int64_t)k * n_local(), k, n_local(), weight_layout | (interleave16 << 1)}; }
     int n_local() const { return n / SParams.world_size; }
     void init_weights(uint64_t seed, uint64_t tensor_id, float stddev = 0.02f) {
-        dev_fill_normal(weights, (int64_t)k * n_local(), seed, tensor_id, 0.f, stddev);
+        if (!lda_view) dev_fill_normal(weights, (int64_t)k * n_local(), seed, tensor_id, 0.f, stddev);
     }
     GemmDesc desc(T* input, T* output, int m) const {
         GemmDesc g;
         g.valid = true; g.dtype = dtype_of<T>::value; g.transa = weight_layout;
         g.m = n_local(); g.n = m; g.k = k;
-        g.A = weights; g.lda = weight_layout ? k : n_local(); g.B = input; g.ldb = k; g.C = output; g.ldc = n_local();
+        g.A = weights; g.lda = lda_view ? lda_view : (weight_layout ? k : n_local()); g.B = input; g.ldb = k; g.C = output; g.ldc = n_local();
         return g;
     }
     std::vector<FuncWrap> forward(T* input, T* output, int m) {
@@ -286,18 +291,30 @@ class Bert_MHA {
     Bert_MHA(const BertInitParam& BertParams_, const StaticInitParam& SParam_, const int& k_, const int& n_, T* workspace_)
         : k(k_), n(n_), SParam(SParam_), BertParams(BertParams_), workspace(workspace_) {
         scalar = 1.0f / sqrtf((float)BertParams.size_per_head);  // bert_layer.h:94
-        linear_q_col = new Linear_Col<T>(SParam, k, n, BertParams.weight_layout);
-        linear_k_col = new Linear_Col<T>(SParam, k, n, BertParams.weight_layout);
-        linear_v_col = new Linear_Col<T>(SParam, k, n, BertParams.weight_layout);
         linear_w_row = new Linear_Row<T>(SParam, k, n, BertParams.weight_layout);
-        q_bias = dev_alloc<T>(hl()); k_bias = dev_alloc<T>(hl()); v_bias = dev_alloc<T>(hl());
         w_bias = dev_alloc<T>(n);
-        dev_fill_const(q_bias, hl(), 0.f); dev_fill_const(k_bias, hl(), 0.f); dev_fill_const(v_bias, hl(), 0.f);
         dev_fill_const(w_bias, n, 0.f);
         if (BertParams.packed_qkv) {
-            linear_qkv_col = new Linear_Col<T>(SParam, k, 3 * n, BertParams.weight_layout);
+            // one [H, 3 Hl] projection, columns [q | k | v]; the three per-projection objects are views of its column blocks
+            // (weights stored [out, in]: row blocks), so every assembly that issues q, k and v separately, or as one grouped
+            // launch, reads the packed parameters
+            const int wl = BertParams.weight_layout;
+            linear_qkv_col = new Linear_Col<T>(SParam, k, 3 * n, wl);
             qkv_bias = dev_alloc<T>(3 * hl());
             dev_fill_const(qkv_bias, 3 * hl(), 0.f);
+            T* w = linear_qkv_col->weights;
+            const int64_t step = wl ? (int64_t)hl() * k : hl();
+            const int lda = wl ? k : 3 * hl();
+            linear_q_col = new Linear_Col<T>(SParam, k, n, wl, w, lda);
+            linear_k_col = new Linear_Col<T>(SParam, k, n, wl, w + step, lda);
+            linear_v_col = new Linear_Col<T>(SParam, k, n, wl, w + 2 * step, lda);
+            q_bias = qkv_bias; k_bias = qkv_bias + hl(); v_bias = qkv_bias + 2 * hl();
+        } else {
+            linear_q_col = new Linear_Col<T>(SParam, k, n, BertParams.weight_layout);
+            linear_k_col = new Linear_Col<T>(SParam, k, n, BertParams.weight_layout);
+            linear_v_col = new Linear_Col<T>(SParam, k, n, BertParams.weight_layout);
+            q_bias = dev_alloc<T>(hl()); k_bias = dev_alloc<T>(hl()); v_bias = dev_alloc<T>(hl());
+            dev_fill_const(q_bias, hl(), 0.f); dev_fill_const(k_bias, hl(), 0.f); dev_fill_const(v_bias, hl(), 0.f);
         }
         if (BertParams.max_cache_len > 0) {
             const size_t ce = (size_t)BertParams.max_batch_size * heads() * BertParams.max_cache_len * BertParams.size_per_head;
@@ -310,13 +327,15 @@ class Bert_MHA {
     int heads() const { return BertParams.head_num / SParam.world_size; }
     int hl() const { return heads() * BertParams.size_per_head; }
     void init_weights(uint64_t seed, uint64_t base) {
-        linear_q_col->init_weights(seed, base + 0);
+        linear_q_col->init_weights(seed, base + 0);  // views of the packed projection fill nothing
         linear_k_col->init_weights(seed, base + 1);
         linear_v_col->init_weights(seed, base + 2);
         linear_w_row->init_weights(seed, base + 3);
-        dev_fill_normal(q_bias, hl(), seed, base + 4, 0.f, 0.02f);
-        dev_fill_normal(k_bias, hl(), seed, base + 5, 0.f, 0.02f);
-        dev_fill_normal(v_bias, hl(), seed, base + 6, 0.f, 0.02f);
+        if (!linear_qkv_col) {
+            dev_fill_normal(q_bias, hl(), seed, base + 4, 0.f, 0.02f);
+            dev_fill_normal(k_bias, hl(), seed, base + 5, 0.f, 0.02f);
+            dev_fill_normal(v_bias, hl(), seed, base + 6, 0.f, 0.02f);
+        }
         dev_fill_normal(w_bias, n, seed, base + 7, 0.f, 0.02f);
         if (linear_qkv_col) {
             linear_qkv_col->init_weights(seed, base + 20);
@@ -397,13 +416,23 @@ class Bert_MHA {
             T* dst[3] = {b.q_buf, kdst, vdst};
             const T* bias[3] = {q_bias, k_bias, v_bias};
             const char* lab[3] = {"q_gemm+bias+heads", "k_gemm+bias+heads", "v_gemm+bias+heads"};
+            GemmDesc gd[3];
             for (int t = 0; t < 3; ++t) {
                 GemmDesc g = lin[t]->desc(input, dst[t], M);
                 g.epilogue = LG_EPI_BIAS_HEADS;
                 g.bias = bias[t];
                 g.epi_seq = seq_len; g.epi_d = d; g.epi_heads_total = h;
                 g.ldc = (t == 0) ? seq_len : kv_rows;  // rows per (batch, head) slot of the destination
-                FuncWrapVec.push_back(FuncWrap(1.0f, GEMM, [g](const DynamicInitParam& D) { GemmEx(D, g); }, g, lab[t]));
+                gd[t] = g;
+                if (!linear_qkv_col) FuncWrapVec.push_back(FuncWrap(1.0f, GEMM, [g](const DynamicInitParam& D) { GemmEx(D, g); }, g, lab[t]));
+            }
+            if (linear_qkv_col) {
+                // packed projection: ONE launch over the [H, 3 Hl] weight whose epilogue routes the q columns to q_buf and the k
+                // and v columns to their buffers or straight into the KV cache (attention_kernels.cu:331-393 does the routing in
+                // a separate kernel after the GEMM)
+                const GemmDesc gq = gd[0], gk = gd[1], gv = gd[2];
+                FuncWrapVec.push_back(FuncWrap(1.0f, COMPUTATION, [gq, gk, gv](const DynamicInitParam& D) { GemmExGrouped3(D, gq, gk, gv); },
+                                               "qkv_gemm+bias+heads", MFMA_BOUND));
             }
             T* qb = b.q_buf; T* ao = b.attn_out;
             const int causal = BertParams.causal;
@@ -716,8 +745,9 @@ class Bert_Model {
     // entries per layer of the vector forward() returns for this configuration
     int kernels_per_layer(bool decode = false) const {
         const bool fused = BertParams.fused && dtype_of<T>::value == LG_F16;
-        int mha = decode ? (BertParams.fused ? 3 : 6) : (fused ? 5 : (BertParams.packed_qkv ? 7 : 9));
-        int mlp = (fused && BertParams.ffn_act != FFN_GEGLU) ? 2 : 3;
+        int mha = decode ? (BertParams.fused ? 3 : 6) : (fused ? (BertParams.packed_qkv ? 3 : 5) : (BertParams.packed_qkv ? 7 : 9));
+        const int hidden = BertParams.head_num * BertParams.size_per_head;
+        int mlp = (fused && (BertParams.ffn_act != FFN_GEGLU || Bert_MLP<T>::geglu_fused(BertParams, SParam, hidden))) ? 2 : 3;
         return mha + mlp + 2 + (BertParams.norm_mode == PRE_LN_RESID ? 1 : 0);
     }
 

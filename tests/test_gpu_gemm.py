@@ -316,6 +316,48 @@ def test_grouped_qkv_gemm_equals_three_plain_calls(dev, po, M, transa):
                        (C.c_int * 3)(*ldc), dev.capi.EPI_BIAS_HEADS, arr([b.data_ptr() for b in dB]), 1, d, h) != 0
 
 
+@pytest.mark.parametrize("transa", [0, 1])
+@pytest.mark.parametrize("B,S,h,d", [(4, 128, 6, 128), (2, 384, 4, 64), (3, 100, 8, 96)])
+def test_grouped_qkv_gemm_on_a_packed_weight_prefill(dev, po, transa, B, S, h, d):
+    """Q, K and V of a prefill as one grouped call on the column blocks of ONE packed [K, 3 N] weight (the pointers of the
+    members are offsets into it, lda is the packed matrix's): with more than 256 token rows the pipelined kernel runs the
+    group as one launch, and its result must equal three plain fused calls bit for bit (same tiles, same k order) and the
+    oracle.  q goes to [B, h, S, d], k and v into cache-shaped buffers with more rows than S."""
+    import ctypes as C
+    K, rows = 512, S + 24
+    N, M = h * d, B * S
+    X = rnd(po, M * K, 70, 1).reshape(M, K)
+    W = rnd(po, K * 3 * N, 71, 1, 0.05).reshape(K, 3 * N)
+    bias = rnd(po, 3 * N, 72, 1, 0.3)
+    dX, dB = dev.up(X, 1), dev.up(bias, 1)
+    dW = dev.up(np.ascontiguousarray(W.T) if transa else W, 1)
+    lda = K if transa else 3 * N
+    step = N * K * 2 if transa else N * 2       # bytes between the members inside the packed weight
+    A = [dW.data_ptr() + t * step for t in range(3)]
+    bp = [dB.data_ptr() + t * N * 2 for t in range(3)]
+    ldc = [S, rows, rows]
+
+    def outputs():
+        o = [dev.empty((B, h, S, d), 1), dev.empty((B, h, rows, d), 1), dev.empty((B, h, rows, d), 1)]
+        for t in o:
+            t.zero_()
+        return o
+
+    plain, grouped = outputs(), outputs()
+    for t in range(3):
+        dev.call("lg_gemm_fused_f16", transa, N, M, K, A[t], lda, dX, K, plain[t], ldc[t], dev.capi.EPI_BIAS_HEADS, bp[t], S, d, h)
+    arr = lambda ptrs: (C.c_void_p * 3)(*ptrs)
+    dev.call("lg_gemm_fused_grouped_f16", transa, N, M, K, 3, arr(A), lda, dX, K, arr([g.data_ptr() for g in grouped]),
+             (C.c_int * 3)(*ldc), dev.capi.EPI_BIAS_HEADS, arr(bp), S, d, h)
+    for t in range(3):
+        got = dev.down(grouped[t])
+        assert np.array_equal(got, dev.down(plain[t]))
+        y = po.round_f16(po.gemm(X, np.ascontiguousarray(W[:, t * N:(t + 1) * N]), 1) + bias[t * N:(t + 1) * N])
+        ref = y.reshape(B, S, h, d).transpose(0, 2, 1, 3)
+        assert max_rel_err(got[:, :, :S], ref) < 4e-3
+        assert np.all(got[:, :, S:] == 0)
+
+
 @pytest.mark.parametrize("M,count,epi", [(1, 2, "bias"), (4, 1, "gelu"), (16, 2, "bias"), (40, 3, "none"), (16, 3, "gelu")])
 def test_grouped_gemm_other_epilogues_and_counts(dev, po, M, count, epi):
     """Groups of one, two and three problems with the plain, bias and bias + GELU epilogues and different leading

@@ -214,3 +214,37 @@ def test_packed_qkv_layer(dev, po, host, dtype, weight_layout):
     labels = [e["label"] for e in m.describe(2, 80)]
     assert labels[:2] == ["qkv_gemm", "fused_qkv_bias_transpose"] and m.kernels_per_layer() == 12
     assert max_rel_err(got, ref) < (2e-5 if dtype == 0 else 1e-2)
+
+
+@pytest.mark.parametrize("weight_layout", [0, 1])
+@pytest.mark.parametrize("B,S", [(2, 80), (3, 256)])
+def test_packed_qkv_fused_layer_and_decode(dev, po, host, weight_layout, B, S):
+    """Packed [H, 3 Hl] projection in the fused assembly: one grouped launch whose epilogue routes q to its buffer and k, v
+    straight into the KV cache (B x S = 768 token rows take the pipelined kernel as ONE launch, 160 rows the per-member
+    path), then a decode step that reads the same packed parameters.  The oracle gets the three column blocks."""
+    heads, d, F = 4, 64, 512
+    H = heads * d
+    m = host.Model(1, B, S, heads, d, layer_num=1, ffn_inner=F, causal=True, fused=True, packed_qkv=True, max_cache_len=S + 8,
+                   weight_layout=weight_layout, seed=9)
+    assert [e["label"] for e in m.describe(B, S)][:2] == ["qkv_gemm+bias+heads", "attn_prefill_fused"]
+    p = {k[len("layer0."):]: v for k, v in m.download_params().items() if k.startswith("layer0.")}
+    w = dict(p)
+    for i, t in enumerate("qkv"):
+        w["w" + t] = np.ascontiguousarray(p["wqkv"][:, i * H:(i + 1) * H])
+        w["b" + t] = np.ascontiguousarray(p["bqkv"][i * H:(i + 1) * H])
+    del w["wqkv"], w["bqkv"]
+    shape = dict(batch=B, seq=S, hidden=H, head_num=heads, size_per_head=d, ffn_inner=F, causal=1, norm_mode=0, dtype=1)
+    x = po.fill_normal(B * S * H, 9, 99, 0.0, 1.0, 1).reshape(B * S, H)
+    dx, dy = dev.up(x, 1), dev.empty((B * S, H), 1)
+    m.run(dx.data_ptr(), dy.data_ptr(), B, S, None, dev.stream, cache_slot=0)
+    assert max_rel_err(dev.down(dy), po.encoder_forward(shape, w, x)) < 1e-2
+    k = po.gemm(x, w["wk"], 1)
+    v = po.gemm(x, w["wv"], 1)
+    _, kb, vb = po.add_qkv_bias_transpose(k, w["bk"], k, w["bk"], v, w["bv"], B, S, heads, d, 1)
+    kc = np.zeros((B, heads, S + 8, d), dtype=np.float32)
+    vc = np.zeros_like(kc)
+    kc[:, :, :S], vc[:, :, :S] = kb, vb
+    tok = po.fill_normal(B * H, 9, 100, 0.0, 1.0, 1).reshape(B, H)
+    dt_in, dt_out = dev.up(tok, 1), dev.empty((B, H), 1)
+    m.run_decode(dt_in.data_ptr(), dt_out.data_ptr(), B, S, 0, None, dev.stream)
+    assert max_rel_err(dev.down(dt_out), po.decoder_step(shape, w, tok, kc, vc, S)) < 1e-2

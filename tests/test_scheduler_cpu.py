@@ -62,8 +62,11 @@ def test_launch_vector_shapes_and_order(fake):
     mp = host.Model(0, 2, 32, 4, 64, packed_qkv=True)
     assert [e["label"] for e in mp.describe(2, 32)][:3] == ["qkv_gemm", "fused_qkv_bias_transpose", "qk_gemm"]
     assert mp.kernels_per_layer() == 12
-    with pytest.raises(host.capi.LigerError):
-        host.Model(1, 2, 32, 4, 64, fused=True, packed_qkv=True)   # packed QKV belongs to the reference-shaped assembly
+    mpf = host.Model(1, 2, 32, 4, 64, fused=True, packed_qkv=True, max_cache_len=40)
+    assert [e["label"] for e in mpf.describe(2, 32)][:3] == ["qkv_gemm+bias+heads", "attn_prefill_fused", "out_proj"]
+    assert mpf.kernels_per_layer() == 7 and sorted(mpf.param_info()) == sorted(mp.param_info())
+    assert [e["label"] for e in mpf.describe(2, 1, decode_past=10)][0] == "qkv_gemm(decode)"
+    assert mg.kernels_per_layer() == 9
     m2 = host.Model(0, 2, 32, 4, 64, layer_num=3, norm_mode=host.PRE_LN_RESID)
     assert len(m2.describe(2, 32)) == 3 * 15
     with pytest.raises(host.capi.LigerError):
