@@ -164,8 +164,10 @@ int launch_gemm_skinny_kn_f16(const GemmArgs& g, const RowMap* rows, int wlayout
     const int nblk = g.N / BN, ktiles = g.K / KN_KT;
     // as few K-slices as fill the stream's compute units (one workgroup per CU keeps 48 .. 80 KiB of loads in flight), each
     // at least 8 k-tiles long, and no more than the workspace holds
-    int nsplit = 1;
-    while (nblk * nsplit < si.cus * 3 / 4 && ktiles / (nsplit * 2) >= 8 && nsplit < 32) nsplit *= 2;
+    int nsplit = si.cus / nblk;   // one workgroup per compute unit, or as close below as the slice length allows
+    if (nsplit > ktiles / 8) nsplit = ktiles / 8;
+    if (nsplit > 32) nsplit = 32;
+    if (nsplit < 1) nsplit = 1;
     const size_t slice_bytes = (size_t)g.M * g.N * sizeof(float);
     while (nsplit > 1 && (size_t)nsplit * slice_bytes > si.ws_bytes) nsplit /= 2;
     if (slice_bytes > si.ws_bytes) return LG_OK;

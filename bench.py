@@ -81,7 +81,7 @@ def kernel_only(args, capi, host, model, x, y, B, S, H, stream):
         capi.call("lg_stream_synchronize", stream)
         print(json.dumps({"kernel": "copy", "bytes_read": src.numel() * 2, "bytes_written": src.numel() * 2, "iters": args.iters}))
         return
-    decode = name in ("attn_decode", "kv_append") or name.endswith("(decode)")
+    decode = args.decode or name in ("attn_decode", "kv_append") or name.endswith("(decode)")
     if decode:
         Bd, L = CFG3["batch"], CFG3["cache_len"]
         xd = torch.empty(Bd, H, device="cuda", dtype=torch.float16)
@@ -101,7 +101,7 @@ def kernel_only(args, capi, host, model, x, y, B, S, H, stream):
     print(json.dumps({"kernel": name, "iters": args.iters, "avg_ms_hip_events": round(ms, 5)}))
 
 
-def bench_cfg4(capi, host, weight_layout, factors=(1, 2, 4, 8), shares=(0, 64, 96, 128), repeats=3, decode_steps=8):
+def bench_cfg4(capi, host, weight_layout, factors=(1, 2, 4, 8), shares=(0, 32, 64, 96, 128), repeats=3, decode_steps=8):
     """BASELINE config 4: a prefill request (batch 4 x seq 512) is decomposed by `factors` (token rows) and interleaved on two
     streams with a decode batch (32 sequences, 1024 cached positions, `decode_steps` steps: 8 steps hold the whole prefill in
     their window, 4 do not, so that a GEMM has to be split); makespan against sequential launch of the same two requests.  The decode batch is the primary request (its HBM-bound kernels open the windows), the prefill's MFMA-bound
@@ -240,11 +240,13 @@ def bench_cfg5(capi, host, weight_layout, n_requests, rates=(4.0, 8.0, 16.0), sh
 
 def derived_peaks(info):
     """Roofline denominators re-derived from the device properties: matrix peak = CUs x 4096 fp16 flop per clock and CU x
-    engine clock; memory peak = bus width x memory clock x 2 transfers per clock (as the runtime reports them)."""
+    engine clock; memory peak = bus width x reported memory clock x 4 transfers per pin and clock (the runtime reports 2.0 GHz
+    for HBM3E pins that run at 8 Gb/s; with 2 transfers per clock the "peak" would be 4.1 TB/s, below the 5.9 TB/s the
+    decode attention kernel measures, so the reported clock is a quarter of the pin rate)."""
     flops = info["cu_count"] * 4096 * info["clock_khz"] * 1e3 / 1e12
-    gbs = info["bus_width_bits"] / 8 * info["mem_clock_khz"] * 1e3 * 2 / 1e9
+    gbs = info["bus_width_bits"] / 8 * info["mem_clock_khz"] * 1e3 * 4 / 1e9
     return {"fp16_mfma_TFLOPs": round(flops, 1), "hbm_GBps": round(gbs, 1),
-            "formula": "%d CUs x 4096 flop/clk x %.3f GHz; %d bit x %.3f GHz x 2" % (info["cu_count"], info["clock_khz"] / 1e6,
+            "formula": "%d CUs x 4096 flop/clk x %.3f GHz; %d bit x %.3f GHz x 4" % (info["cu_count"], info["clock_khz"] / 1e6,
                                                                                      info["bus_width_bits"], info["mem_clock_khz"] / 1e6)}
 
 
@@ -306,6 +308,9 @@ def main():
                     help="launch only the named launch-vector entry (e.g. 'ffn1+bias+gelu', 'attn_decode', 'layer_norm') or "
                          "'copy' (a plain 128 MiB read + 128 MiB write kernel) --iters times; for rocprofv3 runs")
     ap.add_argument("--iters", type=int, default=50)
+    ap.add_argument("--decode", action="store_true",
+                    help="with --kernel-only: take the entry from the decode step's launch vector (batch 32, 1024 cached positions); "
+                         "needed for the entries whose name the prefill vector has too (ffn1+bias+gelu, ffn2, layer_norm)")
     ap.add_argument("--weight-layout", type=int, default=1, choices=[0, 1],
                     help="0: weights stored [in, out] (the reference's cuBLAS (N,N) layout); 1: stored [out, in] (default)")
     args = ap.parse_args()
