@@ -44,9 +44,18 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l16 = lane & 15, g = lane >> 4;
-    const int bh = blockIdx.y;                 // b * head_num + head
+    // Workgroups are handed to the 8 XCDs round-robin by their linear id.  The query blocks of one (batch, head) read the same
+    // K/V rows, so they are placed on ONE XCD, one after the other (its L2 then serves the re-reads: without this the K/V of a
+    // causal 512-token head are fetched 2.5 times), the longest (last) query block first.
+    int bh = blockIdx.y, qblk = blockIdx.x;    // bh = b * head_num + head
+    if ((gridDim.y & 7) == 0) {
+        const int lin = blockIdx.x + gridDim.x * blockIdx.y;
+        const int xcd = lin & 7, slot = lin >> 3;
+        bh = (slot / (int)gridDim.x) * 8 + xcd;
+        qblk = (int)gridDim.x - 1 - slot % (int)gridDim.x;
+    }
     const int b = bh / head_num, head = bh % head_num;
-    const int q0 = blockIdx.x * PF_BQ;         // first query of the block
+    const int q0 = qblk * PF_BQ;               // first query of the block
     const int qw = q0 + wave * 32;             // first query of the wave
 
     const half_t* Q = q_buf + (int64_t)bh * seq * D;

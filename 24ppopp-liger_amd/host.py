@@ -49,6 +49,8 @@ SIGNATURES = {
     "lgh_model_time_kernels": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, C.POINTER(_f), _i]),
     "lgh_model_time_one": (_f, [_p, _p, _p, _i, _i, _i, _i, _i, _i]),
     "lgh_sched_create": (_p, [_p, _i, _f, _i, _i, _i, _i, _i, _i]),
+    "lgh_sched_destroy": (_i, [_p]),
+    "lgh_model_destroy": (_i, [_p]),
     "lgh_sched_profile": (_i, [_p, _i, _i, _i, _i, _i]),
     "lgh_sched_profile_decode": (_i, [_p, _i, _i, _i]),
     "lgh_sched_profile_contention": (_i, [_p, _i, _i, _i, _i, C.POINTER(_f)]),
@@ -155,6 +157,7 @@ class Model:
                                          int(packed_qkv), seed)
         if not self.h:
             check(1, "lgh_model_create")
+        self._lib = lib          # the library the model was created in (tests switch libraries)
         self.dtype = dtype
         self.hidden = head_num * size_per_head
         self.layer_num = layer_num
@@ -169,6 +172,19 @@ class Model:
     @property
     def stream(self):
         return lib.lgh_model_stream(self.h)
+
+    def close(self):
+        """Frees the model's device memory and stream.  Schedulers built on it must be closed first (they hold a reference
+        to the model, so garbage collection keeps that order)."""
+        if getattr(self, "h", None) and self._lib is not None:
+            self._lib.lgh_model_destroy(self.h)
+        self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
     def param_info(self):
         """name -> dict(ptr, elems, rows, cols, transposed, interleave16); rows x cols is the logical [in, out] shape;
@@ -270,6 +286,20 @@ class Scheduler:
                                       pool_count, ctx_batch)
         if not self.h:
             check(1, "lgh_sched_create")
+        self._lib = lib
+
+    def close(self):
+        """Frees the scheduler's streams, events, request contexts and decode-batch buffers (every stream holds a hardware
+        queue: a process that keeps creating schedulers without closing them ends up with streams that share queues)."""
+        if getattr(self, "h", None) and self._lib is not None:
+            self._lib.lgh_sched_destroy(self.h)
+        self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
     def profile(self, bs, seq_lo, seq_hi, seq_step=1, itr=20):
         check(lib.lgh_sched_profile(self.h, bs, seq_lo, seq_hi, seq_step, itr), "lgh_sched_profile")

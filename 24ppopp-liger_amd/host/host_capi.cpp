@@ -49,7 +49,10 @@ struct SchedBase {
 
 struct ModelBase {
     virtual SchedBase* make_scheduler() = 0;
-    virtual ~ModelBase() {}
+    virtual ~ModelBase() {
+        if (stream0) { stream0->destroy(); delete stream0; }
+        dev_free(default_ws); dev_free(io_in); dev_free(io_out);
+    }
     virtual std::vector<FuncWrap> build(void* in, void* out, int batch, int seq, void* ws, int slot) = 0;
     virtual std::vector<FuncWrap> build_decode(void* in, void* out, int batch, int past, int slot, void* ws) = 0;
     virtual std::vector<FuncWrap> build_decode_seqs(void* in, void* out, const std::vector<int>& slots, const std::vector<int>& pasts, void* ws) = 0;
@@ -309,6 +312,16 @@ void* lgh_model_create_ex(int dtype, int max_batch, int max_seq, int head_num, i
     return mb;
 }
 
+// Frees a model: its parameters, KV caches, default workspace and buffers, and its stream.  Schedulers built on the model must be
+// destroyed first.
+int lgh_model_destroy(void* model) {
+    ModelBase* mb = (ModelBase*)model;
+    if (!mb) return LG_OK;
+    lg_device_synchronize();
+    delete mb;
+    return LG_OK;
+}
+
 int lgh_model_kernels_per_layer(void* model, int decode) { return model ? ((ModelBase*)model)->kernels_per_layer(decode != 0) : -1; }
 int64_t lgh_model_workspace_elems(void* model, int batch, int seq) { return model ? ((ModelBase*)model)->workspace_elems(batch, seq) : -1; }
 void* lgh_model_stream(void* model) { return model ? ((ModelBase*)model)->stream0->stream : nullptr; }
@@ -438,6 +451,12 @@ void* lgh_sched_create(void* model, int schedule_deep, float contention_factor, 
     s->configure(schedule_deep, contention_factor, policy, axis, seq_bucket < 1 ? 1 : seq_bucket, ignore_num);
     if (pool_count > 0) s->make_pool(pool_count, ctx_batch);
     return first_error() ? nullptr : s;
+}
+// Frees a scheduler: its streams (every one holds a hardware queue), events, request contexts and decode-batch buffers.
+int lgh_sched_destroy(void* sched) {
+    if (!sched) return LG_OK;
+    delete (SchedBase*)sched;
+    return first_error();
 }
 int lgh_sched_profile(void* sched, int bs, int seq_lo, int seq_hi, int seq_step, int itr) {
     if (!sched || bs <= 0 || seq_lo <= 0 || seq_hi < seq_lo || seq_step <= 0 || itr <= 0) return fail("lgh_sched_profile: bad arguments");

@@ -76,11 +76,22 @@ class DynamicInitParam {
   public:
     void* stream = nullptr;
     int stream_id = 0;  // 0 = primary, 1 = secondary; used by traces
+    // Copies are handed to every launch callback (as in the reference), so the object does not own its stream: whoever created
+    // the context calls destroy() on ONE copy when the stream is idle and no longer needed (a stream that was adopted from
+    // elsewhere is detached from the device library instead and stays alive).
+    bool adopted = false;
+    void destroy() {
+        if (!stream) return;
+        note_status(lg_stream_synchronize(stream), "lg_stream_synchronize");
+        if (adopted) note_status(lg_stream_detach(stream), "lg_stream_detach");
+        else note_status(lg_stream_destroy(stream), "lg_stream_destroy");
+        stream = nullptr;
+    }
     DynamicInitParam() { note_status(lg_stream_create(&stream), "lg_stream_create"); }
     // the reference passes a CUDA stream priority here; priorities are deliberately not used on this platform
     explicit DynamicInitParam(int /*priority*/) { note_status(lg_stream_create(&stream), "lg_stream_create"); }
     // a stream created elsewhere: the device library is told about it (it then owns a split-K workspace for it)
-    DynamicInitParam(void* existing_stream, int id) : stream(existing_stream), stream_id(id) {
+    DynamicInitParam(void* existing_stream, int id) : stream(existing_stream), stream_id(id), adopted(true) {
         note_status(lg_stream_attach(existing_stream, 0), "lg_stream_attach");
     }
     // a stream whose kernels run on the compute units selected by the mask only (see lg_stream_create_cu_mask)

@@ -28,6 +28,9 @@ inline T* dev_alloc(size_t elems) {
     note_status(lg_malloc(&p, (elems ? elems : 1) * sizeof(T)), "lg_malloc");
     return (T*)p;
 }
+inline void dev_free(void* p) {
+    if (p) note_status(lg_free(p), "lg_free");
+}
 template <typename T>
 inline void dev_fill_normal(T* p, int64_t n, uint64_t seed, uint64_t tensor_id, float mean, float stddev) {
     if (dtype_of<T>::value == LG_F16) note_status(lg_fill_normal_f16(p, n, seed, tensor_id, mean, stddev, nullptr), "lg_fill_normal_f16");
@@ -76,6 +79,9 @@ class Linear_Col {  // linear.h:68-109: output features split across ranks
     }
     Linear_Col(const StaticInitParam& SParams_, const int& k_, const int& n_, int weight_layout_, T* view, int lda)
         : k(k_), n(n_), weights(view), SParams(SParams_), weight_layout(weight_layout_), lda_view(lda) {}
+    Linear_Col(const Linear_Col&) = delete;
+    Linear_Col& operator=(const Linear_Col&) = delete;
+    ~Linear_Col() { if (!lda_view) dev_free(weights); }
     ParamRef param(const std::string& name) { return ParamRef{name, weights, (int64_t)k * n_local(), k, n_local(), weight_layout | (interleave16 << 1)}; }
     int n_local() const { return n / SParams.world_size; }
     void init_weights(uint64_t seed, uint64_t tensor_id, float stddev = 0.02f) {
@@ -110,6 +116,9 @@ class Linear_Row {  // linear.h:16-64: input features split across ranks; partia
         : k(k_), n(n_), SParams(SParams_), weight_layout(weight_layout_) {
         weights = dev_alloc<T>((size_t)k * n / SParams.world_size);
     }
+    Linear_Row(const Linear_Row&) = delete;
+    Linear_Row& operator=(const Linear_Row&) = delete;
+    ~Linear_Row() { dev_free(weights); }
     ParamRef param(const std::string& name) { return ParamRef{name, weights, (int64_t)k_local() * n, k_local(), n, weight_layout}; }
     int k_local() const { return k / SParams.world_size; }
     void init_weights(uint64_t seed, uint64_t tensor_id, float stddev = 0.02f) {
@@ -147,6 +156,9 @@ class LayerNorm {  // operator.h:16-41
         dev_fill_const(gamma, k, 1.0f);
         dev_fill_const(beta, k, 0.0f);
     }
+    LayerNorm(const LayerNorm&) = delete;
+    LayerNorm& operator=(const LayerNorm&) = delete;
+    ~LayerNorm() { dev_free(gamma); dev_free(beta); }
     void init_weights(uint64_t seed, uint64_t tensor_id) {
         dev_fill_normal(gamma, k, seed, tensor_id, 1.0f, 0.1f);
         dev_fill_normal(beta, k, seed, tensor_id + 1, 0.0f, 0.1f);
@@ -192,6 +204,9 @@ class Bert_MLP {
         dev_fill_const(bias, f_local() * gate_mult(), 0.f);
         dev_fill_const(bias2, k, 0.f);
     }
+    Bert_MLP(const Bert_MLP&) = delete;
+    Bert_MLP& operator=(const Bert_MLP&) = delete;
+    ~Bert_MLP() { delete linear_col; delete linear_row; dev_free(bias); dev_free(bias2); }
     int f_local() const { return intermediate_size / SParam.world_size; }
     int gate_mult() const { return BertParams.ffn_act == FFN_GEGLU ? 2 : 1; }
     // GeGLU in the fused fp16 assembly: FFN-1's weight and bias are stored with gate and up interleaved in groups of 16 features,
@@ -323,6 +338,14 @@ class Bert_MHA {
             note_status(lg_memset_async(k_cache, 0, ce * sizeof(T), nullptr), "lg_memset_async");
             note_status(lg_memset_async(v_cache, 0, ce * sizeof(T), nullptr), "lg_memset_async");
         }
+    }
+    Bert_MHA(const Bert_MHA&) = delete;
+    Bert_MHA& operator=(const Bert_MHA&) = delete;
+    ~Bert_MHA() {
+        delete linear_q_col; delete linear_k_col; delete linear_v_col; delete linear_w_row;
+        if (linear_qkv_col) { delete linear_qkv_col; dev_free(qkv_bias); }   // q / k / v biases are parts of qkv_bias
+        else { dev_free(q_bias); dev_free(k_bias); dev_free(v_bias); }
+        dev_free(w_bias); dev_free(k_cache); dev_free(v_cache);
     }
     int heads() const { return BertParams.head_num / SParam.world_size; }
     int hl() const { return heads() * BertParams.size_per_head; }
@@ -645,6 +668,9 @@ class Bert_Encoder {
         ln_mha = new LayerNorm<T>(SParam, k);
         ln_mlp = new LayerNorm<T>(SParam, k);
     }
+    Bert_Encoder(const Bert_Encoder&) = delete;
+    Bert_Encoder& operator=(const Bert_Encoder&) = delete;
+    ~Bert_Encoder() { delete MHA; delete MLP; delete ln_mha; delete ln_mlp; }
     void init_weights(uint64_t seed, uint64_t base) {
         MHA->init_weights(seed, base + 0);
         MLP->init_weights(seed, base + 8);
@@ -732,6 +758,9 @@ class Bert_Model {
         : k(k_), n(n_), SParam(SParam_), BertParams(BertParams_), workspace(workspace_) {
         for (int i = 0; i < BertParams.layer_num; i++) encoders.push_back(new Bert_Encoder<T>(BertParams, SParam, k, n, workspace));
     }
+    Bert_Model(const Bert_Model&) = delete;
+    Bert_Model& operator=(const Bert_Model&) = delete;
+    ~Bert_Model() { for (auto* e : encoders) delete e; }   // the workspace belongs to the caller
     void init_weights(uint64_t seed) {
         for (size_t i = 0; i < encoders.size(); ++i) encoders[i]->init_weights(seed, 1000 * (i + 1));
         note_status(lg_device_synchronize(), "lg_device_synchronize");

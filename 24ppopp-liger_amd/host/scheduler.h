@@ -183,9 +183,36 @@ class Scheduler {
         note_status(lg_event_create(&Main_EVENT), "lg_event_create");
         note_status(lg_event_create(&Wait_EVENT), "lg_event_create");
     }
+    // Releases what the scheduler created: its streams (the two of the constructor and the CU-masked ones; every stream holds a
+    // hardware queue, and queues that pile up make streams share one and run in turn), its events, the request contexts and
+    // the decode batch's buffers.  The model and the buffers handed to the constructor belong to the caller.
     ~Scheduler() {
         if (_thread.joinable()) _thread.join();
+        lg_device_synchronize();
+        _drop_queued();
+        {   // samples still in flight or retired but not yet reclaimed (none after a completed run)
+            std::vector<Sample*> left(exe_vec.begin(), exe_vec.end());
+            left.insert(left.end(), _retired.begin(), _retired.end());
+            std::sort(left.begin(), left.end());
+            left.erase(std::unique(left.begin(), left.end()), left.end());
+            for (Sample* smp : left) delete smp;
+        }
+        for (auto& kv : _part_streams)
+            for (int role = 0; role < 2; ++role)
+                for (int cls = 0; cls < 2; ++cls)
+                    if (kv.second.d[role][cls]) kv.second.d[role][cls]->destroy();
+        DParams1.destroy();
+        DParams0.destroy();
+        for (void* e : {Main_EVENT, Wait_EVENT, _epoch_event})
+            if (e) lg_event_destroy(e);
+        for (ReqCtx* c : _all_ctx) {
+            dev_free(c->input); dev_free(c->output); dev_free(c->ws); dev_free(c->dec_a); dev_free(c->dec_b);
+            delete c;
+        }
+        dev_free(_dec_x); dev_free(_dec_ws);
     }
+    Scheduler(const Scheduler&) = delete;
+    Scheduler& operator=(const Scheduler&) = delete;
 
     // Creates the four CU-masked streams of partitioned rounds: [role: primary, secondary] x [class: MFMA-bound, HBM-bound].
     // hbm_cus compute units (a multiple of 8, spread evenly over the 8 dies: mask bits 0 .. hbm_cus-1) go to the HBM-bound
@@ -193,9 +220,14 @@ class Scheduler {
     bool enable_partition(int hbm_cus, int total_cus = 256) {
         if (hbm_cus <= 0 || hbm_cus % 8 != 0 || hbm_cus >= total_cus || total_cus > 256 || total_cus % 8 != 0) return false;
         if (partition_hbm_cus == hbm_cus) return true;
-        // the streams of a share are created once and kept (every CU-masked stream is a hardware queue of its own)
+        // The streams of a share are created once and kept while that share is in use (switching the partition on and off does
+        // not touch them); asking for another share releases them first: every CU-masked stream is a hardware queue of its own.
         auto it = _part_streams.find(hbm_cus);
         if (it == _part_streams.end()) {
+            for (auto& kv : _part_streams)
+                for (int role = 0; role < 2; ++role)
+                    for (int cls = 0; cls < 2; ++cls) kv.second.d[role][cls]->destroy();
+            _part_streams.clear();
             unsigned hbm_mask[8] = {0}, mfma_mask[8] = {0};
             for (int b = 0; b < total_cus; ++b) (b < hbm_cus ? hbm_mask : mfma_mask)[b >> 5] |= 1u << (b & 31);
             PartStreams ps;

@@ -149,9 +149,12 @@ def bench_cfg4(capi, host, weight_layout, factors=(1, 2, 4, 8), shares=(0, 32, 6
             res[key] = best_of(host.MODE_LIGER)
             res[key]["speedup"] = round(res["sequential"]["makespan_ms"] / res[key]["makespan_ms"], 4)
         sched.enable_partition(0)
+        print("cfg4: factor %d done" % factor, file=sys.stderr, flush=True)
         res["speedup"] = round(res["sequential"]["makespan_ms"] / res["interleaved"]["makespan_ms"], 4)
         res["speedup_minor_merged"] = round(res["sequential"]["makespan_ms"] / res["interleaved_minor_merged"]["makespan_ms"], 4)
         out.append(res)
+        sched.close()   # gives its streams back: hardware queues that pile up make later streams share one
+    model.close()
     return {"workload": "cfg4: prefill B4 S512 (split by token rows) || decode B32 L1024 x %d steps, one layer shard" % decode_steps,
             "partition_measurement": {"what": "MFMA-bound kernels of the prefill layer on 256 - n compute units || decode steps on n, "
                                               "against both back to back on the whole chip", "by_hbm_cus": partition},
@@ -177,6 +180,7 @@ def bench_cfg5(capi, host, weight_layout, n_requests, rates=(4.0, 8.0, 16.0), sh
         for past in range(128, 1024 + 64 + 1, 64):
             sched.profile_decode(bs, min(past, 1024 + 63), 3)
     prof_s = time.perf_counter() - t0
+    print("cfg5: profiled in %.1f s" % prof_s, file=sys.stderr, flush=True)
     # measured contention: the MFMA-bound kernels of a 512-token prefill next to batch-1 decode steps at 512 cached positions
     meas = sched.profile_contention(1, 512, 1, 512)
     table = {"mfma_main_hbm_sub": sched.contention(0, 1), "hbm_main_mfma_sub": sched.contention(1, 0)}
@@ -217,6 +221,7 @@ def bench_cfg5(capi, host, weight_layout, n_requests, rates=(4.0, 8.0, 16.0), sh
                 sched.set_partition_factor(1, 0, part_factor[share][1])
             reps = [sched.run_trace(trace, mode) for _ in range(runs)]
             r = reps[0]
+            print("cfg5: lambda %.0f %s: mean %.2f ms" % (lam, name, sum(x["avg_e2e_ms"] for x in reps) / len(reps)), file=sys.stderr, flush=True)
             # latency = arrival -> completion on one clock; the reference's sum (first launch - arrival) + (start event -> stop
             # event) is kept beside it: it under-counts when a start event is held up on the device
             means = [x["avg_e2e_ms"] for x in reps]
@@ -231,8 +236,11 @@ def bench_cfg5(capi, host, weight_layout, n_requests, rates=(4.0, 8.0, 16.0), sh
         out.append(row)
     sched.enable_partition(0)
     sched.enable_batch_decode(False)
+    concurrent = sched.streams_concurrent
+    sched.close()
+    model.close()
     return {"workload": "cfg5: 4 layer shards, Poisson arrivals, prompts U[128,1024] rounded to 64, 32 decode tokens", "profile_seconds": round(prof_s, 1),
-            "streams_verified_concurrent": sched.streams_concurrent,
+            "streams_verified_concurrent": concurrent,
             "contention_measurement": {k: (round(v, 4) if isinstance(v, float) else v) for k, v in meas.items()},
             "contention_table": {k: round(v, 4) for k, v in table.items()},
             "partition_measurement": part_meas, "results": out}

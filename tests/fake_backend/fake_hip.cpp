@@ -44,6 +44,7 @@ double g_share_exp[2] = {1.0, 1.0};  // a kernel on a stream with `cus` of 256 c
                                      // [0] matrix kernels, [1] memory kernels (1 = proportional, < 1 = the share hurts less)
 thread_local int g_cost_kind = 1;    // kind of the cost computed last on this thread (0 matrix, 1 memory)
 std::vector<Stream*> g_streams;
+int g_live_streams = 0, g_live_allocs = 0;   // created and not yet destroyed / allocated and not yet freed
 std::vector<Launch> g_trace;
 Stream g_default;
 
@@ -104,6 +105,8 @@ int fake_trace_get(int i, int* stream, char* name, int name_len, long long* abc,
     return 0;
 }
 double fake_host_now(void) { return g_host_now; }
+int fake_live_streams(void) { return g_live_streams; }
+int fake_live_allocs(void) { return g_live_allocs; }
 
 // ---- library / runtime ------------------------------------------------------------------------------------------------
 const char* lg_last_error(void) { return "fake backend: no error text"; }
@@ -120,9 +123,14 @@ int lg_malloc(void** ptr, size_t bytes) {
     std::lock_guard<std::mutex> lk(g_mu);
     *ptr = (void*)next;
     next += (bytes + 255) / 256 * 256 + 256;
+    ++g_live_allocs;
     return LG_OK;
 }
-int lg_free(void*) { return LG_OK; }
+int lg_free(void* p) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (p) --g_live_allocs;
+    return LG_OK;
+}
 int lg_memcpy_h2d(void*, const void*, size_t) { return LG_OK; }
 int lg_memcpy_d2h(void*, const void*, size_t) { return LG_OK; }
 int lg_memcpy_d2d_async(void* dst, const void* src, size_t bytes, void* stream) { return launch(stream, "memcpy_d2d", (long long)bytes, 0, 0, src, nullptr, dst, mem_cost(2.0 * bytes)); }
@@ -139,6 +147,7 @@ int lg_stream_create(void** stream) {
     s->id = (int)g_streams.size() + 1;
     s->ready = g_host_now;
     g_streams.push_back(s);
+    ++g_live_streams;
     *stream = s;
     return LG_OK;
 }
@@ -158,7 +167,12 @@ int lg_stream_create_cu_mask(void** stream, const unsigned* cu_mask, int mask_wo
     for (int w = 0; w < 8; ++w) s->mask[w] = w < mask_words ? cu_mask[w] : 0u;
     return rc;
 }
-int lg_stream_destroy(void*) { return LG_OK; }
+int lg_stream_destroy(void* stream) {
+    // the object stays (traces refer to it); only the count of streams in existence goes down
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (stream) --g_live_streams;
+    return LG_OK;
+}
 int lg_stream_attach(void*, int cu_count) { return cu_count < 0 ? LG_ERR_INVALID : LG_OK; }
 int lg_stream_detach(void*) { return LG_OK; }
 int lg_stream_cu_count(void* stream) { return stream ? S(stream)->cus : 256; }

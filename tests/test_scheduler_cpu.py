@@ -678,3 +678,34 @@ def test_cfg4_shapes_pieces_cover_the_prefill_exactly(fake, factor, axis):
         total = sum(e["m"] * e["n"] for e in gemms)
         assert total == M * (3 * Hl + H + F + H) and all(e["n"] == M for e in gemms)
         assert len(gemms) > 6
+
+
+def test_closing_a_scheduler_and_a_model_releases_streams_and_memory(fake):
+    """Every stream holds a hardware queue on the GPU, so schedulers must give theirs back: the two streams of the
+    constructor, the four CU-masked streams of the share in use (asking for another share releases the previous four), the
+    request contexts and the decode batch's buffers."""
+    host, lib = fake.host, fake.lib
+    s0, a0 = lib.fake_live_streams(), lib.fake_live_allocs()
+    m = host.Model(1, 9, 64, 4, 64, layer_num=2, ffn_inner=512, fused=True, max_cache_len=96)
+    s1, a1 = lib.fake_live_streams(), lib.fake_live_allocs()
+    assert s1 == s0 + 1 and a1 > a0
+    sch = host.Scheduler(m, pool_count=4, ctx_batch=2)
+    assert lib.fake_live_streams() == s1 + 2
+    sch.enable_partition(64)
+    assert lib.fake_live_streams() == s1 + 6
+    sch.enable_partition(0)
+    sch.enable_partition(64)                      # off and on again: the same four streams
+    assert lib.fake_live_streams() == s1 + 6
+    sch.enable_partition(128)                     # another share: the previous four are released first
+    assert lib.fake_live_streams() == s1 + 6
+    sch.enable_batch_decode(True, 2)
+    sch.profile(2, 32, 64, 32, 1)
+    sch.profile_decode(2, 32, 1)
+    sch.serve(2, 32, 2)
+    sch.run_queued(host.MODE_LIGER)
+    assert lib.fake_live_allocs() > a1
+    sch.close()
+    assert (lib.fake_live_streams(), lib.fake_live_allocs()) == (s1, a1)
+    sch.close()                                   # closing twice is harmless
+    m.close()
+    assert (lib.fake_live_streams(), lib.fake_live_allocs()) == (s0, a0)
