@@ -203,7 +203,7 @@ class Scheduler {
                     if (kv.second.d[role][cls]) kv.second.d[role][cls]->destroy();
         DParams1.destroy();
         DParams0.destroy();
-        for (void* e : {Main_EVENT, Wait_EVENT, _epoch_event})
+        for (void* e : {Main_EVENT, Wait_EVENT, _epoch_event, _dec_prev_stop})
             if (e) lg_event_destroy(e);
         for (ReqCtx* c : _all_ctx) {
             dev_free(c->input); dev_free(c->output); dev_free(c->ws); dev_free(c->dec_a); dev_free(c->dec_b);
@@ -802,6 +802,7 @@ class Scheduler {
         recs.clear();
         for (void* e : _dec_prefill_events) lg_event_destroy(e);
         _dec_prefill_events.clear();
+        if (_dec_prev_stop) { lg_event_destroy(_dec_prev_stop); _dec_prev_stop = nullptr; }
         batched_steps = batched_rows = 0;
         rounds = secondary_launches = splits = partition_rounds = 0;
     }
@@ -960,6 +961,16 @@ class Scheduler {
                 vec.push_back(f);
             }
         }
+        // The steps of this vector work in place on the batch's rows, workspace and cache slots, like the steps of the vector
+        // before it, whose last kernels may still be running on the other stream: the vector's first entry waits for them.
+        if (_dec_prev_stop) {
+            void* prev = _dec_prev_stop;
+            FuncWrap f(0.001f, COMPUTATION, [prev](const DynamicInitParam& D) {
+                note_status(lg_stream_wait_event(D.stream, prev), "lg_stream_wait_event");
+            }, "after_previous_steps");
+            f.minor = true; f.name = 902; f.duration = 0.001f;
+            vec.insert(vec.begin(), f);
+        }
         std::unique_lock<std::mutex> build_lock(_build_mutex);
         for (int st = 0; st < steps; ++st) {
             int rows = 0, longest = 0;
@@ -1016,7 +1027,10 @@ class Scheduler {
         if (_dec_sample && _dec_sample->empty()) {
             exe_vec.erase(std::find(exe_vec.begin(), exe_vec.end(), _dec_sample));
             lg_event_destroy(_dec_sample->start);
-            lg_event_destroy(_dec_sample->stop);
+            // the stop event (recorded behind the vector's last kernel) is what the next vector waits for; the one before it
+            // is no longer needed: whatever waited for it has been launched, and a wait keeps the state it found at launch
+            if (_dec_prev_stop) lg_event_destroy(_dec_prev_stop);
+            _dec_prev_stop = _dec_sample->stop;
             delete _dec_sample;
             _dec_sample = nullptr;
         }
@@ -1032,6 +1046,7 @@ class Scheduler {
         }
     }
     std::vector<void*> _dec_prefill_events;  // destroyed with the run's records
+    void* _dec_prev_stop = nullptr;          // stop event of the previous vector of batched steps
 
     std::atomic<bool> _running{false};
     std::vector<ReqCtx*> _held;   // contexts of finished requests kept back while recycle_contexts is off

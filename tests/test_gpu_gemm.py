@@ -91,6 +91,37 @@ def test_gemm_geglu_epilogue(dev, po, transa, M, F, K):
     assert np.all(got[:, F:] == 7.0) and max_rel_err(got[:, :F], ref) < 4e-3
 
 
+@pytest.mark.parametrize("transa", [0, 1])
+def test_gemm_geglu_subrange_concatenation_is_exact(dev, po, transa):
+    """Decomposition of a GeGLU FFN-1 (decompose_callback: whole groups of 32 stored features = 16 output columns; weight
+    and bias move by c0 features, the output by c0 / 2 columns; token rows as for any GEMM): the pieces reproduce the full
+    call bit for bit."""
+    M, F, K = 512, 768, 256
+    X = rnd(po, M * K, 43, 1).reshape(M, K)
+    Ws = rnd(po, K * 2 * F, 44, 1, 0.05).reshape(K, 2 * F)      # already in the stored (interleaved) order
+    bs = rnd(po, 2 * F, 45, 1, 0.3)
+    dX, dB = dev.up(X, 1), dev.up(bs, 1)
+    dW = dev.up(np.ascontiguousarray(Ws.T) if transa else Ws, 1)
+    lda = K if transa else 2 * F
+    full = dev.empty((M, F), 1)
+    dev.call("lg_gemm_fused_f16", transa, 2 * F, M, K, dW, lda, dX, K, full, F, 5, dB, 0, 0, 0)
+    # stored features split at 3/8 (a multiple of 32)
+    c0 = (2 * F * 3 // 8) // 32 * 32
+    cols = dev.empty((M, F), 1)
+    wstep = c0 * K * 2 if transa else c0 * 2
+    dev.call("lg_gemm_fused_f16", transa, c0, M, K, dW, lda, dX, K, cols, F, 5, dB, 0, 0, 0)
+    dev.call("lg_gemm_fused_f16", transa, 2 * F - c0, M, K, dW.data_ptr() + wstep, lda, dX, K, cols.data_ptr() + (c0 // 2) * 2, F, 5,
+             dB.data_ptr() + c0 * 2, 0, 0, 0)
+    assert np.array_equal(dev.down(cols), dev.down(full))
+    # token rows split at 5/8 (both pieces above 256 rows: every output stays one sequential sum over k)
+    rows = dev.empty((M, F), 1)
+    m1 = 320
+    dev.call("lg_gemm_fused_f16", transa, 2 * F, m1, K, dW, lda, dX, K, rows, F, 5, dB, 0, 0, 0)
+    dev.call("lg_gemm_fused_f16", transa, 2 * F, M - m1, K, dW, lda, dX.data_ptr() + m1 * K * 2, K, rows.data_ptr() + m1 * F * 2, F, 5, dB, 0, 0, 0)
+    got, ref = dev.down(rows), dev.down(full)
+    assert np.array_equal(got[:m1], ref[:m1]) and max_rel_err(got[m1:], ref[m1:]) < 1e-3   # 192 rows may slice K
+
+
 def test_gemm_geglu_epilogue_rejects_bad_shapes(dev):
     x = dev.empty((4, 64), 1)
     w = dev.empty((48, 64), 1)

@@ -66,6 +66,26 @@ def test_cfg1_reference_assembly_fp32(dev, po, host):
     assert max_rel_err(got, ref) < 2e-5
 
 
+@pytest.mark.parametrize("weight_layout", [0, 1])
+@pytest.mark.parametrize("mode,key", [(0, "post_noresid"), (1, "pre_ln_resid")])
+def test_cfg1_layer_against_the_committed_torch_fixture(dev, host, mode, key, weight_layout):
+    """BASELINE config 1 on the GPU against tests/golden/cfg1_layer_torch.npz directly (no oracle in between): the
+    fixture's weights are uploaded into the model, the input is the fixture's input, the output must match what torch
+    computed in float64 from the same numbers."""
+    import os
+    from tests.golden.make_golden import cfg1_weights
+    w, x = cfg1_weights()
+    m = host.Model(0, 2, 32, 4, 64, layer_num=1, ffn_inner=1024, norm_mode=mode, causal=False, fused=False,
+                   weight_layout=weight_layout, seed=3)
+    m.upload_params({"layer0." + k: v for k, v in w.items()})
+    back = m.download_params()
+    assert all(np.array_equal(back["layer0." + k], v) for k, v in w.items())
+    dx, dy = dev.up(x, 0), dev.empty((64, 256), 0)
+    m.run(dx.data_ptr(), dy.data_ptr(), 2, 32, None, dev.stream)
+    want = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "cfg1_layer_torch.npz"))[key]
+    assert max_rel_err(dev.down(dy), want) < 2e-5
+
+
 @pytest.mark.parametrize("norm_mode", [0, 1])
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("fused", [False, True])
