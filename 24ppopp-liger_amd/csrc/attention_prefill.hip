@@ -131,8 +131,8 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
     issue(0, 0);
     for (int k0 = 0, t = 0; k0 < kv_end; k0 += PF_BC, ++t) {
         const int buf = t & 1;
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's part of tile t has landed
-        __syncthreads();  // tile t is visible to every wave, and every wave is done with tile t-1: its buffer is refilled now
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // this thread's part of tile t has landed
+        barrier_keep_loads_in_flight();  // tile t is visible to every wave, and every wave is done with tile t-1: its buffer is refilled now
         if (k0 + PF_BC < kv_end) issue(k0 + PF_BC, buf ^ 1);
         // a wave whose queries all lie before this key tile has nothing to do here (causal), but keeps loading and hitting
         // the barrier, so only the math is skipped
@@ -141,16 +141,28 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
         const half_t* vs = Vs[buf];
 
         // ---- S^T = K Q^T ------------------------------------------------------------------------------------
+        // The LDS reads of this loop are issued by hand (lds_read16_issue / lds_read_tr4_issue): the compiler would put a wait
+        // for the loads of the NEXT tile, issued just above, in front of every read of THIS tile.  The fragments of key tile
+        // kt + 1 are requested before the MFMAs of key tile kt.
         float4_t s[4][2];
+        half8_t kf[2][DC];
+        auto kissue = [&](int kt, int slot) {
+#pragma unroll
+            for (int dc = 0; dc < DC; ++dc) lds_read16_issue(kf[slot][dc], &ks[P2 ? kfrag[0][dc] + kt * 16 * D : kfrag[kt % KG][dc]]);
+        };
+        kissue(0, 0);
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt) {
+            const int slot = kt & 1;
+            if (kt + 1 < 4) kissue(kt + 1, slot ^ 1);
             s[kt][0] = float4_t{0.f, 0.f, 0.f, 0.f};
             s[kt][1] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int dc = 0; dc < DC; ++dc) {
-                const half8_t a = *reinterpret_cast<const half8_t*>(&ks[P2 ? kfrag[0][dc] + kt * 16 * D : kfrag[kt % KG][dc]]);
-                s[kt][0] = mfma16(a, qf[0][dc], s[kt][0]);
-                s[kt][1] = mfma16(a, qf[1][dc], s[kt][1]);
+                if (kt + 1 < 4) lds_read16_wait<DC>(kf[slot][dc]);   // the DC reads of the next key tile may be outstanding
+                else lds_read16_wait<0>(kf[slot][dc]);
+                s[kt][0] = mfma16(kf[slot][dc], qf[0][dc], s[kt][0]);
+                s[kt][1] = mfma16(kf[slot][dc], qf[1][dc], s[kt][1]);
             }
         }
         // ---- scale, mask, online softmax (per query column) -----------------------------------------------------
@@ -224,14 +236,35 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
                 pf[qt] = half8_t{(half_t)lo[0], (half_t)lo[1], (half_t)lo[2], (half_t)lo[3],
                                  (half_t)hi[0], (half_t)hi[1], (half_t)hi[2], (half_t)hi[3]};
             }
+            // The transposed reads are issued by hand (lds_read_tr4_issue: the builtin would make the compiler wait for the
+            // loads of the NEXT tile, issued above, before every read), a group of VGRP fragments ahead of the MFMAs that use
+            // them: logical 32-byte block dt of rows 32 j + 4 g + l16 / 4 and 16 rows further on, this lane's 8 bytes inside it.
+            constexpr int VGRP = 2;
+            static_assert(DT % VGRP == 0, "head size must be a multiple of 32");
+            half4_t vlo[2][VGRP], vhi[2][VGRP];
+            auto vissue = [&](int grp, int slot) {
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                // logical 32-byte block dt of rows 32 j + 4 g + l16 / 4 and 16 rows further on, this lane's 8 bytes inside it
-                const half4_t lo = lds_read_tr4(&vs[P2 ? vfrag[0][dt] + (2 * j) * 16 * D : vfrag[(2 * j) % VG][dt]]);
-                const half4_t hi = lds_read_tr4(&vs[P2 ? vfrag[0][dt] + (2 * j + 1) * 16 * D : vfrag[(2 * j + 1) % VG][dt]]);
-                const half8_t a = half8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                o[dt][0] = mfma16(a, pf[0], o[dt][0]);
-                o[dt][1] = mfma16(a, pf[1], o[dt][1]);
+                for (int i = 0; i < VGRP; ++i) {
+                    const int dt = grp * VGRP + i;
+                    lds_read_tr4_issue(vlo[slot][i], &vs[P2 ? vfrag[0][dt] + (2 * j) * 16 * D : vfrag[(2 * j) % VG][dt]]);
+                    lds_read_tr4_issue(vhi[slot][i], &vs[P2 ? vfrag[0][dt] + (2 * j + 1) * 16 * D : vfrag[(2 * j + 1) % VG][dt]]);
+                }
+            };
+            vissue(0, 0);
+#pragma unroll
+            for (int grp = 0; grp < DT / VGRP; ++grp) {
+                const int slot = grp & 1;
+                if (grp + 1 < DT / VGRP) vissue(grp + 1, slot ^ 1);
+#pragma unroll
+                for (int i = 0; i < VGRP; ++i) {
+                    // the reads of the next group (2 VGRP of them) may still be outstanding
+                    if (grp + 1 < DT / VGRP) lds_tr_wait<2 * VGRP>(vlo[slot][i], vhi[slot][i]);
+                    else lds_tr_wait<0>(vlo[slot][i], vhi[slot][i]);
+                    const half8_t a = join_half4(vlo[slot][i], vhi[slot][i]);
+                    const int dt = grp * VGRP + i;
+                    o[dt][0] = mfma16(a, pf[0], o[dt][0]);
+                    o[dt][1] = mfma16(a, pf[1], o[dt][1]);
+                }
             }
         }
     }

@@ -89,6 +89,44 @@ __device__ __forceinline__ half4_t lds_read_tr4(const half_t* p) {
     return __builtin_bit_cast(half4_t, r);
 }
 
+// The same read issued as inline assembly, for kernels that fill their LDS tiles with direct-to-LDS loads (load_lds16): the
+// compiler cannot tell which outstanding direct-to-LDS load the builtin's read may alias and puts an s_waitcnt vmcnt(0) in front
+// of it, which drains the load pipeline of a ring of tiles at every read.  The kernels order tiles and reads themselves (their
+// own vmcnt wait + barrier before a tile is read), so the read is hidden from that analysis.  The compiler then does not know
+// that `dst` arrives late either: nothing may touch dst before lds_tr_wait has named it.
+__device__ __forceinline__ void lds_read_tr4_issue(half4_t& dst, const half_t* p) {
+    const unsigned addr = (unsigned)(uintptr_t)p;  // a pointer into LDS: its low 32 bits are the LDS address
+    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(dst) : "v"(addr));
+}
+// waits until at most PENDING LDS operations issued after the reads of lo / hi are outstanding, and makes every later use of
+// lo / hi depend on that wait
+template <int PENDING = 0>
+__device__ __forceinline__ void lds_tr_wait(half4_t& lo, half4_t& hi) {
+    asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(lo), "+v"(hi) : "n"(PENDING));
+}
+// the plain 16-byte LDS read and its wait, issued by hand for the same reason
+__device__ __forceinline__ void lds_read16_issue(half8_t& dst, const half_t* p) {
+    const unsigned addr = (unsigned)(uintptr_t)p;
+    asm volatile("ds_read_b128 %0, %1" : "=v"(dst) : "v"(addr));
+}
+template <int PENDING = 0>
+__device__ __forceinline__ void lds_read16_wait(half8_t& v) {
+    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(v) : "n"(PENDING));
+}
+__device__ __forceinline__ half8_t join_half4(half4_t lo, half4_t hi) {
+    return half8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+}
+
+// Workgroup barrier for loops that keep direct-to-LDS loads in flight across it.  __syncthreads() carries a fence for which the
+// compiler waits for ALL such loads (s_waitcnt vmcnt(0)): a ring of tiles would drain at every barrier.  Here the caller waits
+// for exactly the loads and LDS operations it needs (s_waitcnt vmcnt(n) lgkmcnt(0) in front of the call); the empty assembly
+// statements keep the compiler from moving memory accesses across the barrier instruction.
+__device__ __forceinline__ void barrier_keep_loads_in_flight() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
 // ---- direct-to-LDS loads and the bank-conflict swizzles of the LDS-tiled kernels -------------------------------------------
 typedef __attribute__((address_space(3))) void lds_void_t;
 typedef __attribute__((address_space(1))) const void gbl_void_t;

@@ -157,7 +157,17 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, GemmGroup
         for (int j = 0; j < NJ; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     // LDS read unit u of k-step ks: u < NJ -> W fragment u, else X fragment u - NJ (W first: every MFMA row needs all of b)
-    auto read_unit = [&](const half_t* xs, const half_t* ws, int ks, int u, half8_t (&a)[8], half8_t (&b)[NJ]) {
+    // [K, N] weights: the two transposed 8-byte reads of a W fragment are issued by hand (lds_read_tr4_issue) into blo / bhi
+    // [set][u] and joined into the fragment at the start of the phase that multiplies it (finish_b)
+    half4_t blo[2][NJ], bhi[2][NJ];
+    int wfrag[NJ];   // [K, N] weights: offset (halves) inside a W tile of this lane's first transposed read of fragment u at ks = 0
+#pragma unroll
+    for (int u = 0; u < NJ; ++u) {
+        const int blk = wn * NJ + u;             // 32-byte block = 16 output columns
+        const int k = lk * 8 + (l16 >> 2);       // this lane's source row of the first 4x16 read
+        wfrag[u] = k * FB_N + unswz_kn<NJ>(k, blk) * 16 + (l16 & 3) * 4;
+    }
+    auto read_unit = [&](const half_t* xs, const half_t* ws, int ks, int u, half8_t (&a)[8], half8_t (&b)[NJ], int set) {
         if (u >= NJ) {
             const int i = u - NJ;
             const int row = wm * 128 + i * 16 + l16;
@@ -166,11 +176,18 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, GemmGroup
             const int row = wn * (16 * NJ) + u * 16 + l16;
             b[u] = *reinterpret_cast<const half8_t*>(&ws[row * FB_K + swz_a(row, ks * 4 + lk) * 8]);
         } else {
-            const int blk = wn * NJ + u;                     // 32-byte block = 16 output columns
-            const int k = ks * 32 + lk * 8 + (l16 >> 2);     // this lane's source row of the first 4x16 read
-            const half4_t lo = lds_read_tr4(&ws[k * FB_N + unswz_kn<NJ>(k, blk) * 16 + (l16 & 3) * 4]);
-            const half4_t hi = lds_read_tr4(&ws[(k + 4) * FB_N + unswz_kn<NJ>(k + 4, blk) * 16 + (l16 & 3) * 4]);
-            b[u] = half8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            // rows k and k + 4 of the tile, k = 32 ks + 8 lk + l16 / 4; neither ks nor the + 4 changes a block's position in its
+            // row (the swizzles look at bits 0, 1 and 3 of k only), so both are plain offsets from the lane's base for ks = 0
+            lds_read_tr4_issue(blo[set][u], ws + wfrag[u] + ks * 32 * FB_N);
+            lds_read_tr4_issue(bhi[set][u], ws + wfrag[u] + (ks * 32 + 4) * FB_N);
+        }
+    };
+    auto finish_b = [&](half8_t (&b)[NJ], int set) {
+        if (WL != W_KN) return;
+#pragma unroll
+        for (int u = 0; u < NJ; ++u) {
+            lds_tr_wait<0>(blo[set][u], bhi[set][u]);
+            b[u] = join_half4(blo[set][u], bhi[set][u]);
         }
     };
     constexpr int NDS = 8 + NJ;       // LDS read units per k-step
@@ -183,10 +200,12 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, GemmGroup
     // and, if LOADS, the global -> LDS loads of a later k-tile placed between them in exactly this order: the
     // scheduling fence after every MFMA keeps the compiler from regrouping them.  Operands are swapped in the MFMA so
     // that each lane owns 4 consecutive output columns of one row.
-    auto phase = [&](auto with_loads, half8_t (&ma)[8], half8_t (&mb)[NJ], half8_t (&ra)[8], half8_t (&rb)[NJ],
+    auto phase = [&](auto with_loads, auto mset_c, half8_t (&ma)[8], half8_t (&mb)[NJ], half8_t (&ra)[8], half8_t (&rb)[NJ],
                      const half_t* rxs, const half_t* rws, int rks, const char* xg, const char* wg, half_t* lxs,
                      half_t* lws) {
         constexpr bool LOADS = decltype(with_loads)::value;
+        constexpr int MSET = decltype(mset_c)::value;   // which blo / bhi set holds mb's halves; the reads go to the other
+        finish_b(mb, MSET);
 #pragma unroll
         for (int m = 0; m < NMFMA; ++m) {
             const int i = m / NJ, j = m % NJ;
@@ -203,7 +222,7 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, GemmGroup
                 // [N, K] weights: one read unit every DS_SPAN / NDS MFMAs.  [K, N] weights: the W units (two transposed
                 // reads each) go under the first NJ MFMAs, the X units are spread over the rest (measured: 8 % faster)
                 const int at = (WL == W_NK) ? (u * DS_SPAN + DS_SPAN - 1) / NDS : (u < NJ ? u : NJ + (u - NJ) * (DS_SPAN - NJ) / 8);
-                if (at == m) read_unit(rxs, rws, rks, u, ra, rb);
+                if (at == m) read_unit(rxs, rws, rks, u, ra, rb, MSET ^ 1);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -219,7 +238,7 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, GemmGroup
     __syncthreads();
     half8_t a0[8], b0[NJ], a1[8], b1[NJ];
 #pragma unroll
-    for (int u = 0; u < NDS; ++u) read_unit(xring, wring, 0, u, a0, b0);
+    for (int u = 0; u < NDS; ++u) read_unit(xring, wring, 0, u, a0, b0, 0);
 
     int xslot = 0, xnext = 1;  // kt % 3, (kt + 1) % 3
     for (int kt = 0; kt < ktiles; ++kt) {
@@ -227,14 +246,14 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, GemmGroup
         half_t* const xs = xring + xslot * X_TILE;
         half_t* const ws = wring + wslot * W_TILE;
         // first k-step multiplies while the second k-step's fragments stream in
-        phase(std::false_type{}, a0, b0, a1, b1, xs, ws, 1, nullptr, nullptr, nullptr, nullptr);
+        phase(std::false_type{}, std::integral_constant<int, 0>{}, a0, b0, a1, b1, xs, ws, 1, nullptr, nullptr, nullptr, nullptr);
         // all of tile kt is in this wave's registers; its loads of X(kt+1) and W(kt+1) have landed, the four loads of
         // X(kt+2) issued last may stay in flight across the barrier
         asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
         __syncthreads();
         // every wave is past tile kt: its W slot takes W(kt+2), its X slot X(kt+3); tile kt+1's first fragments stream
         // in under the MFMAs of the second k-step
-        phase(std::true_type{}, a1, b1, a0, b0, xring + xnext * X_TILE, wring + (wslot ^ 1) * W_TILE, 0, x_tile(kt + 3),
+        phase(std::true_type{}, std::integral_constant<int, 1>{}, a1, b1, a0, b0, xring + xnext * X_TILE, wring + (wslot ^ 1) * W_TILE, 0, x_tile(kt + 3),
               w_tile(kt + 2), xs, ws);
         xslot = xnext;
         xnext = (xnext == X_STAGES - 1) ? 0 : xnext + 1;

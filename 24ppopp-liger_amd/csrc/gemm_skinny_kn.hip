@@ -91,21 +91,27 @@ __global__ __launch_bounds__(KN_THREADS) void gemm_skinny_kn_kernel(GemmArgs g, 
     for (int t = 0; t < NS - 1; ++t) issue(t);
     for (int t = 0; t < ktiles; ++t) {
         // tile t has landed when at most the loads of tiles t+1 .. t+NS-2 are outstanding
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 2) * LPS) : "memory");
-        __syncthreads();  // tile t is visible to every wave, and every wave is done with tile t-1: its slot is refilled now
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((NS - 2) * LPS) : "memory");
+        barrier_keep_loads_in_flight();  // tile t is visible to every wave, and every wave is done with tile t-1: its slot is refilled now
         issue(t + NS - 1);
         const half_t* ws = wring + (t % NS) * W_TILE;
         const half_t* xs = xring + (t % NS) * X_TILE;
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
-            half8_t b[NU];
+            // transposed reads issued by hand (see lds_read_tr4_issue): all of the k-step's, then one wait
+            half4_t blo[NU], bhi[NU];
 #pragma unroll
             for (int u = 0; u < NU; ++u) {
                 const int blk = wave * NU + u;                   // 32-byte block = 16 output features
                 const int k = ks * 32 + lk * 8 + (l16 >> 2);     // this lane's source row of the first 4x16 read
-                const half4_t lo = lds_read_tr4(&ws[k * KN_BN + swz_b(k, blk) * 16 + (l16 & 3) * 4]);
-                const half4_t hi = lds_read_tr4(&ws[(k + 4) * KN_BN + swz_b(k + 4, blk) * 16 + (l16 & 3) * 4]);
-                b[u] = half8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                lds_read_tr4_issue(blo[u], &ws[k * KN_BN + swz_b(k, blk) * 16 + (l16 & 3) * 4]);
+                lds_read_tr4_issue(bhi[u], &ws[(k + 4) * KN_BN + swz_b(k + 4, blk) * 16 + (l16 & 3) * 4]);
+            }
+            half8_t b[NU];
+#pragma unroll
+            for (int u = 0; u < NU; ++u) {
+                lds_tr_wait<0>(blo[u], bhi[u]);
+                b[u] = join_half4(blo[u], bhi[u]);
             }
 #pragma unroll
             for (int i = 0; i < MT; ++i) {
