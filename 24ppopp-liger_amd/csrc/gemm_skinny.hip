@@ -206,8 +206,8 @@ __global__ __launch_bounds__(64 * NWV) void gemm_skinny_direct_kernel(GemmArgs g
     }
     store_x(0, xq[0]);
     __syncthreads();
-    // one chunk: multiply its 8 fragments (registers b) with the X chunk in LDS buffer `buf`, reloading each fragment's
-    // registers with the chunk DEPTH ahead as soon as it has been used; at its end the X chunk fetched one chunk ago goes
+    // one chunk: multiply its 8 fragments (registers b) with the X chunk in LDS buffer `buf`, reloading each pair of
+    // fragments' registers with the chunk DEPTH ahead as soon as both have been used; at its end the X chunk fetched one chunk ago goes
     // to the other LDS buffer.  Chunks past the
     // end wrap around to valid addresses and are never multiplied.
     auto do_chunk = [&](int ch, int buf, half8_t (&b)[8]) {
@@ -224,7 +224,12 @@ __global__ __launch_bounds__(64 * NWV) void gemm_skinny_direct_kernel(GemmArgs g
                 const half8_t a = *reinterpret_cast<const half8_t*>(&xs[buf][(i * 16 + l16) * SK_XS + s * 32 + lk * 8]);
                 acc[i] = mfma16(b[s], a, acc[i]);  // operands swapped: acc[i][r] = Y[16 i + l16][n0 + 4 lk + r]
             }
-            b[s] = *reinterpret_cast<const half8_t*>(wn + s * 32);
+            // a fragment is one 64-byte half of a 128-byte weight line per row: both halves are requested back to back,
+            // after the second has been used (requested a fragment apart they reach the L2 as two separate half-line reads)
+            if (s & 1) {
+                b[s - 1] = *reinterpret_cast<const half8_t*>(wn + (s - 1) * 32);
+                b[s] = *reinterpret_cast<const half8_t*>(wn + s * 32);
+            }
             asm volatile("" ::: "memory");
             __builtin_amdgcn_sched_barrier(0);
         }
