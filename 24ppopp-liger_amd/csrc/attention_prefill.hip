@@ -17,12 +17,31 @@
 //                                           exactly the accumulator layout S^T came out in (4 consecutive keys per
 //                                           lane), so the probabilities go from MFMA result to MFMA operand in place.
 // Softmax statistics are per query = per (lane % 16); the four 16-lane groups hold different keys and are combined
-// with two shuffles per tile.
+// with two row swaps per tile.
 #include "gemm_common.cuh"
 
 namespace lg {
 
 constexpr int PF_BC = 64;   // keys per LDS tile
+
+// max(x, x of lane ^ 16) and max(x, x of lane ^ 32) through the gfx950 row-swap instructions: with both operands holding
+// x, v_permlane16_swap leaves {row 0, row 0, row 2, row 2} in the first and {row 1, row 1, row 3, row 3} in the second
+// (rows of 16 lanes), v_permlane32_swap {low half, low half} and {high half, high half}.  Plain VALU operations: no trip
+// through the LDS crossbar (ds_bpermute) in the middle of the softmax's dependent chain.
+typedef unsigned uint2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float max_of_swapped(uint2_t r) {
+    float m;
+    asm("v_max_f32 %0, %1, %2" : "=v"(m) : "v"(r[0]), "v"(r[1]));  // by hand: fmaxf would first canonicalise both bit-cast inputs
+    return m;
+}
+__device__ __forceinline__ float max_xor16(float x) {
+    const unsigned u = __float_as_uint(x);
+    return max_of_swapped(__builtin_amdgcn_permlane16_swap(u, u, false, false));
+}
+__device__ __forceinline__ float max_xor32(float x) {
+    const unsigned u = __float_as_uint(x);
+    return max_of_swapped(__builtin_amdgcn_permlane32_swap(u, u, false, false));
+}
 
 template <int D, int NW, bool CAUSAL, bool HAS_MASK>
 // two waves per SIMD (at most 256 registers): the softmax arithmetic of one wave runs under the MFMAs of the other
@@ -44,15 +63,24 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l16 = lane & 15, g = lane >> 4;
-    // Workgroups are handed to the 8 XCDs round-robin by their linear id.  The query blocks of one (batch, head) read the same
-    // K/V rows, so they are placed on ONE XCD, one after the other (its L2 then serves the re-reads: without this the K/V of a
-    // causal 512-token head are fetched 2.5 times), the longest (last) query block first.
+    // Workgroups are handed to the 8 XCDs round-robin by their linear id.  All query blocks of one (batch, head) go to ONE
+    // XCD: without a causal mask one after the other (they read the same K/V rows, which that XCD's L2 then serves); with it,
+    // ordered by their length (below), which costs the L2 re-use (K/V are then fetched about 2.5 times, from the memory-side
+    // cache) and gains an even finish.
     int bh = blockIdx.y, qblk = blockIdx.x;    // bh = b * head_num + head
     if ((gridDim.y & 7) == 0) {
         const int lin = blockIdx.x + gridDim.x * blockIdx.y;
         const int xcd = lin & 7, slot = lin >> 3;
-        bh = (slot / (int)gridDim.x) * 8 + xcd;
-        qblk = (int)gridDim.x - 1 - slot % (int)gridDim.x;
+        if (CAUSAL) {
+            // a causal query block's work grows with its position: every XCD starts the last (longest) query block of all its
+            // heads first, then the one before, ... so that the blocks still running at the end are the short ones
+            const int per_xcd = (int)gridDim.y >> 3;
+            bh = (slot % per_xcd) * 8 + xcd;
+            qblk = (int)gridDim.x - 1 - slot / per_xcd;
+        } else {
+            bh = (slot / (int)gridDim.x) * 8 + xcd;
+            qblk = slot % (int)gridDim.x;
+        }
     }
     const int b = bh / head_num, head = bh % head_num;
     const int q0 = qblk * PF_BQ;               // first query of the block
@@ -146,25 +174,33 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
         // kt + 1 are requested before the MFMAs of key tile kt.
         float4_t s[4][2];
         half8_t kf[2][DC];
-        auto kissue = [&](int kt, int slot) {
+        // one address register per d-chunk when the row is a power of two (the key tile's distance goes into the instruction)
+        unsigned kbase[DC];
 #pragma unroll
-            for (int dc = 0; dc < DC; ++dc) lds_read16_issue(kf[slot][dc], &ks[P2 ? kfrag[0][dc] + kt * 16 * D : kfrag[kt % KG][dc]]);
+        for (int dc = 0; dc < DC; ++dc) kbase[dc] = lds_address(ks + kfrag[0][dc]);
+        auto kissue = [&](auto ktc, int slot) {
+            constexpr int kt = decltype(ktc)::value;
+#pragma unroll
+            for (int dc = 0; dc < DC; ++dc) {
+                if constexpr (P2) lds_read16_issue_at<kt * 16 * D * 2>(kf[slot][dc], kbase[dc]);
+                else lds_read16_issue(kf[slot][dc], &ks[kfrag[kt % KG][dc]]);
+            }
         };
-        kissue(0, 0);
-#pragma unroll
-        for (int kt = 0; kt < 4; ++kt) {
-            const int slot = kt & 1;
-            if (kt + 1 < 4) kissue(kt + 1, slot ^ 1);
+        kissue(std::integral_constant<int, 0>{}, 0);
+        static_for<4>([&](auto ktc) {
+            constexpr int kt = decltype(ktc)::value;
+            constexpr int slot = kt & 1;
+            if constexpr (kt + 1 < 4) kissue(std::integral_constant<int, kt + 1>{}, slot ^ 1);
             s[kt][0] = float4_t{0.f, 0.f, 0.f, 0.f};
             s[kt][1] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int dc = 0; dc < DC; ++dc) {
-                if (kt + 1 < 4) lds_read16_wait<DC>(kf[slot][dc]);   // the DC reads of the next key tile may be outstanding
+                if constexpr (kt + 1 < 4) lds_read16_wait<DC>(kf[slot][dc]);   // the DC reads of the next key tile may be outstanding
                 else lds_read16_wait<0>(kf[slot][dc]);
                 s[kt][0] = mfma16(kf[slot][dc], qf[0][dc], s[kt][0]);
                 s[kt][1] = mfma16(kf[slot][dc], qf[1][dc], s[kt][1]);
             }
-        }
+        });
         // ---- scale, mask, online softmax (per query column) -----------------------------------------------------
         // Scores are kept in log2 units (scale folded with log2 e: exp(t - m) = exp2(t' - m')), so that a score costs one
         // multiply, one max, one subtract, one exp2 and one add.  The causal comparison is only made on tiles that reach above
@@ -208,8 +244,8 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
             for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[kt][qt][r]);
-            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            mx = max_xor16(mx);
+            mx = max_xor32(mx);
             const float m_new = fmaxf(m_run[qt], mx);
             const float corr = __builtin_amdgcn_exp2f(m_run[qt] - m_new);
             m_run[qt] = m_new;
@@ -227,8 +263,11 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
             for (int dt = 0; dt < DT; ++dt) o[dt][qt] *= corr;
         }
         // ---- O^T += V^T P^T ---------------------------------------------------------------------------------------
+        unsigned vbase[DT];   // as for K: one address register per d-tile when the row is a power of two
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {  // two k-steps of 32 keys: key tiles 2j and 2j+1
+        for (int dt = 0; dt < DT; ++dt) vbase[dt] = lds_address(vs + vfrag[0][dt]);
+        static_for<2>([&](auto jc) {  // two k-steps of 32 keys: key tiles 2j and 2j+1
+            constexpr int j = decltype(jc)::value;
             half8_t pf[2];
 #pragma unroll
             for (int qt = 0; qt < 2; ++qt) {
@@ -236,7 +275,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
                 pf[qt] = half8_t{(half_t)lo[0], (half_t)lo[1], (half_t)lo[2], (half_t)lo[3],
                                  (half_t)hi[0], (half_t)hi[1], (half_t)hi[2], (half_t)hi[3]};
             }
-            // The transposed reads are issued by hand (lds_read_tr4_issue: the builtin would make the compiler wait for the
+            // The transposed reads are issued by hand (the builtin would make the compiler wait for the
             // loads of the NEXT tile, issued above, before every read), a group of VGRP fragments ahead of the MFMAs that use
             // them: logical 32-byte block dt of rows 32 j + 4 g + l16 / 4 and 16 rows further on, this lane's 8 bytes inside it.
             constexpr int VGRP = 2;
@@ -246,8 +285,13 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
 #pragma unroll
                 for (int i = 0; i < VGRP; ++i) {
                     const int dt = grp * VGRP + i;
-                    lds_read_tr4_issue(vlo[slot][i], &vs[P2 ? vfrag[0][dt] + (2 * j) * 16 * D : vfrag[(2 * j) % VG][dt]]);
-                    lds_read_tr4_issue(vhi[slot][i], &vs[P2 ? vfrag[0][dt] + (2 * j + 1) * 16 * D : vfrag[(2 * j + 1) % VG][dt]]);
+                    if constexpr (P2) {
+                        lds_read_tr4_issue_at<(2 * j) * 16 * D * 2>(vlo[slot][i], vbase[dt]);
+                        lds_read_tr4_issue_at<(2 * j + 1) * 16 * D * 2>(vhi[slot][i], vbase[dt]);
+                    } else {
+                        lds_read_tr4_issue(vlo[slot][i], &vs[vfrag[(2 * j) % VG][dt]]);
+                        lds_read_tr4_issue(vhi[slot][i], &vs[vfrag[(2 * j + 1) % VG][dt]]);
+                    }
                 }
             };
             vissue(0, 0);
@@ -266,7 +310,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
                     o[dt][1] = mfma16(a, pf[1], o[dt][1]);
                 }
             }
-        }
+        });
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 

@@ -4,6 +4,8 @@
 //     Y[M, N] (ldy) = X[M, K] (ldx) * W,      W given either as [K, N] (W_KN) or as [N, K] (W_NK).
 // M = tokens, N = output features, K = reduction.
 #pragma once
+#include <utility>
+
 #include "common.cuh"
 
 namespace lg {
@@ -113,6 +115,30 @@ template <int PENDING = 0>
 __device__ __forceinline__ void lds_read16_wait(half8_t& v) {
     asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(v) : "n"(PENDING));
 }
+// Both reads at LDS byte address `addr` plus a compile-time byte offset that travels in the instruction (16-bit field): a lane
+// that reads the same position of several rows groups or ring slots needs one address register for all of them.
+template <int OFF>
+__device__ __forceinline__ void lds_read16_issue_at(half8_t& dst, unsigned addr) {
+    static_assert(OFF >= 0 && OFF < 65536, "the offset field of an LDS instruction holds 16 bits");
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+template <int OFF>
+__device__ __forceinline__ void lds_read_tr4_issue_at(half4_t& dst, unsigned addr) {
+    static_assert(OFF >= 0 && OFF < 65536, "the offset field of an LDS instruction holds 16 bits");
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+__device__ __forceinline__ unsigned lds_address(const half_t* p) { return (unsigned)(uintptr_t)p; }
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a compile-time constant in its body
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
 __device__ __forceinline__ half8_t join_half4(half4_t lo, half4_t hi) {
     return half8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
 }
