@@ -20,6 +20,8 @@
 //     operands are swapped in the MFMA so that a lane ends up with 4 consecutive output columns of one row;
 //   * workgroup ids are remapped so that the 32 workgroups resident on one XCD (ids congruent mod 8) form a compact
 //     4 x 8 block of tiles and share their X / W panels in that XCD's L2.
+#include <stdlib.h>
+
 #include "gemm_common.cuh"
 #include <type_traits>
 
@@ -424,6 +426,10 @@ int launch_gemm_fast_f16(const GemmArgs& g, const GemmGroup& grp, int wlayout, i
         const long cost = ((tiles + si.cus - 1) / si.cus) * nj * (nj == 4 ? 100 : nj == 3 ? 103 : 135);
         if (!best_nj || cost < best_cost) { best_nj = nj; best_cost = cost; }
     }
+    // LG_GEMM_TILE_WIDTH=2|3|4 in the environment (read once) overrides the choice where that width divides N: a measurement knob
+    // (256 x 128 tiles leave registers and LDS for a second kernel's waves on the same compute unit)
+    static const int forced_nj = [] { const char* e = getenv("LG_GEMM_TILE_WIDTH"); return e ? atoi(e) : 0; }();
+    if (forced_nj >= 2 && forced_nj <= 4 && g.N % (64 * forced_nj) == 0 && !(forced_nj == 3 && g.epi.kind == LG_EPI_BIAS_GEGLU)) best_nj = forced_nj;
     if (!best_nj) return LG_OK;
     *handled = true;
     const int tiles_n = g.N / (64 * best_nj) * grp.count;

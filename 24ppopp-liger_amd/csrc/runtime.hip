@@ -233,6 +233,9 @@ int lg_stream_attach(void* stream, int cu_count) {
 }
 int lg_stream_detach(void* stream) { return unregister_stream(stream); }
 int lg_stream_cu_count(void* stream) { return stream_info((hipStream_t)stream).cus; }
+__global__ void lg_stream_first_use_kernel(int* sink) {
+    if (sink && threadIdx.x == 1024) *sink = 1;  // never true: an empty kernel
+}
 int lg_stream_create_cu_mask(void** stream, const unsigned* cu_mask, int mask_words) {
     if (!stream || !cu_mask || mask_words <= 0) { set_error("lg_stream_create_cu_mask: bad arguments"); return LG_ERR_INVALID; }
     // Bit i of the mask selects a compute unit of accelerator die i mod 8 (the dies take the bits in turn).  A mask that leaves
@@ -247,7 +250,15 @@ int lg_stream_create_cu_mask(void** stream, const unsigned* cu_mask, int mask_wo
     hipStream_t s = nullptr;
     int rc = rt(hipExtStreamCreateWithCUMask(&s, (uint32_t)mask_words, cu_mask), "hipExtStreamCreateWithCUMask");
     *stream = (void*)s;
-    return rc ? rc : register_stream((void*)s, cus);
+    if (rc) return rc;
+    // The runtime sets a stream's hardware queue up at its first submission.  A CU-masked stream that is destroyed without ever
+    // having run anything has been seen to block in hipStreamDestroy (about one time in four), so every such stream runs one
+    // empty kernel here, at creation, where waiting is allowed.
+    hipLaunchKernelGGL(lg_stream_first_use_kernel, dim3(1), dim3(64), 0, s, (int*)nullptr);
+    rc = rt(hipGetLastError(), "first kernel on a CU-masked stream");
+    if (!rc) rc = rt(hipStreamSynchronize(s), "hipStreamSynchronize");
+    if (rc) { (void)hipStreamDestroy(s); *stream = nullptr; return rc; }
+    return register_stream((void*)s, cus);
 }
 // ---- a second stream that really runs next to the first ----------------------------------------------------------------------
 // HIP multiplexes streams onto a few hardware queues (4 per process by default) and hands a new stream the least used one,

@@ -161,6 +161,49 @@ def bench_cfg4(capi, host, weight_layout, factors=(1, 2, 4, 8), shares=(0, 32, 6
             "results": out}
 
 
+def bench_corun_one(capi, host, weight_layout, dec_bs):
+    """One process of --corun-variants: the MFMA-bound kernels of a prefill layer shard (batch 4 x seq 512) next to decode steps
+    (`dec_bs` sequences, 1024 cached positions) with both streams on the whole chip, and with the HBM-bound side on 64 / 128
+    compute units, each against the same work back to back on the whole chip.  The pipelined GEMM's tile width follows
+    LG_GEMM_TILE_WIDTH (unset: chosen by shape, 256 x 256 here; 2: 256 x 128, which leaves room for other waves on the CU)."""
+    c = CFG2
+    model = host.Model(capi.F16, 64, 512, c["heads_global"], c["d"], layer_num=1, world_size=c["world_size"], ffn_inner=c["ffn_global"],
+                       causal=True, fused=True, max_cache_len=1024 + 64, weight_layout=weight_layout, seed=0)
+    sched = host.Scheduler(model, schedule_deep=6, contention_factor=0.8, policy=host.POLICY_RESOURCE, axis=host.SPLIT_TOKEN_ROWS,
+                           seq_bucket=64, ignore_num=0, pool_count=2, ctx_batch=32)
+    out = {"tile_width": os.environ.get("LG_GEMM_TILE_WIDTH", "auto"), "decode_batch": dec_bs}
+    w = sched.profile_contention(4, 512, dec_bs, 1024)
+    w["gain"] = (w["main_ms"] + w["sub_ms"]) / w["both_ms"]
+    out["whole_chip"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in w.items()}
+    for share in (64, 128):
+        sched.enable_partition(share)
+        meas = sched.profile_partition(4, 512, dec_bs, 1024)
+        out["hbm_cus_%d" % share] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in meas.items()}
+    sched.enable_partition(0)
+    sched.close()
+    model.close()
+    return out
+
+
+def bench_corun_variants(weight_layout):
+    """GEMM variant x CU share: one child process per (tile width, decode batch), because the library reads the tile width once."""
+    import subprocess
+    rows = []
+    for width in ("", "2"):
+        for dec_bs in (32, 16):
+            env = dict(os.environ)
+            env.pop("LG_GEMM_TILE_WIDTH", None)
+            if width:
+                env["LG_GEMM_TILE_WIDTH"] = width
+            r = subprocess.run([sys.executable, os.path.abspath(__file__), "--corun-one", str(dec_bs), "--weight-layout", str(weight_layout)],
+                               env=env, stdout=subprocess.PIPE, text=True, timeout=300)
+            if r.returncode != 0:
+                raise RuntimeError("co-run measurement (tile width %s, decode batch %d) failed with status %d" % (width or "auto", dec_bs, r.returncode))
+            rows.append(json.loads(r.stdout.strip().splitlines()[-1]))
+            print("corun: tile width %s, decode batch %d done" % (width or "auto", dec_bs), file=sys.stderr, flush=True)
+    return {"workload": "prefill B4 S512 MFMA-bound kernels || decode steps at 1024 cached positions, one layer shard", "rows": rows}
+
+
 def bench_cfg5(capi, host, weight_layout, n_requests, rates=(4.0, 8.0, 16.0), shares=(64, 128), runs=1, decode_steps_ahead=2, short=False):
     """BASELINE config 5: Poisson arrivals at 4, 8, 16 req/s through 4 stacked layer shards; prompts U[128, 1024]
     (rounded to 64), 32 decode tokens each; mean and p99 request latency with interleaving on and off.  `runs` > 1 repeats
@@ -312,6 +355,9 @@ def main():
     ap.add_argument("--cfg5", action="store_true", help="run the full mixed request trace (BASELINE config 5; minutes) instead of the short record")
     ap.add_argument("--cfg5-requests", type=int, default=60)
     ap.add_argument("--cfg5-runs", type=int, default=3)
+    ap.add_argument("--corun-variants", action="store_true",
+                    help="GEMM tile width (chosen by shape / 256 x 128) x CU share: prefill MFMA kernels next to decode steps, one JSON line")
+    ap.add_argument("--corun-one", type=int, default=0, help=argparse.SUPPRESS)
     ap.add_argument("--kernel-only", default=None,
                     help="launch only the named launch-vector entry (e.g. 'ffn1+bias+gelu', 'attn_decode', 'layer_norm') or "
                          "'copy' (a plain 128 MiB read + 128 MiB write kernel) --iters times; for rocprofv3 runs")
@@ -327,6 +373,9 @@ def main():
               "(the all-reduce between GPUs is out of scope)" % args.gpus, file=sys.stderr)
         sys.exit(2)
 
+    if args.corun_variants:
+        print(json.dumps(bench_corun_variants(args.weight_layout)), flush=True)
+        return
     import torch
     liger = importlib.import_module("24ppopp-liger_amd")
     host = importlib.import_module("24ppopp-liger_amd.host")
@@ -338,6 +387,9 @@ def main():
     M = B * S
     fused = not args.unfused
 
+    if args.corun_one:
+        print(json.dumps(bench_corun_one(capi, host, args.weight_layout, args.corun_one)), flush=True)
+        return
     if args.kernel_only:
         model = host.Model(capi.F16, 32, S, c["heads_global"], c["d"], layer_num=1, world_size=c["world_size"], ffn_inner=c["ffn_global"],
                            norm_mode=host.POST_NORESID, causal=True, fused=fused, max_cache_len=CFG3["cache_len"] + 32 if fused else 0,

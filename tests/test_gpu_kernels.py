@@ -200,6 +200,24 @@ def test_cu_masked_stream_runs_kernels(dev, po):
     assert lib.lg_stream_create_cu_mask(C.byref(s2), empty, 8) == 1  # LG_ERR_INVALID
 
 
+def test_cu_masked_streams_that_never_ran_a_kernel_can_be_destroyed(dev):
+    """The four streams of a partitioned scheduler are created together, and a run may never use some of them: creating and
+    destroying CU-masked streams without submitting anything must return (the library gives each stream one empty kernel at
+    creation, because destroying one that never ran anything has blocked in the runtime)."""
+    import ctypes as C
+    lib = dev.lib
+    hbm = (C.c_uint * 8)(*([0xFFFFFFFF] * 2 + [0] * 6))     # compute units 0..63: 8 on every die
+    mfma = (C.c_uint * 8)(*([0] * 2 + [0xFFFFFFFF] * 6))
+    streams = []
+    for words in (mfma, hbm, mfma, hbm):
+        s = C.c_void_p()
+        assert lib.lg_stream_create_cu_mask(C.byref(s), words, 8) == 0, dev.capi.last_error()
+        streams.append(s)
+    assert lib.lg_stream_cu_count(streams[0]) == 192 and lib.lg_stream_cu_count(streams[1]) == 64
+    for s in streams:
+        assert lib.lg_stream_destroy(s) == 0, dev.capi.last_error()
+
+
 def test_second_stream_is_verified_to_run_next_to_the_first(dev, po):
     """lg_stream_create_concurrent hands out a stream whose kernels overlap with the given stream's (measured by the
     library) even when the process already holds more streams than there are hardware queues; the stream computes like any
