@@ -66,7 +66,9 @@ int lg_stream_cu_count(void* stream);
  * words, bit i of word w = mask bit 32*w + i; on this GPU bit i selects a unit of accelerator die i mod 8, and every die must
  * keep at least one unit).  The launchers size their grids for the number of selected units.  Takes the place of the two stream priorities
  * the reference gives its streams (context.h:28-29, schedule.h:54-55): on this platform the two streams of the scheduler
- * are separated in space, not by priority. */
+ * are separated in space, not by priority.  The call runs one empty kernel on the new stream and waits for it (a stream of
+ * this kind that is destroyed before anything ran on it has blocked in the runtime's destroy call): it may block, like every
+ * stream creation here; launches never do. */
 int lg_stream_create_cu_mask(void** stream, const unsigned* cu_mask, int mask_words);
 /* Non-blocking stream that is verified, by measurement, to run kernels at the same time as `other` (the scheduler's
  * second stream, schedule.h:54-55).  HIP multiplexes a process's streams onto a few hardware queues and two streams
