@@ -111,9 +111,19 @@ def test_fp16_layer_on_the_pipelined_gemm(dev, po, host, weight_layout):
     assert max_rel_err(got, ref) < 1e-2
 
 
-def test_decode_step_matches_oracle(dev, po, host):
+@pytest.mark.parametrize("fused", [False, True])
+@pytest.mark.parametrize("weight_layout", [0, 1])
+def test_fp16_layer_with_the_published_head_size(dev, po, host, fused, weight_layout):
+    """The reference's published configuration uses 96-wide heads, batch 2 and sequences of 16 to 115 tokens (main.cu:14-21):
+    one TP=2 shard of a two-layer stack with that head size at the longest of those sequences."""
+    got, ref, _ = run_layer_case(dev, po, host, 1, 2, 115, 8, 96, 3072, 0, True, fused, ws=2, layers=2, weight_layout=weight_layout)
+    assert max_rel_err(got, ref) < 1e-2
+
+
+@pytest.mark.parametrize("heads,d", [(4, 64), (4, 96)])
+def test_decode_step_matches_oracle(dev, po, host, heads, d):
     """Fused prefill fills the KV cache, then two decode steps; each is checked against the oracle's decoder step."""
-    B, S, heads, d, F, Lmax = 2, 40, 4, 64, 512, 64
+    B, S, F, Lmax = 2, 40, 512, 64
     H = heads * d
     m = host.Model(1, B, S, heads, d, layer_num=1, ffn_inner=F, causal=True, fused=True, max_cache_len=Lmax, seed=3)
     w = oracle_weights(m.download_params())
