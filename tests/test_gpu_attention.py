@@ -121,7 +121,10 @@ def test_kv_append(dev, po, B, h, d, pos, Lmax):
 @pytest.mark.parametrize("B,h,S,d,mode,kv_rows,layout", [
     (2, 3, 128, 128, "causal", 128, 0), (1, 2, 200, 64, "causal", 256, 1), (2, 2, 77, 128, "mask", 77, 1),
     (1, 1, 512, 128, "none", 512, 0), (1, 2, 1000, 128, "causal", 1024, 1), (1, 1, 5, 64, "causal", 8, 0),
-    (2, 4, 115, 96, "causal", 128, 1), (1, 2, 300, 96, "mask", 300, 0), (1, 3, 64, 96, "none", 64, 1)])
+    (2, 4, 115, 96, "causal", 128, 1), (1, 2, 300, 96, "mask", 300, 0), (1, 3, 64, 96, "none", 64, 1),
+    # batch * heads a multiple of 8 with several query blocks: the block -> (head, query block) placement is remapped
+    (2, 4, 300, 128, "causal", 320, 1), (1, 8, 520, 64, "causal", 520, 0), (2, 4, 300, 128, "none", 300, 0),
+    (1, 16, 260, 96, "causal", 260, 1)])
 def test_attn_prefill_fused(dev, po, B, h, S, d, mode, kv_rows, layout):
     """Fused attention == qk_gemm -> softmax -> qkv_gemm (-> transpose) of the oracle, fp16 semantics."""
     q = rnd(po, B * h * S * d, 70).reshape(B, h, S, d)
