@@ -46,7 +46,7 @@ def _stale(target, deps):
 def build_device(force=True, verbose=False):
     os.makedirs(LIBDIR, exist_ok=True)
     os.makedirs(OBJDIR, exist_ok=True)
-    headers = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".cuh", ".h"))]
+    headers = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".hpp", ".h"))]
     headers.append(os.path.join(ROOT, "include", "liger_hip.h"))
     objs, jobs = [], []
     for src in HIP_SOURCES:

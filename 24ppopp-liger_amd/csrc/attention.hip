@@ -15,7 +15,7 @@
 // t = q.k * scalar, all positions < len unmasked.
 #include <mutex>
 
-#include "common.cuh"
+#include "common.hpp"
 
 namespace lg {
 

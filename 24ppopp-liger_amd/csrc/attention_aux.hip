@@ -1,7 +1,7 @@
 // attention_aux.hip -- the reference-shaped helper kernels around the attention GEMMs:
 // Q/K/V bias + head transpose, scale+mask+softmax (in place), transpose back.
 // All are pure HBM streaming; 16-byte accesses, one wave64 per softmax row.
-#include "common.cuh"
+#include "common.hpp"
 
 namespace lg {
 

@@ -18,7 +18,7 @@
 //                                           lane), so the probabilities go from MFMA result to MFMA operand in place.
 // Softmax statistics are per query = per (lane % 16); the four 16-lane groups hold different keys and are combined
 // with two row swaps per tile.
-#include "gemm_common.cuh"
+#include "gemm_common.hpp"
 
 namespace lg {
 

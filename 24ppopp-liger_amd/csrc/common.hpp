@@ -1,4 +1,4 @@
-// common.cuh -- shared device helpers for the gfx950 (CDNA4, wave64) kernels.
+// common.hpp -- shared device helpers for the gfx950 (CDNA4, wave64) kernels.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>

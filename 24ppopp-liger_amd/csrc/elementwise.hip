@@ -4,7 +4,7 @@
 // in registers (one HBM read, one HBM write per element) and reduce with wave64 shuffles; statistics
 // are two-pass in fp32 exactly as the reference computes them (cuda_kernels.cu:463-508):
 //   mean = sum(x)/n,  var = sum((x-mean)^2)/n,  y = (x-mean) * rsqrt(var + 1e-6) * gamma + beta.
-#include "common.cuh"
+#include "common.hpp"
 
 namespace lg {
 

@@ -5,7 +5,7 @@
 //                      (edge tiles, decomposed sub-ranges, attention GEMMs, small models).
 //   gemm_f32_generic   64x64x16 VALU tiles for the fp32 plumbing configuration.
 // The large aligned prefill shapes are routed to the pipelined kernels in gemm_fast.hip.
-#include "gemm_common.cuh"
+#include "gemm_common.hpp"
 
 namespace lg {
 

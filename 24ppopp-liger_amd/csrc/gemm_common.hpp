@@ -1,4 +1,4 @@
-// gemm_common.cuh -- operand descriptors, epilogues and MFMA helpers shared by the GEMM kernels.
+// gemm_common.hpp -- operand descriptors, epilogues and MFMA helpers shared by the GEMM kernels.
 //
 // All kernels here use the row-major view of the reference's column-major cuBLAS calls:
 //     Y[M, N] (ldy) = X[M, K] (ldx) * W,      W given either as [K, N] (W_KN) or as [N, K] (W_NK).
@@ -6,7 +6,7 @@
 #pragma once
 #include <utility>
 
-#include "common.cuh"
+#include "common.hpp"
 
 namespace lg {
 

@@ -22,7 +22,7 @@
 //     4 x 8 block of tiles and share their X / W panels in that XCD's L2.
 #include <stdlib.h>
 
-#include "gemm_common.cuh"
+#include "gemm_common.hpp"
 #include <type_traits>
 
 namespace lg {

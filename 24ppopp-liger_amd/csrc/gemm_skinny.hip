@@ -13,7 +13,7 @@
 //   * the few X rows are staged once per 256-wide k-chunk in LDS (double buffered) and shared by the block's waves;
 //   * K-slices (when there are any) are summed in fp32 through the stream's workspace and a small second kernel that also
 //     applies the epilogue (bias / GELU / head-transposed store), so results match the single-pass kernels' rounding.
-#include "gemm_common.cuh"
+#include "gemm_common.hpp"
 
 namespace lg {
 

@@ -13,7 +13,7 @@
 //     transposed 8-byte reads (ds_read_b64_tr_b16) and the 16-byte reads of the token rows are spread over the banks;
 //   * K is sliced over the grid until the stream's compute units are filled (N / 128 workgroups per slice); the fp32 partials
 //     go to the stream's workspace and the shared reduce kernel sums them in slice order and applies the epilogue.
-#include "gemm_common.cuh"
+#include "gemm_common.hpp"
 
 namespace lg {
 

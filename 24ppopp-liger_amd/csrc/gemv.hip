@@ -13,7 +13,7 @@
 //     the first weight loads are issued before that staging so that the stream starts at once.
 // Each output is one fixed-order fp32 sum (per-lane partial sums over k in an order fixed by the output's position, then a
 // butterfly), independent of the other token rows.
-#include "gemm_common.cuh"
+#include "gemm_common.hpp"
 
 namespace lg {
 

@@ -5,7 +5,7 @@
 #include <mutex>
 #include <unordered_map>
 
-#include "common.cuh"
+#include "common.hpp"
 
 namespace lg {
 
