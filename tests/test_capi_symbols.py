@@ -36,3 +36,14 @@ def test_version_and_error_text_without_a_gpu(liger):
     assert "bad shape" in liger.capi.last_error()
     assert liger.capi.lib.lg_gemm_f16(0, 1, 4, 4, 4, None, 4, None, 4, None, 4, None) == liger.capi.ERR_INVALID
     assert liger.capi.lib.lg_attn_decode_f16(None, None, None, None, None, 1, 1, 80, 8, 8, 1.0, None) == liger.capi.ERR_INVALID
+
+
+def test_bench_refuses_more_than_one_gpu_with_a_message():
+    """bench.py measures one GPU's shard on one GPU: --gpus 2 exits with status 2 and says so, before anything touches a GPU."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], stdout=subprocess.PIPE, stderr=subprocess.PIPE,
+                       text=True, timeout=120)
+    assert r.returncode == 2
+    assert "--gpus 2 is not supported" in r.stderr and r.stdout == ""
