@@ -448,7 +448,9 @@ def main():
         attn = [k for k in dk if k["kernel"] == "attn_decode"][0]
         kv_bytes = 2 * Bd * 48 * L * 128 * 2
         w_bytes = (3 * H * 6144 + 6144 * H + 2 * H * 16384) * 2
-        gemm_dec_ms = sum(k["ms"] for k in dk if "gemm" in k["kernel"] or "proj" in k["kernel"] or "ffn" in k["kernel"])
+        is_gemm = lambda k: "gemm" in k["kernel"] or "proj" in k["kernel"] or "ffn" in k["kernel"]
+        gemm_dec_ms = sum(k["ms"] for k in dk if is_gemm(k))
+        other_dec_ms = sum(k["ms"] for k in dk if not is_gemm(k))
         decode = {"workload": "cfg3: batch 32, 1 new token, 1024 cached positions", "ms_per_layer_shard": step_ms,
                   "sum_kernel_ms": res["decode"]["sum_kernel_ms"],
                   "tokens_per_s": round(Bd / (step_ms * 1e-3), 1), "kernels": dk,
@@ -457,7 +459,11 @@ def main():
                                            "unit": "GB/s", "frac": round(kv_bytes / (attn["ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
                                            "traffic": measured_traffic("attn_decode")},
                   "skinny_gemms": {"ms": round(gemm_dec_ms, 4), "weight_GBps": round(w_bytes / (gemm_dec_ms * 1e-3) / 1e9, 1),
-                                   "frac": round(w_bytes / (gemm_dec_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}}
+                                   "frac": round(w_bytes / (gemm_dec_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                                   # the same from the end-to-end step: what is left of it after the other kernels (launch gaps
+                                   # included, nothing re-read from the memory-side cache by a repeated launch)
+                                   "in_step_ms": round(step_ms - other_dec_ms, 4),
+                                   "in_step_frac": round(w_bytes / ((step_ms - other_dec_ms) * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}}
 
     out = {
         "metric": "ms/layer-shard prefill (GLM-130B TP=2 shard, B8 S512, causal, fp16)",
