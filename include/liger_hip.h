@@ -196,9 +196,11 @@ int lg_gemm_fused_f16(int transa, int m, int n, int k, const void* A, int lda, c
 
 /* `count` (1..3) lg_gemm_fused_f16 calls that share B (the token rows), the shape, lda and the epilogue arguments
  * and differ in A[i], C[i], ldc[i] and bias[i]: the Q, K and V projections of a decode step (linear.h:99-101 issued
- * three times by bert_layer.h:127-137).  Few-token problems with weights [out, in] run as ONE launch of the
- * weight-streaming kernels; anything else is executed as `count` plain calls.  Results are those of the plain calls
- * up to the order of the fp32 sum over k (the one launch may use another block width).  No reference counterpart. */
+ * three times by bert_layer.h:127-137; also the column blocks of one packed [H, 3 Hl] weight: A[i] = the block's first
+ * column or row, lda = the packed matrix's).  Few-token problems with weights [out, in] run as ONE launch of the
+ * weight-streaming kernels, problems of more than 256 token rows as ONE launch of the pipelined kernel (either weight
+ * layout); anything else is executed as `count` plain calls.  Results are those of the plain calls up to the order of the
+ * fp32 sum over k (the one launch may use another block width).  No reference counterpart. */
 int lg_gemm_fused_grouped_f16(int transa, int m, int n, int k, int count, const void* const* A, int lda, const void* B,
                               int ldb, void* const* C, const int* ldc, int epilogue, const void* const* bias,
                               int epi_arg0, int epi_arg1, int epi_arg2, void* stream);
@@ -207,7 +209,9 @@ int lg_gemm_fused_grouped_f16(int transa, int m, int n, int k, int count, const 
  * steps of different requests batched into one launch): lg_gemm_fused_grouped_f16 with the heads epilogue and one token per
  * sequence, except that a member i with use_rows[i] != 0 writes token row r to position pos[r] of batch entry slot[r] of its
  * destination C[i] = [slots, heads_total, ldc[i], size_per_head] (a KV cache) instead of to position 0 of entry r.  slot and
- * pos are HOST arrays of n ints, copied into the launch (n <= LG_ATTN_DECODE_MAX_SEQS).  No reference counterpart. */
+ * pos are HOST arrays of n ints, copied into the launch (n <= LG_ATTN_DECODE_MAX_SEQS).  pos[r] is checked against ldc[i];
+ * how many entries C[i] has is not known here: slot[r] must be a valid entry (the host runtime checks it against the model's
+ * cache before it builds a launch).  No reference counterpart. */
 int lg_gemm_fused_grouped_rows_f16(int transa, int m, int n, int k, int count, const void* const* A, int lda, const void* B,
                                    int ldb, void* const* C, const int* ldc, const void* const* bias, int size_per_head,
                                    int heads_total, const int* use_rows, const int* slot, const int* pos, void* stream);
