@@ -47,6 +47,7 @@ SIGNATURES = {
     "lgh_model_run_decode": (_i, [_p, _p, _p, _i, _i, _i, _p, _p]),
     "lgh_model_run_decode_seqs": (_i, [_p, _p, _p, _i, C.POINTER(_i), C.POINTER(_i), _p, _p]),
     "lgh_model_time_kernels": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, C.POINTER(_f), _i]),
+    "lgh_model_time_step": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, C.POINTER(_f), _i]),
     "lgh_model_time_one": (_f, [_p, _p, _p, _i, _i, _i, _i, _i, _i]),
     "lgh_sched_create": (_p, [_p, _i, _f, _i, _i, _i, _i, _i, _i]),
     "lgh_sched_destroy": (_i, [_p]),
@@ -268,6 +269,14 @@ class Model:
         n = len(slots)
         check(lib.lgh_model_run_decode_seqs(self.h, input_ptr, output_ptr, n, (C.c_int * n)(*slots), (C.c_int * n)(*pasts),
                                             workspace_ptr, stream), "lgh_model_run_decode_seqs")
+
+    def time_step(self, input_ptr, output_ptr, batch, seq, decode_past=-1, cache_slot=-1, reps=20):
+        """Mean time of every launch-vector entry inside whole steps (an event between every two entries, `reps` steps)."""
+        out = (C.c_float * 4096)()
+        n = lib.lgh_model_time_step(self.h, input_ptr, output_ptr, batch, seq, decode_past, cache_slot, reps, out, 4096)
+        if n < 0:
+            check(1, "lgh_model_time_step")
+        return [out[i] for i in range(n)]
 
     def time_kernels(self, input_ptr, output_ptr, batch, seq, decode_past=-1, cache_slot=-1, iters=20, trials=3):
         out = (C.c_float * 4096)()

@@ -426,6 +426,40 @@ int lgh_model_time_kernels(void* model, void* input, void* output, int batch, in
     return first_error() ? -1 : (int)v.size();
 }
 
+// Times the entries where they run: the whole launch vector is launched `reps` times with an event between every two entries,
+// and ms_out[i] gets the mean distance between the events around entry i (its run time plus the gap to the entry before it).
+// Unlike lgh_model_time_kernels no launch repeats the one before it, so nothing is re-read from a cache that the previous
+// launch of the same kernel filled, and the values add up to the step.  Returns the number of entries.
+int lgh_model_time_step(void* model, void* input, void* output, int batch, int seq, int decode_past, int cache_slot, int reps,
+                        float* ms_out, int ms_cap) {
+    ModelBase* mb = (ModelBase*)model;
+    if (!mb || !input || !output || reps <= 0) { fail("lgh_model_time_step: bad arguments"); return -1; }
+    if (!launch_shape_ok(mb, batch, seq, decode_past, cache_slot)) { fail("lgh_model_time_step: shape, position or cache slot outside the model's buffers"); return -1; }
+    std::vector<FuncWrap> v = decode_past >= 0 ? mb->build_decode(input, output, batch, decode_past, cache_slot, nullptr)
+                                               : mb->build(input, output, batch, seq, nullptr, cache_slot);
+    if ((int)v.size() > ms_cap) { fail("lgh_model_time_step: output array too small"); return -1; }
+    DynamicInitParam& D = *mb->stream0;
+    std::vector<void*> ev(v.size() + 1, nullptr);
+    for (auto& e : ev) note_status(lg_event_create(&e), "lg_event_create");
+    std::vector<double> sum(v.size(), 0.0);
+    for (int r = -2; r < reps; ++r) {   // two untimed passes first
+        note_status(lg_event_record(ev[0], D.stream), "lg_event_record");
+        for (size_t i = 0; i < v.size(); ++i) {
+            v[i].callback(D);
+            note_status(lg_event_record(ev[i + 1], D.stream), "lg_event_record");
+        }
+        note_status(lg_stream_synchronize(D.stream), "lg_stream_synchronize");
+        for (size_t i = 0; i < v.size() && r >= 0; ++i) {
+            float ms = 0.f;
+            note_status(lg_event_elapsed_ms(&ms, ev[i], ev[i + 1]), "lg_event_elapsed_ms");
+            sum[i] += ms;
+        }
+    }
+    for (size_t i = 0; i < v.size(); ++i) ms_out[i] = (float)(sum[i] / reps);
+    for (void* e : ev) if (e) lg_event_destroy(e);
+    return first_error() ? -1 : (int)v.size();
+}
+
 
 // ---- scheduler ---------------------------------------------------------------------------------------------------
 struct LghReport {

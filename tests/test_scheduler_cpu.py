@@ -75,6 +75,23 @@ def test_launch_vector_shapes_and_order(fake):
         host.Model(0, 2, 32, 4, 64, fused=True)        # fused assembly is fp16 only
 
 
+def test_entries_timed_inside_whole_steps_add_up_to_the_step(fake):
+    """time_step launches the whole vector (two untimed passes + reps) with an event between every two entries: every entry is
+    launched once per pass in vector order, and on the virtual-time backend the per-entry means equal the looped per-kernel
+    times plus the host launch cost that separates two entries."""
+    host = fake.host
+    m = small_model(host)
+    n = m.kernels_per_layer()
+    fake.reset()
+    per_entry = m.time_step(0x10000, 0x20000000, 2, 64, reps=3)
+    launches = [e for e in fake.trace() if e["name"] not in ("event_record",)]
+    assert len(per_entry) == n and all(t > 0 for t in per_entry)
+    one_pass = [e["name"] for e in fake_trace_of(fake, m, 2, 64)]
+    assert [e["name"] for e in launches] == one_pass * 5            # 2 untimed passes + 3 timed ones
+    looped = m.time_kernels(0x10000, 0x20000000, 2, 64, iters=2, trials=1)
+    assert per_entry == pytest.approx(looped, abs=0.01)             # virtual durations; 0.002 ms launch cost per entry
+
+
 def test_sequential_run_launches_every_entry_once_in_order(fake):
     host = fake.host
     m = small_model(host)
@@ -437,6 +454,8 @@ def test_requests_that_exceed_the_contexts_are_refused_on_the_host(fake):
         m.time_kernels(0x1000, 0x2000, 5, 64)          # batch beyond max_batch
     with pytest.raises(host.capi.LigerError):
         m.time_kernels(0x1000, 0x2000, 1, 1, decode_past=80, cache_slot=0)
+    with pytest.raises(host.capi.LigerError):
+        m.time_step(0x1000, 0x2000, 5, 64)             # batch beyond max_batch
     nocache = small_model(host, cache=0, fused=False)
     s2 = host.Scheduler(nocache, pool_count=1, ctx_batch=1)
     with pytest.raises(host.capi.LigerError):
