@@ -69,14 +69,23 @@ static int register_stream(void* stream, int cus) {
             return LG_OK;
         }
     }
+    // hipMalloc may synchronise the device, so it runs outside the lock; two threads that attach the same stream at the same
+    // time both get here, and the one that finds the stream registered when it comes back frees its block again
     void* p = nullptr;
     const int rc = rt(hipMalloc(&p, LG_SPLITK_WORKSPACE_BYTES), "hipMalloc (split-K workspace)");
     if (rc) return rc;
     info.ws = (float*)p;
     info.ws_bytes = LG_SPLITK_WORKSPACE_BYTES;
-    std::lock_guard<std::mutex> lk(g_streams_mu);
-    g_streams[stream] = info;
-    return LG_OK;
+    {
+        std::lock_guard<std::mutex> lk(g_streams_mu);
+        auto it = g_streams.find(stream);
+        if (it == g_streams.end()) {
+            g_streams[stream] = info;
+            return LG_OK;
+        }
+        if (cus > 0) it->second.cus = cus;
+    }
+    return rt(hipFree(p), "hipFree (split-K workspace of a stream registered twice)");
 }
 
 static int unregister_stream(void* stream) {

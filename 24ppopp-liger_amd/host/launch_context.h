@@ -78,22 +78,23 @@ class DynamicInitParam {
     int stream_id = 0;  // 0 = primary, 1 = secondary; used by traces
     // Copies are handed to every launch callback (as in the reference), so the object does not own its stream: whoever created
     // the context calls destroy() on ONE copy when the stream is idle and no longer needed (a stream that was adopted from
-    // elsewhere is detached from the device library instead and stays alive).
+    // elsewhere belongs to whoever made it and is left alone).
     bool adopted = false;
     void destroy() {
         if (!stream) return;
-        note_status(lg_stream_synchronize(stream), "lg_stream_synchronize");
-        if (adopted) note_status(lg_stream_detach(stream), "lg_stream_detach");
-        else note_status(lg_stream_destroy(stream), "lg_stream_destroy");
+        if (!adopted) {
+            note_status(lg_stream_synchronize(stream), "lg_stream_synchronize");
+            note_status(lg_stream_destroy(stream), "lg_stream_destroy");
+        }
         stream = nullptr;
     }
     DynamicInitParam() { note_status(lg_stream_create(&stream), "lg_stream_create"); }
     // the reference passes a CUDA stream priority here; priorities are deliberately not used on this platform
     explicit DynamicInitParam(int /*priority*/) { note_status(lg_stream_create(&stream), "lg_stream_create"); }
-    // a stream created elsewhere: the device library is told about it (it then owns a split-K workspace for it)
-    DynamicInitParam(void* existing_stream, int id) : stream(existing_stream), stream_id(id), adopted(true) {
-        note_status(lg_stream_attach(existing_stream, 0), "lg_stream_attach");
-    }
+    // A stream created elsewhere.  Wrapping it costs nothing and touches nothing, so it may be done per call on the launch
+    // path.  Whether K-sliced GEMMs are available on it is the owner's decision: lg_stream_attach (once, at set-up, where
+    // allocating and blocking are allowed) gives it a split-K workspace; without it the launchers simply do not slice K.
+    DynamicInitParam(void* existing_stream, int id) : stream(existing_stream), stream_id(id), adopted(true) {}
     // a stream whose kernels run on the compute units selected by the mask only (see lg_stream_create_cu_mask)
     DynamicInitParam(const unsigned* cu_mask, int mask_words, int id) : stream_id(id) {
         note_status(lg_stream_create_cu_mask(&stream, cu_mask, mask_words), "lg_stream_create_cu_mask");

@@ -197,10 +197,7 @@ class Scheduler {
             left.erase(std::unique(left.begin(), left.end()), left.end());
             for (Sample* smp : left) delete smp;
         }
-        for (auto& kv : _part_streams)
-            for (int role = 0; role < 2; ++role)
-                for (int cls = 0; cls < 2; ++cls)
-                    if (kv.second.d[role][cls]) kv.second.d[role][cls]->destroy();
+        _drop_partition_streams();
         DParams1.destroy();
         DParams0.destroy();
         for (void* e : {Main_EVENT, Wait_EVENT, _epoch_event, _dec_prev_stop})
@@ -224,10 +221,10 @@ class Scheduler {
         // not touch them); asking for another share releases them first: every CU-masked stream is a hardware queue of its own.
         auto it = _part_streams.find(hbm_cus);
         if (it == _part_streams.end()) {
-            for (auto& kv : _part_streams)
-                for (int role = 0; role < 2; ++role)
-                    for (int cls = 0; cls < 2; ++cls) kv.second.d[role][cls]->destroy();
-            _part_streams.clear();
+            // The error state is process-wide and sticky: with one already recorded the outcome of the stream creation below
+            // could not be told apart from it, so nothing is touched and the partition in use (if any) stays as it is.
+            if (first_error()) return false;
+            _drop_partition_streams();
             unsigned hbm_mask[8] = {0}, mfma_mask[8] = {0};
             for (int b = 0; b < total_cus; ++b) (b < hbm_cus ? hbm_mask : mfma_mask)[b >> 5] |= 1u << (b & 31);
             PartStreams ps;
@@ -235,7 +232,13 @@ class Scheduler {
                 ps.d[role][MFMA_BOUND].reset(new DynamicInitParam(mfma_mask, 8, 2 + 2 * role + MFMA_BOUND));
                 ps.d[role][HBM_BOUND].reset(new DynamicInitParam(hbm_mask, 8, 2 + 2 * role + HBM_BOUND));
             }
-            if (first_error()) { partition_hbm_cus = 0; return false; }
+            if (first_error()) {
+                // a stream could not be created: release the ones that were (each holds a hardware queue and a workspace)
+                for (int role = 0; role < 2; ++role)
+                    for (int cls = 0; cls < 2; ++cls)
+                        if (ps.d[role][cls]) ps.d[role][cls]->destroy();
+                return false;
+            }
             it = _part_streams.emplace(hbm_cus, std::move(ps)).first;
         }
         for (int role = 0; role < 2; ++role)
@@ -1062,6 +1065,17 @@ class Scheduler {
         _main_q.clear();
     }
     struct PartStreams { std::unique_ptr<DynamicInitParam> d[2][2]; };
+    // releases every CU-masked stream and leaves partitioning off with no pointer to a released stream behind
+    void _drop_partition_streams() {
+        partition_hbm_cus = 0;
+        for (int role = 0; role < 2; ++role)
+            for (int cls = 0; cls < 2; ++cls) _part[role][cls] = nullptr;
+        for (auto& kv : _part_streams)
+            for (int role = 0; role < 2; ++role)
+                for (int cls = 0; cls < 2; ++cls)
+                    if (kv.second.d[role][cls]) kv.second.d[role][cls]->destroy();
+        _part_streams.clear();
+    }
     std::map<int, PartStreams> _part_streams;                              // by HBM-side share, created once
     DynamicInitParam* _part[2][2] = {{nullptr, nullptr}, {nullptr, nullptr}};  // CU-masked streams of partitioned rounds: [role][class]
     void* _epoch_event = nullptr;
@@ -1085,9 +1099,12 @@ class Scheduler {
     void _finish() {
         note_status(lg_stream_synchronize(DParams0.stream), "lg_stream_synchronize");
         note_status(lg_stream_synchronize(DParams1.stream), "lg_stream_synchronize");
-        for (int role = 0; role < 2; ++role)
-            for (int cls = 0; cls < 2; ++cls)
-                if (_part[role][cls]) note_status(lg_stream_synchronize(_part[role][cls]->stream), "lg_stream_synchronize");
+        // every CU-masked stream that exists, whether or not partitioning is switched on at the moment
+        for (auto& kv : _part_streams)
+            for (int role = 0; role < 2; ++role)
+                for (int cls = 0; cls < 2; ++cls)
+                    if (kv.second.d[role][cls] && kv.second.d[role][cls]->stream)
+                        note_status(lg_stream_synchronize(kv.second.d[role][cls]->stream), "lg_stream_synchronize");
         _reclaim();
         for (auto& d : _dec_done) release_ctx(d.second);   // every stream has been synchronised: their kernels are done
         _dec_done.clear();

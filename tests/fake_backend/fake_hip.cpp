@@ -44,6 +44,7 @@ double g_share_exp[2] = {1.0, 1.0};  // a kernel on a stream with `cus` of 256 c
                                      // [0] matrix kernels, [1] memory kernels (1 = proportional, < 1 = the share hurts less)
 thread_local int g_cost_kind = 1;    // kind of the cost computed last on this thread (0 matrix, 1 memory)
 std::vector<Stream*> g_streams;
+int g_fail_cu_mask_after = -1;  // >= 0: that many CU-masked streams are still created, the ones after them fail
 int g_live_streams = 0, g_live_allocs = 0;   // created and not yet destroyed / allocated and not yet freed
 std::vector<Launch> g_trace;
 Stream g_default;
@@ -106,6 +107,7 @@ int fake_trace_get(int i, int* stream, char* name, int name_len, long long* abc,
 }
 double fake_host_now(void) { return g_host_now; }
 int fake_live_streams(void) { return g_live_streams; }
+void fake_fail_cu_mask_streams_after(int n) { g_fail_cu_mask_after = n; }
 int fake_live_allocs(void) { return g_live_allocs; }
 
 // ---- library / runtime ------------------------------------------------------------------------------------------------
@@ -161,6 +163,8 @@ int lg_stream_create_cu_mask(void** stream, const unsigned* cu_mask, int mask_wo
     int cus = 0;
     for (int b = 0; b < mask_words * 32 && b < 256; ++b) cus += (cu_mask[b >> 5] >> (b & 31)) & 1u;
     if (cus == 0) return LG_ERR_INVALID;
+    if (g_fail_cu_mask_after == 0) { *stream = nullptr; return LG_ERR_LAUNCH; }
+    if (g_fail_cu_mask_after > 0) --g_fail_cu_mask_after;
     const int rc = lg_stream_create(stream);
     Stream* s = (Stream*)*stream;
     s->cus = cus;

@@ -576,6 +576,48 @@ def test_partitioned_rounds_run_only_while_the_other_class_has_work(fake):
     assert r2["partition_rounds"] == 0 and len({e["stream"] for e in fake.trace()}) <= 2
 
 
+def test_a_failed_change_of_share_leaves_no_stream_behind_and_no_stale_pointer(fake):
+    """enable_partition for a new share releases the streams of the old one before it creates its own.  Whatever goes wrong
+    on the way, the scheduler must neither keep a pointer to a released stream (a later run synchronises the partition's
+    streams) nor lose track of a stream it created (each holds a hardware queue and a workspace)."""
+    host, m, s = _partition_setup(fake, factor_hbm_main=1.0)      # share 128 in use
+    lib = fake.lib
+    live = lib.fake_live_streams()
+    # (1) an error recorded earlier (here: a refused request) is sticky and process-wide: the change is refused up front and
+    #     the share in use stays usable
+    assert lib.lgh_sched_serve(s.h, 99, 64, 0) != 0
+    assert lib.lgh_sched_enable_partition(s.h, 64) != 0
+    assert lib.fake_live_streams() == live
+    lib.lgh_clear_error()
+    s.serve_decode(1, 48, 8)
+    s.serve(1, 64, 0)
+    assert s.run_queued(host.MODE_LIGER)["partition_rounds"] >= 1
+    # (2) the third of the four new streams cannot be created: the two that were are released again, the old share's four
+    #     are gone, partitioning is off and runs use the two whole-chip streams only
+    lib.fake_fail_cu_mask_streams_after(2)
+    try:
+        with pytest.raises(host.capi.LigerError):
+            s.enable_partition(64)
+    finally:
+        lib.fake_fail_cu_mask_streams_after(-1)
+    assert lib.fake_live_streams() == live - 4
+    assert s.partition_factor(HBM, MFMA) == pytest.approx(1.0)      # the table is only reset by a successful change
+    fake.reset()
+    s.serve_decode(1, 48, 8)
+    s.serve(1, 64, 0)
+    r = s.run_queued(host.MODE_LIGER)
+    assert r["records"] == 2 and r["partition_rounds"] == 0 and len({e["stream"] for e in fake.trace()}) <= 2
+    # (3) and the share can be switched on again afterwards
+    s.enable_partition(64)
+    assert lib.fake_live_streams() == live
+    s.set_partition_factor(HBM, MFMA, 1.0)
+    s.serve_decode(1, 48, 8)
+    s.serve(1, 64, 0)
+    assert s.run_queued(host.MODE_LIGER)["partition_rounds"] >= 1
+    s.close()
+    assert lib.fake_live_streams() == live - 6
+
+
 @pytest.mark.parametrize("matrix_exp,memory_exp,pays", [(1.0, 1.0, False), (0.5, 0.2, True)])
 def test_measured_partition_follows_the_backend_model(fake, matrix_exp, memory_exp, pays):
     """profile_partition runs the prefill's MFMA-bound kernels on 128 of 256 compute units next to decode steps on the other
