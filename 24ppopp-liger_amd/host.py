@@ -57,6 +57,7 @@ SIGNATURES = {
     "lgh_sched_profile_contention": (_i, [_p, _i, _i, _i, _i, C.POINTER(_f)]),
     "lgh_sched_set_contention": (_i, [_p, _i, _i, _f]),
     "lgh_sched_enable_partition": (_i, [_p, _i]),
+    "lgh_sched_set_decode_step_hook": (_i, [_p, _p, _p]),
     "lgh_sched_enable_batch_decode": (_i, [_p, _i, _i]),
     "lgh_sched_set_recycle_contexts": (_i, [_p, _i]),
     "lgh_sched_ctx_decode_ptrs": (_i, [_p, _i, C.POINTER(_p), C.POINTER(_p)]),
@@ -326,6 +327,20 @@ class Scheduler:
     def enable_batch_decode(self, on=True, steps_ahead=0):
         """Requests that are in their decode steps at the same time share one launch vector per step."""
         check(lib.lgh_sched_enable_batch_decode(self.h, int(bool(on)), steps_ahead), "lgh_sched_enable_batch_decode")
+
+    def set_decode_step_hook(self, fn):
+        """fn(step, slots, pasts, rows_ptr, stream) runs on the scheduler's thread after the kernels of every batched decode step
+        have been launched (slots / pasts: per batch row, before the step); None removes it."""
+        if fn is None:
+            self._hook = None
+            check(lib.lgh_sched_set_decode_step_hook(self.h, None, None), "lgh_sched_set_decode_step_hook")
+            return
+        proto = C.CFUNCTYPE(None, _p, _i, _i, C.POINTER(_i), C.POINTER(_i), _p, _p)
+
+        def tramp(_user, step, rows, slots, pasts, ptr, stream):
+            fn(step, [slots[i] for i in range(rows)], [pasts[i] for i in range(rows)], ptr, stream)
+        self._hook = proto(tramp)      # kept alive with the scheduler
+        check(lib.lgh_sched_set_decode_step_hook(self.h, C.cast(self._hook, _p), None), "lgh_sched_set_decode_step_hook")
 
     def set_recycle_contexts(self, on):
         """False: finished requests keep their context (and results) until the next run starts."""

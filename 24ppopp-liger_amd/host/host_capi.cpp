@@ -45,6 +45,7 @@ struct SchedBase {
     virtual float get_contention(int main_class, int sub_class) = 0;
     virtual bool streams_concurrent() = 0;
     virtual void set_merge_minor(bool on) = 0;
+    virtual void set_decode_step_hook(void (*fn)(void*, int, int, const int*, const int*, void*, void*), void* user) = 0;
 };
 
 struct ModelBase {
@@ -186,6 +187,12 @@ struct SchedT : SchedBase {
     }
     bool streams_concurrent() override { return s->DParams1.concurrent; }
     void set_merge_minor(bool on) override { s->merge_minor = on; }
+    void set_decode_step_hook(void (*fn)(void*, int, int, const int*, const int*, void*, void*), void* user) override {
+        if (!fn) { s->decode_step_hook = nullptr; return; }
+        s->decode_step_hook = [fn, user](int step, const std::vector<int>& slots, const std::vector<int>& pasts, T* rows, const DynamicInitParam& D) {
+            fn(user, step, (int)slots.size(), slots.data(), pasts.data(), (void*)rows, D.stream);
+        };
+    }
 };
 
 template <typename T>
@@ -562,6 +569,14 @@ int lgh_sched_set_contention(void* sched, int main_class, int sub_class, float v
 int lgh_sched_set_merge_minor(void* sched, int on) {
     if (!sched) return fail("lgh_sched_set_merge_minor: null");
     ((SchedBase*)sched)->set_merge_minor(on != 0);
+    return LG_OK;
+}
+// fn(user, step, rows, slots[rows], pasts[rows], batch_rows, stream) is called on the scheduler's thread after the kernels of
+// every batched decode step have been launched on `stream` (Scheduler::decode_step_hook); batch_rows is the device buffer
+// [rows, hidden] the steps work on in place.  fn = NULL removes the hook.
+int lgh_sched_set_decode_step_hook(void* sched, void (*fn)(void*, int, int, const int*, const int*, void*, void*), void* user) {
+    if (!sched) return fail("lgh_sched_set_decode_step_hook: null");
+    ((SchedBase*)sched)->set_decode_step_hook(fn, user);
     return LG_OK;
 }
 // 1 when the scheduler's second stream was verified to execute at the same time as the first

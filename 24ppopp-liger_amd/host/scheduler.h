@@ -160,6 +160,15 @@ class Scheduler {
     bool batch_decode = false;
     int decode_steps_ahead = 4;       // steps per batched launch vector while nothing waits to join (1 otherwise)
     int batched_steps = 0, batched_rows = 0;   // steps launched, and token rows they carried (holes included)
+    // Called by the scheduler thread right after the kernels of every batched decode step have been launched, as an entry of
+    // the step's launch vector (so before the rows of requests that finish with this step are copied out): the place where a
+    // serving loop turns the step's hidden states into the next step's input rows (sampling + embedding), with work it puts
+    // on the stream it is handed.  `step` counts the batched steps of the run; row r of the batch belongs to cache slot
+    // slots[r] at pasts[r] cached positions BEFORE the step (rows of no request point at the spare slot, index
+    // pool contexts x context batch).  Tests use it to check every step against the CPU oracle and to force the oracle's
+    // rows into the next step.
+    std::function<void(int step, const std::vector<int>& slots, const std::vector<int>& pasts, T* rows, const DynamicInitParam&)> decode_step_hook;
+    T* decode_batch_rows() const { return _dec_x; }
     int partition_hbm_cus = 0;
     float partition_table[3][3] = {{-1.f, -1.f, -1.f}, {-1.f, -1.f, -1.f}, {-1.f, -1.f, -1.f}};
     float partition_min_ms = 0.05f;   // less waiting work than this is not worth a partitioned round
@@ -990,6 +999,15 @@ class Scheduler {
                 dv[j].duration = lookup_decode(dv[j].name, rows, longest);
             }
             vec.insert(vec.end(), dv.begin(), dv.end());
+            if (decode_step_hook) {
+                const int step_no = batched_steps;
+                T* x = _dec_x;
+                auto hook = decode_step_hook;
+                FuncWrap f(0.001f, COMPUTATION, [hook, step_no, slots, pasts, x](const DynamicInitParam& D) { hook(step_no, slots, pasts, x, D); },
+                           "decode_step_hook");
+                f.minor = true; f.name = 903; f.duration = 0.001f;
+                vec.push_back(f);
+            }
             batched_steps++;
             batched_rows += rows;
             // retire

@@ -43,3 +43,12 @@ def max_rel_err(a, b):
     a = np.asarray(a, dtype=np.float64)
     b = np.asarray(b, dtype=np.float64)
     return float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-30))
+
+
+def elementwise_err(a, b):
+    """max over the elements of |a - b| / (|b| + rms(b)): a bound of 1e-2 on it says |a - b| <= 1e-2 |b| + 1e-2 rms(b) for
+    every element, which (unlike max_rel_err, whose yardstick is the largest output) a wrong small output cannot hide behind."""
+    a = np.asarray(a, dtype=np.float64)
+    b = np.asarray(b, dtype=np.float64)
+    rms = max(float(np.sqrt(np.mean(b * b))), 1e-30)
+    return float((np.abs(a - b) / (np.abs(b) + rms)).max())

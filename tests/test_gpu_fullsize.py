@@ -13,7 +13,7 @@ import numpy as np
 import pytest
 import torch
 
-from tests.conftest import max_rel_err
+from tests.conftest import elementwise_err, max_rel_err
 
 pytestmark = pytest.mark.gpu
 
@@ -51,11 +51,13 @@ def test_full_size_gemm_one_hot_rows_select_weight_rows(dev, transa, N, K):
     assert torch.equal(Y, expect.half())
 
 
-def test_full_size_layer_batch_independence_and_oracle_slice(dev, po, host):
+@pytest.mark.parametrize("weight_layout", [0, 1])
+def test_full_size_layer_batch_independence_and_oracle_slice(dev, po, host, weight_layout):
     """The cfg2 prefill layer shard (fused assembly, causal) on the full batch: every sequence's result equals, bit for
-    bit, the result of running that sequence alone; one sequence is checked against the CPU oracle."""
+    bit, the result of running that sequence alone; one sequence is checked against the CPU oracle.  Both weight layouts:
+    0 stores weights [in, out] as the reference's cuBLAS calls imply (linear.h:47-49,99-101), 1 stores them [out, in]."""
     m = host.Model(1, B, S, 96, D, layer_num=1, world_size=2, ffn_inner=2 * F, norm_mode=0, causal=True, fused=True,
-                   weight_layout=1, seed=0)
+                   weight_layout=weight_layout, seed=0)
     x = po.fill_normal(M * H, 0, 99, 0.0, 1.0, 1).reshape(M, H)
     dx = dev.up(x, 1)
     dy = dev.empty((M, H), 1)
@@ -74,7 +76,9 @@ def test_full_size_layer_batch_independence_and_oracle_slice(dev, po, host):
     shape = dict(batch=1, seq=S, hidden=H, head_num=48, size_per_head=D, ffn_inner=F, causal=1, norm_mode=0, dtype=1)
     ref = po.encoder_forward(shape, w, x[5 * S:6 * S])
     got = dy[5 * S:6 * S].float().cpu().numpy()
+    print("cfg2 layer, layout %d: max-rel %.3g, element-wise %.3g" % (weight_layout, max_rel_err(got, ref), elementwise_err(got, ref)))
     assert max_rel_err(got, ref) < 1e-2
+    assert elementwise_err(got, ref) < 1e-2
 
 
 def test_full_size_layer_norm_against_oracle(dev, po):
@@ -110,15 +114,16 @@ def test_full_size_decode_attention_against_oracle(dev, po):
     assert max_rel_err(dev.down(out2), got) < 2e-3
 
 
+@pytest.mark.parametrize("weight_layout", [0, 1])
 @pytest.mark.parametrize("batch", [2, 8])
-def test_full_size_decode_step_against_oracle(dev, po, host, batch):
+def test_full_size_decode_step_against_oracle(dev, po, host, batch, weight_layout):
     """One decode step of the full-size layer shard (fused assembly) after a short prefill that fills the KV cache:
     batch 2 takes the matrix-vector kernel, batch 8 the weight-streaming kernel with unsliced blocks, both with the
     grouped Q/K/V launch whose epilogues append the new K/V rows to the cache.  The oracle repeats prefill projections
     and the decoder step on the downloaded weights."""
     S, Lmax = 64, 128
     m = host.Model(1, batch, S, 96, D, layer_num=1, world_size=2, ffn_inner=2 * F, norm_mode=0, causal=True, fused=True,
-                   max_cache_len=Lmax, weight_layout=1, seed=1)
+                   max_cache_len=Lmax, weight_layout=weight_layout, seed=1)
     w = {k[len("layer0."):]: v for k, v in m.download_params().items() if k.startswith("layer0.")}
     x = po.fill_normal(batch * S * H, 1, 99, 0.0, 1.0, 1).reshape(batch * S, H)
     dx, dy = dev.up(x, 1), dev.empty((batch * S, H), 1)
@@ -137,18 +142,20 @@ def test_full_size_decode_step_against_oracle(dev, po, host, batch):
         dt_in, dt_out = dev.up(tok, 1), dev.empty((batch, H), 1)
         m.run_decode(dt_in.data_ptr(), dt_out.data_ptr(), batch, S + step, 0, None, dev.stream)
         ref = po.decoder_step(shape, w, tok, kc, vc, S + step)   # also appends this step's K/V rows to kc / vc
-        assert max_rel_err(dev.down(dt_out), ref) < 1e-2
+        assert max_rel_err(dev.down(dt_out), ref) < 1e-2 and elementwise_err(dev.down(dt_out), ref) < 1e-2
         tok = po.round_f16(ref)
 
 
-def test_cfg3_full_decode_step_against_oracle(dev, po, host):
+@pytest.mark.parametrize("weight_layout", [0, 1])
+def test_cfg3_full_decode_step_against_oracle(dev, po, host, weight_layout):
     """BASELINE config 3 as a whole: batch 32, one new token per sequence, 1024 cached positions with K/V ~ N(0, 1), on the
     full layer shard.  The cache contents are written into the model's KV cache from the host, so the oracle's decoder step
     sees the same numbers; the 32-row Q/K/V, output and FFN GEMMs take the weight-streaming kernel at K = 12288 / 6144 /
-    16384, the grouped Q/K/V launch appends row 1024, the attention reads 1025 positions."""
+    16384 (weights [out, in]) or the LDS-ring kernel that streams [in, out] weights with transposed reads (layout 0, the
+    reference's), the grouped Q/K/V launch appends row 1024, the attention reads 1025 positions."""
     Bd, h, L, Lmax = 32, 48, 1024, 1032
     m = host.Model(1, Bd, 8, 96, D, layer_num=1, world_size=2, ffn_inner=2 * F, norm_mode=0, causal=True, fused=True,
-                   max_cache_len=Lmax, weight_layout=1, seed=2)
+                   max_cache_len=Lmax, weight_layout=weight_layout, seed=2)
     w = {k[len("layer0."):]: v for k, v in m.download_params().items() if k.startswith("layer0.")}
     kc = np.zeros((Bd, h, Lmax, D), dtype=np.float32)
     vc = np.zeros_like(kc)
@@ -166,7 +173,9 @@ def test_cfg3_full_decode_step_against_oracle(dev, po, host):
     got = dev.down(dt_out)
     shape = dict(batch=Bd, seq=L, hidden=H, head_num=h, size_per_head=D, ffn_inner=F, causal=1, norm_mode=0, dtype=1)
     ref = po.decoder_step(shape, w, tok, kc, vc, L)
+    print("cfg3 decode step, layout %d: max-rel %.3g, element-wise %.3g" % (weight_layout, max_rel_err(got, ref), elementwise_err(got, ref)))
     assert max_rel_err(got, ref) < 1e-2
+    assert elementwise_err(got, ref) < 1e-2
     # the step appended its K and V rows at position 1024 of every sequence (the oracle did the same to its arrays)
     back = torch.empty(Bd, h, Lmax, D, device="cuda", dtype=torch.float16)
     dev.capi.call("lg_memcpy_d2d_async", back.data_ptr(), pk, back.numel() * 2, None)

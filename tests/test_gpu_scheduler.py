@@ -80,8 +80,11 @@ def test_batched_decode_equals_every_request_on_its_own(dev, host, mode, partiti
     prefills interleaved into them, optionally on a CU partition) every request must end with the hidden state it gets when it
     runs alone, step by step, on the same model.  A step over several rows may take another weight-streaming kernel than a step
     over one row (which rows share a step depends on the timing of the run), so every step may differ by the rounding of the
-    fp32 summation order, and a later step starts from the earlier steps' differences: the bound grows with the number of
-    steps (4e-3 + 3e-3 per step; the stated 1e-2 at two steps)."""
+    fp32 summation order, and a later step starts from the earlier steps' differences.  This is a free-running comparison of
+    two GPU runs: both sides round to fp16 after every kernel, a difference of one fp16 unit in a step's output (2^-11
+    relative, about 1e-3 of the largest output after LayerNorm) enters the next step as an input perturbation, and up to 12
+    steps x 2 layers compound.  The step-by-step check against the oracle is
+    test_batched_decode_steps_teacher_forced_against_the_oracle (1e-2 at every step); here a fixed 2e-2 bounds the drift."""
     if mode == 0 and partition:
         pytest.skip("partitioned rounds belong to the interleaving scheduler")
     heads, d, F, layers, pool = 8, 128, 2048, 2, 6
@@ -108,6 +111,7 @@ def test_batched_decode_equals_every_request_on_its_own(dev, host, mode, partiti
     assert rep["batched_steps"] < sum(n for _, _, n in reqs)
     if partition and mode:
         assert rep["partition_rounds"] > 0
+    worst = 0.0
     for i, (_, S, n) in enumerate(reqs):
         pin, pout = s.ctx_ptrs(i)
         da, db = s.ctx_decode_ptrs(i)
@@ -127,7 +131,105 @@ def test_batched_decode_equals_every_request_on_its_own(dev, host, mode, partiti
         torch.cuda.synchronize()
         ref = a[0].float()
         err = float((got.float() - ref).abs().max() / ref.abs().max())
-        assert err < 4e-3 + 3e-3 * n, "request %d (prompt %d, %d steps): max rel err %g" % (i, S, n, err)
+        worst = max(worst, err)
+        assert err < 2e-2, "request %d (prompt %d, %d steps): max rel err %g" % (i, S, n, err)
+    print("free-running batched decode vs. per-request steps: worst max-rel %.3g" % worst)
+
+
+@pytest.mark.parametrize("weight_layout", [0, 1])
+@pytest.mark.parametrize("mode", [0, 1])
+def test_batched_decode_steps_teacher_forced_against_the_oracle(dev, po, host, mode, weight_layout):
+    """Batched decode steps through the scheduler (join -> step -> retire vectors built from the requests in flight),
+    checked against the CPU oracle at EVERY step: after the kernels of a step the hook compares each live row with the
+    oracle's decoder step over that request's own cache (two stacked layers) and writes the oracle's rounded row back, so the
+    next step starts from the oracle's state on both sides and no step inherits an earlier step's rounding.  Requests have
+    different prompt and decode lengths, so the batch changes composition while it runs; the bound is the stated 1e-2 at
+    every step, and the element-wise figure is held to the same 1e-2."""
+    from tests.conftest import elementwise_err, max_rel_err
+    heads, d, F, layers, pool, Lmax = 8, 128, 2048, 2, 5, 96
+    H = heads * d
+    m = host.Model(1, pool + 1, 64, heads, d, layer_num=layers, ffn_inner=F, causal=True, fused=True, max_cache_len=Lmax, factor=4,
+                   weight_layout=weight_layout, seed=9)
+    P = m.download_params()
+    W = [{k[len("layer%d." % l):]: v for k, v in P.items() if k.startswith("layer%d." % l)} for l in range(layers)]
+    s = host.Scheduler(m, policy=host.POLICY_RESOURCE, axis=host.SPLIT_TOKEN_ROWS, seq_bucket=32, ignore_num=0, pool_count=pool, ctx_batch=1)
+    s.profile(1, 32, 64, 32, 3)
+    for bs in (1, 2, 3, 4, 5):
+        for past in (32, 64, 96):
+            s.profile_decode(bs, min(past, Lmax - 1), 3)
+    s.set_merge_minor(True)
+    s.enable_batch_decode(True, 2)
+    s.set_recycle_contexts(False)
+    reqs = [(1, 48, 9), (1, 33, 12), (1, 64, 8), (1, 40, 3), (1, 57, 10)]
+    # oracle side: every request's prompt goes through the two layers; K and V of each layer's input fill its caches
+    caches, state = [], {}
+    for i, (_, S, n) in enumerate(reqs):
+        x = _read(dev, s.ctx_ptrs(i)[0], S * H).cpu().numpy().reshape(S, H)
+        shape = dict(batch=1, seq=S, hidden=H, head_num=heads, size_per_head=d, ffn_inner=F, causal=1, norm_mode=0, dtype=1)
+        per_layer = []
+        for l in range(layers):
+            k = po.gemm(x, W[l]["wk"], 1)
+            v = po.gemm(x, W[l]["wv"], 1)
+            _, kb, vb = po.add_qkv_bias_transpose(k, W[l]["bk"], k, W[l]["bk"], v, W[l]["bv"], 1, S, heads, d, 1)
+            kc = np.zeros((1, heads, Lmax, d), dtype=np.float32)
+            vc = np.zeros_like(kc)
+            kc[:, :, :S] = kb
+            vc[:, :, :S] = vb
+            per_layer.append((kc, vc))
+            x = po.round_f16(po.encoder_forward(shape, W[l], x))
+        caches.append(per_layer)
+        state[i] = x[S - 1:S].copy()          # the oracle's own last prompt row: the first decode input if the GPU's agrees
+    worst = {"rel": 0.0, "elem": 0.0, "steps": 0, "rows": 0, "first": 0.0}
+    failures = []
+    row_bytes = H * 2
+
+    def hook(step, slots, pasts, rows_ptr, stream):
+        dev.capi.call("lg_stream_synchronize", stream)
+        got = _read(dev, rows_ptr, len(slots) * H).cpu().numpy().reshape(len(slots), H)
+        forced = got.copy()
+        for r, (slot, past) in enumerate(zip(slots, pasts)):
+            if slot >= pool:
+                continue                       # a row of no request
+            _, S, n = reqs[slot]
+            if past == S:                      # first step: the row was joined from the GPU's own prefill output
+                gpu_in = _read(dev, s.ctx_ptrs(slot)[1] + (S - 1) * row_bytes, H).cpu().numpy().reshape(1, H)
+                worst["first"] = max(worst["first"], max_rel_err(gpu_in, state[slot]))
+                state[slot] = gpu_in
+            x = state[slot]
+            shape = dict(batch=1, seq=S, hidden=H, head_num=heads, size_per_head=d, ffn_inner=F, causal=1, norm_mode=0, dtype=1)
+            for l in range(layers):
+                x = po.round_f16(po.decoder_step(shape, W[l], x, caches[slot][l][0], caches[slot][l][1], past))
+            e1, e2 = max_rel_err(got[r:r + 1], x), elementwise_err(got[r:r + 1], x)
+            worst["rel"], worst["elem"] = max(worst["rel"], e1), max(worst["elem"], e2)
+            worst["rows"] += 1
+            if e1 >= 1e-2 or e2 >= 1e-2:
+                failures.append((step, slot, past, e1, e2))
+            state[slot] = x
+            forced[r] = x[0]
+        t = torch.from_numpy(forced).cuda().half()
+        dev.capi.call("lg_memcpy_d2d_async", rows_ptr, t.data_ptr(), t.numel() * 2, stream)
+        dev.capi.call("lg_stream_synchronize", stream)
+        worst["steps"] += 1
+
+    s.set_decode_step_hook(hook)
+    for r in reqs:
+        s.serve(*r)
+    rep = s.run_queued(host.MODE_LIGER if mode else host.MODE_SEQUENTIAL)
+    s.set_decode_step_hook(None)
+    torch.cuda.synchronize()
+    print("teacher-forced batched decode: %d steps, %d rows, worst max-rel %.3g, worst element-wise %.3g, prefill rows %.3g"
+          % (worst["steps"], worst["rows"], worst["rel"], worst["elem"], worst["first"]))
+    assert rep["records"] == len(reqs) and rep["profile_misses"] == 0
+    assert worst["steps"] == rep["batched_steps"] >= max(n for _, _, n in reqs) >= 8
+    assert worst["rows"] == sum(n for _, _, n in reqs)
+    assert not failures, "steps beyond 1e-2 (step, slot, cached, max-rel, element-wise): %s" % failures[:5]
+    assert worst["first"] < 1e-2
+    # what the requests end with is the forced (oracle) state of their last step: the copy-out comes after the hook
+    for i, (_, S, n) in enumerate(reqs):
+        da, db = s.ctx_decode_ptrs(i)
+        out = _read(dev, db if n % 2 else da, H).cpu().numpy().reshape(1, H)
+        assert np.array_equal(out, state[i])
+    s.close()
 
 
 CFG = dict(hidden=12288, heads_global=96, d=128, ffn_global=32768, world_size=2)   # GLM-130B, one TP=2 shard
@@ -140,7 +242,8 @@ def _read(dev, ptr, elems):
     return t.float()
 
 
-def test_cfg4_decomposition_sweep_at_its_real_shapes(dev, host):
+@pytest.mark.parametrize("weight_layout", [0, 1])
+def test_cfg4_decomposition_sweep_at_its_real_shapes(dev, host, weight_layout):
     """BASELINE config 4: a prefill request of batch 4 x seq 512 on the TP=2 layer shard, decomposed by 1, 2, 4 and 8 along
     its token rows and interleaved on two streams with a decode batch of 32 sequences at 1024 cached positions (3 steps, so
     that the prefill does not fit the decode window whole and something has to be split).  Durations come from profiling on
@@ -150,7 +253,7 @@ def test_cfg4_decomposition_sweep_at_its_real_shapes(dev, host):
     c = CFG
     H = c["hidden"]
     m = host.Model(1, 64, 512, c["heads_global"], c["d"], layer_num=1, world_size=c["world_size"], ffn_inner=c["ffn_global"], causal=True,
-                   fused=True, max_cache_len=1024 + 64, weight_layout=1, seed=0)
+                   fused=True, max_cache_len=1024 + 64, weight_layout=weight_layout, seed=0)
     s = host.Scheduler(m, schedule_deep=6, contention_factor=0.8, policy=host.POLICY_RESOURCE, axis=host.SPLIT_TOKEN_ROWS, seq_bucket=64,
                        ignore_num=0, pool_count=2, ctx_batch=32)
     s.set_merge_minor(True)

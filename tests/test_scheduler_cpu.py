@@ -695,6 +695,58 @@ def test_batched_decode_steps_share_one_launch_vector(fake, mode_name):
         s2.enable_batch_decode(True)
 
 
+@pytest.mark.parametrize("steps_ahead", [1, 3])
+def test_every_batched_step_carries_each_live_request_at_its_own_position(fake, steps_ahead):
+    """The per-step row tables the batched decode vector is built from, seen through the step hook: row r of step k belongs
+    to cache slot r (one-sequence contexts) at the position that request has reached, or to the spare slot at position 0.
+    For every request the steps that carry it are consecutive, start at its prompt length, advance by one and number exactly
+    its decode steps; no step is empty; a step never has more rows than the highest live slot + 1."""
+    host = fake.host
+    pool = 4
+    m = host.Model(1, pool + 1, 64, 4, 64, layer_num=2, ffn_inner=512, causal=True, fused=True, max_cache_len=128, factor=4, seed=0)
+    s = host.Scheduler(m, contention_factor=0.8, policy=host.POLICY_RESOURCE, seq_bucket=16, pool_count=pool, ctx_batch=1)
+    s.profile(1, 16, 64, 16, 2)
+    for bs in (1, 2, 3, 4):
+        for past in (16, 32, 48, 64, 80):
+            s.profile_decode(bs, past, 2)
+    s.set_merge_minor(True)
+    s.enable_batch_decode(True, steps_ahead)
+    seen = []
+    s.set_decode_step_hook(lambda step, slots, pasts, ptr, stream: seen.append((step, slots, pasts)))
+    reqs = [(1, 48, 5), (1, 64, 1), (1, 17, 7), (1, 32, 4)]
+    fake.reset()
+    for r in reqs:
+        s.serve(*r)
+    rep = s.run_queued(host.MODE_LIGER)
+    assert rep["records"] == len(reqs) and rep["batched_steps"] == len(seen)
+    assert [k for k, _, _ in seen] == list(range(len(seen)))
+    spare = pool
+    for i, (_, seq, n) in enumerate(reqs):
+        carried = [(k, pasts[i]) for k, slots, pasts in seen if i < len(slots) and slots[i] == i]
+        assert [p for _, p in carried] == list(range(seq, seq + n)), "request %d" % i
+        assert [k for k, _ in carried] == list(range(carried[0][0], carried[0][0] + n))
+    for k, slots, pasts in seen:
+        live = [r for r, sl in enumerate(slots) if sl != spare]
+        assert live and len(slots) == live[-1] + 1
+        assert all(sl == r for r, sl in enumerate(slots) if sl != spare)
+        assert all(pasts[r] == 0 for r, sl in enumerate(slots) if sl == spare)
+    # launch order around a step: join copies come before the first kernel of the step that first carries the request, the
+    # copy-out after the last kernel of its last step
+    t = fake.trace()
+    steps = [e for e in t if e["name"] == "attn_decode_varlen"][::2]       # first layer's attention of every step
+    assert len(steps) == len(seen)
+    row_bytes = 256 * 2
+    for i, (_, seq, n) in enumerate(reqs):
+        pout = s.ctx_ptrs(i)[1]
+        first = next(k for k, slots, _ in seen if i < len(slots) and slots[i] == i)
+        join = [e for e in t if e["name"] == "memcpy_d2d" and e["A"] == pout + (seq - 1) * row_bytes]
+        assert len(join) == 1 and join[0]["end"] <= steps[first]["start"] + 1e-12
+        if first > 0:
+            assert join[0]["start"] >= steps[first - 1]["end"] - 1e-12       # it joined at a step boundary
+    s.set_decode_step_hook(None)
+    s.close()
+
+
 @pytest.mark.parametrize("factor", [2, 4, 8])
 @pytest.mark.parametrize("axis", [0, 1])
 def test_cfg4_shapes_pieces_cover_the_prefill_exactly(fake, factor, axis):

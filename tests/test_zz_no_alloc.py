@@ -42,6 +42,26 @@ def test_static_scratch_entry_matches_the_workspace_entry_twice(dev, po):
     assert float(np.abs(dev.down(out) - ref).max() / np.abs(ref).max()) < 1e-2
 
 
+def test_static_scratch_entry_leaves_free_device_memory_unchanged(dev, po):
+    """The property the entry exists for: after one warm-up call (the first call on a device looks the array's address up),
+    calls of any size inside the limit change nothing in the device's free memory, and neither does the first call of a shape
+    that was not seen before."""
+    import torch
+    B, h, d, Lmax = 8, 8, 128, 2048
+    q = dev.up(rnd(po, B * h * d, 400).reshape(B, h, d), 1)
+    kc = dev.up(rnd(po, B * h * Lmax * d, 401).reshape(B, h, Lmax, d), 1)
+    vc = dev.up(rnd(po, B * h * Lmax * d, 402).reshape(B, h, Lmax, d), 1)
+    out = dev.empty((B, h, d), 1)
+    scalar = float(1.0 / np.sqrt(d))
+    dev.call("lg_attn_decode_static_f16", q, kc, vc, out, B, h, d, 64, Lmax, scalar)     # warm-up
+    dev.sync()
+    free0 = torch.cuda.mem_get_info()[0]
+    for (b, L) in ((8, 2048), (3, 700), (8, 1), (1, 2048), (5, 1333)):
+        dev.call("lg_attn_decode_static_f16", q, kc, vc, out, b, h, d, L, Lmax, scalar)
+        dev.sync()
+        assert torch.cuda.mem_get_info()[0] == free0, "batch %d, %d keys changed the free device memory" % (b, L)
+
+
 def test_static_scratch_entry_rejects_what_exceeds_its_maximum(dev):
     t = dev.empty((16,), 1)
     rc = dev.call_rc("lg_attn_decode_static_f16", t, t, t, t, 1, 1, 256, 8, 8, 1.0)
