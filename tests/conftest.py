@@ -52,3 +52,10 @@ def elementwise_err(a, b):
     b = np.asarray(b, dtype=np.float64)
     rms = max(float(np.sqrt(np.mean(b * b))), 1e-30)
     return float((np.abs(a - b) / (np.abs(b) + rms)).max())
+
+
+def rms_rel_err(a, b):
+    """rms(a - b) / rms(b): the typical error, next to the two worst-case figures."""
+    a = np.asarray(a, dtype=np.float64)
+    b = np.asarray(b, dtype=np.float64)
+    return float(np.sqrt(np.mean((a - b) ** 2)) / max(float(np.sqrt(np.mean(b * b))), 1e-30))
