@@ -82,6 +82,8 @@ SIGNATURES = {
     "lg_attn_decode_static_f16": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _f, _p]),
     "lg_kv_append_f16": (_i, [_p] * 9 + [_i, _i, _i, _i, _i, _p]),
     "lg_kv_append_varlen_f16": (_i, [_p] * 9 + [_i, _i, _i, C.POINTER(_i), C.POINTER(_i), _i, _p]),
+    "lg_probe_mfma_f16": (_i, [_p, _i64, _p, _sz, _i, C.POINTER(_f), C.POINTER(_f), C.POINTER(_f), _p]),
+    "lg_probe_read": (_i, [_p, _sz, _p, _i, _i, C.POINTER(_f), C.POINTER(_f), _p]),
 }
 
 

@@ -289,6 +289,47 @@ def bench_cfg5(capi, host, weight_layout, n_requests, rates=(4.0, 8.0, 16.0), sh
             "partition_measurement": part_meas, "results": out}
 
 
+def measured_ceilings(capi, iters=3000, read_mib=2048):
+    """What this device sustains, measured now with the library's two probe kernels (lg_probe_mfma_f16, lg_probe_read):
+    a register-only loop of the GEMM's matrix instruction on its wave tile with operands distributed like the bench's data
+    (N(0,1) x N(0,0.02) products are what the layer's GEMMs multiply; both operand sets here are N(0,1) halves, which toggle
+    at least as many bits) and with all-zero operands, and a single-pass read of a buffer eight times the memory-side cache."""
+    import ctypes as C
+    import torch
+    n = 1 << 20
+    ops = torch.empty(n, device="cuda", dtype=torch.float16)
+    scratch = torch.zeros(64, device="cuda", dtype=torch.float32)
+    out = {}
+    ms, tf, ghz = C.c_float(), C.c_float(), C.c_float()
+    for name in ("random_operands", "zero_operands"):
+        if name == "random_operands":
+            capi.call("lg_fill_normal_f16", ops.data_ptr(), n, 0, 77, 0.0, 1.0, None)
+        else:
+            ops.zero_()
+        torch.cuda.synchronize()
+        best = None
+        for _ in range(3):
+            capi.call("lg_probe_mfma_f16", ops.data_ptr(), n, scratch.data_ptr(), 256, iters, C.byref(ms), C.byref(tf), C.byref(ghz), None)
+            if best is None or tf.value > best[0]:
+                best = (tf.value, ghz.value, ms.value)
+        out["mfma_f16_" + name] = {"TFLOPs": round(best[0], 1), "shader_clock_GHz": round(best[1], 3), "kernel_ms": round(best[2], 3),
+                                   "frac_of_published_peak": round(best[0] / PEAK_FP16_TFLOPS, 4)}
+    del ops
+    buf = torch.empty(read_mib << 20, device="cuda", dtype=torch.uint8)
+    capi.call("lg_fill_normal_f16", buf.data_ptr(), buf.numel() // 2, 0, 78, 0.0, 1.0, None)
+    torch.cuda.synchronize()
+    gb = C.c_float()
+    for nt in (0, 1):
+        capi.call("lg_probe_read", buf.data_ptr(), buf.numel(), scratch.data_ptr(), 5, nt, C.byref(ms), C.byref(gb), None)
+        out["read_%d_MiB%s" % (read_mib, "_nontemporal" if nt else "")] = {"GBps": round(gb.value, 1), "ms_per_pass": round(ms.value, 4),
+                                                                          "frac_of_published_peak": round(gb.value / PEAK_HBM_GBS, 4)}
+    del buf
+    torch.cuda.empty_cache()
+    out["what"] = ("lg_probe_mfma_f16: 1024 blocks x 8 waves x %d rounds of 32 v_mfma_f32_16x16x32_f16, operands in registers; "
+                   "lg_probe_read: one pass over %d MiB per launch, 16-byte loads" % (iters, read_mib))
+    return out
+
+
 def derived_peaks(info):
     """Roofline denominators re-derived from the device properties: matrix peak = CUs x 4096 fp16 flop per clock and CU x
     engine clock; memory peak = bus width x reported memory clock x 4 transfers per pin and clock (the runtime reports 2.0 GHz
@@ -377,7 +418,8 @@ def main():
     ap.add_argument("--corun-one", type=int, default=0, help=argparse.SUPPRESS)
     ap.add_argument("--kernel-only", default=None,
                     help="launch only the named launch-vector entry (e.g. 'ffn1+bias+gelu', 'attn_decode', 'layer_norm') or "
-                         "'copy' (a plain 128 MiB read + 128 MiB write kernel) --iters times; for rocprofv3 runs")
+                         "'copy' (a plain 128 MiB read + 128 MiB write kernel) --iters times; for rocprofv3 runs.  "
+                         "'mfma_ceiling' / 'read_ceiling' run the library's probe kernels and print what the device sustains")
     ap.add_argument("--iters", type=int, default=50)
     ap.add_argument("--decode", action="store_true",
                     help="with --kernel-only: take the entry from the decode step's launch vector (batch 32, 1024 cached positions); "
@@ -406,6 +448,10 @@ def main():
 
     if args.corun_one:
         print(json.dumps(bench_corun_one(capi, host, args.weight_layout, args.corun_one)), flush=True)
+        return
+    if args.kernel_only in ("mfma_ceiling", "read_ceiling"):
+        m = measured_ceilings(capi)
+        print(json.dumps({"kernel": args.kernel_only, **{k: v for k, v in m.items() if k == "what" or k.startswith("mfma" if args.kernel_only == "mfma_ceiling" else "read")}}))
         return
     if args.kernel_only:
         model = host.Model(capi.F16, 32, S, c["heads_global"], c["d"], layer_num=1, world_size=c["world_size"], ffn_inner=c["ffn_global"],
@@ -490,6 +536,11 @@ def main():
     }
     del model, x, y
     torch.cuda.empty_cache()
+    # what a kernel that does nothing else sustains on this device, measured in this run: the power-limited matrix ceiling on
+    # data like the bench's, and the memory read ceiling
+    out["peaks"]["measured"] = measured_ceilings(capi)
+    mc = out["peaks"]["measured"]["mfma_f16_random_operands"]["TFLOPs"]
+    out["roofline"]["frac_of_measured_mfma_ceiling"] = round(out["roofline"]["achieved"] / mc, 4) if mc > 0 else None
     # the same layer with the weights stored the other way round (0 = [in, out], the layout the reference's (N,N) cuBLAS call implies)
     other = 1 - args.weight_layout
     m2, x2, y2, r2 = time_layer(capi, host, other, fused, max(5, args.steps // 2), 2)

@@ -259,6 +259,21 @@ int lg_kv_append_varlen_f16(void* q_out, void* k_cache, void* v_cache, const voi
                             const void* bias_K, const void* V, const void* bias_V, int batch, int head_num,
                             int size_per_head, const int* slot, const int* pos, int max_len, void* stream);
 
+/* ---- what the device sustains (no reference counterpart; measurement calls for a bench: they time their own kernel with
+ * two events on `stream` and BLOCK until it has finished; nothing on the launch path calls them) ------------------------- */
+/* A register-only loop of v_mfma_f32_16x16x32_f16 on a 128 x 64 wave tile (no loads, no LDS), 1024 blocks of 8 waves x iters
+ * rounds of 32 matrix instructions.  Operands are read once from `operands` (fp16, >= 106504 elements, 16-byte aligned): with
+ * the data distribution of a GEMM's inputs the pipes draw more power than with zeros and the clock settles lower, so the
+ * figure is the matrix throughput a GEMM on such data cannot exceed on this device.  scratch: >= 64 bytes of device memory.
+ * Returns the kernel's milliseconds, TFLOP/s and the shader clock (GHz) seen by the kernel (either may be NULL). */
+int lg_probe_mfma_f16(const void* operands, int64_t operand_elems, void* scratch, size_t scratch_bytes, int iters, float* ms,
+                      float* tflops, float* shader_ghz, void* stream);
+/* Reads every byte of src[0, bytes) once per pass (16-byte loads, 8 in flight per lane, 1 KiB per wave instruction;
+ * nontemporal != 0 marks them as streaming), `passes` passes after one untimed pass.  On a buffer much larger than the
+ * caches (256 MB memory-side cache) the figure is the device's memory read ceiling.  scratch: >= 4 bytes of device memory.
+ * Returns milliseconds per pass and GB/s (may be NULL). */
+int lg_probe_read(const void* src, size_t bytes, void* scratch, int passes, int nontemporal, float* ms, float* gbps, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -262,5 +262,20 @@ int lg_kv_append_varlen_f16(void* q, void* kc, void*, const void* Q, const void*
     return launch(stream, "kv_append_varlen", (long long)b * h, pos ? pos[0] : 0, slot ? slot[0] : 0, Q, kc, q, mem_cost(12.0 * b * h * d));
 }
 int lg_kv_append_f16(void* q, void* kc, void*, const void* Q, const void*, const void*, const void*, const void*, const void*, int b, int h, int d, int pos, int, void* stream) { return launch(stream, "kv_append", (long long)b * h, pos, d, Q, kc, q, mem_cost(12.0 * b * h * d)); }
+// the measuring entries report the backend's own rates
+int lg_probe_mfma_f16(const void* operands, int64_t n, void* scratch, size_t, int iters, float* ms, float* tflops, float* ghz, void*) {
+    if (!operands || !scratch || iters <= 0 || !ms || n < 106504) return LG_ERR_INVALID;
+    const double flop = 1024.0 * 8.0 * iters * 32.0 * 16384.0;
+    *ms = (float)(flop / g_mfma_rate);
+    if (tflops) *tflops = (float)(g_mfma_rate / 1e9);
+    if (ghz) *ghz = 2.4f;
+    return LG_OK;
+}
+int lg_probe_read(const void* src, size_t bytes, void* scratch, int passes, int, float* ms, float* gbps, void*) {
+    if (!src || !scratch || passes <= 0 || !ms || bytes < (1u << 20)) return LG_ERR_INVALID;
+    *ms = (float)((double)bytes / g_hbm_rate);
+    if (gbps) *gbps = (float)(g_hbm_rate / 1e6);
+    return LG_OK;
+}
 
 }  // extern "C"
