@@ -25,7 +25,7 @@ HIP_FLAGS = [
     "-Wno-unused-command-line-argument", "-Wno-option-ignored",
 ]
 HIP_SOURCES = ["runtime.hip", "elementwise.hip", "attention_aux.hip", "gemm.hip", "gemm_fast.hip", "gemm_skinny.hip", "gemm_skinny_kn.hip", "gemv.hip", "attention.hip",
-               "attention_prefill.hip", "ceilings.hip"]
+               "attention_prefill.hip", "ceilings.hip", "weight_layout.hip"]
 
 
 def _run(cmd):

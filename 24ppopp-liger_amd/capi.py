@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(_PKG, "lib", "libliger_hip.so")
 
 OK, ERR_INVALID, ERR_LAUNCH = 0, 1, 2
 F32, F16 = 0, 1
+OP_N, OP_T, OP_TILED = 0, 1, 2
 EPI_NONE, EPI_BIAS, EPI_BIAS_GELU, EPI_BIAS_HEADS = 0, 1, 2, 3
 
 _i, _i64, _u64, _f, _p, _sz = C.c_int, C.c_int64, C.c_uint64, C.c_float, C.c_void_p, C.c_size_t
@@ -82,6 +83,8 @@ SIGNATURES = {
     "lg_attn_decode_static_f16": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _f, _p]),
     "lg_kv_append_f16": (_i, [_p] * 9 + [_i, _i, _i, _i, _i, _p]),
     "lg_kv_append_varlen_f16": (_i, [_p] * 9 + [_i, _i, _i, C.POINTER(_i), C.POINTER(_i), _i, _p]),
+    "lg_weight_tile_f16": (_i, [_p, _p, _i, _i, _i, _i, _p]),
+    "lg_weight_untile_f16": (_i, [_p, _p, _i, _i, _i, _i, _p]),
     "lg_probe_mfma_f16": (_i, [_p, _i64, _p, _sz, _i, C.POINTER(_f), C.POINTER(_f), C.POINTER(_f), _p]),
     "lg_probe_read": (_i, [_p, _sz, _p, _i, _i, C.POINTER(_f), C.POINTER(_f), _p]),
 }

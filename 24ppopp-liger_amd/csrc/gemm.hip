@@ -38,7 +38,7 @@ __device__ __forceinline__ half8_t load8(const half_t* p, int valid) {
 template <int WL, int EPI, bool ALIGNED>
 __global__ __launch_bounds__(256) void gemm_f16_generic(GemmArgs g) {
     __shared__ __attribute__((aligned(16))) half_t As[GB_M * GA_STRIDE];
-    __shared__ __attribute__((aligned(16))) half_t Bs[(WL == W_NK) ? GB_N * GA_STRIDE : GB_K * GBKN_STRIDE];
+    __shared__ __attribute__((aligned(16))) half_t Bs[(WL == W_KN) ? GB_K * GBKN_STRIDE : GB_N * GA_STRIDE];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;  // 2x2 waves, 64x64 each
@@ -63,7 +63,11 @@ __global__ __launch_bounds__(256) void gemm_f16_generic(GemmArgs g) {
                 const int m = m0 + row, k = k0 + kv * 8;
                 ra[i] = load8<ALIGNED>(X + (int64_t)m * g.ldx + k, (m < g.M) ? (g.K - k) : 0);
             }
-            if (WL == W_NK) {  // W tile: 128 n-rows x 4 k-vectors
+            if (WL == W_TILED) {  // W tile: 8 fragment blocks (16 features x 32 k each), one lane's 16 bytes per thread
+                const int blk = v >> 6, ln = v & 63;
+                const int n = n0 + blk * 16;   // N % 16 == 0 and K % 32 == 0: a block is there as a whole or not at all
+                rb[i] = load8<true>(W + ((int64_t)(n >> 4) * (g.K >> 5) + (k0 >> 5)) * 512 + ln * 8, (n < g.N) ? 8 : 0);
+            } else if (WL == W_NK) {  // W tile: 128 n-rows x 4 k-vectors
                 const int row = v >> 2, kv = v & 3;
                 const int n = n0 + row, k = k0 + kv * 8;
                 rb[i] = load8<ALIGNED>(W + (int64_t)n * g.ldw + k, (n < g.N) ? (g.K - k) : 0);
@@ -79,7 +83,9 @@ __global__ __launch_bounds__(256) void gemm_f16_generic(GemmArgs g) {
         for (int i = 0; i < 2; ++i) {
             const int v = tid + 256 * i;
             *reinterpret_cast<half8_t*>(&As[(v >> 2) * GA_STRIDE + (v & 3) * 8]) = ra[i];
-            if (WL == W_NK)
+            if (WL == W_TILED)
+                *reinterpret_cast<half8_t*>(&Bs[v * 8]) = rb[i];   // block v / 64 keeps its register order
+            else if (WL == W_NK)
                 *reinterpret_cast<half8_t*>(&Bs[(v >> 2) * GA_STRIDE + (v & 3) * 8]) = rb[i];
             else
                 *reinterpret_cast<half8_t*>(&Bs[(v >> 4) * GBKN_STRIDE + (v & 15) * 8]) = rb[i];
@@ -100,7 +106,9 @@ __global__ __launch_bounds__(256) void gemm_f16_generic(GemmArgs g) {
             a[i] = *reinterpret_cast<const half8_t*>(&As[(wm * 64 + i * 16 + l16) * GA_STRIDE + lk * 8]);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            if (WL == W_NK) {
+            if (WL == W_TILED) {
+                b[j] = *reinterpret_cast<const half8_t*>(&Bs[((wn * 4 + j) * 64 + lane) * 8]);
+            } else if (WL == W_NK) {
                 b[j] = *reinterpret_cast<const half8_t*>(&Bs[(wn * 64 + j * 16 + l16) * GA_STRIDE + lk * 8]);
             } else {
                 const int col = wn * 64 + j * 16 + 4 * (l16 & 3);
@@ -173,7 +181,9 @@ static int gemm_f16_dispatch(GemmArgs g, int wlayout, int batch, hipStream_t str
                          (g.epi.kind == LG_EPI_BIAS_HEADS || (((uintptr_t)g.Y & 7u) == 0));
     dim3 grid((g.N + GB_N - 1) / GB_N, (g.M + GB_M - 1) / GB_M, batch);
     if (grid.y > 65535 || grid.z > 65535) { set_error("gemm: problem too large for the generic grid"); return LG_ERR_INVALID; }
-    if (wlayout == W_NK) {
+    if (wlayout == W_TILED) {
+        if (aligned) launch_generic_epi<W_TILED, true>(g, grid, stream); else launch_generic_epi<W_TILED, false>(g, grid, stream);
+    } else if (wlayout == W_NK) {
         if (aligned) launch_generic_epi<W_NK, true>(g, grid, stream); else launch_generic_epi<W_NK, false>(g, grid, stream);
     } else {
         if (aligned) launch_generic_epi<W_KN, true>(g, grid, stream); else launch_generic_epi<W_KN, false>(g, grid, stream);
@@ -258,10 +268,14 @@ static int gemm_f32_dispatch(const GemmArgsF32& g, int wlayout, int batch, hipSt
 // cuBLAS column-major arguments -> row-major problem; returns LG_OK or sets the error text
 static int check_blas_args(const char* what, int transa, int transb, int m, int n, int k, const void* A, int lda,
                            const void* B, int ldb, const void* C, int ldc, int batch) {
-    if (transb != 0 || (transa != 0 && transa != 1)) { set_error("%s: only (N,N) and (T,N) are supported", what); return LG_ERR_INVALID; }
+    if (transb != 0 || (transa != 0 && transa != 1 && transa != LG_OP_TILED)) { set_error("%s: only (N,N), (T,N) and (tiled,N) are supported", what); return LG_ERR_INVALID; }
     if (m < 0 || n < 0 || k < 0 || batch < 0) { set_error("%s: negative dimension", what); return LG_ERR_INVALID; }
     if (m == 0 || n == 0 || batch == 0) return LG_OK;
     if (!A || !B || !C) { set_error("%s: null pointer", what); return LG_ERR_INVALID; }
+    if (transa == LG_OP_TILED && (m % 16 != 0 || k % 32 != 0 || lda != k || batch > 1 || ((uintptr_t)A & 15u))) {
+        set_error("%s: tiled weights need features %% 16 == 0, k %% 32 == 0, lda == k, a 16-byte aligned pointer and no batch (m=%d k=%d lda=%d)", what, m, k, lda);
+        return LG_ERR_INVALID;
+    }
     const int min_lda = transa ? k : m;
     if (lda < (min_lda > 1 ? min_lda : 1) || ldb < (k > 1 ? k : 1) || ldc < (m > 1 ? m : 1)) {
         set_error("%s: leading dimension too small (lda=%d ldb=%d ldc=%d for m=%d n=%d k=%d)", what, lda, ldb, ldc, m, n, k);
@@ -287,7 +301,7 @@ int lg_gemm_strided_batched_f16(int transa, int transb, int m, int n, int k, con
     g.W = (const half_t*)A; g.ldw = lda; g.strideW = strideA;
     g.Y = (half_t*)C; g.ldy = ldc; g.strideY = strideC;
     g.epi = Epilogue{LG_EPI_NONE, nullptr, 0, 0, 0, 0};
-    return gemm_f16_dispatch(g, transa ? W_NK : W_KN, batch, (hipStream_t)stream);
+    return gemm_f16_dispatch(g, transa == LG_OP_TILED ? W_TILED : (transa ? W_NK : W_KN), batch, (hipStream_t)stream);
 }
 
 int lg_gemm_f16(int transa, int transb, int m, int n, int k, const void* A, int lda, const void* B, int ldb, void* C,
@@ -319,7 +333,7 @@ int lg_gemm_fused_f16(int transa, int m, int n, int k, const void* A, int lda, c
     g.W = (const half_t*)A; g.ldw = lda; g.strideW = 0;
     g.Y = (half_t*)C; g.ldy = ldc; g.strideY = 0;
     g.epi = Epilogue{epilogue, (const half_t*)bias, epi_arg0, epi_arg1, epi_arg2, 0};
-    return gemm_f16_dispatch(g, transa ? W_NK : W_KN, 1, (hipStream_t)stream);
+    return gemm_f16_dispatch(g, transa == LG_OP_TILED ? W_TILED : (transa ? W_NK : W_KN), 1, (hipStream_t)stream);
 }
 
 int lg_gemm_fused_grouped_f16(int transa, int m, int n, int k, int count, const void* const* A, int lda, const void* B, int ldb,
@@ -365,12 +379,13 @@ int lg_gemm_fused_grouped_f16(int transa, int m, int n, int k, int count, const 
             g.Y = grp.Y[0]; g.ldy = grp.ldy[0]; g.strideY = 0;
             g.epi = Epilogue{epilogue, grp.bias[0], epi_arg0, epi_arg1, heads_total, 0};
             bool handled = false;
-            int rc = launch_gemm_fast_f16(g, grp, transa ? W_NK : W_KN, 1, (hipStream_t)stream, &handled);
+            const int wl = transa == LG_OP_TILED ? W_TILED : (transa ? W_NK : W_KN);
+            int rc = launch_gemm_fast_f16(g, grp, wl, 1, (hipStream_t)stream, &handled);
             if (handled) return rc;
-            if (transa == 1) {
-                rc = launch_gemv_f16(g, grp, nullptr, W_NK, 1, (hipStream_t)stream, &handled);
+            if (transa != 0) {
+                rc = launch_gemv_f16(g, grp, nullptr, wl, 1, (hipStream_t)stream, &handled);
                 if (handled) return rc;
-                rc = launch_gemm_skinny_f16(g, grp, nullptr, W_NK, 1, (hipStream_t)stream, &handled);
+                rc = launch_gemm_skinny_f16(g, grp, nullptr, wl, 1, (hipStream_t)stream, &handled);
                 if (handled) return rc;
             }
         }
@@ -421,17 +436,18 @@ int lg_gemm_fused_grouped_rows_f16(int transa, int m, int n, int k, int count, c
         grp.ldy[i] = ldc[i];
         grp.rows[i] = use_rows[i] ? 1 : 0;
     }
-    if (transa == 1) {
+    if (transa != 0) {
         GemmArgs g;
         g.M = n; g.N = m; g.K = k;
         g.X = (const half_t*)B; g.ldx = ldb; g.strideX = 0;
         g.W = grp.W[0]; g.ldw = lda; g.strideW = 0;
         g.Y = grp.Y[0]; g.ldy = grp.ldy[0]; g.strideY = 0;
         g.epi = Epilogue{LG_EPI_BIAS_HEADS_ROWS, grp.bias[0], 1, d, heads_total, grp.rows[0]};
+        const int wl = transa == LG_OP_TILED ? W_TILED : W_NK;
         bool handled = false;
-        int rc = launch_gemv_f16(g, grp, &rm, W_NK, 1, (hipStream_t)stream, &handled);
+        int rc = launch_gemv_f16(g, grp, &rm, wl, 1, (hipStream_t)stream, &handled);
         if (handled) return rc;
-        rc = launch_gemm_skinny_f16(g, grp, &rm, W_NK, 1, (hipStream_t)stream, &handled);
+        rc = launch_gemm_skinny_f16(g, grp, &rm, wl, 1, (hipStream_t)stream, &handled);
         if (handled) return rc;
     }
     if (transa == 0) {
@@ -473,6 +489,7 @@ int lg_gemm_fused_grouped_rows_f16(int transa, int m, int n, int k, int count, c
 int lg_gemm_strided_batched_f32(int transa, int transb, int m, int n, int k, const float* A, int lda, int64_t strideA,
                                 const float* B, int ldb, int64_t strideB, float* C, int ldc, int64_t strideC, int batch,
                                 void* stream) {
+    if (transa == LG_OP_TILED) { set_error("gemm_f32: tiled weights are an fp16 layout"); return LG_ERR_INVALID; }
     int rc = check_blas_args("gemm_f32", transa, transb, m, n, k, A, lda, B, ldb, C, ldc, batch);
     if (rc) return rc;
     GemmArgsF32 g;

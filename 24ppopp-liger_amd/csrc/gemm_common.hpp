@@ -10,7 +10,18 @@
 
 namespace lg {
 
-enum WLayout { W_KN = 0, W_NK = 1 };
+// W_TILED: the [N, K] matrix cut into 16-feature x 32-k blocks, each stored as the 1 KiB an MFMA B operand of
+// v_mfma_f32_16x16x32_f16 occupies in a wave's registers: lane l (feature l % 16, k-group l / 16) owns bytes [16 l, 16 l + 16)
+// of its block = W[16 t + l % 16][32 c + 8 (l / 16) .. + 8); block (t, c) is block number t * (K / 32) + c.  A wave-wide
+// 16-byte load of one block is one contiguous KiB, and the blocks a feature tile needs along k follow each other in memory:
+// a weight-streaming kernel reads its weights as one sequential stream per wave (which is what lets it mark the loads
+// non-temporal), a tile kernel copies blocks to LDS and reads fragments back without any swizzle.  Feature tile t starts
+// 16 t * K elements into the matrix, exactly where row 16 t of the [N, K] layout starts, so sub-ranges and packed row blocks
+// keep the pointer arithmetic of W_NK as long as they start at multiples of 16 features.  Needs N % 16 == 0, K % 32 == 0.
+enum WLayout { W_KN = 0, W_NK = 1, W_TILED = 2 };
+__host__ __device__ __forceinline__ int64_t tiled_offset(int n, int k, int64_t K) {
+    return ((int64_t)(n >> 4) * (K >> 5) + (k >> 5)) * 512 + ((((k >> 3) & 3) << 4) + (n & 15)) * 8 + (k & 7);
+}
 
 struct Epilogue {
     int kind;             // LG_EPI_*

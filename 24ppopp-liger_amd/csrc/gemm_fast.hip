@@ -114,7 +114,10 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, GemmGroup
     const int kt0 = split * kt_per_split;
     const int ktiles = min(g.K / FB_K - kt0, kt_per_split);
     const half_t* X = g.X + (int64_t)m0 * g.ldx + (int64_t)kt0 * FB_K;
-    const half_t* W = (WL == W_KN) ? g.W + n0 + (int64_t)kt0 * FB_K * g.ldw : g.W + (int64_t)n0 * g.ldw + (int64_t)kt0 * FB_K;
+    // tiled weights: feature tile n0 / 16 starts n0 * K elements in, and a k-tile of 64 is two consecutive 512-element blocks
+    const half_t* W = (WL == W_KN)   ? g.W + n0 + (int64_t)kt0 * FB_K * g.ldw
+                      : (WL == W_NK) ? g.W + (int64_t)n0 * g.ldw + (int64_t)kt0 * FB_K
+                                     : g.W + (int64_t)n0 * g.ldw + (int64_t)kt0 * 1024;
 
     // ---- per-lane global offsets of the 8 direct-to-LDS loads of one k-tile ---------------------------------------------
     // X tile (and W tile when [N, K]): 32 chunks of 1 KiB = 8 rows x 128 B; wave w fills chunks w, w+8, w+16, w+24.
@@ -128,7 +131,11 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, GemmGroup
         const int xrow = min(row, g.M - 1 - m0);
         xoff[i] = (unsigned)(xrow * (int)g.ldx + c * 8) * 2u;
         if (i >= WCH) continue;
-        if (WL == W_NK) {
+        if (WL == W_TILED) {
+            // chunk q of the W tile = fragment block (feature tile q / 2, k-step q % 2): one contiguous KiB in memory that lands
+            // as one contiguous KiB of LDS, each lane's 16 bytes where the lane will read them back
+            woff[i] = ((unsigned)(q >> 1) * (unsigned)(g.K >> 5) * 512u + (unsigned)(q & 1) * 512u + (unsigned)lane * 8u) * 2u;
+        } else if (WL == W_NK) {
             woff[i] = (unsigned)(row * (int)g.ldw + c * 8) * 2u;
         } else {
             // W tile [64 k][FB_N n]: a k-row is FB_N / 8 lanes wide, chunk q = 64 / (FB_N / 8) consecutive k-rows
@@ -140,7 +147,7 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, GemmGroup
             woff[i] = (unsigned)(k * (int)g.ldw + (blk * 2 + (p & 1)) * 8) * 2u;
         }
     }
-    const int64_t wstep = (WL == W_KN) ? (int64_t)FB_K * g.ldw : FB_K;
+    const int64_t wstep = (WL == W_KN) ? (int64_t)FB_K * g.ldw : (WL == W_NK ? FB_K : 1024);
 
     // tile index clamped to the last one: the loop body is branch-free, the extra loads of the last iterations
     // refill slots nobody reads any more
@@ -174,6 +181,8 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, GemmGroup
             const int i = u - NJ;
             const int row = wm * 128 + i * 16 + l16;
             a[i] = *reinterpret_cast<const half8_t*>(&xs[row * FB_K + swz_a(row, ks * 4 + lk) * 8]);
+        } else if (WL == W_TILED) {
+            b[u] = *reinterpret_cast<const half8_t*>(&ws[(((wn * NJ + u) * 2 + ks) * 64 + lane) * 8]);
         } else if (WL == W_NK) {
             const int row = wn * (16 * NJ) + u * 16 + l16;
             b[u] = *reinterpret_cast<const half8_t*>(&ws[row * FB_K + swz_a(row, ks * 4 + lk) * 8]);
@@ -223,7 +232,7 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, GemmGroup
             for (int u = 0; u < NDS; ++u) {
                 // [N, K] weights: one read unit every DS_SPAN / NDS MFMAs.  [K, N] weights: the W units (two transposed
                 // reads each) go under the first NJ MFMAs, the X units are spread over the rest (measured: 8 % faster)
-                const int at = (WL == W_NK) ? (u * DS_SPAN + DS_SPAN - 1) / NDS : (u < NJ ? u : NJ + (u - NJ) * (DS_SPAN - NJ) / 8);
+                const int at = (WL != W_KN) ? (u * DS_SPAN + DS_SPAN - 1) / NDS : (u < NJ ? u : NJ + (u - NJ) * (DS_SPAN - NJ) / 8);
                 if (at == m) read_unit(rxs, rws, rks, u, ra, rb, MSET ^ 1);
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -407,6 +416,7 @@ int launch_gemm_fast_f16(const GemmArgs& g, const GemmGroup& grp, int wlayout, i
     if (g.M <= 64) return LG_OK;
     if (!aligned16(g.X) || (g.ldx % 8) || (g.ldw % 8)) return LG_OK;
     if (g.ldx >= (1 << 22) || g.ldw >= (1 << 22)) return LG_OK;  // 256 rows x ld must fit the 31-bit tile offsets
+    if (wlayout == W_TILED && g.ldw != g.K) return LG_OK;
     for (int i = 0; i < grp.count; ++i) {
         if (!aligned16(grp.W[i]) || !aligned16(grp.Y[i])) return LG_OK;
         if (g.epi.kind == LG_EPI_BIAS_HEADS ? (g.epi.d % 4 != 0) : (grp.ldy[i] % 4 != 0)) return LG_OK;
@@ -434,7 +444,11 @@ int launch_gemm_fast_f16(const GemmArgs& g, const GemmGroup& grp, int wlayout, i
     *handled = true;
     const int tiles_n = g.N / (64 * best_nj) * grp.count;
     int rc;
-    if (wlayout == W_NK) {
+    if (wlayout == W_TILED) {
+        if (best_nj == 4) rc = launch_fast_epi<W_TILED, 4>(g, grp, tiles_m, tiles_n, si, stream);
+        else if (best_nj == 3) rc = launch_fast_epi<W_TILED, 3>(g, grp, tiles_m, tiles_n, si, stream);
+        else rc = launch_fast_epi<W_TILED, 2>(g, grp, tiles_m, tiles_n, si, stream);
+    } else if (wlayout == W_NK) {
         if (best_nj == 4) rc = launch_fast_epi<W_NK, 4>(g, grp, tiles_m, tiles_n, si, stream);
         else if (best_nj == 3) rc = launch_fast_epi<W_NK, 3>(g, grp, tiles_m, tiles_n, si, stream);
         else rc = launch_fast_epi<W_NK, 2>(g, grp, tiles_m, tiles_n, si, stream);

@@ -134,6 +134,17 @@ def make_poisson_trace(lam, n, batch, seq_lo, seq_hi, seq_round, n_decode, seed)
     return [{"arrival_s": arr[i], "batch": batch, "seq": seq[i], "n_decode": n_decode} for i in range(n)]
 
 
+def _tile(a):
+    """[features, k] -> the tiled storage order of lg_weight_tile_f16 (flat): blocks of 16 features x 32 k, inside a block
+    element (f, j) at ((j // 8) * 16 + f) * 8 + j % 8."""
+    n, k = a.shape
+    return a.reshape(n // 16, 16, k // 32, 4, 8).transpose(0, 2, 3, 1, 4).reshape(-1)
+
+
+def _untile(flat, n, k):
+    return flat.reshape(n // 16, k // 32, 4, 16, 8).transpose(0, 3, 1, 2, 4).reshape(n * k)
+
+
 def _interleave16(n, inverse=False):
     """Index vector of the stored order of n = 2 f features [first half | second half] interleaved in groups of 16:
     stored[p] = logical[idx[p]] (inverse: logical[c] = stored[idx[c]])."""
@@ -199,7 +210,7 @@ class Model:
             check(lib.lgh_model_param_info(self.h, i, name, 128, C.byref(ptr), C.byref(n), C.byref(r), C.byref(c), C.byref(t)),
                   "lgh_model_param_info")
             out[name.value.decode()] = dict(ptr=ptr.value, elems=n.value, rows=r.value, cols=c.value, transposed=t.value & 1,
-                                            interleave16=(t.value >> 1) & 1)
+                                            interleave16=(t.value >> 1) & 1, tiled=(t.value >> 2) & 1)
         return out
 
     def params(self):
@@ -216,6 +227,8 @@ class Model:
             capi.check(capi.lib.lg_memcpy_d2h(raw.ctypes.data_as(_p), _p(info["ptr"]), n * self.es), "lg_memcpy_d2h")
             a = raw.astype(np.float32)
             if info["rows"] > 1:
+                if info["tiled"]:
+                    a = _untile(a, info["cols"], info["rows"])      # -> [out, in]
                 a = a.reshape(info["cols"], info["rows"]).T if info["transposed"] else a.reshape(info["rows"], info["cols"])
             if info["interleave16"]:
                 a = a[..., _interleave16(a.shape[-1], inverse=True)]
@@ -239,6 +252,8 @@ class Model:
                 a = a[..., _interleave16(a.shape[-1])]
             if i["rows"] > 1:
                 a = a.T if i["transposed"] else a
+                if i["tiled"]:
+                    a = _tile(np.ascontiguousarray(a))
             raw = np.ascontiguousarray(a, dtype=dt).ravel()
             if raw.size != i["elems"]:
                 raise ValueError("%s: expected %d elements, got %d" % (name, i["elems"], raw.size))

@@ -284,7 +284,8 @@ void* lgh_model_create_ex(int dtype, int max_batch, int max_seq, int head_num, i
     BertInitParam P(max_batch, max_seq, head_num, size_per_head, layer_num, 0, factor, 0);
     P.ffn_act = ffn_act; P.packed_qkv = packed_qkv;
     P.ffn_inner = ffn_inner; P.norm_mode = norm_mode; P.causal = causal; P.fused = fused; P.max_cache_len = max_cache_len;
-    P.weight_layout = weight_layout ? 1 : 0;
+    if (weight_layout < 0 || weight_layout > 2 || (weight_layout == 2 && dtype != 1)) { fail("lgh_model_create: weight_layout is 0 ([in, out]), 1 ([out, in]) or 2 (tiled, fp16 only)"); return nullptr; }
+    P.weight_layout = weight_layout;
     StaticInitParam S(0, world_size, dtype);
     const int hidden = head_num * size_per_head;
     ModelBase* mb = nullptr;

@@ -143,7 +143,8 @@ class BertInitParam {
     int fused = 0;          // 1 -> bias/GELU/transposes folded into GEMM epilogues, one fused attention kernel
     int max_cache_len = 0;  // > 0 -> layers own a KV cache [max_batch, heads, max_cache_len, d] for decode steps
     int weight_layout = 0;  // 0: weights stored [in, out] (what the reference's (N,N) cuBLAS call implies);
-                            // 1: stored [out, in] and multiplied with transa = T (both operands K-contiguous)
+                            // 1: stored [out, in] and multiplied with transa = T (both operands K-contiguous);
+                            // 2: the [out, in] matrix in the tiled layout of lg_weight_tile_f16 (transa = LG_OP_TILED; fp16)
     int ffn_act = 0;        // 0: FFN-1 -> bias + GELU -> FFN-2 (bert_layer.h:43-62); 1: GeGLU, FFN-1 is [H, 2F] = [gate | up]
     int packed_qkv = 0;     // 1 (reference-shaped assembly only): one [H, 3 Hl] GEMM + add_fusedQKV_bias_transpose
                             // (attention_kernels.cuh:23-34) instead of three GEMMs + add_QKV_bias_transpose

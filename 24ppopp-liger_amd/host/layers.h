@@ -52,8 +52,18 @@ struct ParamRef {
     int rows = 1, cols = 0;   // logical shape [in, out] of a weight matrix (vectors: rows = 1)
     int transposed = 0;       // bit 0: stored as [out, in]; bit 1: the out dimension (or the vector) is stored with its two
                               // halves interleaved in groups of 16 (stored group 2g = logical [16g, 16g+16) of the first
-                              // half, stored group 2g+1 = the same range of the second half)
+                              // half, stored group 2g+1 = the same range of the second half); bit 2: the [out, in] matrix is
+                              // stored in the tiled layout of lg_weight_tile_f16 (16 x 32 fragment blocks)
 };
+
+// ParamRef::transposed bits of a weight layout, and the shapes the tiled layout can hold
+inline int layout_bits(int weight_layout) { return weight_layout == 2 ? (1 | 4) : (weight_layout ? 1 : 0); }
+inline void check_tiled_shape(int weight_layout, int dtype, int features, int k, const char* who) {
+    if (weight_layout != 2) return;
+    if (dtype != LG_F16 || features % 16 != 0 || k % 32 != 0)
+        set_error_state(LG_ERR_INVALID, std::string(who) + ": the tiled weight layout is fp16 only and needs features % 16 == 0 and k % 32 == 0 (features " +
+                        std::to_string(features) + ", k " + std::to_string(k) + ")");
+}
 
 // ---------------------------------------------------------------------------------------------------
 // Linear layers.  Y[M, N'] = X[M, K'] * W with W stored row-major [K', N'] (the layout cuBLAS's (N,N) call in
@@ -67,7 +77,8 @@ class Linear_Col {  // linear.h:68-109: output features split across ranks
     StaticInitParam SParams;
     std::vector<FuncWrap> FuncWrapVec;
 
-    int weight_layout = 0;  // 0: [k, n_local] row-major; 1: [n_local, k] row-major (multiplied with transa = T)
+    int weight_layout = 0;  // 0: [k, n_local] row-major; 1: [n_local, k] row-major (multiplied with transa = T); 2: [n_local, k] in
+                            // the tiled layout (transa = LG_OP_TILED; fp16, n_local % 16 == 0, k % 32 == 0)
     int interleave16 = 0;   // 1: output features stored as (gate, up) groups of 16 (the GeGLU epilogue's order)
 
     int lda_view = 0;       // > 0: `weights` points into a wider matrix with this leading dimension (one of q / k / v inside the
@@ -76,13 +87,14 @@ class Linear_Col {  // linear.h:68-109: output features split across ranks
     Linear_Col(const StaticInitParam& SParams_, const int& k_, const int& n_, int weight_layout_ = 0)
         : k(k_), n(n_), SParams(SParams_), weight_layout(weight_layout_) {
         weights = dev_alloc<T>((size_t)k * n / SParams.world_size);
+        check_tiled_shape(weight_layout, dtype_of<T>::value, n_local(), k, "Linear_Col");
     }
     Linear_Col(const StaticInitParam& SParams_, const int& k_, const int& n_, int weight_layout_, T* view, int lda)
         : k(k_), n(n_), weights(view), SParams(SParams_), weight_layout(weight_layout_), lda_view(lda) {}
     Linear_Col(const Linear_Col&) = delete;
     Linear_Col& operator=(const Linear_Col&) = delete;
     ~Linear_Col() { if (!lda_view) dev_free(weights); }
-    ParamRef param(const std::string& name) { return ParamRef{name, weights, (int64_t)k * n_local(), k, n_local(), weight_layout | (interleave16 << 1)}; }
+    ParamRef param(const std::string& name) { return ParamRef{name, weights, (int64_t)k * n_local(), k, n_local(), layout_bits(weight_layout) | (interleave16 << 1)}; }
     int n_local() const { return n / SParams.world_size; }
     void init_weights(uint64_t seed, uint64_t tensor_id, float stddev = 0.02f) {
         if (!lda_view) dev_fill_normal(weights, (int64_t)k * n_local(), seed, tensor_id, 0.f, stddev);
@@ -110,16 +122,17 @@ class Linear_Row {  // linear.h:16-64: input features split across ranks; partia
     StaticInitParam SParams;
     std::vector<FuncWrap> FuncWrapVec;
 
-    int weight_layout = 0;  // 0: [k_local, n] row-major; 1: [n, k_local] row-major (multiplied with transa = T)
+    int weight_layout = 0;  // 0: [k_local, n] row-major; 1: [n, k_local] row-major (multiplied with transa = T); 2: [n, k_local] tiled
 
     Linear_Row(const StaticInitParam& SParams_, const int& k_, const int& n_, int weight_layout_ = 0)
         : k(k_), n(n_), SParams(SParams_), weight_layout(weight_layout_) {
         weights = dev_alloc<T>((size_t)k * n / SParams.world_size);
+        check_tiled_shape(weight_layout, dtype_of<T>::value, n, k_local(), "Linear_Row");
     }
     Linear_Row(const Linear_Row&) = delete;
     Linear_Row& operator=(const Linear_Row&) = delete;
     ~Linear_Row() { dev_free(weights); }
-    ParamRef param(const std::string& name) { return ParamRef{name, weights, (int64_t)k_local() * n, k_local(), n, weight_layout}; }
+    ParamRef param(const std::string& name) { return ParamRef{name, weights, (int64_t)k_local() * n, k_local(), n, layout_bits(weight_layout)}; }
     int k_local() const { return k / SParams.world_size; }
     void init_weights(uint64_t seed, uint64_t tensor_id, float stddev = 0.02f) {
         dev_fill_normal(weights, (int64_t)k_local() * n, seed, tensor_id, 0.f, stddev);

@@ -189,7 +189,9 @@ inline FuncWrap decompose_callback(const FuncWrap& old_func, int factor, int n, 
     if (g.epilogue == LG_EPI_BIAS_HEADS) axis = SPLIT_OUT_COLS;  // token rows would move the (batch, seq) decode of rows
     if (axis == SPLIT_OUT_COLS) {
         // GeGLU: whole (gate, up) groups of 32 features, which produce 16 output columns
-        const int gran = (g.epilogue == LG_EPI_BIAS_HEADS) ? g.epi_d : (g.epilogue == LG_EPI_BIAS_GEGLU ? 32 : 8);
+        int gran = (g.epilogue == LG_EPI_BIAS_HEADS) ? g.epi_d : (g.epilogue == LG_EPI_BIAS_GEGLU ? 32 : 8);
+        // tiled weights: a piece starts at a whole 16-feature tile (their feature counts are multiples of 16, so it divides)
+        while (g.transa == LG_OP_TILED && gran % 16 != 0) gran *= 2;
         const int c0 = split_point(g.m, start, factor, gran), c1 = split_point(g.m, start + n, factor, gran);
         g.A = (const char*)g.A + (g.transa ? (size_t)c0 * g.lda : (size_t)c0) * es;
         if (g.bias) g.bias = (const char*)g.bias + (size_t)c0 * es;

@@ -35,6 +35,12 @@ extern "C" {
 #define LG_F32 0
 #define LG_F16 1
 
+/* values of transa in the GEMM entry points: the two cuBLAS operations the reference uses, and a third with no cuBLAS
+ * counterpart for weights the caller has re-laid with lg_weight_tile_f16 (fp16 only; see there) */
+#define LG_OP_N 0
+#define LG_OP_T 1
+#define LG_OP_TILED 2
+
 /* most sequences one launch of the per-sequence (varlen / rows) decode entry points can carry */
 #define LG_ATTN_DECODE_MAX_SEQS 64
 
@@ -160,7 +166,10 @@ int lg_transpose_f16(void* dst, const void* src, int batch, int seq, int head_nu
 /* cublasGemmEx subset the reference uses: column-major, alpha = 1, beta = 0, C = op(A) * B.
  * transa: 0 = N (linear.h:47-49,99-101), 1 = T (bert_layer.h:145-149); transb must be 0.
  * In row-major words: C'[n, m] = B'[n, k] * W where W is A seen row-major: [k, m] (transa = 0) or
- * [m, k] (transa = 1).  fp16: fp32 accumulate (the reference accumulates in fp16). */
+ * [m, k] (transa = 1).  fp16: fp32 accumulate (the reference accumulates in fp16).
+ * transa = LG_OP_TILED (fp16, single problems and groups): A is the [m, k] matrix in the tiled layout written by
+ * lg_weight_tile_f16, lda must equal k, m % 16 == 0, k % 32 == 0.  A sub-range of features that starts at a multiple of
+ * 16 starts (first feature) * k elements into A, as in the [m, k] layout. */
 int lg_gemm_f32(int transa, int transb, int m, int n, int k, const float* A, int lda, const float* B, int ldb,
                 float* C, int ldc, void* stream);
 int lg_gemm_f16(int transa, int transb, int m, int n, int k, const void* A, int lda, const void* B, int ldb,
@@ -258,6 +267,18 @@ int lg_kv_append_f16(void* q_out, void* k_cache, void* v_cache, const void* Q, c
 int lg_kv_append_varlen_f16(void* q_out, void* k_cache, void* v_cache, const void* Q, const void* bias_Q, const void* K,
                             const void* bias_K, const void* V, const void* bias_V, int batch, int head_num,
                             int size_per_head, const int* slot, const int* pos, int max_len, void* stream);
+
+/* ---- weights in the tiled layout (no reference counterpart: linear.h:40,92 allocate the weights and never say how they
+ * are laid out, so a layer that owns its weights may store them as its kernels read them fastest) -------------------- */
+/* tiled = the [features, k] matrix cut into blocks of 16 features x 32 k, block (t, c) at element ((t * k / 32) + c) * 512;
+ * inside a block, element (feature f, position j) sits at ((j / 8) * 16 + f) * 8 + j % 8 -- the order in which the lanes of a
+ * wave hold the B operand of v_mfma_f32_16x16x32_f16.  Every wave-wide load of a block is one contiguous KiB and the blocks
+ * of a feature tile follow each other along k: decode GEMMs stream such weights 15-20 % faster than row-major ones (whole
+ * 128-byte lines per load, marked non-temporal), prefill GEMMs copy blocks to LDS without a swizzle.
+ * plain_transa says how the plain matrix is stored: 0 = [k, features] (ld_plain >= features), 1 = [features, k]
+ * (ld_plain >= k, a multiple of 8).  features % 16 == 0, k % 32 == 0, both pointers 16-byte aligned and distinct. */
+int lg_weight_tile_f16(void* tiled, const void* plain, int features, int k, int plain_transa, int ld_plain, void* stream);
+int lg_weight_untile_f16(void* plain, const void* tiled, int features, int k, int plain_transa, int ld_plain, void* stream);
 
 /* ---- what the device sustains (no reference counterpart; measurement calls for a bench: they time their own kernel with
  * two events on `stream` and BLOCK until it has finished; nothing on the launch path calls them) ------------------------- */

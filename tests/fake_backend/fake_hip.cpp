@@ -262,6 +262,8 @@ int lg_kv_append_varlen_f16(void* q, void* kc, void*, const void* Q, const void*
     return launch(stream, "kv_append_varlen", (long long)b * h, pos ? pos[0] : 0, slot ? slot[0] : 0, Q, kc, q, mem_cost(12.0 * b * h * d));
 }
 int lg_kv_append_f16(void* q, void* kc, void*, const void* Q, const void*, const void*, const void*, const void*, const void*, int b, int h, int d, int pos, int, void* stream) { return launch(stream, "kv_append", (long long)b * h, pos, d, Q, kc, q, mem_cost(12.0 * b * h * d)); }
+int lg_weight_tile_f16(void* t, const void* p, int f, int k, int, int, void* stream) { return launch(stream, "weight_tile", f, k, 0, p, nullptr, t, mem_cost(4.0 * f * k)); }
+int lg_weight_untile_f16(void* p, const void* t, int f, int k, int, int, void* stream) { return launch(stream, "weight_untile", f, k, 0, t, nullptr, p, mem_cost(4.0 * f * k)); }
 // the measuring entries report the backend's own rates
 int lg_probe_mfma_f16(const void* operands, int64_t n, void* scratch, size_t, int iters, float* ms, float* tflops, float* ghz, void*) {
     if (!operands || !scratch || iters <= 0 || !ms || n < 106504) return LG_ERR_INVALID;

@@ -51,7 +51,7 @@ def test_full_size_gemm_one_hot_rows_select_weight_rows(dev, transa, N, K):
     assert torch.equal(Y, expect.half())
 
 
-@pytest.mark.parametrize("weight_layout", [0, 1])
+@pytest.mark.parametrize("weight_layout", [0, 1, 2])
 def test_full_size_layer_batch_independence_and_oracle_slice(dev, po, host, weight_layout):
     """The cfg2 prefill layer shard (fused assembly, causal) on the full batch: every sequence's result equals, bit for
     bit, the result of running that sequence alone; one sequence is checked against the CPU oracle.  Both weight layouts:
@@ -118,7 +118,7 @@ def test_full_size_decode_attention_against_oracle(dev, po):
     assert max_rel_err(dev.down(out2), got) < 2e-3
 
 
-@pytest.mark.parametrize("weight_layout", [0, 1])
+@pytest.mark.parametrize("weight_layout", [0, 1, 2])
 @pytest.mark.parametrize("batch", [2, 8])
 def test_full_size_decode_step_against_oracle(dev, po, host, batch, weight_layout):
     """One decode step of the full-size layer shard (fused assembly) after a short prefill that fills the KV cache:
@@ -150,7 +150,7 @@ def test_full_size_decode_step_against_oracle(dev, po, host, batch, weight_layou
         tok = po.round_f16(ref)
 
 
-@pytest.mark.parametrize("weight_layout", [0, 1])
+@pytest.mark.parametrize("weight_layout", [0, 1, 2])
 def test_cfg3_full_decode_step_against_oracle(dev, po, host, weight_layout):
     """BASELINE config 3 as a whole: batch 32, one new token per sequence, 1024 cached positions with K/V ~ N(0, 1), on the
     full layer shard.  The cache contents are written into the model's KV cache from the host, so the oracle's decoder step

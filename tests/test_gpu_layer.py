@@ -95,7 +95,7 @@ def test_fp16_layer_small(dev, po, host, norm_mode, causal, fused):
 
 
 @pytest.mark.parametrize("fused", [False, True])
-@pytest.mark.parametrize("weight_layout", [0, 1])
+@pytest.mark.parametrize("weight_layout", [0, 1, 2])
 def test_fp16_tp2_shard_two_layers(dev, po, host, fused, weight_layout):
     """One TP=2 shard (half the heads, half the FFN) of a 2-layer stack, GLM-like head size 128, ragged seq; weights
     stored [in, out] (the reference's layout) or [out, in]."""
@@ -103,7 +103,7 @@ def test_fp16_tp2_shard_two_layers(dev, po, host, fused, weight_layout):
     assert max_rel_err(got, ref) < 1e-2 and elementwise_err(got, ref) < 1e-2
 
 
-@pytest.mark.parametrize("weight_layout", [0, 1])
+@pytest.mark.parametrize("weight_layout", [0, 1, 2])
 def test_fp16_layer_on_the_pipelined_gemm(dev, po, host, weight_layout):
     """Shapes that are multiples of the 256 x 256 x 64 tile, so every weight GEMM takes the pipelined kernel
     (hidden 1024, 8 heads x 128, FFN 2048, 512 tokens)."""
@@ -112,7 +112,7 @@ def test_fp16_layer_on_the_pipelined_gemm(dev, po, host, weight_layout):
 
 
 @pytest.mark.parametrize("fused", [False, True])
-@pytest.mark.parametrize("weight_layout", [0, 1])
+@pytest.mark.parametrize("weight_layout", [0, 1, 2])
 def test_fp16_layer_with_the_published_head_size(dev, po, host, fused, weight_layout):
     """The reference's published configuration uses 96-wide heads, batch 2 and sequences of 16 to 115 tokens (main.cu:14-21):
     one TP=2 shard of a two-layer stack with that head size at the longest of those sequences."""
@@ -202,7 +202,7 @@ def test_geglu_layer(dev, po, host, dtype, fused, norm_mode):
     assert max_rel_err(got, ref) < (2e-5 if dtype == 0 else 1e-2)
 
 
-@pytest.mark.parametrize("weight_layout", [0, 1])
+@pytest.mark.parametrize("weight_layout", [0, 1, 2])
 def test_geglu_fused_upload_round_trip_and_decode(dev, po, host, weight_layout):
     """Fused GeGLU with weights uploaded in the logical [gate | up] order (the model stores them interleaved): prefill and
     one decode step against the oracle, and download(upload(w)) == w."""
@@ -246,7 +246,7 @@ def test_packed_qkv_layer(dev, po, host, dtype, weight_layout):
     assert max_rel_err(got, ref) < (2e-5 if dtype == 0 else 1e-2)
 
 
-@pytest.mark.parametrize("weight_layout", [0, 1])
+@pytest.mark.parametrize("weight_layout", [0, 1, 2])
 @pytest.mark.parametrize("B,S", [(2, 80), (3, 256)])
 def test_packed_qkv_fused_layer_and_decode(dev, po, host, weight_layout, B, S):
     """Packed [H, 3 Hl] projection in the fused assembly: one grouped launch whose epilogue routes q to its buffer and k, v
