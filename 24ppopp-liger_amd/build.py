@@ -86,20 +86,32 @@ def build_host(force=True, verbose=False):
     return lib
 
 
-def build_fake_host(force=True):
+def build_fake_host(force=True, sanitize=None):
     """The same host runtime linked against tests/fake_backend (virtual-time stand-in for the device library):
-    lets the scheduler logic be unit-tested without a GPU.  Test infrastructure; never loaded by the product."""
+    lets the scheduler logic be unit-tested without a GPU.  Test infrastructure; never loaded by the product.
+    sanitize = "thread" | "address": an instrumented build (libliger_host_fake_tsan.so / _asan.so) for the two-thread
+    scheduler tests; the process that loads it must have the sanitizer's runtime preloaded."""
     fake_dir = os.path.join(ROOT, "tests", "fake_backend")
     src = os.path.join(fake_dir, "fake_hip.cpp")
     if not os.path.exists(src):
         return None
-    lib = os.path.join(fake_dir, "libliger_host_fake.so")
+    if sanitize not in (None, "thread", "address"):
+        raise ValueError("sanitize must be None, 'thread' or 'address'")
+    suffix = {None: "", "thread": "_tsan", "address": "_asan"}[sanitize]
+    lib = os.path.join(fake_dir, "libliger_host_fake%s.so" % suffix)
     srcs = [os.path.join(HOST, f) for f in sorted(os.listdir(HOST)) if f.endswith(".cpp") and f != "liger_main.cpp"] + [src]
     hdrs = [os.path.join(HOST, f) for f in os.listdir(HOST) if f.endswith(".h")] + [os.path.join(ROOT, "include", "liger_hip.h")]
+    san = ["-fsanitize=" + sanitize, "-fno-omit-frame-pointer"] if sanitize else []
     if force or _stale(lib, srcs + hdrs):
         _run(["g++", "-O1", "-g", "-std=c++17", "-fPIC", "-Wall", "-Wextra", "-Wno-unused-parameter", "-pthread", "-I",
-              os.path.join(ROOT, "include"), "-I", HOST, "-shared", "-Wl,-Bsymbolic", "-o", lib] + srcs)
+              os.path.join(ROOT, "include"), "-I", HOST, "-shared", "-Wl,-Bsymbolic"] + san + ["-o", lib] + srcs)
     return lib
+
+
+def sanitizer_runtime(sanitize):
+    """Path of the sanitizer's shared runtime (to preload into a process that loads an instrumented library)."""
+    name = {"thread": "libtsan.so", "address": "libasan.so"}[sanitize]
+    return subprocess.run(["g++", "-print-file-name=" + name], stdout=subprocess.PIPE, text=True).stdout.strip()
 
 
 def build_all(force=True, verbose=False):

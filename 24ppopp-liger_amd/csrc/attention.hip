@@ -13,6 +13,7 @@
 //     independent 1 KiB loads in flight.
 // Softmax semantics are the reference's (attention_kernels.cu:480-519): p = exp(t - max t) / (sum + 1e-6),
 // t = q.k * scalar, all positions < len unmasked.
+#include <stdlib.h>
 #include <mutex>
 
 #include "common.hpp"
@@ -32,7 +33,10 @@ struct DecodeSeqs {
 // A key row of D halves is D/8 16-byte chunks; lane `sub` of an LPK-lane group holds chunks sub, sub + LPK, ... (CPL of
 // them), so one wave-wide load covers 64 / LPK keys with LPK * 16 contiguous bytes of each (D = 128: LPK 16, whole rows;
 // D = 64: LPK 8; D = 96: LPK 4 x 3 chunks).
-template <int D, int LPK, int UNROLL, bool VARLEN>
+// NT: the K / V loads are marked non-temporal.  Every load instruction covers whole 128-byte lines and every byte is used once,
+// so nothing is lost by not keeping the lines; the launcher sets it when the keys and values of the launch exceed what the
+// memory-side cache could hold for the next step anyway.
+template <int D, int LPK, int UNROLL, bool VARLEN, bool NT>
 __global__ __launch_bounds__(256) void attn_decode_kernel(const half_t* __restrict__ q, const half_t* __restrict__ kc,
                                                           const half_t* __restrict__ vc, half_t* out, float* ws,
                                                           int len, int max_len, int nsplit, float scalar, int head_num,
@@ -86,8 +90,10 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const half_t* __restri
 #pragma unroll
             for (int c = 0; c < CPL; ++c) {
                 if (key < w_end) {
-                    kv[u][c] = *reinterpret_cast<const half8_t*>(kbase + (int64_t)key * D + c * LPK * 8);
-                    vv[u][c] = *reinterpret_cast<const half8_t*>(vbase + (int64_t)key * D + c * LPK * 8);
+                    const half8_t* kp = reinterpret_cast<const half8_t*>(kbase + (int64_t)key * D + c * LPK * 8);
+                    const half8_t* vp = reinterpret_cast<const half8_t*>(vbase + (int64_t)key * D + c * LPK * 8);
+                    kv[u][c] = NT ? __builtin_nontemporal_load(kp) : *kp;
+                    vv[u][c] = NT ? __builtin_nontemporal_load(vp) : *vp;
                 } else {
                     kv[u][c] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
                     vv[u][c] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
@@ -186,10 +192,16 @@ template <int D, int LPK, int UNROLL>
 static void launch_decode(const half_t* q, const half_t* kc, const half_t* vc, half_t* out, float* ws, int bh, int head_num,
                           int len, int max_len, int ns, float scalar, const DecodeSeqs* seqs, hipStream_t st) {
     const dim3 grid(bh, ns);
-    if (seqs)
-        hipLaunchKernelGGL((attn_decode_kernel<D, LPK, UNROLL, true>), grid, dim3(256), 0, st, q, kc, vc, out, ws, len, max_len, ns, scalar, head_num, *seqs);
-    else
-        hipLaunchKernelGGL((attn_decode_kernel<D, LPK, UNROLL, false>), grid, dim3(256), 0, st, q, kc, vc, out, ws, len, max_len, ns, scalar, head_num, DecodeSeqs{});
+    // more keys and values than half the 256 MB memory-side cache: the next step would not find them there anyway
+    static const int nt_forced = [] { const char* e = getenv("LG_ATTN_DECODE_NT"); return e ? atoi(e) : -1; }();
+    const bool nt = nt_forced >= 0 ? nt_forced != 0 : (int64_t)bh * len * D * 4 > ((int64_t)128 << 20);
+    if (seqs) {
+        if (nt) hipLaunchKernelGGL((attn_decode_kernel<D, LPK, UNROLL, true, true>), grid, dim3(256), 0, st, q, kc, vc, out, ws, len, max_len, ns, scalar, head_num, *seqs);
+        else hipLaunchKernelGGL((attn_decode_kernel<D, LPK, UNROLL, true, false>), grid, dim3(256), 0, st, q, kc, vc, out, ws, len, max_len, ns, scalar, head_num, *seqs);
+    } else {
+        if (nt) hipLaunchKernelGGL((attn_decode_kernel<D, LPK, UNROLL, false, true>), grid, dim3(256), 0, st, q, kc, vc, out, ws, len, max_len, ns, scalar, head_num, DecodeSeqs{});
+        else hipLaunchKernelGGL((attn_decode_kernel<D, LPK, UNROLL, false, false>), grid, dim3(256), 0, st, q, kc, vc, out, ws, len, max_len, ns, scalar, head_num, DecodeSeqs{});
+    }
     if (ns > 1) hipLaunchKernelGGL((attn_decode_merge_kernel<D>), dim3(bh), dim3(D), 0, st, (const float*)ws, out, ns);
 }
 

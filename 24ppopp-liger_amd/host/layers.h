@@ -298,6 +298,22 @@ struct MhaBuffers {  // per-request slices, all in elements of T
     void* decode_ws;  // split-KV partials of the decode attention
 };
 
+// Which (batch, seq, causal) the attr_mask slice of a workspace was last written for.  The slices of a workspace are a function of
+// its base and the request's shape, so as long as the same shape keeps using the workspace nothing else overlaps the mask.
+// Launch callbacks run on the scheduler's thread, the profiler's on the caller's: hence the lock.
+struct MaskState {
+    std::mutex mu;
+    std::map<const void*, std::tuple<int, int, int>> last;
+    bool in_place(const void* ws_base, int batch, int seq, int causal) {
+        std::lock_guard<std::mutex> lk(mu);
+        const auto want = std::make_tuple(batch, seq, causal);
+        auto it = last.find(ws_base);
+        if (it != last.end() && it->second == want) return true;
+        last[ws_base] = want;
+        return false;
+    }
+};
+
 template <typename T>
 class Bert_MHA {
   public:
@@ -314,6 +330,7 @@ class Bert_MHA {
     T *q_bias, *k_bias, *v_bias, *w_bias;
     T* workspace;
     T *k_cache = nullptr, *v_cache = nullptr;  // [max_batch, heads, max_cache_len, d] when max_cache_len > 0
+    std::shared_ptr<MaskState> mask_state = std::make_shared<MaskState>();
     std::vector<FuncWrap> FuncWrapVec;
 
     Bert_MHA(const BertInitParam& BertParams_, const StaticInitParam& SParam_, const int& k_, const int& n_, T* workspace_)
@@ -512,10 +529,16 @@ class Bert_MHA {
                                  (long long)seq_len * d, b.qk_buf, seq_len, (long long)seq_len * seq_len, batch_size * h);
         }, "qk_gemm", MFMA_BOUND));
         // softmax  (:153-155).  The mask (all ones, or lower-triangular) is written into the request's workspace by the same
-        // entry, on the launch stream: building the vector neither allocates nor synchronises.
+        // entry, on the launch stream: building the vector neither allocates nor synchronises.  It is written when the
+        // workspace last held another shape's slices (or nothing): the layers of one request, the requests of one shape that
+        // follow each other on a context and the repeated launches of the profiler find it in place, so a profiled softmax is
+        // the softmax alone.
         const int causal_mask = BertParams.causal;
+        std::shared_ptr<MaskState> ms = mask_state;
         FuncWrapVec.push_back(FuncWrap(0.2f, COMPUTATION, [=](const DynamicInitParam& D) {
-            if (dt == LG_F16) {
+            if (ms->in_place(b.q, batch_size, seq_len, causal_mask)) {
+                // nothing to write
+            } else if (dt == LG_F16) {
                 if (causal_mask) note_status(lg_fill_causal_mask_f16(b.mask, batch_size, seq_len, D.stream), "lg_fill_causal_mask_f16");
                 else note_status(lg_fill_const_f16(b.mask, (int64_t)batch_size * seq_len * seq_len, 1.0f, D.stream), "lg_fill_const_f16");
             } else {
@@ -770,6 +793,8 @@ class Bert_Model {
     Bert_Model(const BertInitParam& BertParams_, const StaticInitParam& SParam_, const int& k_, const int& n_, T* workspace_)
         : k(k_), n(n_), SParam(SParam_), BertParams(BertParams_), workspace(workspace_) {
         for (int i = 0; i < BertParams.layer_num; i++) encoders.push_back(new Bert_Encoder<T>(BertParams, SParam, k, n, workspace));
+        // the layers share their workspaces, so they share what is known about the mask slices in them
+        for (auto* e : encoders) e->MHA->mask_state = encoders[0]->MHA->mask_state;
     }
     Bert_Model(const Bert_Model&) = delete;
     Bert_Model& operator=(const Bert_Model&) = delete;

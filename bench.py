@@ -424,8 +424,9 @@ def main():
     ap.add_argument("--decode", action="store_true",
                     help="with --kernel-only: take the entry from the decode step's launch vector (batch 32, 1024 cached positions); "
                          "needed for the entries whose name the prefill vector has too (ffn1+bias+gelu, ffn2, layer_norm)")
-    ap.add_argument("--weight-layout", type=int, default=1, choices=[0, 1],
-                    help="0: weights stored [in, out] (the reference's cuBLAS (N,N) layout); 1: stored [out, in] (default)")
+    ap.add_argument("--weight-layout", type=int, default=1, choices=[0, 1, 2],
+                    help="0: weights stored [in, out] (the reference's cuBLAS (N,N) layout); 1: stored [out, in] (default); "
+                         "2: [out, in] re-laid into 16 x 32 fragment blocks (lg_weight_tile_f16)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs one GPU's tensor-parallel shard on one GPU; --gpus %d is not supported "
@@ -523,7 +524,7 @@ def main():
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": "cfg2 prefill: hidden 12288, 48/96 heads x 128, FFN 16384/32768, batch 8 x seq 512, causal; "
                                + ("fused assembly (9 launches/layer)" if fused else "reference-shaped assembly (14 launches/layer)")
-                               + ("; weights stored [out, in]" if args.weight_layout else "; weights stored [in, out]")},
+                               + "; weights stored " + {0: "[in, out]", 1: "[out, in]", 2: "[out, in] in 16 x 32 fragment blocks"}[args.weight_layout]},
         "tokens_per_s": round(M / (ms_per_step * 1e-3), 1),
         "roofline": roofline,
         "layer_norm_GBps": round(ln_gbs, 1) if ln_gbs else None,
@@ -541,16 +542,21 @@ def main():
     out["peaks"]["measured"] = measured_ceilings(capi)
     mc = out["peaks"]["measured"]["mfma_f16_random_operands"]["TFLOPs"]
     out["roofline"]["frac_of_measured_mfma_ceiling"] = round(out["roofline"]["achieved"] / mc, 4) if mc > 0 else None
-    # the same layer with the weights stored the other way round (0 = [in, out], the layout the reference's (N,N) cuBLAS call implies)
-    other = 1 - args.weight_layout
-    m2, x2, y2, r2 = time_layer(capi, host, other, fused, max(5, args.steps // 2), 2)
-    out["reference_layout" if other == 0 else "out_in_layout"] = {
-        "weights": "[in, out]" if other == 0 else "[out, in]", "ms_per_layer_shard_prefill": round(r2["ms_per_step"], 4),
-        "ms_per_layer_shard_decode": r2["decode"]["ms_per_layer_shard"] if r2["decode"] else None,
-        "prefill_gemm_tflops": {k["kernel"]: round(label_flops[k["kernel"]] / (k["ms"] * 1e-3) / 1e12, 1) for k in r2["kernels"] if k["kernel"] in label_flops},
-        "decode_kernels_ms": {k["kernel"]: k["ms"] for k in r2["decode"]["kernels"]} if r2["decode"] else None}
-    del m2, x2, y2
-    torch.cuda.empty_cache()
+    # the same layer (prefill and decode step) in the other weight layouts: 0 = [in, out], the layout the reference's (N,N)
+    # cuBLAS call implies; 1 = [out, in]; 2 = [out, in] re-laid into 16 x 32 fragment blocks
+    names = {0: ("reference_layout", "[in, out]"), 1: ("out_in_layout", "[out, in]"), 2: ("tiled_layout", "[out, in] in 16 x 32 fragment blocks")}
+    for other in (0, 1, 2):
+        if other == args.weight_layout:
+            continue
+        m2, x2, y2, r2 = time_layer(capi, host, other, fused, max(5, args.steps // 2), 2)
+        out[names[other][0]] = {
+            "weights": names[other][1], "ms_per_layer_shard_prefill": round(r2["ms_per_step"], 4),
+            "ms_per_layer_shard_decode": r2["decode"]["ms_per_layer_shard"] if r2["decode"] else None,
+            "prefill_gemm_tflops": {k["kernel"]: round(label_flops[k["kernel"]] / (k["ms"] * 1e-3) / 1e12, 1) for k in r2["kernels"] if k["kernel"] in label_flops},
+            "decode_kernels_ms": {k["kernel"]: k["ms"] for k in r2["decode"]["kernels"]} if r2["decode"] else None,
+            "decode_kernels_in_step_ms": {k["kernel"]: k["in_step_ms"] for k in r2["decode"]["kernels"]} if r2["decode"] else None}
+        del m2, x2, y2
+        torch.cuda.empty_cache()
     if not args.no_cpu_baseline:
         from oracle import pyoracle as po
         out["cpu_baseline"] = cpu_baseline(po)

@@ -3,7 +3,8 @@ import ctypes as C
 import importlib
 import os
 
-FAKE_LIB = os.path.join(os.path.dirname(os.path.abspath(__file__)), "fake_backend", "libliger_host_fake.so")
+# LIGER_FAKE_LIB selects another build of the same library (the sanitizer runs load an instrumented one)
+FAKE_LIB = os.environ.get("LIGER_FAKE_LIB") or os.path.join(os.path.dirname(os.path.abspath(__file__)), "fake_backend", "libliger_host_fake.so")
 
 
 class Fake:
