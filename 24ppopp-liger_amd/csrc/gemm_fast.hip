@@ -49,7 +49,7 @@ template <int NJ> __device__ __forceinline__ int unswz_kn(int k, int blk) {
 }
 
 template <int WL, int EPI, int NJ>
-__global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, GemmGroup grp, int tiles_m, int tiles_n, float* partial, int kt_per_split, int cus) {
+__global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, GemmGroup grp, int tiles_m, int tiles_n, float* partial, int kt_per_split, int cus, int wide_store) {
     constexpr int FB_N = 64 * NJ;
     constexpr int X_TILE = FB_M * FB_K, W_TILE = FB_K * FB_N;  // halves per ring slot
     constexpr int WCH = (FB_K * FB_N) / 512 / 8;  // 1 KiB chunks of the W tile per wave (= NJ)
@@ -330,6 +330,51 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, GemmGroup
         if (EPI == LG_EPI_BIAS_HEADS) col_off[j] = (int64_t)(n / g.epi.d) * g.ldy * g.epi.d + (n % g.epi.d);
         else col_off[j] = n;
     }
+    if (wide_store) {
+        // The tile goes through LDS (the ring is idle now) and leaves in whole rows: in the accumulator layout a wave's store
+        // instruction writes 32 bytes of 16 different rows; read back row by row, 32 lanes write 512 contiguous bytes of one
+        // row.  Rows are 16 bytes apart from a multiple of 128 in LDS, so the 8-byte writes of a half-wave (16 rows x 2 lane
+        // groups) and the 16-byte reads fall on distinct banks.
+        constexpr int PITCH = FB_N + 8;  // halves
+        __syncthreads();                 // every wave has read its last fragments
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                float v[4] = {acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
+                if (EPI != LG_EPI_NONE) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) v[r] += bias_v[j][r];
+                }
+                if (EPI == LG_EPI_BIAS_GELU) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) v[r] = gelu_tanh(v[r]);
+                }
+                const half4_t o = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+                *reinterpret_cast<half4_t*>(&smem[(wm * 128 + i * 16 + l16) * PITCH + wn * (16 * NJ) + j * 16 + 4 * lk]) = o;
+            }
+        }
+        __syncthreads();
+        constexpr int CPR = FB_N / 8;                 // 16-byte chunks per tile row
+        constexpr int ITERS = FB_M * CPR / F_THREADS;  // 16, 12 or 8
+#pragma unroll 4
+        for (int it = 0; it < ITERS; ++it) {
+            const int c = it * F_THREADS + tid;
+            const int row = c / CPR, cc = c % CPR;
+            const int m = m0 + row, n = n0 + cc * 8;
+            if (m >= g.M) continue;
+            const half8_t o = *reinterpret_cast<const half8_t*>(&smem[row * PITCH + cc * 8]);
+            int64_t off;
+            if (EPI == LG_EPI_BIAS_HEADS) {
+                const int b = m / g.epi.seq, sq = m % g.epi.seq;
+                off = (((int64_t)b * g.epi.heads_total + n / g.epi.d) * g.ldy + sq) * (int64_t)g.epi.d + (n % g.epi.d);
+            } else {
+                off = (int64_t)m * g.ldy + n;
+            }
+            *reinterpret_cast<half8_t*>(g.Y + off) = o;
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         const int m = m0 + wm * 128 + i * 16 + l16;
@@ -381,12 +426,18 @@ static int launch_fast_epi(const GemmArgs& g, const GemmGroup& grp, int tiles_m,
     float* partial = nsplit > 1 ? si.ws : nullptr;
     const dim3 grid(tiles, nsplit), block(F_THREADS);
     const size_t smem = lds_halves(NJ) * sizeof(half_t);
+    // whole-row stores through LDS need 16-byte aligned rows (heads epilogue: rows of size_per_head halves)
+    static const int wide_forced = [] { const char* e = getenv("LG_GEMM_WIDE_STORE"); return e ? atoi(e) : -1; }();
+    int wide = 1;
+    for (int i = 0; i < grp.count; ++i)
+        if (g.epi.kind == LG_EPI_BIAS_HEADS ? (g.epi.d % 8 != 0) : (grp.ldy[i] % 8 != 0)) wide = 0;
+    if (wide_forced >= 0) wide = wide && wide_forced;
 #define LG_FAST(E)                                                                                                  \
     do {                                                                                                            \
         /* set once per instantiation; the initialisation of a function-local static is thread-safe */              \
         static const hipError_t attr_rc = hipFuncSetAttribute((const void*)gemm_f16_fast<WL, E, NJ>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
         (void)attr_rc;                                                                                              \
-        hipLaunchKernelGGL((gemm_f16_fast<WL, E, NJ>), grid, block, smem, stream, g, grp, tiles_m, tiles_n, partial, kt_per_split, cus); \
+        hipLaunchKernelGGL((gemm_f16_fast<WL, E, NJ>), grid, block, smem, stream, g, grp, tiles_m, tiles_n, partial, kt_per_split, cus, wide); \
     } while (0)
     if (nsplit > 1) {
         LG_FAST(LG_EPI_PARTIAL);

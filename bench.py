@@ -424,9 +424,9 @@ def main():
     ap.add_argument("--decode", action="store_true",
                     help="with --kernel-only: take the entry from the decode step's launch vector (batch 32, 1024 cached positions); "
                          "needed for the entries whose name the prefill vector has too (ffn1+bias+gelu, ffn2, layer_norm)")
-    ap.add_argument("--weight-layout", type=int, default=1, choices=[0, 1, 2],
-                    help="0: weights stored [in, out] (the reference's cuBLAS (N,N) layout); 1: stored [out, in] (default); "
-                         "2: [out, in] re-laid into 16 x 32 fragment blocks (lg_weight_tile_f16)")
+    ap.add_argument("--weight-layout", type=int, default=2, choices=[0, 1, 2],
+                    help="0: weights stored [in, out] (the reference's cuBLAS (N,N) layout); 1: stored [out, in]; "
+                         "2 (default): [out, in] re-laid into 16 x 32 fragment blocks when the layer takes them over (lg_weight_tile_f16)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs one GPU's tensor-parallel shard on one GPU; --gpus %d is not supported "
