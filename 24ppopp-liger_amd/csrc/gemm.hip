@@ -3,8 +3,11 @@
 //   gemm_f16_generic   128x128x32 tiles, 4 waves (2x2), MFMA 16x16x32 f16 -> fp32, any shape / stride /
 //                      alignment, both weight layouts, optional fused epilogue.  Correctness workhorse
 //                      (edge tiles, decomposed sub-ranges, attention GEMMs, small models).
-//   gemm_f32_generic   64x64x16 VALU tiles for the fp32 plumbing configuration.
+//   gemm_f32_mfma      128x128x16 tiles on v_mfma_f32_32x32x2_f32 for the fp32 instantiation (any shape, both layouts);
+//   gemm_f32_generic   64x64x16 VALU tiles, kept as a cross-check.
 // The large aligned prefill shapes are routed to the pipelined kernels in gemm_fast.hip.
+#include <stdlib.h>
+
 #include "gemm_common.hpp"
 
 namespace lg {
@@ -255,9 +258,142 @@ __global__ __launch_bounds__(256) void gemm_f32_generic(GemmArgsF32 g) {
         }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// fp32 on the matrix cores: 128 x 128 x 16 tiles, 4 waves (2 x 2), v_mfma_f32_32x32x2_f32
+// ---------------------------------------------------------------------------------------------------
+// The reference instantiates every layer for float through cublasGemmEx(..., CUDA_R_32F, ...) (context.h:49-55,
+// linear.h:47-49,99-101).  A wave owns 64 x 64 outputs = 2 x 2 MFMA tiles (64 accumulator registers); operands are swapped as
+// in the fp16 kernels (the weight tile is the A operand), so a lane ends up with 4 consecutive output features of one token
+// row: acc[i][j][v] = Y[token 32 i + lane % 32][feature 32 j + 8 (v / 4) + 4 (lane / 32) + v % 4].  Both tiles sit in LDS
+// k-major ([16][128 + 32] floats): a wave-wide operand read is two runs of 32 consecutive floats, 32 banks apart.
+typedef float float16v_t __attribute__((ext_vector_type(16)));
+constexpr int SB_M = 128, SB_N = 128, SB_K = 16, SB_PITCH = 128 + 32;
+
+template <int WL, bool ALIGNED>
+__global__ __launch_bounds__(256) void gemm_f32_mfma(GemmArgsF32 g) {
+    __shared__ __attribute__((aligned(16))) float Xs[SB_K * SB_PITCH];
+    __shared__ __attribute__((aligned(16))) float Ws[SB_K * SB_PITCH];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int m0 = blockIdx.y * SB_M, n0 = blockIdx.x * SB_N;
+    const float* X = g.X + (int64_t)blockIdx.z * g.strideX;
+    const float* W = g.W + (int64_t)blockIdx.z * g.strideW;
+    float* Y = g.Y + (int64_t)blockIdx.z * g.strideY;
+
+    float16v_t acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+    // 8 consecutive floats p[0..7] with `valid` of them inside the matrix
+    auto load8f = [](const float* p, int valid, float (&r)[8]) {
+        if (ALIGNED && valid >= 8) {
+            const float4_t a = *reinterpret_cast<const float4_t*>(p), b = *reinterpret_cast<const float4_t*>(p + 4);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { r[i] = a[i]; r[4 + i] = b[i]; }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) r[i] = i < valid ? p[i] : 0.f;
+        }
+    };
+    float rx[8], rw[8];
+    auto gload = [&](int k0) {
+        {   // X tile: 128 token rows x 16 k; thread = (row, half of the k range)
+            const int row = tid >> 1, kh = (tid & 1) * 8;
+            const int m = m0 + row, k = k0 + kh;
+            load8f(X + (int64_t)m * g.ldx + k, m < g.M ? g.K - k : 0, rx);
+        }
+        if (WL == W_NK) {
+            const int row = tid >> 1, kh = (tid & 1) * 8;
+            const int n = n0 + row, k = k0 + kh;
+            load8f(W + (int64_t)n * g.ldw + k, n < g.N ? g.K - k : 0, rw);
+        } else {  // [K, N]: 16 k-rows x 128 features; thread = (k, 8 consecutive features)
+            const int kr = tid >> 4, ns = (tid & 15) * 8;
+            const int k = k0 + kr, n = n0 + ns;
+            load8f(W + (int64_t)k * g.ldw + n, k < g.K ? g.N - n : 0, rw);
+        }
+    };
+    auto lstore = [&]() {
+        {
+            const int row = tid >> 1, kh = (tid & 1) * 8;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) Xs[(kh + i) * SB_PITCH + row] = rx[i];
+        }
+        if (WL == W_NK) {
+            const int row = tid >> 1, kh = (tid & 1) * 8;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) Ws[(kh + i) * SB_PITCH + row] = rw[i];
+        } else {
+            const int kr = tid >> 4, ns = (tid & 15) * 8;
+            *reinterpret_cast<float4_t*>(&Ws[kr * SB_PITCH + ns]) = float4_t{rw[0], rw[1], rw[2], rw[3]};
+            *reinterpret_cast<float4_t*>(&Ws[kr * SB_PITCH + ns + 4]) = float4_t{rw[4], rw[5], rw[6], rw[7]};
+        }
+    };
+
+    const int l32 = lane & 31, lh = lane >> 5;
+    gload(0);
+    for (int k0 = 0; k0 < g.K; k0 += SB_K) {
+        __syncthreads();
+        lstore();
+        __syncthreads();
+        if (k0 + SB_K < g.K) gload(k0 + SB_K);
+#pragma unroll
+        for (int ks = 0; ks < SB_K / 2; ++ks) {
+            float a[2], b[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) a[i] = Xs[(ks * 2 + lh) * SB_PITCH + wm * 64 + i * 32 + l32];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) b[j] = Ws[(ks * 2 + lh) * SB_PITCH + wn * 64 + j * 32 + l32];
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(b[j], a[i], acc[i][j], 0, 0, 0);
+        }
+    }
+    const bool vec_ok = ALIGNED && (g.ldy % 4 == 0);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int m = m0 + wm * 64 + i * 32 + l32;
+        if (m >= g.M) continue;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int n = n0 + wn * 64 + j * 32 + 8 * q + 4 * lh;
+                float* p = Y + (int64_t)m * g.ldy + n;
+                if (vec_ok && n + 3 < g.N) {
+                    *reinterpret_cast<float4_t*>(p) = float4_t{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (n + r < g.N) p[r] = acc[i][j][4 * q + r];
+                }
+            }
+    }
+}
+
 static int gemm_f32_dispatch(const GemmArgsF32& g, int wlayout, int batch, hipStream_t stream) {
     if (g.M == 0 || g.N == 0 || batch == 0) return LG_OK;
     if (g.K == 0) { set_error("gemm: k == 0 is not supported"); return LG_ERR_INVALID; }
+    // LG_GEMM_F32_VALU=1 in the environment (read once) selects the vector-ALU tile kernel instead: a cross-check for tests
+    static const bool valu = [] { const char* e = getenv("LG_GEMM_F32_VALU"); return e && atoi(e) != 0; }();
+    if (!valu) {
+        dim3 grid((g.N + SB_N - 1) / SB_N, (g.M + SB_M - 1) / SB_M, batch);
+        if (grid.y > 65535 || grid.z > 65535) { set_error("gemm: problem too large for the grid"); return LG_ERR_INVALID; }
+        const bool aligned = aligned16(g.X) && aligned16(g.W) && aligned16(g.Y) && (g.ldx % 4 == 0) && (g.ldw % 4 == 0) &&
+                             (g.strideX % 4 == 0) && (g.strideW % 4 == 0) && (g.strideY % 4 == 0);
+        if (wlayout == W_NK) {
+            if (aligned) hipLaunchKernelGGL((gemm_f32_mfma<W_NK, true>), grid, dim3(256), 0, stream, g);
+            else hipLaunchKernelGGL((gemm_f32_mfma<W_NK, false>), grid, dim3(256), 0, stream, g);
+        } else {
+            if (aligned) hipLaunchKernelGGL((gemm_f32_mfma<W_KN, true>), grid, dim3(256), 0, stream, g);
+            else hipLaunchKernelGGL((gemm_f32_mfma<W_KN, false>), grid, dim3(256), 0, stream, g);
+        }
+        return check_launch("gemm_f32");
+    }
     dim3 grid((g.N + 63) / 64, (g.M + 63) / 64, batch);
     if (grid.y > 65535 || grid.z > 65535) { set_error("gemm: problem too large for the generic grid"); return LG_ERR_INVALID; }
     if (wlayout == W_NK) hipLaunchKernelGGL((gemm_f32_generic<W_NK>), grid, dim3(256), 0, stream, g);

@@ -330,6 +330,50 @@ def measured_ceilings(capi, iters=3000, read_mib=2048):
     return out
 
 
+def bench_fp32(capi, host):
+    """The fp32 instantiation (the reference builds every layer for float as well, context.h:49-55): BASELINE config 1 (hidden 256,
+    4 heads x 64, FFN 1024, pre-LayerNorm, batch 2 x seq 32) as one launch vector, and the fp32 GEMM on the matrix cores at a
+    size that fills the chip, against the published fp32 matrix peak."""
+    import ctypes as C
+    import torch
+    m = host.Model(capi.F32, 2, 32, 4, 64, layer_num=1, ffn_inner=1024, norm_mode=host.PRE_LN_RESID, causal=False, fused=False, seed=0)
+    x = torch.empty(64, 256, device="cuda", dtype=torch.float32)
+    capi.call("lg_fill_normal_f32", x.data_ptr(), x.numel(), 0, 99, 0.0, 1.0, None)
+    y = torch.empty_like(x)
+    torch.cuda.synchronize()
+    for _ in range(5):
+        m.run(x.data_ptr(), y.data_ptr(), 2, 32, None, m.stream)
+    capi.call("lg_stream_synchronize", m.stream)
+    t0 = time.perf_counter()
+    for _ in range(200):
+        m.run(x.data_ptr(), y.data_ptr(), 2, 32, None, m.stream)
+    capi.call("lg_stream_synchronize", m.stream)
+    cfg1_ms = (time.perf_counter() - t0) * 1e3 / 200
+    launches = m.kernels_per_layer()
+    m.close()
+    out = {"cfg1_layer_ms": round(cfg1_ms, 4), "cfg1_launches": launches}
+    n = 4096
+    a = torch.empty(n, n, device="cuda", dtype=torch.float32)
+    b = torch.empty(n, n, device="cuda", dtype=torch.float32)
+    c = torch.empty(n, n, device="cuda", dtype=torch.float32)
+    capi.call("lg_fill_normal_f32", a.data_ptr(), a.numel(), 0, 5, 0.0, 0.02, None)
+    capi.call("lg_fill_normal_f32", b.data_ptr(), b.numel(), 0, 6, 0.0, 1.0, None)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for transa, name in ((0, "[in, out]"), (1, "[out, in]")):
+        for _ in range(2):
+            capi.call("lg_gemm_f32", transa, 0, n, n, n, a.data_ptr(), n, b.data_ptr(), n, c.data_ptr(), n, None)
+        e0.record()
+        for _ in range(10):
+            capi.call("lg_gemm_f32", transa, 0, n, n, n, a.data_ptr(), n, b.data_ptr(), n, c.data_ptr(), n, None)
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / 10
+        out["gemm_4096_cubed_weights_" + name] = {"ms": round(ms, 4), "TFLOPs": round(2 * n ** 3 / ms / 1e9, 1),
+                                                  "frac_of_fp32_matrix_peak": round(2 * n ** 3 / ms / 1e9 / 157.3, 4)}
+    return out
+
+
 def derived_peaks(info):
     """Roofline denominators re-derived from the device properties: matrix peak = CUs x 4096 fp16 flop per clock and CU x
     engine clock; memory peak = bus width x reported memory clock x 4 transfers per pin and clock (the runtime reports 2.0 GHz
@@ -557,6 +601,16 @@ def main():
             "decode_kernels_in_step_ms": {k["kernel"]: k["in_step_ms"] for k in r2["decode"]["kernels"]} if r2["decode"] else None}
         del m2, x2, y2
         torch.cuda.empty_cache()
+    if fused:
+        # the reference-shaped assembly (bert.h:59-79: 14 launches per layer, three batched-GEMM / softmax / transpose kernels
+        # instead of the fused attention, separate bias kernels) on the same shard and weights layout: what a maintainer who binds
+        # the C ABI entry by entry gets before adopting the fused entries
+        m3, x3, y3, r3 = time_layer(capi, host, args.weight_layout, False, max(5, args.steps // 2), 2)
+        out["reference_assembly"] = {"launches_per_layer": len(r3["kernels"]), "ms_per_layer_shard_prefill": round(r3["ms_per_step"], 4),
+                                     "kernels_ms": {"%d:%s" % (k["idx"], k["kernel"]): k["ms"] for k in r3["kernels"]}}
+        del m3, x3, y3
+        torch.cuda.empty_cache()
+    out["fp32"] = bench_fp32(capi, host)
     if not args.no_cpu_baseline:
         from oracle import pyoracle as po
         out["cpu_baseline"] = cpu_baseline(po)
