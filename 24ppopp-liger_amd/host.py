@@ -58,6 +58,8 @@ SIGNATURES = {
     "lgh_sched_set_contention": (_i, [_p, _i, _i, _f]),
     "lgh_sched_enable_partition": (_i, [_p, _i]),
     "lgh_sched_set_decode_step_hook": (_i, [_p, _p, _p]),
+    "lgh_sched_set_partition_feedback": (_i, [_p, _i, _i, _i, _f]),
+    "lgh_sched_partition_feedback_state": (_i, [_p, C.POINTER(C.c_double)]),
     "lgh_sched_enable_batch_decode": (_i, [_p, _i, _i]),
     "lgh_sched_set_recycle_contexts": (_i, [_p, _i]),
     "lgh_sched_ctx_decode_ptrs": (_i, [_p, _i, C.POINTER(_p), C.POINTER(_p)]),
@@ -369,6 +371,18 @@ class Scheduler:
     def enable_partition(self, hbm_cus):
         """Co-running rounds give the HBM-bound side `hbm_cus` compute units and the MFMA-bound side the rest (0 = off)."""
         check(lib.lgh_sched_enable_partition(self.h, hbm_cus), "lgh_sched_enable_partition")
+
+    def set_partition_feedback(self, on, min_samples=0, probe=-1, margin=0.0):
+        """While a run goes on, rounds that could be partitioned are run both ways and partitioned only while that delivers more
+        (on by default).  min_samples / probe / margin: samples of each kind before deciding, every n-th such round takes the other
+        side, required ratio of the two progress rates; non-positive (probe: negative) values keep what is set."""
+        check(lib.lgh_sched_set_partition_feedback(self.h, int(bool(on)), min_samples, probe, margin), "lgh_sched_set_partition_feedback")
+
+    def partition_feedback_state(self):
+        out = (C.c_double * 5)()
+        check(lib.lgh_sched_partition_feedback_state(self.h, out), "lgh_sched_partition_feedback_state")
+        return {"rate_whole_chip": out[0], "rate_partitioned": out[1], "samples_whole_chip": int(out[2]), "samples_partitioned": int(out[3]),
+                "declined": int(out[4])}
 
     def profile_partition(self, bs, seq, dec_bs, past):
         """Measures a partitioned co-run (prefill MFMA-bound kernels || decode steps) and installs the budget factors when

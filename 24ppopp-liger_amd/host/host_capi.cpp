@@ -45,6 +45,8 @@ struct SchedBase {
     virtual float get_contention(int main_class, int sub_class) = 0;
     virtual bool streams_concurrent() = 0;
     virtual void set_merge_minor(bool on) = 0;
+    virtual void set_partition_feedback(bool on, int min_samples, int probe, float margin) = 0;
+    virtual void feedback_state(double* out5) = 0;
     virtual void set_decode_step_hook(void (*fn)(void*, int, int, const int*, const int*, void*, void*), void* user) = 0;
 };
 
@@ -187,6 +189,16 @@ struct SchedT : SchedBase {
     }
     bool streams_concurrent() override { return s->DParams1.concurrent; }
     void set_merge_minor(bool on) override { s->merge_minor = on; }
+    void set_partition_feedback(bool on, int min_samples, int probe, float margin) override {
+        s->partition_feedback = on;
+        if (min_samples > 0) s->partition_feedback_min = min_samples;
+        if (probe >= 0) s->partition_feedback_probe = probe;
+        if (margin > 0.f) s->partition_feedback_margin = margin;
+    }
+    void feedback_state(double* out5) override {
+        out5[0] = s->feedback_rate(1); out5[1] = s->feedback_rate(2); out5[2] = s->feedback_samples(1); out5[3] = s->feedback_samples(2);
+        out5[4] = s->partition_declined;
+    }
     void set_decode_step_hook(void (*fn)(void*, int, int, const int*, const int*, void*, void*), void* user) override {
         if (!fn) { s->decode_step_hook = nullptr; return; }
         s->decode_step_hook = [fn, user](int step, const std::vector<int>& slots, const std::vector<int>& pasts, T* rows, const DynamicInitParam& D) {
@@ -570,6 +582,20 @@ int lgh_sched_set_contention(void* sched, int main_class, int sub_class, float v
 int lgh_sched_set_merge_minor(void* sched, int on) {
     if (!sched) return fail("lgh_sched_set_merge_minor: null");
     ((SchedBase*)sched)->set_merge_minor(on != 0);
+    return LG_OK;
+}
+// Whether partitioned rounds are checked against whole-chip rounds while a run goes on (Scheduler::partition_feedback; on by
+// default).  min_samples <= 0, probe < 0, margin <= 0 keep the current value.
+int lgh_sched_set_partition_feedback(void* sched, int on, int min_samples, int probe, float margin) {
+    if (!sched) return fail("lgh_sched_set_partition_feedback: null");
+    ((SchedBase*)sched)->set_partition_feedback(on != 0, min_samples, probe, margin);
+    return LG_OK;
+}
+// out5 = {progress rate of whole-chip rounds, of partitioned rounds (stand-alone ms of work per ms), samples of each, rounds that
+// could have been partitioned and were not} of the last run
+int lgh_sched_partition_feedback_state(void* sched, double* out5) {
+    if (!sched || !out5) return fail("lgh_sched_partition_feedback_state: bad arguments");
+    ((SchedBase*)sched)->feedback_state(out5);
     return LG_OK;
 }
 // fn(user, step, rows, slots[rows], pasts[rows], batch_rows, stream) is called on the scheduler's thread after the kernels of

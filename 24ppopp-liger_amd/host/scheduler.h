@@ -172,6 +172,26 @@ class Scheduler {
     int partition_hbm_cus = 0;
     float partition_table[3][3] = {{-1.f, -1.f, -1.f}, {-1.f, -1.f, -1.f}, {-1.f, -1.f, -1.f}};
     float partition_min_ms = 0.05f;   // less waiting work than this is not worth a partitioned round
+    // ---- does partitioning pay in THIS run?  (partition_feedback) -----------------------------------------------------------
+    // partition_table comes from one measured pair of shapes in steady state; a trace has other shapes, short rounds and a host
+    // synchronisation per round.  While a run is going on the scheduler therefore measures what its rounds deliver: every round
+    // starts with an event on the primary's stream (behind the end of the round before it), and a round's progress rate is the
+    // stand-alone milliseconds of work launched in it (primary and secondaries) per millisecond until the next round starts.
+    // Rounds in which a partition is possible are run partitioned and on the whole chip in turn until both kinds have
+    // partition_feedback_min samples; from then on they are partitioned only while the partitioned rounds' rate is at least
+    // partition_feedback_margin times the whole-chip rounds', and every partition_feedback_probe-th such round takes the other
+    // side so that both figures stay current.  The figures carry over from run to run (older samples at half weight) until the
+    // share changes.  No reference counterpart.
+    bool partition_feedback = true;
+    int partition_feedback_min = 6, partition_feedback_probe = 16;
+    float partition_feedback_margin = 1.02f;
+    int partition_declined = 0;       // rounds that could have been partitioned and were run on the whole chip instead
+    void reset_partition_feedback() {
+        for (int k = 0; k < 3; ++k) { _fb_work[k] = _fb_time[k] = 0; _fb_n[k] = 0; }
+        _fb_eligible = 0;
+    }
+    double feedback_rate(int kind) const { return _fb_time[kind] > 0 ? _fb_work[kind] / _fb_time[kind] : 0.0; }  // 1: whole chip, 2: partitioned
+    int feedback_samples(int kind) const { return _fb_n[kind]; }
     StaticInitParam SParams;
     DynamicInitParam DParams0;
     DynamicInitParam DParams1;
@@ -211,6 +231,8 @@ class Scheduler {
         DParams0.destroy();
         for (void* e : {Main_EVENT, Wait_EVENT, _epoch_event, _dec_prev_stop})
             if (e) lg_event_destroy(e);
+        for (RoundRec& r : _round_log) lg_event_destroy(r.begin);
+        for (void* e : _round_events) lg_event_destroy(e);
         for (ReqCtx* c : _all_ctx) {
             dev_free(c->input); dev_free(c->output); dev_free(c->ws); dev_free(c->dec_a); dev_free(c->dec_b);
             delete c;
@@ -253,9 +275,10 @@ class Scheduler {
         for (int role = 0; role < 2; ++role)
             for (int cls = 0; cls < 2; ++cls) _part[role][cls] = it->second.d[role][cls].get();
         partition_hbm_cus = hbm_cus;
-        // factors measured for another share do not carry over
+        // factors measured for another share do not carry over, nor does what rounds on it delivered
         for (int a = 0; a < 3; ++a)
             for (int b = 0; b < 3; ++b) partition_table[a][b] = -1.f;
+        reset_partition_feedback();
         return true;
     }
     void disable_partition() { partition_hbm_cus = 0; }
@@ -739,6 +762,7 @@ class Scheduler {
             const DynamicInitParam* Dp = &DParams0;
             const DynamicInitParam* Ds = &DParams1;
             float part_factor = -1.f, cap = 0.f;
+            int round_kind = 0;   // 0: no partition possible, 1: possible but run on the whole chip, 2: partitioned
             if (partition_hbm_cus > 0 && policy == RESOURCE && !head->empty()) {
                 const int mc = head->next_class();
                 const int sc = mc == MFMA_BOUND ? HBM_BOUND : (mc == HBM_BOUND ? MFMA_BOUND : -1);
@@ -747,11 +771,16 @@ class Scheduler {
                     for (size_t s = 1; s < exe_vec.size(); s++)
                         if (!exe_vec[s]->empty()) need += exe_vec[s]->run_ahead_duration(mc);
                     if (need >= partition_min_ms) {
-                        part_factor = partition_table[mc][sc];
-                        cap = need / part_factor;
-                        Dp = _part[0][mc];
-                        Ds = _part[1][sc];
-                        partition_rounds++;
+                        round_kind = _partition_pays() ? 2 : 1;
+                        if (round_kind == 2) {
+                            part_factor = partition_table[mc][sc];
+                            cap = need / part_factor;
+                            Dp = _part[0][mc];
+                            Ds = _part[1][sc];
+                            partition_rounds++;
+                        } else {
+                            partition_declined++;
+                        }
                     }
                 }
             }
@@ -759,6 +788,8 @@ class Scheduler {
             // the secondary stream waits (on the device) for the end of the previous round
             note_status(lg_event_synchronize(Wait_EVENT), "lg_event_synchronize");
             note_status(lg_stream_wait_event(Ds->stream, Main_EVENT), "lg_stream_wait_event");
+            if (partition_feedback && partition_hbm_cus > 0) _round_begin(*Dp, round_kind);
+            float round_work = 0.f;
             while (!head->empty()) {
                 main_class = head->next_class();
                 const bool capped = part_factor > 0.f && time_planned + head->duration(1, time_planned) >= cap;
@@ -770,6 +801,7 @@ class Scheduler {
                 }
                 time_planned += head->dequeue(*Dp, 1, time_planned);
             }
+            round_work += time_planned;
             rounds++;
             // time_planned stays in units of the primary's time; a secondary kernel of stand-alone duration d uses up
             // d / contention(main, sub) of it (with the constant factor this is the reference's 0.8 x time_planned budget)
@@ -786,12 +818,15 @@ class Scheduler {
                         }
                         time_planned = 0.0f;
                     } else {
-                        time_planned -= sub->dequeue(*Ds, 0, avail) / f;
+                        const float d = sub->dequeue(*Ds, 0, avail);
+                        time_planned -= d / f;
+                        round_work += d;
                         secondary_launches++;
                     }
                 }
             }
             time_planned = 0.0f;
+            if (!_round_log.empty()) _round_log.back().work = round_work;
         }
         _finish();
     }
@@ -816,7 +851,12 @@ class Scheduler {
         _dec_prefill_events.clear();
         if (_dec_prev_stop) { lg_event_destroy(_dec_prev_stop); _dec_prev_stop = nullptr; }
         batched_steps = batched_rows = 0;
-        rounds = secondary_launches = splits = partition_rounds = 0;
+        rounds = secondary_launches = splits = partition_rounds = partition_declined = 0;
+        // what the rounds of earlier runs delivered is kept (it is a property of the device and the workload, and a run may have
+        // few rounds in which a partition is possible); older samples count half at every new run
+        for (RoundRec& r : _round_log) _round_events.push_back(r.begin);
+        _round_log.clear();
+        for (int k = 0; k < 3; ++k) { _fb_work[k] *= 0.5; _fb_time[k] *= 0.5; }
     }
 
     // ---- request simulator  (schedule.h:285-321) ---------------------------------------------------------------------
@@ -1081,6 +1121,48 @@ class Scheduler {
         std::lock_guard<std::mutex> lk(_q_mutex);
         for (Sample* smp : _main_q) delete smp;
         _main_q.clear();
+    }
+    // ---- partition feedback ------------------------------------------------------------------------------------------------
+    struct RoundRec { void* begin; float work; int kind; };
+    std::deque<RoundRec> _round_log;     // rounds whose duration is not known yet (the last one is the round being launched)
+    std::vector<void*> _round_events;    // pool of events for the log
+    double _fb_work[3] = {0, 0, 0}, _fb_time[3] = {0, 0, 0};
+    int _fb_n[3] = {0, 0, 0}, _fb_eligible = 0;
+    void* _round_event() {
+        if (!_round_events.empty()) { void* e = _round_events.back(); _round_events.pop_back(); return e; }
+        void* e = nullptr;
+        note_status(lg_event_create(&e), "lg_event_create");
+        return e;
+    }
+    // The round's first event: on the primary's stream, behind the end of the primary run before it (Main_EVENT), so that the
+    // distance between two such events is the time the earlier round took, whichever streams the two rounds use.
+    void _round_begin(const DynamicInitParam& Dp, int kind) {
+        note_status(lg_stream_wait_event(Dp.stream, Main_EVENT), "lg_stream_wait_event");
+        RoundRec r{_round_event(), 0.f, kind};
+        note_status(lg_event_record(r.begin, Dp.stream), "lg_event_record");
+        _round_log.push_back(r);
+        // every round but the newest has an end (the next round's beginning): account for those whose events have completed
+        while (_round_log.size() >= 2 && lg_event_query(_round_log[1].begin) == LG_OK) {
+            RoundRec done = _round_log.front();
+            _round_log.pop_front();
+            float ms = 0.f;
+            if (lg_event_elapsed_ms(&ms, done.begin, _round_log.front().begin) == LG_OK && ms > 0.f && done.kind > 0 && done.work > 0.f) {
+                _fb_work[done.kind] += done.work;
+                _fb_time[done.kind] += ms;
+                _fb_n[done.kind]++;
+            }
+            _round_events.push_back(done.begin);
+        }
+    }
+    // whether the round that is about to start, in which a partition is possible, should be partitioned
+    bool _partition_pays() {
+        if (!partition_feedback) return true;
+        const int n = _fb_eligible++;
+        // both kinds in turn while either lacks samples (launched rounds count: their durations arrive a little later)
+        if (_fb_n[1] < partition_feedback_min || _fb_n[2] < partition_feedback_min) return (n & 1) == 0;
+        const bool pays = feedback_rate(2) >= (double)partition_feedback_margin * feedback_rate(1);
+        if (partition_feedback_probe > 0 && n % partition_feedback_probe == 0) return !pays;
+        return pays;
     }
     struct PartStreams { std::unique_ptr<DynamicInitParam> d[2][2]; };
     // releases every CU-masked stream and leaves partitioning off with no pointer to a released stream behind

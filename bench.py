@@ -204,10 +204,11 @@ def bench_corun_variants(weight_layout):
     return {"workload": "prefill B4 S512 MFMA-bound kernels || decode steps at 1024 cached positions, one layer shard", "rows": rows}
 
 
-def bench_cfg5(capi, host, weight_layout, n_requests, rates=(4.0, 8.0, 16.0), shares=(64, 128), runs=1, decode_steps_ahead=2, short=False):
-    """BASELINE config 5: Poisson arrivals at 4, 8, 16 req/s through 4 stacked layer shards; prompts U[128, 1024]
-    (rounded to 64), 32 decode tokens each; mean and p99 request latency with interleaving on and off.  `runs` > 1 repeats
-    every (rate, mode) and reports the mean and the spread of the mean latency over the runs."""
+def bench_cfg5(capi, host, weight_layout, n_requests, rates=(4.0, 8.0, 16.0, 24.0, 32.0), shares=(64, 128), runs=1, decode_steps_ahead=2, short=False):
+    """BASELINE config 5: Poisson arrivals at 4, 8, 16 req/s -- and at 24 and 32 req/s, which is at and beyond what one request
+    at a time can serve (about 28 req/s) -- through 4 stacked layer shards; prompts U[128, 1024] (rounded to 64), 32 decode
+    tokens each; mean and p99 request latency with interleaving on and off.  `runs` > 1 repeats every (rate, mode) and reports
+    the mean and the spread of the mean latency over the runs."""
     c = CFG2
     pool = 16
     model = host.Model(capi.F16, pool + 1, 1024, c["heads_global"], c["d"], layer_num=4, world_size=c["world_size"], ffn_inner=c["ffn_global"],
@@ -274,7 +275,9 @@ def bench_cfg5(capi, host, weight_layout, n_requests, rates=(4.0, 8.0, 16.0), sh
                          "mean_gpu_ms": round(r["avg_gpu_ms"], 3), "mean_queue_ms": round(r["avg_queue_ms"], 3),
                          "throughput_req_s": round(r["throughput"], 3), "records": r["records"],
                          "secondary_launches": r["secondary_launches"], "splits": r["splits"], "profile_misses": r["profile_misses"],
-                         "partition_rounds": r["partition_rounds"], "batched_steps": r["batched_steps"],
+                         "partition_rounds": r["partition_rounds"],
+                         "partition_feedback": sched.partition_feedback_state() if share else None,
+                         "batched_steps": r["batched_steps"],
                          "rows_per_batched_step": round(r["batched_rows"] / r["batched_steps"], 2) if r["batched_steps"] else None}
         out.append(row)
     sched.enable_partition(0)
@@ -627,7 +630,7 @@ def main():
         if args.cfg5:
             out["cfg5"] = bench_cfg5(capi, host, args.weight_layout, args.cfg5_requests, runs=args.cfg5_runs)
         else:
-            out["cfg5"] = bench_cfg5(capi, host, args.weight_layout, 40, rates=(16.0,), shares=(128,), runs=3, short=True)
+            out["cfg5"] = bench_cfg5(capi, host, args.weight_layout, 40, rates=(16.0, 32.0), shares=(128,), runs=3, short=True)
     print(json.dumps(out))
 
 

@@ -533,6 +533,7 @@ def _partition_setup(fake, factor_hbm_main=None):
         s.profile_decode(1, past, 2)
     s.set_merge_minor(True)
     s.enable_partition(128)
+    s.set_partition_feedback(False)     # these tests look at the partition mechanism itself, round by round
     if factor_hbm_main is not None:
         s.set_partition_factor(HBM, MFMA, factor_hbm_main)
         s.set_partition_factor(MFMA, HBM, 1.0 / factor_hbm_main)
@@ -616,6 +617,56 @@ def test_a_failed_change_of_share_leaves_no_stream_behind_and_no_stale_pointer(f
     assert s.run_queued(host.MODE_LIGER)["partition_rounds"] >= 1
     s.close()
     assert lib.fake_live_streams() == live - 6
+
+
+@pytest.mark.parametrize("matrix_exp,memory_exp,corun,pays", [(1.0, 1.0, 1.0, False), (0.5, 0.2, 0.5, True)])
+def test_partition_feedback_follows_what_the_rounds_deliver(fake, matrix_exp, memory_exp, corun, pays):
+    """Prefill requests (MFMA-bound) and decode requests (HBM-bound) queued in turn, with a partition table that says every
+    co-running round should be partitioned.  The backend decides what is true: (a) a share of the compute units costs in
+    proportion and the whole chip overlaps two streams for free -> partitioned rounds deliver less than whole-chip rounds;
+    (b) a share hurts less than in proportion and the whole chip only time-slices -> partitioned rounds deliver more.
+    With feedback the scheduler runs both kinds of round in turn, then keeps the better kind (and probes the other now and
+    then); without it every such round is partitioned, whatever it delivers."""
+    host = fake.host
+    m = host.Model(1, 41, 64, 4, 64, layer_num=2, ffn_inner=512, causal=True, fused=True, max_cache_len=128, factor=4, seed=0)
+    s = host.Scheduler(m, contention_factor=0.8, policy=host.POLICY_RESOURCE, seq_bucket=16, pool_count=40, ctx_batch=1)
+    s.profile(1, 48, 64, 16, 2)
+    for past in (48, 64, 80, 96, 112):
+        s.profile_decode(1, past, 2)
+    s.set_merge_minor(True)
+    s.enable_partition(128)
+    s.set_partition_factor(HBM, MFMA, 1.0)
+    s.set_partition_factor(MFMA, HBM, 1.0)
+
+    def run(feedback):
+        s.set_partition_feedback(feedback, 3, 8, 1.02)
+        fake.reset()
+        fake.set_share_model(matrix_exp, memory_exp)
+        fake.set_corun_speed(corun)
+        for _ in range(20):
+            s.serve(1, 64, 0)
+            s.serve_decode(1, 48, 60)
+        r = s.run_queued(host.MODE_LIGER)
+        assert r["records"] == 40 and r["profile_misses"] == 0
+        return r, s.partition_feedback_state()
+
+    r, st = run(True)
+    eligible = r["partition_rounds"] + st["declined"]
+    assert eligible >= 15 and st["samples_whole_chip"] >= 3 and st["samples_partitioned"] >= 3
+    if pays:
+        assert st["rate_partitioned"] > 1.02 * st["rate_whole_chip"]
+        assert r["partition_rounds"] >= 0.65 * eligible
+    else:
+        assert st["rate_partitioned"] < 1.02 * st["rate_whole_chip"]
+        assert r["partition_rounds"] <= 0.45 * eligible
+    # a second run starts from what the first one measured: no more turns, only the occasional probe of the other side
+    r1, st1 = run(True)
+    eligible1 = r1["partition_rounds"] + st1["declined"]
+    assert (r1["partition_rounds"] >= 0.8 * eligible1) if pays else (r1["partition_rounds"] <= 0.2 * eligible1)
+    r2, st2 = run(False)
+    assert st2["declined"] == 0 and r2["partition_rounds"] >= 15
+    s.close()
+    m.close()
 
 
 @pytest.mark.parametrize("matrix_exp,memory_exp,pays", [(1.0, 1.0, False), (0.5, 0.2, True)])
