@@ -77,6 +77,7 @@ SIGNATURES = {
     "lg_gemm_fused_grouped_f16": (_i, [_i, _i, _i, _i, _i, _p, _i, _p, _i, _p, _p, _i, _p, _i, _i, _i, _p]),
     "lg_gemm_fused_grouped_rows_f16": (_i, [_i, _i, _i, _i, _i, _p, _i, _p, _i, _p, _p, _p, _i, _i, _p, _p, _p, _p]),
     "lg_attn_prefill_f16": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _i, _p]),
+    "lg_attn_prefill_past_f16": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p]),
     "lg_attn_decode_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "lg_attn_decode_f16": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _f, _p]),
     "lg_attn_decode_varlen_f16": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, C.POINTER(_i), C.POINTER(_i), _i, _f, _p]),

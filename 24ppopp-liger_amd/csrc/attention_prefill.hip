@@ -48,7 +48,7 @@ template <int D, int NW, bool CAUSAL, bool HAS_MASK>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(const half_t* __restrict__ q_buf, const half_t* __restrict__ k_buf,
                                                            const half_t* __restrict__ v_buf, const half_t* __restrict__ mask,
                                                            half_t* out, int seq, int head_num, int kv_rows, float scalar,
-                                                           int out_layout) {
+                                                           int out_layout, int q_off) {
     constexpr int DC = D / 32;      // 32-wide d chunks (k steps of the S^T GEMM)
     constexpr int DT = D / 16;      // 16-wide d tiles (rows of O^T)
     constexpr int CPR = D / 8;      // 16-byte chunks per row
@@ -85,6 +85,10 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
     const int b = bh / head_num, head = bh % head_num;
     const int q0 = qblk * PF_BQ;               // first query of the block
     const int qw = q0 + wave * 32;             // first query of the wave
+    // q_off > 0: the `seq` queries are positions q_off .. q_off + seq - 1 of a sequence whose first q_off keys and values are
+    // already in k_buf / v_buf (a prefill continued in chunks over a KV cache); keys 0 .. kv_len - 1 exist
+    const int kv_len = q_off + seq;
+    const int qwa = q_off + qw;                // absolute position of the wave's first query
 
     const half_t* Q = q_buf + (int64_t)bh * seq * D;
     const half_t* K = k_buf + (int64_t)bh * kv_rows * D;
@@ -127,7 +131,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
     auto issue = [&](int k0, int buf) {
 #pragma unroll
         for (int i = 0; i < LPT; ++i) {
-            const int64_t row = min(k0 + lrow[i], seq - 1);             // rows beyond the sequence: its last row, masked later
+            const int64_t row = min(k0 + lrow[i], kv_len - 1);          // rows beyond the sequence: its last row, masked later
             load_lds16(K + row * D + koff[i], &Ks[buf][(i * NW + wave) * 512]);
             load_lds16(V + row * D + voff[i], &Vs[buf][(i * NW + wave) * 512]);
         }
@@ -155,7 +159,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
 
     const float sl2 = scalar * 1.4426950408889634f;            // scores in log2 units
     constexpr float MASK_L2 = -10000.0f * 1.4426950408889634f;  // the reference's additive mask term, in the same units
-    const int kv_end = CAUSAL ? min(seq, q0 + PF_BQ) : seq;
+    const int kv_end = CAUSAL ? min(kv_len, q_off + q0 + PF_BQ) : kv_len;
     issue(0, 0);
     for (int k0 = 0, t = 0; k0 < kv_end; k0 += PF_BC, ++t) {
         const int buf = t & 1;
@@ -164,7 +168,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
         if (k0 + PF_BC < kv_end) issue(k0 + PF_BC, buf ^ 1);
         // a wave whose queries all lie before this key tile has nothing to do here (causal), but keeps loading and hitting
         // the barrier, so only the math is skipped
-        if (CAUSAL && k0 > qw + 31) continue;
+        if (CAUSAL && k0 > qwa + 31) continue;
         const half_t* ks = Ks[buf];
         const half_t* vs = Vs[buf];
 
@@ -205,8 +209,8 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
         // Scores are kept in log2 units (scale folded with log2 e: exp(t - m) = exp2(t' - m')), so that a score costs one
         // multiply, one max, one subtract, one exp2 and one add.  The causal comparison is only made on tiles that reach above
         // the diagonal of the wave's first query, the end-of-sequence test only on the last tile (both wave-uniform).
-        const bool diag = CAUSAL && (k0 + PF_BC - 1 > qw);
-        const bool tail = k0 + PF_BC > seq;
+        const bool diag = CAUSAL && (k0 + PF_BC - 1 > qwa);
+        const bool tail = k0 + PF_BC > kv_len;
 #pragma unroll
         for (int qt = 0; qt < 2; ++qt) {
             const int q = qw + qt * 16 + l16;
@@ -230,14 +234,14 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
                 for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
                     for (int r = 0; r < 4; ++r)
-                        if (k0 + kt * 16 + 4 * g + r > q) s[kt][qt][r] += MASK_L2;
+                        if (k0 + kt * 16 + 4 * g + r > q_off + q) s[kt][qt][r] += MASK_L2;
             }
             if (tail) {
 #pragma unroll
                 for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
                     for (int r = 0; r < 4; ++r)
-                        if (k0 + kt * 16 + 4 * g + r >= seq) s[kt][qt][r] = -1e30f;  // beyond the sequence: not part of the row at all
+                        if (k0 + kt * 16 + 4 * g + r >= kv_len) s[kt][qt][r] = -1e30f;  // beyond the sequence: not part of the row at all
             }
             float mx = -1e30f;
 #pragma unroll
@@ -336,45 +340,60 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
 
 template <int D, int NW>
 static void launch_prefill(const half_t* q, const half_t* k, const half_t* v, const half_t* mask, half_t* out, int batch,
-                           int seq, int head_num, int kv_rows, float scalar, int causal, int out_layout, hipStream_t st) {
+                           int seq, int head_num, int kv_rows, float scalar, int causal, int out_layout, int q_off, hipStream_t st) {
     constexpr int BQ = 32 * NW;
     dim3 grid((seq + BQ - 1) / BQ, batch * head_num), block(64 * NW);
     if (causal)
-        hipLaunchKernelGGL((attn_prefill_kernel<D, NW, true, false>), grid, block, 0, st, q, k, v, mask, out, seq, head_num, kv_rows, scalar, out_layout);
+        hipLaunchKernelGGL((attn_prefill_kernel<D, NW, true, false>), grid, block, 0, st, q, k, v, mask, out, seq, head_num, kv_rows, scalar, out_layout, q_off);
     else if (mask)
-        hipLaunchKernelGGL((attn_prefill_kernel<D, NW, false, true>), grid, block, 0, st, q, k, v, mask, out, seq, head_num, kv_rows, scalar, out_layout);
+        hipLaunchKernelGGL((attn_prefill_kernel<D, NW, false, true>), grid, block, 0, st, q, k, v, mask, out, seq, head_num, kv_rows, scalar, out_layout, q_off);
     else
-        hipLaunchKernelGGL((attn_prefill_kernel<D, NW, false, false>), grid, block, 0, st, q, k, v, mask, out, seq, head_num, kv_rows, scalar, out_layout);
+        hipLaunchKernelGGL((attn_prefill_kernel<D, NW, false, false>), grid, block, 0, st, q, k, v, mask, out, seq, head_num, kv_rows, scalar, out_layout, q_off);
 }
 
 }  // namespace lg
 
 using namespace lg;
 
-extern "C" int lg_attn_prefill_f16(const void* q_buf, const void* k_buf, const void* v_buf, const void* attr_mask,
-                                   void* out, int batch, int seq, int head_num, int size_per_head, int kv_rows,
-                                   float scalar, int causal, int out_layout, void* stream) {
-    if (batch < 0 || seq < 0 || head_num <= 0 || kv_rows < seq || (out_layout != 0 && out_layout != 1)) {
-        set_error("attn_prefill: bad shape (seq=%d kv_rows=%d)", seq, kv_rows);
+static int attn_prefill_entry(const char* what, const void* q_buf, const void* k_buf, const void* v_buf, const void* attr_mask,
+                              void* out, int batch, int seq, int past, int head_num, int size_per_head, int kv_rows,
+                              float scalar, int causal, int out_layout, void* stream) {
+    if (batch < 0 || seq < 0 || past < 0 || head_num <= 0 || (int64_t)past + seq > kv_rows || (out_layout != 0 && out_layout != 1)) {
+        set_error("%s: bad shape (seq=%d past=%d kv_rows=%d)", what, seq, past, kv_rows);
         return LG_ERR_INVALID;
     }
-    if (size_per_head != 64 && size_per_head != 96 && size_per_head != 128) { set_error("attn_prefill: size_per_head must be 64, 96 or 128"); return LG_ERR_INVALID; }
+    if (past > 0 && attr_mask) { set_error("%s: an explicit mask covers [seq, seq] positions only; past > 0 needs causal or no mask", what); return LG_ERR_INVALID; }
+    if (size_per_head != 64 && size_per_head != 96 && size_per_head != 128) { set_error("%s: size_per_head must be 64, 96 or 128", what); return LG_ERR_INVALID; }
     if (batch == 0 || seq == 0) return LG_OK;
-    if (!q_buf || !k_buf || !v_buf || !out) { set_error("attn_prefill: null pointer"); return LG_ERR_INVALID; }
+    if (!q_buf || !k_buf || !v_buf || !out) { set_error("%s: null pointer", what); return LG_ERR_INVALID; }
     if (!aligned16(q_buf) || !aligned16(k_buf) || !aligned16(v_buf) || !aligned16(out)) {
-        set_error("attn_prefill: pointers must be 16-byte aligned");
+        set_error("%s: pointers must be 16-byte aligned", what);
         return LG_ERR_INVALID;
     }
-    if ((int64_t)batch * head_num > 65535) { set_error("attn_prefill: batch * head_num > 65535"); return LG_ERR_INVALID; }
+    if ((int64_t)batch * head_num > 65535) { set_error("%s: batch * head_num > 65535", what); return LG_ERR_INVALID; }
     scalar = (float)(half_t)scalar;
     if (size_per_head == 128)
         launch_prefill<128, 4>((const half_t*)q_buf, (const half_t*)k_buf, (const half_t*)v_buf, (const half_t*)attr_mask,
-                            (half_t*)out, batch, seq, head_num, kv_rows, scalar, causal, out_layout, (hipStream_t)stream);
+                            (half_t*)out, batch, seq, head_num, kv_rows, scalar, causal, out_layout, past, (hipStream_t)stream);
     else if (size_per_head == 96)
         launch_prefill<96, 4>((const half_t*)q_buf, (const half_t*)k_buf, (const half_t*)v_buf, (const half_t*)attr_mask,
-                           (half_t*)out, batch, seq, head_num, kv_rows, scalar, causal, out_layout, (hipStream_t)stream);
+                           (half_t*)out, batch, seq, head_num, kv_rows, scalar, causal, out_layout, past, (hipStream_t)stream);
     else
         launch_prefill<64, 4>((const half_t*)q_buf, (const half_t*)k_buf, (const half_t*)v_buf, (const half_t*)attr_mask,
-                           (half_t*)out, batch, seq, head_num, kv_rows, scalar, causal, out_layout, (hipStream_t)stream);
-    return check_launch("attn_prefill");
+                           (half_t*)out, batch, seq, head_num, kv_rows, scalar, causal, out_layout, past, (hipStream_t)stream);
+    return check_launch(what);
+}
+
+extern "C" int lg_attn_prefill_f16(const void* q_buf, const void* k_buf, const void* v_buf, const void* attr_mask,
+                                   void* out, int batch, int seq, int head_num, int size_per_head, int kv_rows,
+                                   float scalar, int causal, int out_layout, void* stream) {
+    return attn_prefill_entry("attn_prefill", q_buf, k_buf, v_buf, attr_mask, out, batch, seq, 0, head_num, size_per_head, kv_rows, scalar,
+                              causal, out_layout, stream);
+}
+
+extern "C" int lg_attn_prefill_past_f16(const void* q_buf, const void* k_buf, const void* v_buf, void* out, int batch, int seq,
+                                        int past, int head_num, int size_per_head, int kv_rows, float scalar, int causal,
+                                        int out_layout, void* stream) {
+    return attn_prefill_entry("attn_prefill_past", q_buf, k_buf, v_buf, nullptr, out, batch, seq, past, head_num, size_per_head, kv_rows,
+                              scalar, causal, out_layout, stream);
 }

@@ -44,6 +44,7 @@ SIGNATURES = {
     "lgh_model_kv_cache": (_i, [_p, _i, C.POINTER(_p), C.POINTER(_p)]),
     "lgh_model_describe": (_i, [_p, _i, _i, _i, C.c_char_p, _i]),
     "lgh_model_run": (_i, [_p, _p, _p, _i, _i, _p, _p, _i]),
+    "lgh_model_run_chunked": (_i, [_p, _p, _p, _i, _i, _p, _p, _i]),
     "lgh_model_run_decode": (_i, [_p, _p, _p, _i, _i, _i, _p, _p]),
     "lgh_model_run_decode_seqs": (_i, [_p, _p, _p, _i, C.POINTER(_i), C.POINTER(_i), _p, _p]),
     "lgh_model_time_kernels": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, C.POINTER(_f), _i]),
@@ -277,6 +278,10 @@ class Model:
 
     def run(self, input_ptr, output_ptr, batch, seq, workspace_ptr=None, stream=None, cache_slot=-1):
         check(lib.lgh_model_run(self.h, input_ptr, output_ptr, batch, seq, workspace_ptr, stream, cache_slot), "lgh_model_run")
+
+    def run_chunked(self, input_ptr, output_ptr, seq, chunk, cache_slot, workspace_ptr=None, stream=None):
+        """The prefill of one sequence in chunks of `chunk` tokens over the KV cache of `cache_slot` (fused assembly)."""
+        check(lib.lgh_model_run_chunked(self.h, input_ptr, output_ptr, seq, chunk, workspace_ptr, stream, cache_slot), "lgh_model_run_chunked")
 
     def run_decode(self, input_ptr, output_ptr, batch, past, cache_slot=0, workspace_ptr=None, stream=None):
         check(lib.lgh_model_run_decode(self.h, input_ptr, output_ptr, batch, past, cache_slot, workspace_ptr, stream),

@@ -58,6 +58,7 @@ struct ModelBase {
     }
     virtual std::vector<FuncWrap> build(void* in, void* out, int batch, int seq, void* ws, int slot) = 0;
     virtual std::vector<FuncWrap> build_decode(void* in, void* out, int batch, int past, int slot, void* ws) = 0;
+    virtual std::vector<FuncWrap> build_prefill_past(void* in, void* out, int batch, int seq, int past, void* ws, int slot) = 0;
     virtual std::vector<FuncWrap> build_decode_seqs(void* in, void* out, const std::vector<int>& slots, const std::vector<int>& pasts, void* ws) = 0;
     virtual int64_t workspace_elems(int batch, int seq) = 0;
     virtual int kernels_per_layer(bool decode) = 0;
@@ -221,6 +222,9 @@ struct ModelT : ModelBase {
     }
     std::vector<FuncWrap> build_decode(void* in, void* out, int batch, int past, int slot, void* ws) override {
         return m->forward_decode((T*)in, (T*)out, batch, past, slot, (T*)(ws ? ws : default_ws));
+    }
+    std::vector<FuncWrap> build_prefill_past(void* in, void* out, int batch, int seq, int past, void* ws, int slot) override {
+        return m->forward_prefill_past((T*)in, (T*)out, batch, seq, past, (T*)(ws ? ws : default_ws), slot);
     }
     std::vector<FuncWrap> build_decode_seqs(void* in, void* out, const std::vector<int>& slots, const std::vector<int>& pasts, void* ws) override {
         return m->forward_decode_seqs((T*)in, (T*)out, slots, pasts, (T*)(ws ? ws : default_ws));
@@ -392,6 +396,24 @@ int lgh_model_run(void* model, void* input, void* output, int batch, int seq, vo
         return fail("lgh_model_run: sequence or cache slot outside the KV cache");
     DynamicInitParam D(stream ? stream : mb->stream0->stream, 0);
     for (auto& f : mb->build(input, output, batch, seq, workspace, cache_slot)) f.callback(D);
+    return first_error();
+}
+
+// The prefill of ONE sequence of `seq` tokens taken in chunks of `chunk` tokens (the last one shorter), every chunk through all
+// layers before the next: chunk c attends to the keys and values chunks 0 .. c left in the KV cache of `cache_slot`.  input /
+// output are [seq, hidden].  The result equals lgh_model_run(batch 1) up to the rounding of another summation order.
+int lgh_model_run_chunked(void* model, void* input, void* output, int seq, int chunk, void* workspace, void* stream, int cache_slot) {
+    ModelBase* mb = (ModelBase*)model;
+    if (!shape_ok(mb, 1, seq) || !input || !output || chunk <= 0) return fail("lgh_model_run_chunked: bad arguments");
+    if (!mb->P.fused || cache_slot < 0 || mb->P.max_cache_len <= 0 || seq > mb->P.max_cache_len || cache_slot >= mb->P.max_batch_size)
+        return fail("lgh_model_run_chunked: needs the fused assembly and a KV-cache slot that holds the sequence");
+    DynamicInitParam D(stream ? stream : mb->stream0->stream, 0);
+    const size_t row_bytes = (size_t)mb->P.head_num * mb->P.size_per_head * mb->elem_size();
+    for (int p0 = 0; p0 < seq; p0 += chunk) {
+        const int c = std::min(chunk, seq - p0);
+        for (auto& f : mb->build_prefill_past((char*)input + (size_t)p0 * row_bytes, (char*)output + (size_t)p0 * row_bytes, 1, c, p0, workspace, cache_slot))
+            f.callback(D);
+    }
     return first_error();
 }
 

@@ -445,15 +445,22 @@ class Bert_MHA {
     }
     // idx 0..8 of the launch vector (9 entries); fused assembly: 5 entries.
     // cache_slot >= 0 (fused only): K/V are written straight into the KV cache rows [cache_slot, cache_slot+batch).
-    std::vector<FuncWrap> forward(T* input, T* output, int batch_size, int seq_len, T* ws = nullptr, int cache_slot = -1) {
+    // past > 0 (fused assembly with a cache slot only): the seq_len tokens continue sequences whose first `past` positions are
+    // in the KV cache already (a long prompt prefilled in chunks): K / V go to cache rows past .., the attention sees the past
+    // and the chunk's own keys.  No reference counterpart.
+    std::vector<FuncWrap> forward(T* input, T* output, int batch_size, int seq_len, T* ws = nullptr, int cache_slot = -1, int past = 0) {
         FuncWrapVec.clear();
         if (!ws) ws = workspace;
         const MhaBuffers<T> b = slice(ws, batch_size, seq_len);
         const int M = batch_size * seq_len, h = heads(), d = BertParams.size_per_head;
         const int dt = dtype_of<T>::value;
         const float sc = scalar;
-        if (cache_slot >= 0 && k_cache && (seq_len > BertParams.max_cache_len || cache_slot + batch_size > BertParams.max_batch_size)) {
+        if (cache_slot >= 0 && k_cache && (past + seq_len > BertParams.max_cache_len || cache_slot + batch_size > BertParams.max_batch_size)) {
             set_error_state(LG_ERR_INVALID, "Bert_MHA::forward: sequence or cache slot outside the KV cache");
+            return FuncWrapVec;
+        }
+        if (past < 0 || (past > 0 && !(BertParams.fused && dt == LG_F16 && cache_slot >= 0 && k_cache))) {
+            set_error_state(LG_ERR_INVALID, "Bert_MHA::forward: a prefill that continues a sequence needs the fused assembly and a KV-cache slot");
             return FuncWrapVec;
         }
         if (BertParams.fused && dt == LG_F16) {
@@ -466,7 +473,7 @@ class Bert_MHA {
                 vdst = v_cache + (int64_t)cache_slot * h * kv_rows * d;
             }
             Linear_Col<T>* lin[3] = {linear_q_col, linear_k_col, linear_v_col};
-            T* dst[3] = {b.q_buf, kdst, vdst};
+            T* dst[3] = {b.q_buf, kdst + (int64_t)past * d, vdst + (int64_t)past * d};  // row `past` of every (sequence, head) slot
             const T* bias[3] = {q_bias, k_bias, v_bias};
             const char* lab[3] = {"q_gemm+bias+heads", "k_gemm+bias+heads", "v_gemm+bias+heads"};
             GemmDesc gd[3];
@@ -490,8 +497,12 @@ class Bert_MHA {
             T* qb = b.q_buf; T* ao = b.attn_out;
             const int causal = BertParams.causal;
             FuncWrapVec.push_back(FuncWrap(0.8f, COMPUTATION, [=](const DynamicInitParam& D) {
-                note_status(lg_attn_prefill_f16(qb, kdst, vdst, nullptr, ao, batch_size, seq_len, h, d, kv_rows, sc, causal, 1,
-                                                D.stream), "lg_attn_prefill_f16");
+                if (past > 0)
+                    note_status(lg_attn_prefill_past_f16(qb, kdst, vdst, ao, batch_size, seq_len, past, h, d, kv_rows, sc, causal, 1, D.stream),
+                                "lg_attn_prefill_past_f16");
+                else
+                    note_status(lg_attn_prefill_f16(qb, kdst, vdst, nullptr, ao, batch_size, seq_len, h, d, kv_rows, sc, causal, 1,
+                                                    D.stream), "lg_attn_prefill_f16");
             }, "attn_prefill_fused", MFMA_BOUND));
             std::vector<FuncWrap> v = linear_w_row->forward(b.attn_out, output, M);
             v[0].label = "out_proj";
@@ -731,8 +742,10 @@ class Bert_Encoder {
     // bert.h:59-79: MHA -> LN -> MLP -> LN (POST_NORESID).  PRE_LN_RESID chains layer_norm -> MHA ->
     // add_bias_input_layernorm_2 -> MLP -> add_bias_input.
     // slots / pasts (both or neither): a decode step over sequences in arbitrary cache slots at different positions
+    // prefill_past > 0: the seq_len tokens continue sequences with that many positions in the KV cache (see Bert_MHA::forward)
     std::vector<FuncWrap> forward(T* input, T* output, int batch_size, int seq_len, T* ws = nullptr, int cache_slot = -1,
-                                  int decode_past = -1, const std::vector<int>* slots = nullptr, const std::vector<int>* pasts = nullptr) {
+                                  int decode_past = -1, const std::vector<int>* slots = nullptr, const std::vector<int>* pasts = nullptr,
+                                  int prefill_past = 0) {
         FuncWrapVec.clear();
         if (!ws) ws = workspace;
         const bool decode = decode_past >= 0 || slots;
@@ -748,7 +761,7 @@ class Bert_Encoder {
         auto mha = [&](T* in, T* out) {
             if (slots) return MHA->forward_decode_seqs(in, out, *slots, *pasts, attn_ws);
             return decode ? MHA->forward_decode(in, out, batch_size, decode_past, cache_slot, attn_ws)
-                          : MHA->forward(in, out, batch_size, seq_len, attn_ws, cache_slot);
+                          : MHA->forward(in, out, batch_size, seq_len, attn_ws, cache_slot, prefill_past);
         };
         auto mlp = [&](T* in, T* out) {
             std::vector<FuncWrap> v = MLP->forward(in, out, M, mlp_inner);
@@ -824,6 +837,17 @@ class Bert_Model {
         if (!ws) ws = workspace;
         for (int i = 0; i < BertParams.layer_num; i++) {
             std::vector<FuncWrap> v = encoders[i]->forward(i == 0 ? input : output, output, batch_size, seq_len, ws, cache_slot);
+            FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
+        }
+        return FuncWrapVec;
+    }
+    // A prefill that continues sequences whose first `past` positions are already in the KV cache of `cache_slot` (a long prompt
+    // taken in chunks, each chunk through all layers): input / output are the chunk's own rows [batch, seq_len, hidden].
+    std::vector<FuncWrap> forward_prefill_past(T* input, T* output, int batch_size, int seq_len, int past, T* ws, int cache_slot) {
+        FuncWrapVec.clear();
+        if (!ws) ws = workspace;
+        for (int i = 0; i < BertParams.layer_num; i++) {
+            std::vector<FuncWrap> v = encoders[i]->forward(i == 0 ? input : output, output, batch_size, seq_len, ws, cache_slot, -1, nullptr, nullptr, past);
             FuncWrapVec.insert(FuncWrapVec.end(), v.begin(), v.end());
         }
         return FuncWrapVec;

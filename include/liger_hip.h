@@ -235,6 +235,13 @@ int lg_gemm_fused_grouped_rows_f16(int transa, int m, int n, int k, int count, c
 int lg_attn_prefill_f16(const void* q_buf, const void* k_buf, const void* v_buf, const void* attr_mask,
                         void* out, int batch, int seq, int head_num, int size_per_head, int kv_rows,
                         float scalar, int causal, int out_layout, void* stream);
+/* The same for a prefill that continues a sequence (a long prompt processed in chunks over a KV cache): the `seq` queries of
+ * q_buf [B,h,seq,d] are positions past .. past + seq - 1, k_buf / v_buf [B,h,kv_rows,d] hold the past + seq keys and values
+ * (the chunk's own rows included, past + seq <= kv_rows).  causal != 0: query i sees keys 0 .. past + i; causal == 0: all
+ * past + seq keys.  No explicit mask. */
+int lg_attn_prefill_past_f16(const void* q_buf, const void* k_buf, const void* v_buf, void* out, int batch, int seq, int past,
+                             int head_num, int size_per_head, int kv_rows, float scalar, int causal, int out_layout,
+                             void* stream);
 /* Decode attention: q [B,h,d]; k_cache, v_cache [B,h,max_len,d] with `len` valid positions; out [B,h,d].
  * size_per_head: 64, 96 or 128.  workspace: float buffer of lg_attn_decode_workspace_bytes(...) bytes (split-KV partials),
  * caller-owned; that size is an upper bound for every batch and every len <= max_len, so a buffer sized once for the

@@ -250,6 +250,7 @@ int lg_gemm_fused_grouped_rows_f16(int, int m, int n, int k, int count, const vo
     return launch(stream, "gemm_fused_grouped_rows", (long long)m * count, n, k, A[0], B, C[0], gemm_cost((long long)m * count, n, k));
 }
 int lg_attn_prefill_f16(const void* q, const void* k, const void*, const void*, void* out, int b, int s, int h, int d, int, float, int, int, void* stream) { return launch(stream, "attn_prefill", (long long)b * h, s, d, q, k, out, gemm_cost((long long)b * h * s, s, 2 * d)); }
+int lg_attn_prefill_past_f16(const void* q, const void* k, const void*, void* out, int b, int s, int past, int h, int d, int, float, int, int, void* stream) { return launch(stream, "attn_prefill_past", (long long)b * h, s, past, q, k, out, gemm_cost((long long)b * h * s, past + s, 2 * d)); }
 size_t lg_attn_decode_workspace_bytes(int, int, int, int) { return 1024; }
 int lg_attn_decode_f16(const void* q, const void* kc, const void*, void* out, void*, int b, int h, int d, int len, int, float, void* stream) { return launch(stream, "attn_decode", (long long)b * h, len, d, q, kc, out, mem_cost(4.0 * b * h * len * d)); }
 int lg_attn_decode_static_f16(const void* q, const void* kc, const void*, void* out, int b, int h, int d, int len, int, float, void* stream) { return launch(stream, "attn_decode", (long long)b * h, len, d, q, kc, out, mem_cost(4.0 * b * h * len * d)); }

@@ -168,3 +168,33 @@ def test_attn_prefill_fused(dev, po, B, h, S, d, mode, kv_rows, layout):
         got = np.delete(got, 3, axis=2)
         ref = np.delete(ref, 3, axis=2)
     assert max_rel_err(got, ref) < 1e-2
+
+
+@pytest.mark.parametrize("B,h,d,S,past,kv_rows,causal", [
+    (2, 4, 128, 128, 128, 256, 1), (1, 8, 128, 200, 312, 512, 1), (1, 3, 64, 64, 1, 80, 1), (2, 2, 96, 100, 57, 160, 1),
+    (1, 8, 128, 128, 896, 1024, 1), (1, 4, 128, 70, 130, 200, 0), (1, 48, 128, 256, 768, 1088, 1)])
+def test_attn_prefill_that_continues_a_sequence(dev, po, B, h, d, S, past, kv_rows, causal):
+    """A chunk of S queries at positions past .. past + S - 1 over past + S keys and values (chunked prefill over a KV cache)
+    must equal rows past .. of the oracle's attention over the whole sequence: with a causal mask row i sees keys 0 .. past + i;
+    without one every query sees all past + S keys, which is the last S rows of the full non-causal attention."""
+    L = past + S
+    q = rnd(po, B * h * L * d, 80).reshape(B, h, L, d)
+    k = rnd(po, B * h * L * d, 81).reshape(B, h, L, d)
+    v = rnd(po, B * h * L * d, 82).reshape(B, h, L, d)
+    scalar = 1.0 / np.sqrt(d)
+    ref = po.attn_prefill(q, k, v, scalar, bool(causal), 1)[:, :, past:]
+    kpad = np.zeros((B, h, kv_rows, d), dtype=np.float32); vpad = np.full((B, h, kv_rows, d), 7.0, dtype=np.float32)
+    kpad[:, :, :L] = k; vpad[:, :, :L] = v
+    out = dev.empty((B, S, h, d), 1)
+    dev.call("lg_attn_prefill_past_f16", dev.up(np.ascontiguousarray(q[:, :, past:]), 1), dev.up(kpad, 1), dev.up(vpad, 1), out,
+             B, S, past, h, d, kv_rows, float(scalar), causal, 1)
+    got = dev.down(out).transpose(0, 2, 1, 3)
+    assert max_rel_err(got, ref) < 4e-3
+    # past = 0 is the plain entry, bit for bit
+    a, b = dev.empty((B, L, h, d), 1), dev.empty((B, L, h, d), 1)
+    dq = dev.up(q, 1)
+    dev.call("lg_attn_prefill_past_f16", dq, dev.up(kpad, 1), dev.up(vpad, 1), a, B, L, 0, h, d, kv_rows, float(scalar), causal, 1)
+    dev.call("lg_attn_prefill_f16", dq, dev.up(kpad, 1), dev.up(vpad, 1), 0, b, B, L, h, d, kv_rows, float(scalar), causal, 1)
+    assert np.array_equal(dev.down(a), dev.down(b))
+    # more positions than the buffers hold are refused on the host
+    assert dev.call_rc("lg_attn_prefill_past_f16", dq, dq, dq, a, B, S, kv_rows - S + 1, h, d, kv_rows, float(scalar), causal, 1) == dev.capi.ERR_INVALID

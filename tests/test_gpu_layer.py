@@ -278,3 +278,47 @@ def test_packed_qkv_fused_layer_and_decode(dev, po, host, weight_layout, B, S):
     dt_in, dt_out = dev.up(tok, 1), dev.empty((B, H), 1)
     m.run_decode(dt_in.data_ptr(), dt_out.data_ptr(), B, S, 0, None, dev.stream)
     assert max_rel_err(dev.down(dt_out), po.decoder_step(shape, w, tok, kc, vc, S)) < 1e-2
+
+
+@pytest.mark.parametrize("weight_layout", [1, 2])
+@pytest.mark.parametrize("S,chunk", [(256, 64), (200, 96), (130, 128)])
+def test_chunked_prefill_equals_the_whole_prefill_and_the_oracle(dev, po, host, S, chunk, weight_layout):
+    """One sequence prefilled in chunks over its KV-cache slot (every chunk through both layers before the next): the hidden
+    states must equal the oracle's two stacked layers on the whole prompt, and the whole-prompt launch vector up to rounding;
+    the caches must end up the same, so that a decode step after either gives the same token."""
+    heads, d, F, layers, Lmax = 8, 128, 2048, 2, 320
+    H = heads * d
+    m = host.Model(1, 3, 256, heads, d, layer_num=layers, ffn_inner=F, causal=True, fused=True, max_cache_len=Lmax,
+                   weight_layout=weight_layout, seed=4)
+    P = m.download_params()
+    x = po.fill_normal(S * H, 4, 99, 0.0, 1.0, 1).reshape(S, H)
+    dx = dev.up(x, 1)
+    whole, parts = dev.empty((S, H), 1), dev.empty((S, H), 1)
+    m.run(dx.data_ptr(), whole.data_ptr(), 1, S, None, dev.stream, cache_slot=0)
+    m.run_chunked(dx.data_ptr(), parts.data_ptr(), S, chunk, 2, None, dev.stream)
+    shape = dict(batch=1, seq=S, hidden=H, head_num=heads, size_per_head=d, ffn_inner=F, causal=1, norm_mode=0, dtype=1)
+    ref = x
+    for l in range(layers):
+        w = {k[len("layer%d." % l):]: v for k, v in P.items() if k.startswith("layer%d." % l)}
+        ref = po.round_f16(po.encoder_forward(shape, w, ref))
+    got = dev.down(parts)
+    assert max_rel_err(got, ref) < 1e-2 and elementwise_err(got, ref) < 1e-2
+    assert max_rel_err(got, dev.down(whole)) < 4e-3
+    # the caches of both slots hold the same keys and values (up to rounding), in every layer
+    for l in range(layers):
+        pk, pv = m.kv_cache(l)
+        for ptr in (pk, pv):
+            c = dev.empty((3, heads, Lmax, d), 1)
+            dev.capi.call("lg_memcpy_d2d_async", c.data_ptr(), ptr, c.numel() * 2, None)
+            c = dev.down(c)
+            assert max_rel_err(c[2, :, :S], c[0, :, :S]) < 4e-3
+    # a decode step on top of the chunked prefill against the oracle's decoder step on the whole-prompt caches
+    tok = po.fill_normal(H, 4, 100, 0.0, 1.0, 1).reshape(1, H)
+    o = dev.empty((1, H), 1)
+    m.run_decode(dev.up(tok, 1).data_ptr(), o.data_ptr(), 1, S, 2, None, dev.stream)
+    o0 = dev.empty((1, H), 1)
+    m.run_decode(dev.up(tok, 1).data_ptr(), o0.data_ptr(), 1, S, 0, None, dev.stream)
+    assert max_rel_err(dev.down(o), dev.down(o0)) < 4e-3
+    # refusals: a chunked run needs a cache slot that holds the sequence
+    with pytest.raises(host.capi.LigerError):
+        m.run_chunked(dx.data_ptr(), parts.data_ptr(), S, chunk, -1, None, dev.stream)
