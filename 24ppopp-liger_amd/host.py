@@ -59,6 +59,8 @@ SIGNATURES = {
     "lgh_sched_set_contention": (_i, [_p, _i, _i, _f]),
     "lgh_sched_enable_partition": (_i, [_p, _i]),
     "lgh_sched_set_decode_step_hook": (_i, [_p, _p, _p]),
+    "lgh_sched_set_prefill_chunk": (_i, [_p, _i]),
+    "lgh_sched_chunk_counters": (_i, [_p, C.POINTER(_i)]),
     "lgh_sched_set_partition_feedback": (_i, [_p, _i, _i, _i, _f]),
     "lgh_sched_partition_feedback_state": (_i, [_p, C.POINTER(C.c_double)]),
     "lgh_sched_enable_batch_decode": (_i, [_p, _i, _i]),
@@ -376,6 +378,16 @@ class Scheduler:
     def enable_partition(self, hbm_cus):
         """Co-running rounds give the HBM-bound side `hbm_cus` compute units and the MFMA-bound side the rest (0 = off)."""
         check(lib.lgh_sched_enable_partition(self.h, hbm_cus), "lgh_sched_enable_partition")
+
+    def set_prefill_chunk(self, rows):
+        """With batched decode steps: single-sequence prompts longer than `rows` tokens are prefilled in chunks of `rows` over their
+        KV-cache slot and the batched decode step runs between two chunks (0 = off)."""
+        check(lib.lgh_sched_set_prefill_chunk(self.h, rows), "lgh_sched_set_prefill_chunk")
+
+    def chunk_counters(self):
+        out = (_i * 2)()
+        check(lib.lgh_sched_chunk_counters(self.h, out), "lgh_sched_chunk_counters")
+        return {"chunked_prefills": out[0], "yield_turns": out[1]}
 
     def set_partition_feedback(self, on, min_samples=0, probe=-1, margin=0.0):
         """While a run goes on, rounds that could be partitioned are run both ways and partitioned only while that delivers more

@@ -45,6 +45,8 @@ struct SchedBase {
     virtual float get_contention(int main_class, int sub_class) = 0;
     virtual bool streams_concurrent() = 0;
     virtual void set_merge_minor(bool on) = 0;
+    virtual void set_prefill_chunk(int rows) = 0;
+    virtual void chunk_counters(int* out2) = 0;
     virtual void set_partition_feedback(bool on, int min_samples, int probe, float margin) = 0;
     virtual void feedback_state(double* out5) = 0;
     virtual void set_decode_step_hook(void (*fn)(void*, int, int, const int*, const int*, void*, void*), void* user) = 0;
@@ -190,6 +192,8 @@ struct SchedT : SchedBase {
     }
     bool streams_concurrent() override { return s->DParams1.concurrent; }
     void set_merge_minor(bool on) override { s->merge_minor = on; }
+    void set_prefill_chunk(int rows) override { s->prefill_chunk = rows; }
+    void chunk_counters(int* out2) override { out2[0] = s->chunked_prefills; out2[1] = s->yield_turns; }
     void set_partition_feedback(bool on, int min_samples, int probe, float margin) override {
         s->partition_feedback = on;
         if (min_samples > 0) s->partition_feedback_min = min_samples;
@@ -604,6 +608,19 @@ int lgh_sched_set_contention(void* sched, int main_class, int sub_class, float v
 int lgh_sched_set_merge_minor(void* sched, int on) {
     if (!sched) return fail("lgh_sched_set_merge_minor: null");
     ((SchedBase*)sched)->set_merge_minor(on != 0);
+    return LG_OK;
+}
+// With batched decode steps: single-sequence prompts longer than `rows` tokens are prefilled in chunks of `rows`, and the batched
+// decode step runs between two chunks (Scheduler::prefill_chunk).  0 switches it off.
+int lgh_sched_set_prefill_chunk(void* sched, int rows) {
+    if (!sched || rows < 0) return fail("lgh_sched_set_prefill_chunk: bad arguments");
+    ((SchedBase*)sched)->set_prefill_chunk(rows);
+    return LG_OK;
+}
+// out2 = {requests of the last run whose prefill was cut into chunks, turns given to the batched decode step between chunks}
+int lgh_sched_chunk_counters(void* sched, int* out2) {
+    if (!sched || !out2) return fail("lgh_sched_chunk_counters: bad arguments");
+    ((SchedBase*)sched)->chunk_counters(out2);
     return LG_OK;
 }
 // Whether partitioned rounds are checked against whole-chip rounds while a run goes on (Scheduler::partition_feedback; on by

@@ -185,6 +185,9 @@ class FuncWrap {
     // a small kernel between the big ones of its layer (normalisation, residual, cache append, row gather): a scheduler that
     // is told to merge minor entries lets it take the scheduling class of the entry before it
     bool minor = false;
+    // the primary's round ends behind this entry even though the next one has the same class: the end of a chunk of a long
+    // prefill, where the scheduler may give the turn to the decode steps of other requests (no reference counterpart)
+    bool yield_after = false;
     const char* label = "";
 
     FuncWrap() {}

@@ -89,6 +89,7 @@ class Sample {
     int key_seq = 0;            // seq_len on the profile grid (set by the scheduler; seq_len when there is no grid)
     int sub_profile_misses = 0; // GEMMs that could not be split because the decomposition table has no entry for them
     int id = 0;
+    bool chunked = false;       // the launch vector is a prefill cut into chunks (entries with yield_after mark their ends)
     int n_decode_pending = 0;   // decode steps the owner still has to run for this request once the prefill vector is done
     bool merge_minor = false;  // see _neutral(); false = every entry keeps its own class (the reference's behaviour)
     void* user = nullptr;  // owner's per-request context (buffers), opaque here
@@ -127,9 +128,13 @@ class Sample {
     int next_class() const { return _sub_empty() ? _class_at(exe_num) : _class_of(_SubFuncWrapVec[_sub_exe_num].func); }
     layer_type type() const { return _sub_empty() ? FuncWrapVec.at(exe_num).type : GEMM; }  // init.h:151-157
 
+    // the next launch is marked as the end of a chunk (FuncWrap::yield_after); marked entries are never decomposed
+    bool next_yields() const { return _sub_empty() && !main_empty() && FuncWrapVec[exe_num].yield_after; }
+
     // true when the next launch is the last of a run of same-class launches  (init.h:99-129)
     bool is_switch() const {
         if (next_empty()) return true;
+        if (next_yields()) return true;
         if (_sub_empty()) return _class_at(exe_num) != _class_at(exe_num + 1);
         if (_sub_size() >= 2) return false;  // next two launches are pieces of the same GEMM
         const size_t after = (_sub_exe_num > 0) ? exe_num : exe_num + 1;

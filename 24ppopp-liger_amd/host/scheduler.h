@@ -158,6 +158,11 @@ class Scheduler {
     // prefill.  No reference counterpart (the reference has no
     // decode phase); without it every request runs its own decode steps, as in run_sequential.
     bool batch_decode = false;
+    // With batched decode steps: a single-sequence prompt longer than prefill_chunk tokens is prefilled in chunks of that many
+    // (each chunk through all layers, over the request's KV-cache slot), and after every chunk the batched decode step gets the
+    // primary's turn once, so that requests in their decode steps wait for a chunk, not for a whole prompt.  0 = off.
+    int prefill_chunk = 0;
+    int chunked_prefills = 0, yield_turns = 0;   // requests whose prefill was cut into chunks; turns given to the decode batch
     int decode_steps_ahead = 4;       // steps per batched launch vector while nothing waits to join (1 otherwise)
     int batched_steps = 0, batched_rows = 0;   // steps launched, and token rows they carried (holes included)
     // Called by the scheduler thread right after the kernels of every batched decode step have been launched, as an entry of
@@ -600,14 +605,32 @@ class Scheduler {
         T* ws = ctx ? ctx->ws : nullptr;
         const int slot = (ctx && BertParams.max_cache_len > 0) ? ctx->slot : -1;
         std::unique_lock<std::mutex> build_lock(_build_mutex);  // the layer classes keep per-call state: one builder at a time
-        std::vector<FuncWrap> vec = _model->forward(in, out, batch_size, seq_len, ws, slot);
-        for (int i = 0; i < BertParams.layer_num; i++)
-            for (int j = 0; j < BertParams.kernel_num; j++) {
-                FuncWrap& f = vec[i * BertParams.kernel_num + j];
-                f.name = j;
-                f.duration = lookup(j, batch_size, seq_len);
-            }
         const bool defer_decode = batch_decode && n_decode > 0 && ctx && slot >= 0;  // the decode steps join the batched launch vector
+        const bool chunked = defer_decode && prefill_chunk > 0 && batch_size == 1 && seq_len > prefill_chunk && BertParams.fused;
+        std::vector<FuncWrap> vec;
+        int key_len = seq_len;
+        if (chunked) {
+            const int H = BertParams.head_num * BertParams.size_per_head;
+            for (int p0 = 0; p0 < seq_len; p0 += prefill_chunk) {
+                const int c = std::min(prefill_chunk, seq_len - p0);
+                std::vector<FuncWrap> cv = _model->forward_prefill_past(in + (int64_t)p0 * H, out + (int64_t)p0 * H, 1, c, p0, ws, slot);
+                for (size_t j = 0; j < cv.size(); ++j) {
+                    cv[j].name = (int)(j % (size_t)BertParams.kernel_num);
+                    cv[j].duration = lookup(cv[j].name, 1, c);
+                }
+                if (p0 + c < seq_len && !cv.empty()) cv.back().yield_after = true;
+                vec.insert(vec.end(), cv.begin(), cv.end());
+            }
+            key_len = prefill_chunk;
+        } else {
+            vec = _model->forward(in, out, batch_size, seq_len, ws, slot);
+            for (int i = 0; i < BertParams.layer_num; i++)
+                for (int j = 0; j < BertParams.kernel_num; j++) {
+                    FuncWrap& f = vec[i * BertParams.kernel_num + j];
+                    f.name = j;
+                    f.duration = lookup(j, batch_size, seq_len);
+                }
+        }
         if (n_decode > 0 && ctx && slot >= 0 && !defer_decode) {
             const int H = BertParams.head_num * BertParams.size_per_head;
             const int kd = _model->kernels_per_layer(true);
@@ -643,8 +666,9 @@ class Scheduler {
         Sample* sample = new Sample(vec, profiling_decompse_res_dict, batch_size, seq_len, BertParams.factor, policy, axis);
         sample->user = ctx;
         sample->merge_minor = merge_minor;
-        sample->key_seq = seq_bucket > 1 ? (seq_len + seq_bucket - 1) / seq_bucket * seq_bucket : seq_len;
+        sample->key_seq = seq_bucket > 1 ? (key_len + seq_bucket - 1) / seq_bucket * seq_bucket : key_len;  // chunks: a chunk's GEMMs are what gets split
         sample->n_decode_pending = defer_decode ? n_decode : 0;
+        sample->chunked = chunked;
         {
             std::lock_guard<std::mutex> lk(_q_mutex);
             sample->id = _next_id++;
@@ -714,6 +738,7 @@ class Scheduler {
             if (_main_q.empty()) break;
             // the batched decode step stays last: a request's prefill goes ahead of it (the request then joins the batch)
             exe_vec.insert(_dec_sample ? exe_vec.end() - 1 : exe_vec.end(), _main_q.front());
+            if (_main_q.front()->chunked) chunked_prefills++;
             _main_q.pop_front();
         }
         if (exe_vec.empty()) std::this_thread::sleep_for(std::chrono::microseconds(100));
@@ -730,7 +755,15 @@ class Scheduler {
             update_vec();
             if (!exe_vec.empty()) {
                 note_status(lg_event_synchronize(Wait_EVENT), "lg_event_synchronize");
-                while (!exe_vec.at(0)->empty()) exe_vec.at(0)->dequeue(DParams0, 1, time_planned);
+                // one request at a time, to its end -- or to the end of a chunk of a chunked prefill, after which the batched
+                // decode step (if there is one) has its turn before the next chunk
+                Sample* cur = _pick_head();
+                bool yielded = false;
+                while (!cur->empty() && !yielded) {
+                    yielded = cur->next_yields();
+                    cur->dequeue(DParams0, 1, time_planned);
+                }
+                _yield_turn = yielded;
                 note_status(lg_event_record(Wait_EVENT, DParams0.stream), "lg_event_record");
                 rounds++;
             }
@@ -754,7 +787,7 @@ class Scheduler {
         while (!(_stop.load() && drained())) {
             update_vec();
             if (exe_vec.empty()) continue;
-            Sample* head = exe_vec.at(0);
+            Sample* head = _pick_head();
             // Partitioned round?  Only while a waiting request has work of the other class at its head, and only for as much
             // primary time as that work needs; the primary then runs on its class's share of the compute units, the
             // secondaries on the other share.  Otherwise (and always without enable_partition) the round is the reference's:
@@ -768,8 +801,8 @@ class Scheduler {
                 const int sc = mc == MFMA_BOUND ? HBM_BOUND : (mc == HBM_BOUND ? MFMA_BOUND : -1);
                 if (sc >= 0 && partition_table[mc][sc] > 0.f) {
                     float need = 0.f;
-                    for (size_t s = 1; s < exe_vec.size(); s++)
-                        if (!exe_vec[s]->empty()) need += exe_vec[s]->run_ahead_duration(mc);
+                    for (Sample* other : exe_vec)
+                        if (other != head && !other->empty()) need += other->run_ahead_duration(mc);
                     if (need >= partition_min_ms) {
                         round_kind = _partition_pays() ? 2 : 1;
                         if (round_kind == 2) {
@@ -794,6 +827,7 @@ class Scheduler {
                 main_class = head->next_class();
                 const bool capped = part_factor > 0.f && time_planned + head->duration(1, time_planned) >= cap;
                 if (head->is_switch() || capped) {
+                    _yield_turn = head->next_yields();
                     note_status(lg_event_record(Wait_EVENT, Dp->stream), "lg_event_record");
                     time_planned += head->dequeue(*Dp, 1, time_planned);
                     note_status(lg_event_record(Main_EVENT, Dp->stream), "lg_event_record");
@@ -805,8 +839,8 @@ class Scheduler {
             rounds++;
             // time_planned stays in units of the primary's time; a secondary kernel of stand-alone duration d uses up
             // d / contention(main, sub) of it (with the constant factor this is the reference's 0.8 x time_planned budget)
-            for (size_t s = 1; s < exe_vec.size(); s++) {
-                Sample* sub = exe_vec.at(s);
+            for (Sample* sub : exe_vec) {
+                if (sub == head) continue;
                 while (time_planned > 0 && !sub->empty()) {
                     if (sub->is_same_class(main_class)) break;
                     const float f = part_factor > 0.f ? part_factor : contention(main_class, sub->next_class());
@@ -852,6 +886,8 @@ class Scheduler {
         if (_dec_prev_stop) { lg_event_destroy(_dec_prev_stop); _dec_prev_stop = nullptr; }
         batched_steps = batched_rows = 0;
         rounds = secondary_launches = splits = partition_rounds = partition_declined = 0;
+        chunked_prefills = yield_turns = 0;
+        _yield_turn = false;
         // what the rounds of earlier runs delivered is kept (it is a property of the device and the workload, and a run may have
         // few rounds in which a partition is possible); older samples count half at every new run
         for (RoundRec& r : _round_log) _round_events.push_back(r.begin);
@@ -1109,6 +1145,18 @@ class Scheduler {
     std::vector<void*> _dec_prefill_events;  // destroyed with the run's records
     void* _dec_prev_stop = nullptr;          // stop event of the previous vector of batched steps
 
+    // The primary of the next round: the first request in line -- or, right after a chunk of a chunked prefill, the batched
+    // decode step once (if it has launches left), so that the requests in their decode steps advance between two chunks.
+    bool _yield_turn = false;
+    Sample* _pick_head() {
+        Sample* head = exe_vec.at(0);
+        if (_yield_turn && _dec_sample && head != _dec_sample && !_dec_sample->empty()) {
+            head = _dec_sample;
+            yield_turns++;
+        }
+        _yield_turn = false;
+        return head;
+    }
     std::atomic<bool> _running{false};
     std::vector<ReqCtx*> _held;   // contexts of finished requests kept back while recycle_contexts is off
     int _ctx_batch = 0;

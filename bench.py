@@ -216,7 +216,7 @@ def bench_cfg5(capi, host, weight_layout, n_requests, rates=(4.0, 8.0, 16.0, 24.
     sched = host.Scheduler(model, schedule_deep=6, contention_factor=0.8, policy=host.POLICY_RESOURCE, axis=host.SPLIT_TOKEN_ROWS,
                            seq_bucket=64, ignore_num=5, pool_count=pool, ctx_batch=1)
     t0 = time.perf_counter()
-    sched.profile(1, 128, 1024, 64, 5)
+    sched.profile(1, 64, 1024, 64, 5)     # from 64 tokens: the last chunk of a chunked prefill may be that short
     for past in range(128, 1024 + 64 + 1, 64):
         sched.profile_decode(1, min(past, 1024 + 63), 5)
     # batched decode steps: a few batch sizes on a coarser grid of cached positions (looked up at or below the batch)
@@ -250,6 +250,12 @@ def bench_cfg5(capi, host, weight_layout, n_requests, rates=(4.0, 8.0, 16.0, 24.
     for share in shares:
         if part_factor[share][0] > 0:
             modes.append((host.MODE_LIGER, "scheduling_on_batched_decode_partitioned_%d_hbm_cus" % share, False, True, share, True))
+    # prompts longer than 256 (512) tokens prefilled in chunks of that many, the batched decode step taking the turn between two
+    # chunks (full sweep only)
+    if not short:
+        for chunk in (256, 512):
+            modes.append((host.MODE_SEQUENTIAL, "batched_decode_chunked_prefill_%d_without_interleaving" % chunk, False, True, 0, chunk))
+            modes.append((host.MODE_LIGER, "scheduling_on_batched_decode_chunked_prefill_%d" % chunk, False, True, 0, chunk))
     out = []
     for lam in rates:
         trace = host.make_poisson_trace(lam, n_requests, 1, 128, 1024, 64, 32, 0)
@@ -258,11 +264,14 @@ def bench_cfg5(capi, host, weight_layout, n_requests, rates=(4.0, 8.0, 16.0, 24.
             sched.set_contention(0, 1, table["mfma_main_hbm_sub"] if measured else -1.0)
             sched.set_contention(1, 0, table["hbm_main_mfma_sub"] if measured else -1.0)
             sched.set_merge_minor(merge_minor)
-            sched.enable_batch_decode(batched, decode_steps_ahead)
+            sched.enable_batch_decode(bool(batched), decode_steps_ahead)
+            sched.set_prefill_chunk(batched if batched not in (True, False) else 0)
             sched.enable_partition(share)
             if share:
                 sched.set_partition_factor(0, 1, part_factor[share][0])
                 sched.set_partition_factor(1, 0, part_factor[share][1])
+            if share:
+                sched.run_trace(trace, mode)   # untimed: the partition feedback settles on what this workload's rounds deliver
             reps = [sched.run_trace(trace, mode) for _ in range(runs)]
             r = reps[0]
             print("cfg5: lambda %.0f %s: mean %.2f ms" % (lam, name, sum(x["avg_e2e_ms"] for x in reps) / len(reps)), file=sys.stderr, flush=True)
@@ -277,10 +286,11 @@ def bench_cfg5(capi, host, weight_layout, n_requests, rates=(4.0, 8.0, 16.0, 24.
                          "secondary_launches": r["secondary_launches"], "splits": r["splits"], "profile_misses": r["profile_misses"],
                          "partition_rounds": r["partition_rounds"],
                          "partition_feedback": sched.partition_feedback_state() if share else None,
-                         "batched_steps": r["batched_steps"],
+                         "batched_steps": r["batched_steps"], "chunking": sched.chunk_counters() if batched not in (True, False) else None,
                          "rows_per_batched_step": round(r["batched_rows"] / r["batched_steps"], 2) if r["batched_steps"] else None}
         out.append(row)
     sched.enable_partition(0)
+    sched.set_prefill_chunk(0)
     sched.enable_batch_decode(False)
     concurrent = sched.streams_concurrent
     sched.close()

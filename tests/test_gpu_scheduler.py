@@ -136,6 +136,60 @@ def test_batched_decode_equals_every_request_on_its_own(dev, host, mode, partiti
     print("free-running batched decode vs. per-request steps: worst max-rel %.3g" % worst)
 
 
+@pytest.mark.parametrize("mode", [0, 1])
+def test_chunked_prefills_between_batched_decode_steps_equal_every_request_on_its_own(dev, host, mode):
+    """Prompts longer than prefill_chunk are prefilled in chunks over their cache slots, with the batched decode step taking the
+    turn between two chunks: every request must still end with the hidden state it gets when it runs alone (whole-prompt
+    prefill, then its decode steps one by one).  Chunks change the summation order of the attention (another split of the
+    keys into tiles of the online softmax), and batched steps that of the decode GEMMs: a fixed 2e-2 bounds the free-running
+    drift over up to 10 steps x 2 layers, as in the unchunked test."""
+    heads, d, F, layers, pool = 8, 128, 2048, 2, 6
+    H = heads * d
+    m = host.Model(1, pool + 1, 128, heads, d, layer_num=layers, ffn_inner=F, causal=True, fused=True, max_cache_len=192, factor=4,
+                   weight_layout=2, seed=5)
+    s = host.Scheduler(m, policy=host.POLICY_RESOURCE, axis=host.SPLIT_TOKEN_ROWS, seq_bucket=16, ignore_num=0, pool_count=pool, ctx_batch=1)
+    s.profile(1, 16, 128, 16, 3)
+    for bs in (1, 2, 4, 6):
+        for past in (32, 64, 96, 128, 160):
+            s.profile_decode(bs, past, 3)
+    s.set_merge_minor(True)
+    s.enable_batch_decode(True, 2)
+    s.set_prefill_chunk(48)
+    reqs = [(1, 96, 7), (1, 33, 10), (1, 128, 3), (1, 64, 9), (1, 50, 1), (1, 120, 10)]
+    for r in reqs:
+        s.serve(*r)
+    rep = s.run_queued(host.MODE_LIGER if mode else host.MODE_SEQUENTIAL)
+    torch.cuda.synchronize()
+    cc = s.chunk_counters()
+    assert rep["records"] == len(reqs) and cc["chunked_prefills"] == 5 and cc["yield_turns"] > 0
+    worst = 0.0
+    for i, (_, S, n) in enumerate(reqs):
+        pin, pout = s.ctx_ptrs(i)
+        da, db = s.ctx_decode_ptrs(i)
+        got = torch.empty(H, device="cuda", dtype=torch.float16)
+        dev.capi.call("lg_memcpy_d2d_async", got.data_ptr(), db if n % 2 else da, H * 2, None)
+        y = torch.empty(S, H, device="cuda", dtype=torch.float16)
+        torch.cuda.synchronize()
+        # the prompt's hidden states, as the scheduler left them, against the whole-prompt prefill
+        mine = _read(dev, pout, S * H).reshape(S, H)
+        m.run(pin, y.data_ptr(), 1, S, None, None, cache_slot=i)
+        torch.cuda.synchronize()
+        e_pre = float((mine - y.float()).abs().max() / y.float().abs().max())
+        assert e_pre < 4e-3, "request %d: chunked prefill differs from the whole-prompt prefill (%g)" % (i, e_pre)
+        a = y[S - 1:S].clone()
+        b = torch.empty_like(a)
+        for t in range(n):
+            m.run_decode(a.data_ptr(), b.data_ptr(), 1, S + t, i, None, None)
+            a, b = b, a
+        torch.cuda.synchronize()
+        ref = a[0].float()
+        err = float((got.float() - ref).abs().max() / ref.abs().max())
+        worst = max(worst, err)
+        assert err < 2e-2, "request %d (prompt %d, %d steps): max rel err %g" % (i, S, n, err)
+    print("chunked prefills + batched decode vs. per-request runs: worst max-rel %.3g" % worst)
+    s.close()
+
+
 @pytest.mark.parametrize("weight_layout", [0, 1, 2])
 @pytest.mark.parametrize("mode", [0, 1])
 def test_batched_decode_steps_teacher_forced_against_the_oracle(dev, po, host, mode, weight_layout):

@@ -798,6 +798,63 @@ def test_every_batched_step_carries_each_live_request_at_its_own_position(fake, 
     s.close()
 
 
+@pytest.mark.parametrize("mode_name", ["sequential", "liger"])
+def test_chunked_prefill_lets_the_decode_batch_step_between_chunks(fake, mode_name):
+    """Request A (prompt 32, 12 decode tokens) is in its decode steps when request B (prompt 128) has its prefill.  With
+    prefill_chunk = 32 B's prefill is four chunks of 32 tokens, each through both layers over B's cache slot: the attention of
+    chunk c is the continuing kind with past = 32 c, every other kernel works on 32 token rows, and between two chunks the
+    batched decode step gets the primary's turn.  Without chunking B's prefill is one vector of 128-token kernels."""
+    host = fake.host
+    pool = 3
+    m = host.Model(1, pool + 1, 128, 4, 64, layer_num=2, ffn_inner=512, causal=True, fused=True, max_cache_len=192, factor=4, seed=0)
+    s = host.Scheduler(m, contention_factor=0.8, policy=host.POLICY_RESOURCE, seq_bucket=32, pool_count=pool, ctx_batch=1)
+    s.profile(1, 32, 128, 32, 2)
+    for bs in (1, 2):
+        for past in (32, 64, 128, 160):
+            s.profile_decode(bs, past, 2)
+    s.set_merge_minor(True)
+    s.enable_batch_decode(True, 1)
+    mode = host.MODE_LIGER if mode_name == "liger" else host.MODE_SEQUENTIAL
+
+    def run(chunk):
+        s.set_prefill_chunk(chunk)
+        fake.reset()
+        s.serve(1, 32, 12)      # A: as long as a chunk, so never cut
+        s.serve(1, 128, 3)      # B
+        r = s.run_queued(mode)
+        assert r["records"] == 2 and r["profile_misses"] == 0
+        return r, fake.trace(), s.chunk_counters()
+
+    r0, t0, c0 = run(0)
+    assert c0 == {"chunked_prefills": 0, "yield_turns": 0}
+    assert not [e for e in t0 if e["name"] == "attn_prefill_past"]
+    assert sorted(e["n"] for e in t0 if e["name"] == "attn_prefill") == [32, 32, 128, 128]
+    r1, t1, c1 = run(32)
+    assert c1["chunked_prefills"] == 1 and c1["yield_turns"] >= 2
+    # B's chunks: one plain attention (past 0) and three continuing ones per layer, pasts 32, 64, 96, each over 32 queries
+    past_attn = [e for e in t1 if e["name"] == "attn_prefill_past"]
+    assert [(e["n"], e["k"]) for e in past_attn] == [(32, p) for p in (32, 32, 64, 64, 96, 96)]
+    assert sorted(e["n"] for e in t1 if e["name"] == "attn_prefill") == [32, 32, 32, 32]     # A's two layers, B's first chunk
+    # nothing of B works on 128 token rows any more (GEMMs: n = token rows; LayerNorm: m)
+    assert not [e for e in t1 if (e["name"] in ("gemm", "gemm_fused") and e["n"] == 128) or (e["name"] == "layer_norm" and e["m"] == 128)]
+    # every decode step of A and B is still there
+    assert len([e for e in t1 if e["name"] == "attn_decode_varlen"]) == len([e for e in t0 if e["name"] == "attn_decode_varlen"])
+    # between two consecutive chunks of B at least one batched decode step was launched (A is decoding all the while)
+    marks = [i for i, e in enumerate(t1) if e["name"] == "attn_prefill_past"][::2]     # layer 0 of chunks 1, 2, 3
+    assert len(marks) == 3
+    for a, b in zip(marks, marks[1:]):
+        assert any(e["name"] == "attn_decode_varlen" for e in t1[a:b]), "no decode step between two chunks"
+
+    if mode_name == "sequential":
+        # A's first decode steps no longer wait for the whole of B's prefill, only for its first chunk
+        first = lambda t, k: [e["start"] for e in t if e["name"] == "attn_decode_varlen"][2 * k]
+        b_done = lambda t: max(e["end"] for e in t if e["name"] in ("attn_prefill", "attn_prefill_past"))
+        assert first(t0, 0) > b_done(t0)                 # unchunked: every decode step comes after B's last attention
+        assert first(t1, 0) < 0.5 * first(t0, 0) and first(t1, 2) < b_done(t1)
+    s.set_prefill_chunk(0)
+    s.close()
+
+
 @pytest.mark.parametrize("factor", [2, 4, 8])
 @pytest.mark.parametrize("axis", [0, 1])
 def test_cfg4_shapes_pieces_cover_the_prefill_exactly(fake, factor, axis):
