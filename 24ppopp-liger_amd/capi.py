@@ -34,6 +34,7 @@ SIGNATURES = {
     "lg_stream_cu_count": (_i, [_p]),
     "lg_stream_create_cu_mask": (_i, [C.POINTER(_p), C.POINTER(C.c_uint), _i]),
     "lg_stream_create_concurrent": (_i, [_p, _p, _p]),
+    "lg_streams_run_concurrently": (_i, [_p, _p, _p]),
     "lg_stream_destroy": (_i, [_p]),
     "lg_stream_synchronize": (_i, [_p]),
     "lg_stream_wait_event": (_i, [_p, _p]),

@@ -332,6 +332,14 @@ int lg_stream_create_concurrent(void** stream, void* other, int* verified) {
     *stream = (void*)cand[pick];
     return register_stream(*stream, 0);
 }
+int lg_streams_run_concurrently(void* a, void* b, int* concurrent) {
+    if (!a || !b || a == b || !concurrent) { set_error("lg_streams_run_concurrently: needs two different created streams"); return LG_ERR_INVALID; }
+    bool ok = false;
+    const bool conc = runs_concurrently((hipStream_t)a, (hipStream_t)b, &ok);
+    if (!ok) { set_error("lg_streams_run_concurrently: the concurrency probe failed"); return LG_ERR_LAUNCH; }
+    *concurrent = conc ? 1 : 0;
+    return LG_OK;
+}
 int lg_stream_destroy(void* stream) {
     const int rc = unregister_stream(stream);
     const int rc2 = rt(hipStreamDestroy((hipStream_t)stream), "hipStreamDestroy");

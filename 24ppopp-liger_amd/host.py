@@ -40,6 +40,7 @@ SIGNATURES = {
     "lgh_model_workspace_elems": (_i64, [_p, _i, _i]),
     "lgh_model_stream": (_p, [_p]),
     "lgh_model_param_count": (_i, [_p]),
+    "lgh_model_load_param": (_i, [_p, _i, _p, _i, _p]),
     "lgh_model_param_info": (_i, [_p, _i, C.c_char_p, _i, C.POINTER(_p), C.POINTER(_i64), C.POINTER(_i), C.POINTER(_i), C.POINTER(_i)]),
     "lgh_model_kv_cache": (_i, [_p, _i, C.POINTER(_p), C.POINTER(_p)]),
     "lgh_model_describe": (_i, [_p, _i, _i, _i, C.c_char_p, _i]),
@@ -71,6 +72,8 @@ SIGNATURES = {
     "lgh_sched_get_partition_factor": (_f, [_p, _i, _i]),
     "lgh_sched_get_contention": (_f, [_p, _i, _i]),
     "lgh_sched_streams_concurrent": (_i, [_p]),
+    "lgh_sched_partition_streams_concurrent": (_i, [_p]),
+    "lgh_sched_set_verify_partition_streams": (_i, [_p, _i]),
     "lgh_sched_set_merge_minor": (_i, [_p, _i]),
     "lgh_sched_save": (_i, [_p, C.c_char_p, C.c_char_p]),
     "lgh_sched_load": (_i, [_p, C.c_char_p, C.c_char_p]),
@@ -239,6 +242,16 @@ class Model:
                 a = a[..., _interleave16(a.shape[-1], inverse=True)]
             res[name] = np.ascontiguousarray(a)
         return res
+
+    def load_param(self, name, device_ptr, src_layout, stream=None):
+        """Takes parameter `name` over from device memory: a plain row-major array, weight matrices [in, out] (src_layout 0)
+        or [out, in] (1), vectors flat.  The layer re-lays it into its own storage layout on the device (asynchronous on
+        `stream`, default the model's)."""
+        names = list(self.param_info().keys())
+        if name not in names:
+            raise KeyError("no parameter named %r" % name)
+        check(lib.lgh_model_load_param(self.h, names.index(name), _p(device_ptr), int(src_layout), _p(stream) if stream else None),
+              "lgh_model_load_param")
 
     def upload_params(self, values):
         """Overwrites parameters with host values: name -> array in the logical orientation download_params returns
@@ -429,6 +442,17 @@ class Scheduler:
     def streams_concurrent(self):
         """True when the second stream was verified (by measurement) to execute at the same time as the first."""
         return bool(lib.lgh_sched_streams_concurrent(self.h))
+
+    @property
+    def partition_streams_concurrent(self):
+        """True when the CU-masked streams of the share in use were measured to overlap pair by pair (primary, secondary),
+        False when a pair could not be made to, None when they were not probed."""
+        v = lib.lgh_sched_partition_streams_concurrent(self.h)
+        return None if v < 0 else bool(v)
+
+    def set_verify_partition_streams(self, on):
+        """enable_partition probes the stream pairs of a share it creates and replaces secondaries that take turns (off by default)."""
+        check(lib.lgh_sched_set_verify_partition_streams(self.h, int(bool(on))), "lgh_sched_set_verify_partition_streams")
 
     def save(self, main_file, sub_file):
         check(lib.lgh_sched_save(self.h, main_file.encode(), sub_file.encode()), "lgh_sched_save")

@@ -44,6 +44,8 @@ struct SchedBase {
     virtual bool set_contention(int main_class, int sub_class, float v) = 0;
     virtual float get_contention(int main_class, int sub_class) = 0;
     virtual bool streams_concurrent() = 0;
+    virtual int partition_streams_concurrent() = 0;
+    virtual void set_verify_partition_streams(bool on) = 0;
     virtual void set_merge_minor(bool on) = 0;
     virtual void set_prefill_chunk(int rows) = 0;
     virtual void chunk_counters(int* out2) = 0;
@@ -191,6 +193,8 @@ struct SchedT : SchedBase {
         return n;
     }
     bool streams_concurrent() override { return s->DParams1.concurrent; }
+    int partition_streams_concurrent() override { return s->partition_hbm_cus > 0 ? s->partition_streams_concurrent : -1; }
+    void set_verify_partition_streams(bool on) override { s->verify_partition_streams = on; }
     void set_merge_minor(bool on) override { s->merge_minor = on; }
     void set_prefill_chunk(int rows) override { s->prefill_chunk = rows; }
     void chunk_counters(int* out2) override { out2[0] = s->chunked_prefills; out2[1] = s->yield_turns; }
@@ -366,6 +370,40 @@ int lgh_model_param_info(void* model, int idx, char* name, int name_len, void** 
     if (rows) *rows = ps[idx].rows;
     if (cols) *cols = ps[idx].cols;
     if (transposed) *transposed = ps[idx].transposed;
+    return LG_OK;
+}
+
+// Takes a parameter over from device memory the caller owns: `src` holds parameter `idx` as a plain row-major array, weight
+// matrices either [in, out] (src_layout 0: what the reference's (N,N) cuBLAS call implies, linear.h:47-49,99-101) or [out, in]
+// (src_layout 1), vectors flat.  The layer re-lays it into its own storage layout on the device (one kernel on `stream`, null =
+// the model's stream; nothing is allocated, the caller synchronises): a copy when the layouts agree, a transpose between the
+// two plain layouts, lg_weight_tile_f16 for a layer that stores fragment blocks.  So a model whose weights arrive [in, out]
+// runs at the speed of the layout its kernels read fastest.  Parameters stored with interleaved halves (fused GeGLU FFN-1)
+// are refused: their order is private to the layer and they are written through the host (upload in logical order).
+int lgh_model_load_param(void* model, int idx, const void* src, int src_layout, void* stream) {
+    ModelBase* mb = (ModelBase*)model;
+    if (!mb || !src) return fail("lgh_model_load_param: null model or source");
+    if (src_layout != 0 && src_layout != 1) return fail("lgh_model_load_param: src_layout must be 0 ([in, out]) or 1 ([out, in])");
+    auto ps = mb->params();
+    if (idx < 0 || idx >= (int)ps.size()) return fail("lgh_model_load_param: index out of range");
+    const ParamRef& p = ps[idx];
+    if (p.transposed & 2) return fail(("lgh_model_load_param: " + p.name + " is stored with interleaved halves; upload it in logical order through the host").c_str());
+    if (src == p.ptr) return fail("lgh_model_load_param: the source is the parameter itself");
+    void* st = stream ? stream : mb->stream0->stream;
+    const size_t es = mb->elem_size();
+    int rc;
+    if (p.rows <= 1) {
+        rc = lg_memcpy_d2d_async(p.ptr, src, (size_t)p.elems * es, st);
+    } else if (p.transposed & 4) {   // fragment blocks of the [out, in] matrix (fp16 by construction)
+        rc = lg_weight_tile_f16(p.ptr, src, p.cols, p.rows, src_layout, src_layout ? p.rows : p.cols, st);
+    } else if ((p.transposed & 1) == src_layout) {
+        rc = lg_memcpy_d2d_async(p.ptr, src, (size_t)p.elems * es, st);
+    } else {
+        // [a, b] -> [b, a]: the head transpose [1, a, b, 1] -> [1, b, a, 1]
+        const int a = src_layout ? p.cols : p.rows, b = src_layout ? p.rows : p.cols;
+        rc = es == 2 ? lg_transpose_f16(p.ptr, src, 1, b, a, 1, st) : lg_transpose_f32((float*)p.ptr, (const float*)src, 1, b, a, 1, st);
+    }
+    if (rc != LG_OK) { note_status(rc, "lgh_model_load_param"); return rc; }
     return LG_OK;
 }
 
@@ -647,6 +685,15 @@ int lgh_sched_set_decode_step_hook(void* sched, void (*fn)(void*, int, int, cons
 }
 // 1 when the scheduler's second stream was verified to execute at the same time as the first
 int lgh_sched_streams_concurrent(void* sched) { return (sched && ((SchedBase*)sched)->streams_concurrent()) ? 1 : 0; }
+// 1 when both (primary, secondary) pairs of CU-masked streams of the share in use were measured to overlap, 0 when a pair could
+// not be made to, -1 when they were not probed (no share in use, or verification off when the share's streams were created)
+int lgh_sched_partition_streams_concurrent(void* sched) { return sched ? ((SchedBase*)sched)->partition_streams_concurrent() : -1; }
+// Whether enable_partition probes the stream pairs of a share it creates (and replaces secondaries that take turns)
+int lgh_sched_set_verify_partition_streams(void* sched, int on) {
+    if (!sched) return fail("lgh_sched_set_verify_partition_streams: null scheduler");
+    ((SchedBase*)sched)->set_verify_partition_streams(on != 0);
+    return LG_OK;
+}
 float lgh_sched_get_contention(void* sched, int main_class, int sub_class) {
     return sched ? ((SchedBase*)sched)->get_contention(main_class, sub_class) : -1.f;
 }

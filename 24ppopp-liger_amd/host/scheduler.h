@@ -186,10 +186,12 @@ class Scheduler {
     // partition_feedback_min samples; from then on they are partitioned only while the partitioned rounds' rate is at least
     // partition_feedback_margin times the whole-chip rounds', and every partition_feedback_probe-th such round takes the other
     // side so that both figures stay current.  The figures carry over from run to run (older samples at half weight) until the
-    // share changes.  No reference counterpart.
+    // share changes.  The margin is well above 1 because the estimate flatters partitioned rounds (see _round_begin): measured
+    // ratios of 1.02-1.05 went with mean latencies 0.2-1.5 % behind the unpartitioned run's, ratios of 1.37-1.39 with gains.
+    // No reference counterpart.
     bool partition_feedback = true;
-    int partition_feedback_min = 6, partition_feedback_probe = 16;
-    float partition_feedback_margin = 1.02f;
+    int partition_feedback_min = 6, partition_feedback_probe = 32;
+    float partition_feedback_margin = 1.08f;
     int partition_declined = 0;       // rounds that could have been partitioned and were run on the whole chip instead
     void reset_partition_feedback() {
         for (int k = 0; k < 3; ++k) { _fb_work[k] = _fb_time[k] = 0; _fb_n[k] = 0; }
@@ -275,8 +277,35 @@ class Scheduler {
                         if (ps.d[role][cls]) ps.d[role][cls]->destroy();
                 return false;
             }
+            // The two streams of a partitioned round must sit on different hardware queues, or their kernels run strictly in
+            // turn and the round is a slower sequential one.  Each (primary, secondary) pair of different classes is probed; a
+            // secondary that runs in turn with its primary is replaced, the rejected candidates kept alive meanwhile so that the
+            // next one is handed another queue.
+            ps.verified = -1;
+            if (verify_partition_streams) ps.verified = 1;
+            for (int mc = 0; mc < 2 && verify_partition_streams && !first_error(); ++mc) {
+                const int sc = 1 - mc;
+                std::vector<std::unique_ptr<DynamicInitParam>> rejected;
+                int conc = 0;
+                for (int tries = 0; tries < PARTITION_STREAM_TRIES; ++tries) {
+                    note_status(lg_streams_run_concurrently(ps.d[0][mc]->stream, ps.d[1][sc]->stream, &conc), "lg_streams_run_concurrently");
+                    if (conc || first_error() || tries + 1 == PARTITION_STREAM_TRIES) break;
+                    rejected.push_back(std::move(ps.d[1][sc]));
+                    ps.d[1][sc].reset(new DynamicInitParam(sc == MFMA_BOUND ? mfma_mask : hbm_mask, 8, 2 + 2 * 1 + sc));
+                    if (first_error()) break;
+                }
+                for (auto& r : rejected) r->destroy();
+                if (!conc) ps.verified = 0;
+            }
+            if (first_error()) {
+                for (int role = 0; role < 2; ++role)
+                    for (int cls = 0; cls < 2; ++cls)
+                        if (ps.d[role][cls]) ps.d[role][cls]->destroy();
+                return false;
+            }
             it = _part_streams.emplace(hbm_cus, std::move(ps)).first;
         }
+        partition_streams_concurrent = it->second.verified;
         for (int role = 0; role < 2; ++role)
             for (int cls = 0; cls < 2; ++cls) _part[role][cls] = it->second.d[role][cls].get();
         partition_hbm_cus = hbm_cus;
@@ -287,6 +316,13 @@ class Scheduler {
         return true;
     }
     void disable_partition() { partition_hbm_cus = 0; }
+    // verify_partition_streams (set before enable_partition creates a share's streams): probe both (primary, secondary) pairs
+    // for overlap and replace a secondary that takes turns with its primary.  partition_streams_concurrent: 1 both pairs were
+    // measured to overlap, 0 a pair could not be made to, -1 not probed; profile_partition installs no factor at 0.  Off by
+    // default: profile_partition's own measurement already rejects a share whose streams take turns (its co-run then takes
+    // as long as both sides back to back: gain below 1).
+    bool verify_partition_streams = false;
+    int partition_streams_concurrent = -1;
     const DynamicInitParam* partition_stream(int role, int cls) const {
         return (partition_hbm_cus > 0 && (cls == MFMA_BOUND || cls == HBM_BOUND)) ? _part[role][cls] : nullptr;
     }
@@ -581,7 +617,7 @@ class Scheduler {
         // decode work per millisecond of co-run, times how long the prefill kernels take there, per millisecond of their own
         r.factor = ((float)reps * sub_full / std::max(best_b, 1e-6f)) * best_a / std::max(main_full, 1e-6f);
         r.gain = (main_full + (float)reps * sub_full) / std::max(std::max(best_a, best_b), 1e-6f);
-        if (r.gain >= min_gain && r.factor > 0.f) {
+        if (r.gain >= min_gain && r.factor > 0.f && partition_streams_concurrent != 0) {
             partition_table[MFMA_BOUND][HBM_BOUND] = r.factor;
             partition_table[HBM_BOUND][MFMA_BOUND] = 1.0f / r.factor;
         } else {
@@ -1183,7 +1219,10 @@ class Scheduler {
         return e;
     }
     // The round's first event: on the primary's stream, behind the end of the primary run before it (Main_EVENT), so that the
-    // distance between two such events is the time the earlier round took, whichever streams the two rounds use.
+    // distance between two such events is the time the earlier round's primary run took, whichever streams the two rounds use.
+    // A round's secondary work may still be running then (nothing makes the next primary wait for it) and is then paid for by
+    // the round it runs into: the estimate flatters the kind of round whose secondaries run long, which is the partitioned
+    // kind (its primary is cut short on purpose).  partition_feedback_margin allows for that.
     void _round_begin(const DynamicInitParam& Dp, int kind) {
         note_status(lg_stream_wait_event(Dp.stream, Main_EVENT), "lg_stream_wait_event");
         RoundRec r{_round_event(), 0.f, kind};
@@ -1212,7 +1251,8 @@ class Scheduler {
         if (partition_feedback_probe > 0 && n % partition_feedback_probe == 0) return !pays;
         return pays;
     }
-    struct PartStreams { std::unique_ptr<DynamicInitParam> d[2][2]; };
+    struct PartStreams { std::unique_ptr<DynamicInitParam> d[2][2]; int verified = -1; };
+    static constexpr int PARTITION_STREAM_TRIES = 6;
     // releases every CU-masked stream and leaves partitioning off with no pointer to a released stream behind
     void _drop_partition_streams() {
         partition_hbm_cus = 0;

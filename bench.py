@@ -23,12 +23,17 @@ CFG2 = dict(hidden=12288, heads_global=96, d=128, ffn_global=32768, world_size=2
 CFG3 = dict(batch=32, cache_len=1024)
 
 
-def measured_traffic(label):
+def measured_traffic(label, weight_layout=2):
     """HBM bytes per launch of `label` from the committed rocprofv3 counter runs (FETCH_SIZE + WRITE_SIZE, calibrated
-    against a copy kernel of known size; see profiles/).  None when no measurement is on file."""
+    against a copy kernel of known size; see profiles/).  None when no measurement is on file for this weight layout."""
     try:
         with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
-            k = json.load(f)["kernels"].get(label)
+            j = json.load(f)
+        base = j.get("weight_layout", 1)
+        suffix = "" if weight_layout == base else {0: "[in,out]", 1: "[out,in]", 2: "[tiled]"}[weight_layout]
+        k = j["kernels"].get(label + suffix)
+        if k is None and "gemm" not in label and "ffn" not in label and "proj" not in label:
+            k = j["kernels"].get(label)    # kernels that read no weights
         return int(k["fetch_bytes"] + k["write_bytes"]) if k else None
     except (OSError, KeyError, ValueError):
         return None
@@ -142,9 +147,11 @@ def bench_cfg4(capi, host, weight_layout, factors=(1, 2, 4, 8), shares=(0, 32, 6
             sched.enable_partition(share)
             meas = sched.profile_partition(4, 512, 32, 1024)
             partition[share] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in meas.items()}
+            partition[share]["streams_verified_concurrent"] = sched.partition_streams_concurrent
             key = "partitioned_%d_hbm_cus" % share
             if sched.partition_factor(1, 0) <= 0:
-                res[key] = {"skipped": "a partitioned co-run does not beat back-to-back execution (gain %.3f)" % meas["gain"]}
+                res[key] = {"skipped": ("a partitioned co-run does not beat back-to-back execution (gain %.3f)" % meas["gain"])
+                            if sched.partition_streams_concurrent else "the partition's streams could not be made to overlap"}
                 continue
             res[key] = best_of(host.MODE_LIGER)
             res[key]["speedup"] = round(res["sequential"]["makespan_ms"] / res[key]["makespan_ms"], 4)
@@ -204,9 +211,10 @@ def bench_corun_variants(weight_layout):
     return {"workload": "prefill B4 S512 MFMA-bound kernels || decode steps at 1024 cached positions, one layer shard", "rows": rows}
 
 
-def bench_cfg5(capi, host, weight_layout, n_requests, rates=(4.0, 8.0, 16.0, 24.0, 32.0), shares=(64, 128), runs=1, decode_steps_ahead=2, short=False):
-    """BASELINE config 5: Poisson arrivals at 4, 8, 16 req/s -- and at 24 and 32 req/s, which is at and beyond what one request
-    at a time can serve (about 28 req/s) -- through 4 stacked layer shards; prompts U[128, 1024] (rounded to 64), 32 decode
+def bench_cfg5(capi, host, weight_layout, n_requests, rates=(8.0, 16.0, 24.0, 32.0), shares=(128,), runs=1, decode_steps_ahead=2, short=False):
+    """BASELINE config 5: Poisson arrivals at 8 and 16 req/s -- and at 24 and 32 req/s, which is at and beyond what one request
+    at a time can serve (about 28 req/s; at the reference's 4 req/s nothing ever queues on this device) -- through 4 stacked
+    layer shards; prompts U[128, 1024] (rounded to 64), 32 decode
     tokens each; mean and p99 request latency with interleaving on and off.  `runs` > 1 repeats every (rate, mode) and reports
     the mean and the spread of the mean latency over the runs."""
     c = CFG2
@@ -234,6 +242,7 @@ def bench_cfg5(capi, host, weight_layout, n_requests, rates=(4.0, 8.0, 16.0, 24.
         sched.enable_partition(share)
         pm = sched.profile_partition(1, 512, 1, 512)
         part_meas[share] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in pm.items()}
+        part_meas[share]["streams_verified_concurrent"] = sched.partition_streams_concurrent
         part_factor[share] = (sched.partition_factor(0, 1), sched.partition_factor(1, 0))
     sched.enable_partition(0)
     # (mode, name, measured contention, minor kernels merged, HBM-side compute units of partitioned rounds, batched decode)
@@ -341,6 +350,36 @@ def measured_ceilings(capi, iters=3000, read_mib=2048):
     out["what"] = ("lg_probe_mfma_f16: 1024 blocks x 8 waves x %d rounds of 32 v_mfma_f32_16x16x32_f16, operands in registers; "
                    "lg_probe_read: one pass over %d MiB per launch, 16-byte loads" % (iters, read_mib))
     return out
+
+
+def bench_weight_relay(capi, host, weight_layout):
+    """One-off cost of taking the cfg2 layer shard's six weight matrices over from plain [in, out] device arrays (the layout the
+    reference's (N,N) GEMM call implies) into the layer's storage layout: lgh_model_load_param, one kernel per matrix."""
+    import torch
+    c = CFG2
+    model = host.Model(capi.F16, 1, 64, c["heads_global"], c["d"], layer_num=1, world_size=c["world_size"], ffn_inner=c["ffn_global"],
+                       causal=True, fused=True, weight_layout=weight_layout, seed=0)
+    srcs = {}
+    for name, i in model.param_info().items():
+        if i["rows"] > 1:
+            t = torch.empty(i["rows"] * i["cols"], device="cuda", dtype=torch.float16)
+            capi.call("lg_fill_normal_f16", t.data_ptr(), t.numel(), 0, 5, 0.0, 0.02, None)
+            srcs[name] = t
+    torch.cuda.synchronize()
+    best = None
+    for _ in range(3):
+        t0 = time.perf_counter()
+        for name, t in srcs.items():
+            model.load_param(name, t.data_ptr(), 0)
+        capi.call("lg_stream_synchronize", model.stream)
+        dt = (time.perf_counter() - t0) * 1e3
+        best = dt if best is None else min(best, dt)
+    nbytes = sum(t.numel() * 2 for t in srcs.values())
+    model.close()
+    del srcs
+    torch.cuda.empty_cache()
+    return {"what": "lgh_model_load_param on the %d weight matrices of one cfg2 layer shard, sources [in, out]" % 6, "ms": round(best, 3),
+            "weight_MB": round(nbytes / 1e6, 1), "read_plus_write_GBps": round(2 * nbytes / (best * 1e-3) / 1e9, 1)}
 
 
 def bench_fp32(capi, host):
@@ -458,6 +497,41 @@ def time_layer(capi, host, weight_layout, fused, steps, warmup):
     return model, x, y, {"ms_per_step": ms_per_step, "kernels": kernels, "sum_kernel_ms": sum(times), "decode": decode}
 
 
+def timed_only(capi, host, args, fused):
+    """The bench's timed region and nothing else: `warmup` untimed and `steps` timed launches of the cfg2 prefill layer shard (or,
+    with --decode, of the cfg3 decode step), the same calls `time_layer` times.  Every launch-vector entry is one kernel dispatch,
+    so a kernel trace of this run holds (warmup + steps) x len(entries) dispatches after the set-up fills, in launch order."""
+    import torch
+    c = CFG2
+    B, S, H = c["batch"], c["seq"], c["hidden"]
+    model = host.Model(capi.F16, 32, S, c["heads_global"], c["d"], layer_num=1, world_size=c["world_size"], ffn_inner=c["ffn_global"],
+                       norm_mode=host.POST_NORESID, causal=True, fused=fused, max_cache_len=CFG3["cache_len"] + 32 if fused else 0,
+                       weight_layout=args.weight_layout, seed=0)
+    stream = model.stream
+    if args.decode:
+        Bd, L = CFG3["batch"], CFG3["cache_len"]
+        x = torch.empty(Bd, H, device="cuda", dtype=torch.float16)
+        desc = model.describe(Bd, 1, decode_past=L - 1)
+        step = lambda: model.run_decode(x.data_ptr(), y.data_ptr(), Bd, L - 1, 0, None, stream)
+    else:
+        x = torch.empty(B * S, H, device="cuda", dtype=torch.float16)
+        desc = model.describe(B, S)
+        step = lambda: model.run(x.data_ptr(), y.data_ptr(), B, S, None, stream)
+    capi.call("lg_fill_normal_f16", x.data_ptr(), x.numel(), 0, 99, 0.0, 1.0, None)
+    y = torch.empty_like(x)
+    torch.cuda.synchronize()
+    for _ in range(args.warmup):
+        step()
+    capi.call("lg_stream_synchronize", stream)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    capi.call("lg_stream_synchronize", stream)
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    return {"timed_only": "cfg3 decode step" if args.decode else "cfg2 prefill layer shard", "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(ms, 4), "entries": [e["label"] for e in desc], "weight_layout": args.weight_layout}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -478,12 +552,16 @@ def main():
                          "'copy' (a plain 128 MiB read + 128 MiB write kernel) --iters times; for rocprofv3 runs.  "
                          "'mfma_ceiling' / 'read_ceiling' run the library's probe kernels and print what the device sustains")
     ap.add_argument("--iters", type=int, default=50)
+    ap.add_argument("--timed-only", action="store_true",
+                    help="run nothing but the warm-up steps and the timed steps of the prefill layer shard (with --decode: of the decode "
+                         "step) and print their launch vector; for rocprofv3 runs whose rows are then the timed dispatches alone")
     ap.add_argument("--decode", action="store_true",
                     help="with --kernel-only: take the entry from the decode step's launch vector (batch 32, 1024 cached positions); "
                          "needed for the entries whose name the prefill vector has too (ffn1+bias+gelu, ffn2, layer_norm)")
     ap.add_argument("--weight-layout", type=int, default=2, choices=[0, 1, 2],
                     help="0: weights stored [in, out] (the reference's cuBLAS (N,N) layout); 1: stored [out, in]; "
-                         "2 (default): [out, in] re-laid into 16 x 32 fragment blocks when the layer takes them over (lg_weight_tile_f16)")
+                         "2 (default): [out, in] in 16 x 32 fragment blocks, the layout a layer re-lays weights into when it takes them over "
+                         "(lgh_model_load_param -> lg_weight_tile_f16; cost in the weight_relay_at_load record)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs one GPU's tensor-parallel shard on one GPU; --gpus %d is not supported "
@@ -511,6 +589,9 @@ def main():
         m = measured_ceilings(capi)
         print(json.dumps({"kernel": args.kernel_only, **{k: v for k, v in m.items() if k == "what" or k.startswith("mfma" if args.kernel_only == "mfma_ceiling" else "read")}}))
         return
+    if args.timed_only:
+        print(json.dumps(timed_only(capi, host, args, fused)))
+        return
     if args.kernel_only:
         model = host.Model(capi.F16, 32, S, c["heads_global"], c["d"], layer_num=1, world_size=c["world_size"], ffn_inner=c["ffn_global"],
                            norm_mode=host.POST_NORESID, causal=True, fused=fused, max_cache_len=CFG3["cache_len"] + 32 if fused else 0,
@@ -532,7 +613,7 @@ def main():
     for k in kernels:
         if k["kernel"] in label_flops:
             k["tflops"] = round(label_flops[k["kernel"]] / (k["ms"] * 1e-3) / 1e12, 1)
-            k["traffic"] = measured_traffic(k["kernel"])
+            k["traffic"] = measured_traffic(k["kernel"], args.weight_layout)
             gemm_ms += k["ms"]
             gemm_fl += label_flops[k["kernel"]]
     # dominant kernel = FFN-1 (with FFN-2 the largest share of the step's flops; always the same one, so that the counter
@@ -541,7 +622,7 @@ def main():
     dom_fl = label_flops[dom["kernel"]]
     achieved = dom_fl / (dom["ms"] * 1e-3) / 1e12
     roofline = {"bound": "mfma", "kernel": dom["kernel"], "achieved": round(achieved, 1), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(achieved / PEAK_FP16_TFLOPS, 4), "traffic": measured_traffic(dom["kernel"]),
+                "frac": round(achieved / PEAK_FP16_TFLOPS, 4), "traffic": measured_traffic(dom["kernel"], args.weight_layout),
                 "all_gemms_tflops": round(gemm_fl / (gemm_ms * 1e-3) / 1e12, 1),
                 "all_gemms_frac": round(gemm_fl / (gemm_ms * 1e-3) / 1e12 / PEAK_FP16_TFLOPS, 4)}
     ln = [k for k in kernels if k["kernel"] == "layer_norm"]
@@ -623,6 +704,7 @@ def main():
                                      "kernels_ms": {"%d:%s" % (k["idx"], k["kernel"]): k["ms"] for k in r3["kernels"]}}
         del m3, x3, y3
         torch.cuda.empty_cache()
+    out["weight_relay_at_load"] = bench_weight_relay(capi, host, args.weight_layout)
     out["fp32"] = bench_fp32(capi, host)
     if not args.no_cpu_baseline:
         from oracle import pyoracle as po

@@ -82,6 +82,10 @@ int lg_stream_create_cu_mask(void** stream, const unsigned* cu_mask, int mask_wo
  * to a one-wave kernel on the candidate) until one overlaps.  *verified = 1 if such a stream was found, 0 if the
  * returned stream is an unverified fallback.  `other` must be a created stream (not the null stream). */
 int lg_stream_create_concurrent(void** stream, void* other, int* verified);
+/* The same probe for two streams that exist already (both created, not the null stream; CU-masked ones included):
+ * *concurrent = 1 when a one-wave kernel on `b` finishes while a 0.4 ms one-wave spin on `a` still runs.  Blocks until
+ * both have run (set-up time only).  No reference counterpart: schedule.h:54-55 trusts its two streams to overlap. */
+int lg_streams_run_concurrently(void* a, void* b, int* concurrent);
 int lg_stream_destroy(void* stream);
 int lg_stream_synchronize(void* stream);
 int lg_stream_wait_event(void* stream, void* event);

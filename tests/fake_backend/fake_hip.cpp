@@ -45,6 +45,8 @@ double g_share_exp[2] = {1.0, 1.0};  // a kernel on a stream with `cus` of 256 c
 thread_local int g_cost_kind = 1;    // kind of the cost computed last on this thread (0 matrix, 1 memory)
 std::vector<Stream*> g_streams;
 int g_fail_cu_mask_after = -1;  // >= 0: that many CU-masked streams are still created, the ones after them fail
+int g_serial_probes = 0;        // that many of the next concurrency probes report streams that run in turn
+int g_cu_mask_created = 0;     // CU-masked streams created since the last reset of this counter
 int g_live_streams = 0, g_live_allocs = 0;   // created and not yet destroyed / allocated and not yet freed
 std::vector<Launch> g_trace;
 Stream g_default;
@@ -108,6 +110,8 @@ int fake_trace_get(int i, int* stream, char* name, int name_len, long long* abc,
 double fake_host_now(void) { return g_host_now; }
 int fake_live_streams(void) { return g_live_streams; }
 void fake_fail_cu_mask_streams_after(int n) { g_fail_cu_mask_after = n; }
+void fake_serialise_probes(int n) { g_serial_probes = n; }
+int fake_cu_mask_streams_created(int reset) { const int n = g_cu_mask_created; if (reset) g_cu_mask_created = 0; return n; }
 int fake_live_allocs(void) { return g_live_allocs; }
 
 // ---- library / runtime ------------------------------------------------------------------------------------------------
@@ -166,10 +170,18 @@ int lg_stream_create_cu_mask(void** stream, const unsigned* cu_mask, int mask_wo
     if (g_fail_cu_mask_after == 0) { *stream = nullptr; return LG_ERR_LAUNCH; }
     if (g_fail_cu_mask_after > 0) --g_fail_cu_mask_after;
     const int rc = lg_stream_create(stream);
+    ++g_cu_mask_created;
     Stream* s = (Stream*)*stream;
     s->cus = cus;
     for (int w = 0; w < 8; ++w) s->mask[w] = w < mask_words ? cu_mask[w] : 0u;
     return rc;
+}
+int lg_streams_run_concurrently(void* a, void* b, int* concurrent) {
+    if (!a || !b || a == b || !concurrent) return LG_ERR_INVALID;
+    std::lock_guard<std::mutex> lk(g_mu);
+    *concurrent = g_serial_probes > 0 ? 0 : 1;   // virtual streams overlap unless a test says otherwise
+    if (g_serial_probes > 0) --g_serial_probes;
+    return LG_OK;
 }
 int lg_stream_destroy(void* stream) {
     // the object stays (traces refer to it); only the count of streams in existence goes down

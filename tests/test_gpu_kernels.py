@@ -244,6 +244,12 @@ def test_second_stream_is_verified_to_run_next_to_the_first(dev, po):
         assert lib.lg_layer_norm_f32(ptr(dx), ptr(dg), ptr(db), ptr(out), m, n, second) == 0, dev.capi.last_error()
         assert lib.lg_stream_synchronize(second) == 0
         assert max_rel_err(dev.down(out), po.layer_norm(x, g, b, 0)) < tol(0)
+        # the probe on its own agrees with what the creation reported; one stream with itself, and a null stream, are refused
+        conc = C.c_int(-1)
+        assert lib.lg_streams_run_concurrently(first, second, C.byref(conc)) == 0, dev.capi.last_error()
+        assert conc.value == verified.value
+        assert lib.lg_streams_run_concurrently(first, first, C.byref(conc)) == 1
+        assert lib.lg_streams_run_concurrently(first, None, C.byref(conc)) == 1
     finally:
         assert lib.lg_stream_destroy(second) == 0
         for s in crowd:

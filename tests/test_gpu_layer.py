@@ -322,3 +322,40 @@ def test_chunked_prefill_equals_the_whole_prefill_and_the_oracle(dev, po, host, 
     # refusals: a chunked run needs a cache slot that holds the sequence
     with pytest.raises(host.capi.LigerError):
         m.run_chunked(dx.data_ptr(), parts.data_ptr(), S, chunk, -1, None, dev.stream)
+
+
+@pytest.mark.parametrize("dtype,fused,packed", [(1, True, False), (1, True, True), (1, False, False), (0, False, False)])
+@pytest.mark.parametrize("weight_layout", [0, 1, 2])
+@pytest.mark.parametrize("src_layout", [0, 1])
+def test_parameters_loaded_from_device_memory_are_relaid_exactly(dev, po, host, dtype, fused, packed, weight_layout, src_layout):
+    """lgh_model_load_param: every parameter of a donor model, handed over as a plain [in, out] (what the reference's (N,N)
+    GEMM call implies) or [out, in] device array, lands in the receiving layer's storage layout bit for bit -- the
+    downloaded parameters are equal and the layer's output equals the donor's bit for bit."""
+    if weight_layout == 2 and dtype == 0:
+        pytest.skip("fragment blocks are fp16 only")
+    B, S, heads, d, F = 2, 48, 4, 64, 512
+    H = heads * d
+    mk = lambda seed: host.Model(dtype, B, S, heads, d, ffn_inner=F, causal=True, fused=fused, packed_qkv=packed,
+                                 weight_layout=weight_layout, seed=seed)
+    donor, m = mk(3), mk(4)
+    want = donor.download_params()
+    before = m.download_params()
+    assert any(not np.array_equal(before[k], want[k]) for k in want)
+    keep = []
+    for name, a in want.items():
+        plain = a if (a.ndim == 1 or src_layout == 0) else np.ascontiguousarray(a.T)
+        t = dev.up(plain, dtype)
+        keep.append(t)
+        m.load_param(name, t.data_ptr(), src_layout, dev.stream)
+    dev.sync()
+    got = m.download_params()
+    for k in want:
+        assert np.array_equal(got[k], want[k]), k
+    x = po.fill_normal(B * S * H, 0, 99, 0.0, 1.0, dtype).reshape(B * S, H)
+    dx = dev.up(x, dtype)
+    y0, y1 = dev.empty((B * S, H), dtype), dev.empty((B * S, H), dtype)
+    donor.run(dx.data_ptr(), y0.data_ptr(), B, S, None, dev.stream)
+    m.run(dx.data_ptr(), y1.data_ptr(), B, S, None, dev.stream)
+    assert np.array_equal(dev.down(y0), dev.down(y1))
+    donor.close()
+    m.close()

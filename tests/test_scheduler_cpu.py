@@ -619,6 +619,37 @@ def test_a_failed_change_of_share_leaves_no_stream_behind_and_no_stale_pointer(f
     assert lib.fake_live_streams() == live - 6
 
 
+def test_the_streams_of_a_partitioned_round_are_probed_pair_by_pair(fake):
+    """Two CU-masked streams may share a hardware queue and then take turns.  enable_partition probes both (primary,
+    secondary) pairs, replaces a secondary that does not overlap with its primary (rejected candidates are released once
+    a good one is found) and reports the outcome; a share whose pairs cannot be made to overlap gets no measured factor.
+    The verification is opt-in (set_verify_partition_streams)."""
+    host, m, s = _partition_setup(fake)                 # share 128, created without verification
+    lib = fake.lib
+    live = lib.fake_live_streams()
+    assert s.partition_streams_concurrent is None
+    s.set_verify_partition_streams(True)
+    # the next three probes see streams that take turns: the first pair needs two replacements, the second pair one
+    lib.fake_cu_mask_streams_created(1)
+    lib.fake_serialise_probes(3)
+    s.enable_partition(64)
+    assert lib.fake_cu_mask_streams_created(1) == 4 + 3
+    assert lib.fake_live_streams() == live             # the old share's four and the three rejected ones are gone
+    assert s.partition_streams_concurrent
+    fake.set_share_model(0.5, 0.2)                      # a backend on which a partition pays
+    assert s.profile_partition(1, 48, 1, 48)["gain"] > 1.02 and s.partition_factor(MFMA, HBM) > 0
+    # no candidate overlaps: the share is usable but flagged, and the measurement installs nothing
+    lib.fake_serialise_probes(1000)
+    s.enable_partition(32)
+    lib.fake_serialise_probes(0)
+    assert lib.fake_live_streams() == live
+    assert s.partition_streams_concurrent is False
+    assert s.profile_partition(1, 48, 1, 48)["gain"] > 1.02 and s.partition_factor(MFMA, HBM) < 0
+    s.enable_partition(0)
+    assert s.partition_streams_concurrent is None
+    s.close()
+
+
 @pytest.mark.parametrize("matrix_exp,memory_exp,corun,pays", [(1.0, 1.0, 1.0, False), (0.5, 0.2, 0.5, True)])
 def test_partition_feedback_follows_what_the_rounds_deliver(fake, matrix_exp, memory_exp, corun, pays):
     """Prefill requests (MFMA-bound) and decode requests (HBM-bound) queued in turn, with a partition table that says every
@@ -899,6 +930,42 @@ def test_cfg4_shapes_pieces_cover_the_prefill_exactly(fake, factor, axis):
         total = sum(e["m"] * e["n"] for e in gemms)
         assert total == M * (3 * Hl + H + F + H) and all(e["n"] == M for e in gemms)
         assert len(gemms) > 6
+
+
+@pytest.mark.parametrize("weight_layout", [0, 1, 2])
+def test_loading_a_parameter_relays_it_into_the_layers_storage_layout(fake, weight_layout):
+    """lgh_model_load_param: one launch per parameter on the model's stream -- a copy when the source layout is the layer's,
+    a transpose between the two plain layouts, the tiling kernel for a layer that stores fragment blocks; vectors are
+    copied; interleaved (fused GeGLU) parameters, bad layouts and a parameter loaded from itself are refused."""
+    host = fake.host
+    m = host.Model(1, 2, 32, 4, 64, ffn_inner=512, fused=True, weight_layout=weight_layout, max_cache_len=40)
+    info = m.param_info()
+    name = [k for k, v in info.items() if v["rows"] > 1][0]
+    vec = [k for k, v in info.items() if v["rows"] == 1][0]
+    src = info[vec]["ptr"]    # any other device address will do for the fake backend
+    for src_layout in (0, 1):
+        fake.reset()
+        m.load_param(name, src, src_layout)
+        tr = fake.trace()
+        assert len(tr) == 1 and tr[0]["C"] == info[name]["ptr"] and tr[0]["A"] == src
+        want = "weight_tile" if weight_layout == 2 else ("memcpy_d2d" if src_layout == weight_layout else "transpose")
+        assert tr[0]["name"] == want, (weight_layout, src_layout, tr[0]["name"])
+    fake.reset()
+    m.load_param(vec, info[name]["ptr"], 0)
+    assert [t["name"] for t in fake.trace()] == ["memcpy_d2d"]
+    with pytest.raises(Exception, match="src_layout"):
+        m.load_param(name, src, 2)
+    with pytest.raises(Exception, match="itself"):
+        m.load_param(name, info[name]["ptr"], 0)
+    with pytest.raises(KeyError):
+        m.load_param("no_such_parameter", src, 0)
+    m.close()
+    g = host.Model(1, 2, 32, 4, 64, ffn_inner=512, fused=True, ffn_act=host.FFN_GEGLU, weight_layout=weight_layout)
+    gi = g.param_info()
+    inter = [k for k, v in gi.items() if v["interleave16"] and v["rows"] > 1][0]
+    with pytest.raises(Exception, match="interleaved"):
+        g.load_param(inter, gi[vec]["ptr"], 0)
+    g.close()
 
 
 def test_closing_a_scheduler_and_a_model_releases_streams_and_memory(fake):
