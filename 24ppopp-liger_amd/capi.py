@@ -88,6 +88,7 @@ SIGNATURES = {
     "lg_weight_tile_f16": (_i, [_p, _p, _i, _i, _i, _i, _p]),
     "lg_weight_untile_f16": (_i, [_p, _p, _i, _i, _i, _i, _p]),
     "lg_probe_mfma_f16": (_i, [_p, _i64, _p, _sz, _i, C.POINTER(_f), C.POINTER(_f), C.POINTER(_f), _p]),
+    "lg_probe_mfma_stream_f16": (_i, [_p, _i64, _p, _sz, _i, _i, _i, C.POINTER(_f), C.POINTER(_f), C.POINTER(_f), _p]),
     "lg_probe_read": (_i, [_p, _sz, _p, _i, _i, C.POINTER(_f), C.POINTER(_f), _p]),
 }
 

@@ -270,6 +270,13 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f16_fast(GemmArgs g, GemmGroup
         xnext = (xnext == X_STAGES - 1) ? 0 : xnext + 1;
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the clamped refills of the last iterations
+    if (WL == W_KN) {
+        // the last phase has issued the transposed reads of a tile that is never multiplied: they are waited for and named
+        // here, so that nothing may reuse their registers while they can still land (hand-issued reads are invisible to
+        // the compiler's own bookkeeping)
+#pragma unroll
+        for (int u = 0; u < NJ; ++u) lds_tr_wait<0>(blo[0][u], bhi[0][u]);
+    }
 
     // ---- epilogue: acc[i][j][r] = Y[m0 + wm*128 + i*16 + l16][n0 + wn*16*NJ + j*16 + 4*lk + r] -----------------------------
     // Everything that depends only on the column (bias, head offset) or only on the row (batch / position split) is

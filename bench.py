@@ -311,7 +311,7 @@ def bench_cfg5(capi, host, weight_layout, n_requests, rates=(8.0, 16.0, 24.0, 32
             "partition_measurement": part_meas, "results": out}
 
 
-def measured_ceilings(capi, iters=3000, read_mib=2048):
+def measured_ceilings(capi, iters=3000, read_mib=2048, traffic_variants=False):
     """What this device sustains, measured now with the library's two probe kernels (lg_probe_mfma_f16, lg_probe_read):
     a register-only loop of the GEMM's matrix instruction on its wave tile with operands distributed like the bench's data
     (N(0,1) x N(0,0.02) products are what the layer's GEMMs multiply; both operand sets here are N(0,1) halves, which toggle
@@ -336,6 +336,23 @@ def measured_ceilings(capi, iters=3000, read_mib=2048):
                 best = (tf.value, ghz.value, ms.value)
         out["mfma_f16_" + name] = {"TFLOPs": round(best[0], 1), "shader_clock_GHz": round(best[1], 3), "kernel_ms": round(best[2], 3),
                                    "frac_of_published_peak": round(best[0] / PEAK_FP16_TFLOPS, 4)}
+    # the same instruction stream with the operands travelling L2 -> LDS -> registers at the pipelined GEMM's rate (random data)
+    capi.call("lg_fill_normal_f16", ops.data_ptr(), n, 0, 77, 0.0, 1.0, None)
+    torch.cuda.synchronize()
+    def streamed(loads, reads):
+        best = None
+        for _ in range(3):
+            capi.call("lg_probe_mfma_stream_f16", ops.data_ptr(), n, scratch.data_ptr(), 256, iters // 2, loads, reads, C.byref(ms), C.byref(tf), C.byref(ghz), None)
+            if best is None or tf.value > best[0]:
+                best = (tf.value, ghz.value, ms.value)
+        return {"TFLOPs": round(best[0], 1), "shader_clock_GHz": round(best[1], 3), "kernel_ms": round(best[2], 3),
+                "frac_of_published_peak": round(best[0] / PEAK_FP16_TFLOPS, 4)}
+    out["mfma_f16_random_operands_streamed_through_lds"] = streamed(8, 12)
+    if traffic_variants:
+        # what half or none of either kind of operand traffic would leave (per wave and k-tile: L2 -> LDS loads of 1 KiB, LDS -> register
+        # reads of 1 KiB per k-step)
+        out["mfma_f16_streamed_traffic_variants"] = {"loads_%d_reads_%d" % (l, r): streamed(l, r)["TFLOPs"]
+                                                     for l, r in ((8, 12), (4, 12), (0, 12), (8, 6), (8, 0), (4, 6), (0, 0))}
     del ops
     buf = torch.empty(read_mib << 20, device="cuda", dtype=torch.uint8)
     capi.call("lg_fill_normal_f16", buf.data_ptr(), buf.numel() // 2, 0, 78, 0.0, 1.0, None)
@@ -348,7 +365,8 @@ def measured_ceilings(capi, iters=3000, read_mib=2048):
     del buf
     torch.cuda.empty_cache()
     out["what"] = ("lg_probe_mfma_f16: 1024 blocks x 8 waves x %d rounds of 32 v_mfma_f32_16x16x32_f16, operands in registers; "
-                   "lg_probe_read: one pass over %d MiB per launch, 16-byte loads" % (iters, read_mib))
+                   "lg_probe_mfma_stream_f16: %d rounds of 64, per round 8 KiB per wave L2 -> LDS and 24 KiB LDS -> registers (the pipelined GEMM's "
+                   "operand traffic, nothing else of it); lg_probe_read: one pass over %d MiB per launch, 16-byte loads" % (iters, iters // 2, read_mib))
     return out
 
 
@@ -586,7 +604,7 @@ def main():
         print(json.dumps(bench_corun_one(capi, host, args.weight_layout, args.corun_one)), flush=True)
         return
     if args.kernel_only in ("mfma_ceiling", "read_ceiling"):
-        m = measured_ceilings(capi)
+        m = measured_ceilings(capi, traffic_variants=args.kernel_only == "mfma_ceiling")
         print(json.dumps({"kernel": args.kernel_only, **{k: v for k, v in m.items() if k == "what" or k.startswith("mfma" if args.kernel_only == "mfma_ceiling" else "read")}}))
         return
     if args.timed_only:
@@ -680,6 +698,8 @@ def main():
     out["peaks"]["measured"] = measured_ceilings(capi)
     mc = out["peaks"]["measured"]["mfma_f16_random_operands"]["TFLOPs"]
     out["roofline"]["frac_of_measured_mfma_ceiling"] = round(out["roofline"]["achieved"] / mc, 4) if mc > 0 else None
+    ms_ = out["peaks"]["measured"]["mfma_f16_random_operands_streamed_through_lds"]["TFLOPs"]
+    out["roofline"]["frac_of_measured_mfma_ceiling_with_operand_traffic"] = round(out["roofline"]["achieved"] / ms_, 4) if ms_ > 0 else None
     # the same layer (prefill and decode step) in the other weight layouts: 0 = [in, out], the layout the reference's (N,N)
     # cuBLAS call implies; 1 = [out, in]; 2 = [out, in] re-laid into 16 x 32 fragment blocks
     names = {0: ("reference_layout", "[in, out]"), 1: ("out_in_layout", "[out, in]"), 2: ("tiled_layout", "[out, in] in 16 x 32 fragment blocks")}

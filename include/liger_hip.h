@@ -300,6 +300,15 @@ int lg_weight_untile_f16(void* plain, const void* tiled, int features, int k, in
  * Returns the kernel's milliseconds, TFLOP/s and the shader clock (GHz) seen by the kernel (either may be NULL). */
 int lg_probe_mfma_f16(const void* operands, int64_t operand_elems, void* scratch, size_t scratch_bytes, int iters, float* ms,
                       float* tflops, float* shader_ghz, void* stream);
+/* The same wave tile and instruction with the operand traffic of the pipelined GEMM's k-loop and nothing else of it: per 64
+ * matrix instructions a wave copies 8 KiB from `operands` (a region that stays in L2) to LDS with direct-to-LDS loads and
+ * reads 24 fragments of 1 KiB from LDS (two LDS slots of 64 KiB, fragments double-buffered in registers); no barrier and no
+ * wait for a particular tile, no epilogue, no stores, no traffic beyond L2.  1024 blocks x 8 waves x iters rounds of 64 matrix
+ * instructions.  loads_per_round = 8 and reads_per_step = 12 are the GEMM's traffic; 4 / 0 and 6 / 0 show what half or none of
+ * either would leave.  Other arguments and results as lg_probe_mfma_f16: an upper bound for a k-loop whose operands travel
+ * L2 -> LDS -> registers at that rate, whatever its synchronisation costs on top. */
+int lg_probe_mfma_stream_f16(const void* operands, int64_t operand_elems, void* scratch, size_t scratch_bytes, int iters, int loads_per_round,
+                             int reads_per_step, float* ms, float* tflops, float* shader_ghz, void* stream);
 /* Reads every byte of src[0, bytes) once per pass (16-byte loads, 8 in flight per lane, 1 KiB per wave instruction;
  * nontemporal != 0 marks them as streaming), `passes` passes after one untimed pass.  On a buffer much larger than the
  * caches (256 MB memory-side cache) the figure is the device's memory read ceiling.  scratch: >= 4 bytes of device memory.

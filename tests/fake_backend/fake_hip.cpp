@@ -286,6 +286,13 @@ int lg_probe_mfma_f16(const void* operands, int64_t n, void* scratch, size_t, in
     if (ghz) *ghz = 2.4f;
     return LG_OK;
 }
+int lg_probe_mfma_stream_f16(const void* operands, int64_t n, void* scratch, size_t sb, int iters, int loads, int reads, float* ms, float* tflops,
+                             float* ghz, void* st) {
+    if ((loads != 0 && loads != 4 && loads != 8) || (reads != 0 && reads != 6 && reads != 12)) return LG_ERR_INVALID;
+    const int rc = lg_probe_mfma_f16(operands, n, scratch, sb, iters, ms, tflops, ghz, st);
+    if (rc == LG_OK) *ms *= 2.f;   // twice the matrix instructions per round
+    return rc;
+}
 int lg_probe_read(const void* src, size_t bytes, void* scratch, int passes, int, float* ms, float* gbps, void*) {
     if (!src || !scratch || passes <= 0 || !ms || bytes < (1u << 20)) return LG_ERR_INVALID;
     *ms = (float)((double)bytes / g_hbm_rate);
