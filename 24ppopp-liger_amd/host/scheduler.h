@@ -354,6 +354,8 @@ class Scheduler {
     // Batched decode needs one more cache slot than the contexts use (rows of the batch that belong to no request in its
     // decode steps are pointed at it) and the batch's own token-row buffer and workspace.
     bool enable_batch_decode(bool on = true) {
+        // batching changes what the rounds of a run look like: what partitioned rounds delivered without it says nothing about them
+        if (on != batch_decode) reset_partition_feedback();
         if (!on) { batch_decode = false; return true; }
         const int rows = _pool_total * _ctx_batch;
         if (rows <= 0 || BertParams.max_cache_len <= 0 || rows + 1 > BertParams.max_batch_size || rows > LG_ATTN_DECODE_MAX_SEQS) return false;

@@ -456,7 +456,7 @@ def derived_peaks(info):
                                                                                      info["bus_width_bits"], info["mem_clock_khz"] / 1e6)}
 
 
-def time_layer(capi, host, weight_layout, fused, steps, warmup):
+def time_layer(capi, host, weight_layout, fused, steps, warmup, packed_qkv=False):
     """Times the cfg2 prefill layer shard and the cfg3 decode step in one weight layout; returns (model, x, y, results)."""
     import torch
     c = CFG2
@@ -464,7 +464,7 @@ def time_layer(capi, host, weight_layout, fused, steps, warmup):
     M = B * S
     model = host.Model(capi.F16, 32, S, c["heads_global"], c["d"], layer_num=1, world_size=c["world_size"], ffn_inner=c["ffn_global"],
                        norm_mode=host.POST_NORESID, causal=True, fused=fused, max_cache_len=CFG3["cache_len"] + 32 if fused else 0,
-                       weight_layout=weight_layout, seed=0)
+                       weight_layout=weight_layout, seed=0, packed_qkv=packed_qkv)
     x = torch.empty(M, H, device="cuda", dtype=torch.float16)
     capi.call("lg_fill_normal_f16", x.data_ptr(), x.numel(), 0, 99, 0.0, 1.0, None)
     y = torch.empty_like(x)
@@ -723,6 +723,15 @@ def main():
         out["reference_assembly"] = {"launches_per_layer": len(r3["kernels"]), "ms_per_layer_shard_prefill": round(r3["ms_per_step"], 4),
                                      "kernels_ms": {"%d:%s" % (k["idx"], k["kernel"]): k["ms"] for k in r3["kernels"]}}
         del m3, x3, y3
+        torch.cuda.empty_cache()
+    if fused:
+        # the same shard with the Q, K and V projections stored as ONE [H, 3 Hl] weight (the layout of GLM checkpoints): the three
+        # GEMM entries become one grouped launch whose 18432 features fill six full rounds of 256 x 192 tiles
+        m4, x4, y4, r4 = time_layer(capi, host, args.weight_layout, True, max(5, args.steps // 2), 2, packed_qkv=True)
+        out["packed_qkv"] = {"launches_per_layer": len(r4["kernels"]), "ms_per_layer_shard_prefill": round(r4["ms_per_step"], 4),
+                             "ms_per_layer_shard_decode": r4["decode"]["ms_per_layer_shard"] if r4["decode"] else None,
+                             "kernels_ms": {"%d:%s" % (k["idx"], k["kernel"]): k["ms"] for k in r4["kernels"]}}
+        del m4, x4, y4
         torch.cuda.empty_cache()
     out["weight_relay_at_load"] = bench_weight_relay(capi, host, args.weight_layout)
     out["fp32"] = bench_fp32(capi, host)
