@@ -258,3 +258,51 @@ def test_second_stream_is_verified_to_run_next_to_the_first(dev, po):
     assert lib.lg_stream_create_concurrent(C.byref(second), None, C.byref(verified)) == 1  # LG_ERR_INVALID
     if ok != 1:
         pytest.skip("no candidate stream overlapped with the first one on this box (a single hardware queue?)")
+
+
+def test_ceiling_probes_report_plausible_figures_and_refuse_bad_arguments(dev):
+    """lg_probe_mfma_f16 / lg_probe_mfma_stream_f16 / lg_probe_read (measurement entries of the bench): short runs return
+    figures inside what the device can do at all (no more than the published peaks, a sensible fraction of them), the matrix
+    loop with operand traffic does not beat the one without, zero operands are not slower than random ones; arguments the
+    kernels' indexing does not allow are refused before any launch."""
+    import ctypes as C
+    import torch
+    lib = dev.lib
+    n = 1 << 20
+    ops = torch.empty(n, device="cuda", dtype=torch.float16)
+    dev.call("lg_fill_normal_f16", ops, n, 0, 77, 0.0, 1.0)
+    scratch = torch.zeros(64, device="cuda", dtype=torch.float32)
+    dev.sync()
+    ms, tf, ghz = C.c_float(), C.c_float(), C.c_float()
+    ptr = lambda t: C.c_void_p(t.data_ptr())
+
+    def mfma(stream_traffic, t, iters=400, loads=8, reads=12, elems=n):
+        if stream_traffic:
+            rc = lib.lg_probe_mfma_stream_f16(ptr(t), elems, ptr(scratch), 256, iters, loads, reads, C.byref(ms), C.byref(tf), C.byref(ghz), None)
+        else:
+            rc = lib.lg_probe_mfma_f16(ptr(t), elems, ptr(scratch), 256, iters, C.byref(ms), C.byref(tf), C.byref(ghz), None)
+        return rc, tf.value, ghz.value
+
+    rc, plain, clock = mfma(False, ops)
+    assert rc == 0, dev.capi.last_error()
+    assert 800.0 < plain < 2600.0 and 1.0 < clock < 2.6, (plain, clock)
+    rc, zeros, _ = mfma(False, torch.zeros_like(ops))
+    assert rc == 0 and zeros > 0.98 * plain and zeros < 2600.0, (zeros, plain)
+    rc, streamed, clock = mfma(True, ops)
+    assert rc == 0, dev.capi.last_error()
+    assert 600.0 < streamed < 1.03 * plain and 1.0 < clock < 2.6, (streamed, plain, clock)
+    rc, bare, _ = mfma(True, ops, loads=0, reads=0)
+    assert rc == 0 and bare > streamed, (bare, streamed)
+    print("matrix loop: %.0f TFLOP/s on N(0,1) operands, %.0f on zeros; with the GEMM's operand traffic %.0f, same kernel without it %.0f"
+          % (plain, zeros, streamed, bare))
+    assert mfma(True, ops, loads=3)[0] == 1 and mfma(True, ops, reads=5)[0] == 1          # LG_ERR_INVALID
+    assert mfma(False, ops, elems=1000)[0] == 1 and mfma(True, ops, elems=1000)[0] == 1
+    assert mfma(False, ops, iters=0)[0] == 1
+    assert lib.lg_probe_mfma_f16(None, n, ptr(scratch), 256, 10, C.byref(ms), None, None, None) == 1
+    buf = torch.empty(64 << 20, device="cuda", dtype=torch.uint8)
+    gb = C.c_float()
+    for nt in (0, 1):
+        assert lib.lg_probe_read(ptr(buf), buf.numel(), ptr(scratch), 3, nt, C.byref(ms), C.byref(gb), None) == 0, dev.capi.last_error()
+        assert 1000.0 < gb.value < 40000.0, gb.value       # 64 MiB stays in the memory-side cache: above the HBM peak is possible
+    assert lib.lg_probe_read(ptr(buf), 1000, ptr(scratch), 3, 0, C.byref(ms), C.byref(gb), None) == 1
+    assert lib.lg_probe_read(ptr(buf), buf.numel(), ptr(scratch), 0, 0, C.byref(ms), C.byref(gb), None) == 1
