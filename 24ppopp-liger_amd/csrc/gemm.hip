@@ -491,6 +491,27 @@ int lg_gemm_fused_grouped_f16(int transa, int m, int n, int k, int count, const 
         grp.ldy[i] = ldc[i];
         if (!A[i] || !C[i] || (epilogue != LG_EPI_NONE && !bias[i])) one_launch = false;  // the plain call reports it
     }
+    if (one_launch && n > 256) {
+        // Many token rows (the pipelined kernel's regime): one launch or member by member?  The members' tiles side by side may
+        // fill a round of workgroups that one member alone leaves half empty (384-768 token rows x 6144 features: one launch is
+        // 7-13 % faster per layer), or they may end in a mostly empty last round that three launches with a narrower tile avoid
+        // (1024 rows: 6 % slower).  What decides is rounds of workgroups x tile width for the best width either way, the
+        // quantity the pipelined kernel's launcher minimises; ties go to separate launches.  Both ways give the same bits.
+        const int cus = stream_info((hipStream_t)stream).cus;
+        const int tiles_m = (n + 255) / 256;
+        auto round_widths = [&](int members) {
+            long best = -1;
+            for (int nj = 4; nj >= 2; --nj) {
+                if (m % (64 * nj)) continue;
+                const long tiles = (long)tiles_m * (m / (64 * nj)) * members;
+                const long u = ((tiles + cus - 1) / cus) * nj;
+                if (best < 0 || u < best) best = u;
+            }
+            return best;
+        };
+        const long together = round_widths(count), apart = round_widths(1);
+        if (together > 0 && apart > 0 && together >= (long)count * apart) one_launch = false;
+    }
     if (one_launch) {
         // same argument checks as the plain entry, member by member, before anything is launched
         for (int i = 0; i < count; ++i) {

@@ -359,7 +359,8 @@ def test_cfg4_decomposition_sweep_at_its_real_shapes(dev, host, weight_layout):
     assert e_dec < 8e-3 and e_pre < 4e-3
 
 
-def test_cfg5_mixed_trace_at_its_real_shapes(dev, host):
+@pytest.mark.parametrize("packed_qkv", [False, True])
+def test_cfg5_mixed_trace_at_its_real_shapes(dev, host, packed_qkv):
     """BASELINE config 5, shortened: 12 Poisson arrivals at 16 requests/s through 4 stacked TP=2 layer shards, prompts uniform
     in [128, 1024] (rounded to 64), 32 decode tokens each, durations profiled on the device.  Every request must end with the
     hidden state of its sequential run -- with interleaving, and with interleaving plus batched decode steps (where a step over
@@ -367,7 +368,7 @@ def test_cfg5_mixed_trace_at_its_real_shapes(dev, host):
     c = CFG
     H, n = c["hidden"], 12
     m = host.Model(1, n + 1, 1024, c["heads_global"], c["d"], layer_num=4, world_size=c["world_size"], ffn_inner=c["ffn_global"], causal=True,
-                   fused=True, max_cache_len=1024 + 64, weight_layout=1, factor=8, seed=0)
+                   fused=True, max_cache_len=1024 + 64, weight_layout=1, factor=8, seed=0, packed_qkv=packed_qkv)
     s = host.Scheduler(m, schedule_deep=6, contention_factor=0.8, policy=host.POLICY_RESOURCE, axis=host.SPLIT_TOKEN_ROWS, seq_bucket=64,
                        ignore_num=0, pool_count=n, ctx_batch=1)
     s.profile(1, 128, 1024, 64, 3)
