@@ -472,9 +472,10 @@ int lg_gemm_fused_f16(int transa, int m, int n, int k, const void* A, int lda, c
     return gemm_f16_dispatch(g, transa == LG_OP_TILED ? W_TILED : (transa ? W_NK : W_KN), 1, (hipStream_t)stream);
 }
 
-int lg_gemm_fused_grouped_f16(int transa, int m, int n, int k, int count, const void* const* A, int lda, const void* B, int ldb,
-                              void* const* C, const int* ldc, int epilogue, const void* const* bias, int epi_arg0, int epi_arg1,
-                              int epi_arg2, void* stream) {
+// mode: -1 = choose the plan, 1 = one launch if the kernels allow it (a sub-group of a plan), 0 = member by member
+static int gemm_fused_grouped_f16_impl(int mode, int transa, int m, int n, int k, int count, const void* const* A, int lda, const void* B, int ldb,
+                                       void* const* C, const int* ldc, int epilogue, const void* const* bias, int epi_arg0, int epi_arg1,
+                                       int epi_arg2, void* stream) {
     if (count < 1 || count > LG_MAX_GROUP || !A || !C || !ldc || (epilogue != LG_EPI_NONE && !bias)) {
         set_error("gemm_fused_grouped_f16: count must be 1..%d and the pointer arrays non-null", LG_MAX_GROUP);
         return LG_ERR_INVALID;
@@ -511,6 +512,47 @@ int lg_gemm_fused_grouped_f16(int transa, int m, int n, int k, int count, const 
         };
         const long together = round_widths(count), apart = round_widths(1);
         if (together > 0 && apart > 0 && together >= (long)count * apart) one_launch = false;
+        // A third plan for groups that are many full rounds plus a remainder (Q, K, V of 4096 rows x 6144 features: 72 columns
+        // of 256-wide tiles, 16 columns to a round of 256 workgroups, 8 left over): the members before the last as one launch
+        // of whole rounds of the widest tile, the last member's leading features as whole rounds too, and its remaining features
+        // as one round of 128-wide tiles -- instead of six rounds of 192-wide tiles either way (4.6-6.6 % faster, measured).
+        // Only taken when every launch but the last is whole rounds; pieces are addressed like any feature sub-range.
+        int split_at = 0;   // feature at which the last member is cut (0: no such plan)
+        const bool range_ok = epilogue == LG_EPI_NONE || epilogue == LG_EPI_BIAS || epilogue == LG_EPI_BIAS_GELU ||
+                              (epilogue == LG_EPI_BIAS_HEADS && epi_arg1 > 0 && 256 % epi_arg1 == 0);
+        if (mode < 0 && range_ok && m % 256 == 0 && cus % tiles_m == 0 && (transa != LG_OP_TILED || lda == k)) {
+            const int cols = m / 256, per_round = cus / tiles_m, rem = (count * cols) % per_round;
+            if (rem > 0 && rem < cols && ((count - 1) * cols) % per_round == 0 && (cols - rem) % per_round == 0 && 2 * rem * tiles_m <= cus)
+                split_at = (cols - rem) * 256;
+        }
+        // LG_GEMM_GROUP=1|0 in the environment (read once) forces one launch / member by member: a measurement knob
+        static const int forced = [] { const char* e = getenv("LG_GEMM_GROUP"); return e ? atoi(e) : -1; }();
+        if (forced == 0) { one_launch = false; split_at = 0; }
+        else if (forced == 1) { one_launch = true; split_at = 0; }
+        if (mode == 0) one_launch = false;
+        else if (mode == 1) one_launch = true;
+        if (split_at > 0) {
+            int rc = count - 1 > 1 ? gemm_fused_grouped_f16_impl(1, transa, m, n, k, count - 1, A, lda, B, ldb, C, ldc, epilogue, bias, epi_arg0, epi_arg1,
+                                                                 epilogue == LG_EPI_BIAS_HEADS && epi_arg2 == 0 ? m / epi_arg1 : epi_arg2, stream)
+                                   : lg_gemm_fused_f16(transa, m, n, k, A[0], lda, B, ldb, C[0], ldc[0], epilogue, epilogue != LG_EPI_NONE ? bias[0] : nullptr,
+                                                       epi_arg0, epi_arg1, epi_arg2, stream);
+            if (rc) return rc;
+            const int last = count - 1;
+            const int heads_total = epilogue == LG_EPI_BIAS_HEADS ? (epi_arg2 ? epi_arg2 : m / epi_arg1) : epi_arg2;
+            const int cut[3] = {0, split_at, m};
+            for (int piece = 0; piece < 2; ++piece) {
+                const int f0 = cut[piece], f1 = cut[piece + 1];
+                // features [f0, f1) of the last member: rows f0.. of an [out, in] weight (row-major or in fragment blocks, where
+                // feature tile t starts 16 t k elements in), columns f0.. of an [in, out] one; heads f0 / d .. of a
+                // head-transposed destination, columns f0.. of a plain one
+                const int64_t w_off = transa == 0 ? (int64_t)f0 : (int64_t)f0 * (transa == LG_OP_TILED ? k : lda);
+                const int64_t c_off = epilogue == LG_EPI_BIAS_HEADS ? (int64_t)(f0 / epi_arg1) * ldc[last] * epi_arg1 : (int64_t)f0;
+                rc = lg_gemm_fused_f16(transa, f1 - f0, n, k, (const half_t*)A[last] + w_off, lda, B, ldb, (half_t*)C[last] + c_off, ldc[last], epilogue,
+                                       epilogue != LG_EPI_NONE ? (const void*)((const half_t*)bias[last] + f0) : nullptr, epi_arg0, epi_arg1, heads_total, stream);
+                if (rc) return rc;
+            }
+            return LG_OK;
+        }
     }
     if (one_launch) {
         // same argument checks as the plain entry, member by member, before anything is launched
@@ -553,6 +595,12 @@ int lg_gemm_fused_grouped_f16(int transa, int m, int n, int k, int count, const 
         if (rc) return rc;
     }
     return LG_OK;
+}
+
+int lg_gemm_fused_grouped_f16(int transa, int m, int n, int k, int count, const void* const* A, int lda, const void* B, int ldb,
+                              void* const* C, const int* ldc, int epilogue, const void* const* bias, int epi_arg0, int epi_arg1,
+                              int epi_arg2, void* stream) {
+    return gemm_fused_grouped_f16_impl(-1, transa, m, n, k, count, A, lda, B, ldb, C, ldc, epilogue, bias, epi_arg0, epi_arg1, epi_arg2, stream);
 }
 
 int lg_gemm_fused_grouped_rows_f16(int transa, int m, int n, int k, int count, const void* const* A, int lda, const void* B, int ldb,

@@ -527,7 +527,7 @@ def timed_only(capi, host, args, fused):
     B, S, H = c["batch"], c["seq"], c["hidden"]
     model = host.Model(capi.F16, 32, S, c["heads_global"], c["d"], layer_num=1, world_size=c["world_size"], ffn_inner=c["ffn_global"],
                        norm_mode=host.POST_NORESID, causal=True, fused=fused, max_cache_len=CFG3["cache_len"] + 32 if fused else 0,
-                       weight_layout=args.weight_layout, seed=0)
+                       weight_layout=args.weight_layout, seed=0, packed_qkv=fused and not args.separate_qkv)
     stream = model.stream
     if args.decode:
         Bd, L = CFG3["batch"], CFG3["cache_len"]
@@ -565,10 +565,10 @@ def main():
     ap.add_argument("--cfg5", action="store_true", help="run the full mixed request trace (BASELINE config 5; minutes) instead of the short record")
     ap.add_argument("--cfg5-requests", type=int, default=60)
     ap.add_argument("--cfg5-runs", type=int, default=3)
-    ap.add_argument("--cfg5-separate-qkv", action="store_true",
-                    help="config 5 with three separate Q / K / V weights instead of the packed [H, 3 Hl] one of GLM checkpoints (with the "
-                         "packed weight the three projections are one launch-vector entry, which the library runs as one grouped launch "
-                         "where that fills the chip better: prompts of 384-768 tokens prefill 7-13 %% faster)")
+    ap.add_argument("--separate-qkv", "--cfg5-separate-qkv", dest="separate_qkv", action="store_true",
+                    help="three separate Q / K / V weights (9 launch-vector entries per fused layer) instead of the packed [H, 3 Hl] one of GLM "
+                         "checkpoints (7 entries: the three projections are one entry, for which the library picks the launches that fill the "
+                         "rounds of workgroups best: the cfg2 batch 1.3 %% faster, prompts of 384-768 tokens 7-13 %%)")
     ap.add_argument("--corun-variants", action="store_true",
                     help="GEMM tile width (chosen by shape / 256 x 128) x CU share: prefill MFMA kernels next to decode steps, one JSON line")
     ap.add_argument("--corun-one", type=int, default=0, help=argparse.SUPPRESS)
@@ -620,7 +620,7 @@ def main():
     if args.kernel_only:
         model = host.Model(capi.F16, 32, S, c["heads_global"], c["d"], layer_num=1, world_size=c["world_size"], ffn_inner=c["ffn_global"],
                            norm_mode=host.POST_NORESID, causal=True, fused=fused, max_cache_len=CFG3["cache_len"] + 32 if fused else 0,
-                           weight_layout=args.weight_layout, seed=0)
+                           weight_layout=args.weight_layout, seed=0, packed_qkv=fused and not args.separate_qkv)
         x = torch.empty(M, H, device="cuda", dtype=torch.float16)
         capi.call("lg_fill_normal_f16", x.data_ptr(), x.numel(), 0, 99, 0.0, 1.0, None)
         y = torch.empty_like(x)
@@ -628,11 +628,13 @@ def main():
         kernel_only(args, capi, host, model, x, y, B, S, H, model.stream)
         return
 
-    model, x, y, res = time_layer(capi, host, args.weight_layout, fused, args.steps, args.warmup)
+    packed = fused and not args.separate_qkv
+    model, x, y, res = time_layer(capi, host, args.weight_layout, fused, args.steps, args.warmup, packed_qkv=packed)
     ms_per_step, kernels = res["ms_per_step"], res["kernels"]
     fl = gemm_flops_cfg2()
     label_flops = {"q_gemm": fl["q"], "k_gemm": fl["k"], "v_gemm": fl["v"], "out_proj": fl["out"], "ffn1": fl["ffn1"], "ffn2": fl["ffn2"],
-                   "q_gemm+bias+heads": fl["q"], "k_gemm+bias+heads": fl["k"], "v_gemm+bias+heads": fl["v"], "ffn1+bias+gelu": fl["ffn1"]}
+                   "q_gemm+bias+heads": fl["q"], "k_gemm+bias+heads": fl["k"], "v_gemm+bias+heads": fl["v"], "ffn1+bias+gelu": fl["ffn1"],
+                   "qkv_gemm+bias+heads": fl["q"] + fl["k"] + fl["v"]}
     gemm_ms = 0.0
     gemm_fl = 0.0
     for k in kernels:
@@ -686,7 +688,9 @@ def main():
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": "cfg2 prefill: hidden 12288, 48/96 heads x 128, FFN 16384/32768, batch 8 x seq 512, causal; "
-                               + ("fused assembly (9 launches/layer)" if fused else "reference-shaped assembly (14 launches/layer)")
+                               + (("fused assembly, Q / K / V as one packed weight (7 launch-vector entries/layer)" if packed else
+                                   "fused assembly, separate Q / K / V weights (9 launch-vector entries/layer)") if fused
+                                  else "reference-shaped assembly (14 launches/layer)")
                                + "; weights stored " + {0: "[in, out]", 1: "[out, in]", 2: "[out, in] in 16 x 32 fragment blocks"}[args.weight_layout]},
         "tokens_per_s": round(M / (ms_per_step * 1e-3), 1),
         "roofline": roofline,
@@ -713,7 +717,7 @@ def main():
     for other in (0, 1, 2):
         if other == args.weight_layout:
             continue
-        m2, x2, y2, r2 = time_layer(capi, host, other, fused, max(5, args.steps // 2), 2)
+        m2, x2, y2, r2 = time_layer(capi, host, other, fused, max(5, args.steps // 2), 2, packed_qkv=packed)
         out[names[other][0]] = {
             "weights": names[other][1], "ms_per_layer_shard_prefill": round(r2["ms_per_step"], 4),
             "ms_per_layer_shard_decode": r2["decode"]["ms_per_layer_shard"] if r2["decode"] else None,
@@ -732,12 +736,15 @@ def main():
         del m3, x3, y3
         torch.cuda.empty_cache()
     if fused:
-        # the same shard with the Q, K and V projections stored as ONE [H, 3 Hl] weight (the layout of GLM checkpoints): the three
-        # GEMM entries become one grouped launch whose 18432 features fill six full rounds of 256 x 192 tiles
-        m4, x4, y4, r4 = time_layer(capi, host, args.weight_layout, True, max(5, args.steps // 2), 2, packed_qkv=True)
-        out["packed_qkv"] = {"launches_per_layer": len(r4["kernels"]), "ms_per_layer_shard_prefill": round(r4["ms_per_step"], 4),
-                             "ms_per_layer_shard_decode": r4["decode"]["ms_per_layer_shard"] if r4["decode"] else None,
-                             "kernels_ms": {"%d:%s" % (k["idx"], k["kernel"]): k["ms"] for k in r4["kernels"]}}
+        # the same shard with the other storage of the Q, K and V projections: packed as ONE [H, 3 Hl] weight (the layout of GLM
+        # checkpoints) they are one launch-vector entry, for which the library picks the launches that fill the rounds of workgroups
+        # best (at cfg2: Q and K as one launch of three full rounds, V as a full round and a round of 128-wide tiles); stored
+        # separately they are three entries of two rounds of 192-wide tiles each
+        m4, x4, y4, r4 = time_layer(capi, host, args.weight_layout, True, max(5, args.steps // 2), 2, packed_qkv=not packed)
+        out["separate_qkv" if packed else "packed_qkv"] = {
+            "launches_per_layer": len(r4["kernels"]), "ms_per_layer_shard_prefill": round(r4["ms_per_step"], 4),
+            "ms_per_layer_shard_decode": r4["decode"]["ms_per_layer_shard"] if r4["decode"] else None,
+            "kernels_ms": {"%d:%s" % (k["idx"], k["kernel"]): k["ms"] for k in r4["kernels"]}}
         del m4, x4, y4
         torch.cuda.empty_cache()
     out["weight_relay_at_load"] = bench_weight_relay(capi, host, args.weight_layout)
@@ -756,10 +763,10 @@ def main():
             out["cfg4_split_forced"] = bench_cfg4(capi, host, args.weight_layout, factors=(8,), shares=(0, 128), repeats=3, decode_steps=4)
         torch.cuda.empty_cache()
         if args.cfg5:
-            out["cfg5"] = bench_cfg5(capi, host, args.weight_layout, args.cfg5_requests, runs=args.cfg5_runs, packed_qkv=not args.cfg5_separate_qkv)
+            out["cfg5"] = bench_cfg5(capi, host, args.weight_layout, args.cfg5_requests, runs=args.cfg5_runs, packed_qkv=not args.separate_qkv)
         else:
             out["cfg5"] = bench_cfg5(capi, host, args.weight_layout, 40, rates=(16.0, 32.0), shares=(128,), runs=3, short=True,
-                                     packed_qkv=not args.cfg5_separate_qkv)
+                                     packed_qkv=not args.separate_qkv)
     print(json.dumps(out))
 
 

@@ -348,14 +348,15 @@ def test_grouped_qkv_gemm_equals_three_plain_calls(dev, po, M, transa):
 
 
 @pytest.mark.parametrize("transa", [0, 1])
-@pytest.mark.parametrize("B,S,h,d", [(4, 128, 6, 128), (2, 384, 4, 64), (3, 100, 8, 96), (8, 512, 16, 128)])
+@pytest.mark.parametrize("B,S,h,d", [(4, 128, 6, 128), (2, 384, 4, 64), (3, 100, 8, 96), (8, 512, 16, 128), (8, 512, 48, 128)])
 def test_grouped_qkv_gemm_on_a_packed_weight_prefill(dev, po, transa, B, S, h, d):
     """Q, K and V of a prefill as one grouped call on the column blocks of ONE packed [K, 3 N] weight (the pointers of the
     members are offsets into it, lda is the packed matrix's): with more than 256 token rows the pipelined kernel runs the
     group as one launch where the members' tiles side by side need fewer rounds of workgroups than each member's own, else
     member by member (the last shape: 4096 rows x 2048 features fill one round per member with 128-wide tiles, three
-    members together would need three); either way the result must equal three plain fused calls bit for bit (same tiles,
-    same k order) and the oracle.  q goes to [B, h, S, d], k and v into cache-shaped buffers with more rows than S."""
+    members together would need three; the one after it, 4096 rows x 6144 features, runs as Q and K in one launch and V in two
+    pieces, whole rounds of 256-wide tiles and a last round of 128-wide ones); either way the result must equal three plain
+    fused calls bit for bit (same tiles, same k order) and the oracle.  q goes to [B, h, S, d], k and v into cache-shaped buffers with more rows than S."""
     import ctypes as C
     K, rows = 512, S + 24
     N, M = h * d, B * S

@@ -143,10 +143,12 @@ def test_geglu_epilogue_on_tiled_weights(dev, po, M, F, K):
     assert max_rel_err(dev.down(dY), ref) < 4e-3
 
 
-@pytest.mark.parametrize("M", [1, 8, 32, 64, 300])
+@pytest.mark.parametrize("M", [1, 8, 32, 64, 300, 4096])
 def test_grouped_qkv_on_tiled_weights_equals_three_plain_calls(dev, po, M):
     """Q, K and V as one grouped call on three tiled weights -- and on the three row blocks of ONE packed tiled weight -- against
-    three plain calls on the same weights; per-row destinations (rows entry) at decode sizes."""
+    three plain calls on the same weights; per-row destinations (rows entry) at decode sizes.  4096 rows x 6144 features is the
+    shape the library runs as Q and K in one launch + V in two pieces (whole rounds of 256-wide tiles and one round of 128-wide
+    ones): the pieces must land exactly where the plain calls put them."""
     h, d, K, rows, past = 48, 128, 2048, 6, 3
     N = h * d
     S = 1 if M <= 64 else M
@@ -183,6 +185,8 @@ def test_grouped_qkv_on_tiled_weights_equals_three_plain_calls(dev, po, M):
         got = dev.down(grouped[t])[:, :, (past if t else 0):(past if t else 0) + S]
         assert max_rel_err(got, ref) < 2e-3
         assert max_rel_err(dev.down(grouped[t]), dev.down(plain[t])) < 1e-3
+        if M > 256:
+            assert np.array_equal(dev.down(grouped[t]), dev.down(plain[t]))     # the pipelined kernel: same bits whatever the plan
     if M <= 64:
         # every token row to its own (slot, position) of the K / V destinations
         slots = [(5 * r + 2) % M for r in range(M)]
