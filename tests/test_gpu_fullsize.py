@@ -51,13 +51,17 @@ def test_full_size_gemm_one_hot_rows_select_weight_rows(dev, transa, N, K):
     assert torch.equal(Y, expect.half())
 
 
-@pytest.mark.parametrize("weight_layout", [0, 1, 2])
-def test_full_size_layer_batch_independence_and_oracle_slice(dev, po, host, weight_layout):
+@pytest.mark.parametrize("weight_layout,packed_qkv", [(0, False), (1, False), (2, False), (2, True), (0, True)])
+def test_full_size_layer_batch_independence_and_oracle_slice(dev, po, host, weight_layout, packed_qkv):
     """The cfg2 prefill layer shard (fused assembly, causal) on the full batch: every sequence's result equals, bit for
-    bit, the result of running that sequence alone; one sequence is checked against the CPU oracle.  Both weight layouts:
-    0 stores weights [in, out] as the reference's cuBLAS calls imply (linear.h:47-49,99-101), 1 stores them [out, in]."""
+    bit, the result of running that sequence alone; one sequence is checked against the CPU oracle.  Every weight layout:
+    0 stores weights [in, out] as the reference's cuBLAS calls imply (linear.h:47-49,99-101), 1 stores them [out, in], 2 in
+    fragment blocks; with the packed Q/K/V weight (the assembly the bench times) the three projections are one entry that
+    the library runs as Q and K in one launch and V in two pieces on the full batch, and as one grouped launch on a
+    sequence alone -- still the same bits."""
     m = host.Model(1, B, S, 96, D, layer_num=1, world_size=2, ffn_inner=2 * F, norm_mode=0, causal=True, fused=True,
-                   weight_layout=weight_layout, seed=0)
+                   weight_layout=weight_layout, seed=0, packed_qkv=packed_qkv)
+    assert m.kernels_per_layer() == (7 if packed_qkv else 9)
     x = po.fill_normal(M * H, 0, 99, 0.0, 1.0, 1).reshape(M, H)
     dx = dev.up(x, 1)
     dy = dev.empty((M, H), 1)
@@ -73,6 +77,10 @@ def test_full_size_layer_batch_independence_and_oracle_slice(dev, po, host, weig
     # oracle on sequence 5 (the weights are downloaded, so both sides see the same bits)
     params = m.download_params()
     w = {k[len("layer0."):]: v for k, v in params.items() if k.startswith("layer0.")}
+    if "wqkv" in w:     # the oracle takes the three column blocks of the packed projection
+        for i, n in enumerate("qkv"):
+            w["w" + n] = np.ascontiguousarray(w["wqkv"][:, i * HL:(i + 1) * HL])
+            w["b" + n] = np.ascontiguousarray(w["bqkv"][i * HL:(i + 1) * HL])
     shape = dict(batch=1, seq=S, hidden=H, head_num=48, size_per_head=D, ffn_inner=F, causal=1, norm_mode=0, dtype=1)
     ref = po.encoder_forward(shape, w, x[5 * S:6 * S])
     got = dy[5 * S:6 * S].float().cpu().numpy()
